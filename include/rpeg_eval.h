@@ -1,0 +1,188 @@
+/*
+ * rpeg_eval.h - C ABI of the MI355X batched plan evaluator.
+ *
+ * The reference (spcl/RPEG) is pure Python and has no FFI; its drop-in boundary is the Python
+ * call `search.evaluate._eval_worker / evaluate_cached` (RPEG/search/evaluate.py:329-442), which
+ * the simulated-annealing driver maps over the K_x candidates of one step
+ * (RPEG/search/optimizer.py:793-798).  This library replaces that map by one batched call on the
+ * GPU.  All entry points use plain pointers and sizes; plan tensors and outputs are DEVICE
+ * pointers (structure-of-arrays, see rpeg_plan_soa_t), everything else is host memory.
+ *
+ * Status codes: 0 ok, negative = error (text via rpeg_last_error).
+ */
+#ifndef RPEG_EVAL_H
+#define RPEG_EVAL_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RPEG_ABI_VERSION 1
+
+#define RPEG_MAX_V 6       /* template vertices per structure                */
+#define RPEG_MAX_E 9       /* within-step data edges                          */
+#define RPEG_MAX_PUB 2     /* publication edges                               */
+#define RPEG_MAX_PAIR 4    /* consecutive same-model vertex pairs             */
+#define RPEG_MAX_REL 13    /* vertex pairs whose relation decides the lowering */
+#define RPEG_MAX_PH 6      /* generation phases (quantiles)                   */
+#define RPEG_MAX_SPLIT 7   /* split variants: 0 = unsplit, j = quantiles[j-1:] */
+#define RPEG_MAX_MODEL 5
+#define RPEG_MAX_STRUCT 2
+#define RPEG_FIELDS 10     /* per-vertex plan fields: dp pp tp mb o_r o_n o_g e_r e_n e_g */
+
+enum { RPEG_ROLE_GEN = 0, RPEG_ROLE_INF = 1, RPEG_ROLE_TRAIN = 2 };
+enum { RPEG_MODEL_ACTOR = 0, RPEG_MODEL_CRITIC = 1, RPEG_MODEL_REFERENCE = 2, RPEG_MODEL_REWARD = 3,
+       RPEG_MODEL_AC_SHARE = 4 };
+
+/* need flags of a relation pair */
+enum { RPEG_NEED_DISJ = 1, RPEG_NEED_PI = 2 };
+
+/* mask bits written per plan */
+enum {
+  RPEG_MASK_VALID = 1,     /* integer validity rules of is_valid (evaluate.py:172-196) hold   */
+  RPEG_MASK_STALE_OK = 2,  /* stale_publication_layout_valid (evaluate.py:115-140)            */
+  RPEG_MASK_MEM_OK = 4,    /* no device peak above capacity (memory.py:864-887)               */
+  RPEG_MASK_ERROR = 8      /* the reference would raise (division by zero, cycle) or an engine
+                              limit was hit; the numeric outputs of this plan are NaN           */
+};
+
+/* eval flags */
+enum {
+  RPEG_GATE_STALE = 1      /* score := 0 when the stale-layout rule fails (evaluate_cached, :372-374);
+                              without it the score is what _eval_worker returns (:406-442)      */
+};
+
+/* hardware parameter indices (RPEG/model/hardware.py:17-68, in field order) */
+enum {
+  RPEG_HW_FLOPS = 0, RPEG_HW_MEM, RPEG_HW_BW,
+  RPEG_HW_A_COLL_G, RPEG_HW_B_COLL_G, RPEG_HW_A_COLL_N, RPEG_HW_B_COLL_N, RPEG_HW_A_COLL_R, RPEG_HW_B_COLL_R,
+  RPEG_HW_A_P2P_G, RPEG_HW_B_P2P_G, RPEG_HW_A_P2P_N, RPEG_HW_B_P2P_N, RPEG_HW_A_P2P_R, RPEG_HW_B_P2P_R,
+  RPEG_HW_M_HALF, RPEG_HW_K_HALF, RPEG_HW_DECODE_EFF, RPEG_HW_NG_CONST, RPEG_HW_NG_SCALE, RPEG_HW_NG_BCAL,
+  RPEG_HW_SCALE_GEN, RPEG_HW_SCALE_INF, RPEG_HW_SCALE_TRAIN, RPEG_HW_ACT_OVERHEAD, RPEG_HW_W_COMM_SCALE,
+  RPEG_HW_RESHARD_SCALE, RPEG_HW_COUNT
+};
+
+typedef struct rpeg_model_s {
+  int32_t L, d, d_ff, V, sb, kind;
+  int64_t w_layer;        /* 4 d^2 + 2 d d_ff                                        */
+  int64_t params_formula; /* L*w_layer + V*d (cost.py:188)                           */
+  int64_t n_params;       /* ModelSuite.n_params (models.py:51-82): lowering payloads */
+} rpeg_model_t;
+
+/* plan-independent constants of one operator-node variant, evaluated on the host with exact
+   Python integer/float semantics (cost.py:481-535, lower.py:288-327) */
+typedef struct rpeg_opconst_s {
+  double W;          /* float(_work_cost(node))                                  */
+  double W_prefill;  /* float(prefill work) for generation nodes with a prefill   */
+  double avg_past;   /* generation: S + t_start + steps/2, or S + T/2 unsplit     */
+  int32_t n_eff;     /* _effective_batch(node)                                    */
+  int32_t steps;     /* decode steps of a generation node                         */
+  int32_t prefill;   /* generation node includes the prefill                      */
+  int32_t sub;       /* 1: quantile sub-node, 0: unsplit node                     */
+} rpeg_opconst_t;
+
+typedef struct rpeg_vertex_s {
+  int32_t role, model, topo_idx, tau_slot; /* topo_idx: rank of the id among sorted ids (scheduler.py:385-397) */
+  rpeg_opconst_t unsplit;
+  rpeg_opconst_t sub[RPEG_MAX_SPLIT][RPEG_MAX_PH];
+} rpeg_vertex_t;
+
+typedef struct rpeg_edge_s {
+  int32_t src, dst, is_weight, gen_inf;
+  int64_t full_bytes;                              /* container bytes                   */
+  int64_t sub_bytes[RPEG_MAX_SPLIT][RPEG_MAX_PH];  /* max(1,int(full*n_seq/BK)), lower.py:562-563 */
+} rpeg_edge_t;
+
+typedef struct rpeg_pub_s { int32_t src, dst, model, tau_slot; } rpeg_pub_t;
+typedef struct rpeg_pair_s { int32_t u, v, model, tau_slot, reach, pad; } rpeg_pair_t;
+typedef struct rpeg_rel_s { int32_t u, v, flags, pad; } rpeg_rel_t;
+
+typedef struct rpeg_struct_s {
+  int32_t n_vertex, n_edge, n_pub, n_pair, n_rel, n_tau;
+  rpeg_vertex_t vertex[RPEG_MAX_V];
+  rpeg_edge_t edge[RPEG_MAX_E];
+  rpeg_pub_t pub[RPEG_MAX_PUB];
+  rpeg_pair_t pair[RPEG_MAX_PAIR];     /* within_step_priors over the LIFO topological order (lower.py:135-220) */
+  rpeg_rel_t rel[RPEG_MAX_REL];
+  uint8_t reach[RPEG_MAX_V][RPEG_MAX_V];  /* transitive closure of data edges (lower.py:170-193) */
+  uint8_t trainable[RPEG_MAX_MODEL + 3];
+} rpeg_struct_t;
+
+typedef struct rpeg_phase_s { int32_t n_active, n_seqs, steps, t_start, prefill, pad; } rpeg_phase_t;
+
+typedef struct rpeg_problem_s {
+  int32_t abi_version;
+  int32_t n_struct, n_split, K_eval;
+  int32_t R, N, G;
+  int32_t B, K, S, T;
+  int32_t optimizer_stage, ckpt, max_groups;
+  int32_t n_phase[RPEG_MAX_SPLIT];
+  int32_t pad;
+  rpeg_phase_t phase[RPEG_MAX_SPLIT][RPEG_MAX_PH];
+  double hw[RPEG_HW_COUNT];
+  double cap;             /* (1 - eps_rt) * memory_per_gpu (memory.py:291-298)          */
+  double group_overhead;  /* worker_overhead_bytes + semantic_activation_cache_bytes      */
+  double score_num;       /* float(K_eval * B*K*(S+T)) (evaluate.py:288, trace.py:40-51)  */
+  rpeg_model_t model[RPEG_MAX_MODEL];
+  rpeg_struct_t st[RPEG_MAX_STRUCT];
+} rpeg_problem_t;
+
+/* Candidate plans, structure of arrays, DEVICE memory.
+   vert[(slot*RPEG_FIELDS + f) * stride + i]  field f of vertex slot `slot` of plan i
+   head[h * stride + i]                       h = 0 structure, 1 split index, 2 tau slot 0, 3 tau slot 1 */
+typedef struct rpeg_plan_soa_s {
+  const int16_t* vert;
+  const uint8_t* head;
+  uint64_t stride;
+} rpeg_plan_soa_t;
+
+typedef struct rpeg_engine_s rpeg_engine_t;
+
+/* Creates an engine for one problem on the current HIP device.  Replaces the per-call construction
+   of NodeCostModel / NodeMemoryModel / template graph in evaluate() (evaluate.py:261-287). */
+int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out);
+void rpeg_engine_destroy(rpeg_engine_t* e);
+const char* rpeg_last_error(const rpeg_engine_t* e);
+
+/* Evaluates n plans: the batched form of Pool.map(_eval_worker, ...) (optimizer.py:793-798).
+   makespan: Trace.makespan() (trace.py:31-38); peak: largest per-device peak in bytes
+   (memory.py:608-841); score: throughput times the soft OOM penalty (evaluate.py:288, 396-401);
+   mask: RPEG_MASK_* bits.  All four are device arrays of n elements; any may be NULL.
+   `stream` is a hipStream_t (NULL = default stream).  The call is synchronous with respect to
+   the host only where it must read back the list of new lowering classes. */
+int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
+                    double* makespan, double* peak, double* score, uint8_t* mask, void* stream);
+
+/* Single-node durations and isolated peaks: the batched form of the candidate-directory loop
+   (RPEG/search/moves.py:532-549): for strategy i, time = NodeCostModel.time(mock node) and
+   peak = NodeMemoryModel.peak_bytes(mock node) of vertex `vertex` of structure `structure` placed at
+   origin (0,0,0).  strat[(f)*stride + i], f = dp pp tp mb r_ext n_ext g_ext (int16, device). */
+int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t vertex,
+                       const int16_t* strat, uint64_t stride, double* time, double* peak, void* stream);
+
+/* Start/finish time of every lowered node of ONE plan (host arrays of capacity cap), in the
+   reference's node order; what move_gen reads from Trace (moves.py:590-619).  Returns the node
+   count, or a negative status. */
+int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4,
+                    double* start, double* finish, int32_t* node_kind, int32_t* node_vertex,
+                    int32_t* node_step, int32_t cap);
+
+/* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
+   by this call, [2] wave tasks, [3] kernel-C dynamic LDS bytes, [4] workspace bytes. */
+int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
+
+/* Kernel time of the dominant kernel in the last rpeg_eval_batch call, measured with HIP events on
+   the launch stream (milliseconds); negative when timing was not enabled. */
+int rpeg_engine_set_timing(rpeg_engine_t* e, int32_t enabled);
+double rpeg_engine_last_kernel_ms(const rpeg_engine_t* e);
+
+/* exp() as the host C library of an FMA-capable x86-64 computes it, evaluated on the device for n
+   inputs; exported for the parity test of the OOM penalty. */
+int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
