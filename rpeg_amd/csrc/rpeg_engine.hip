@@ -1,0 +1,466 @@
+// rpeg_engine.hip - HIP kernels and C ABI of the batched plan evaluator (gfx950).
+//
+// Pipeline of rpeg_eval_batch:
+//   k_signature   one thread per plan: integer validity gate, 64-bit class signature
+//   host          new signatures are lowered once into class blobs (rpeg_lower.h) and cached in
+//                 the engine; plans are ordered by class so that the lanes of a wavefront walk the
+//                 same graph tables
+//   k_eval        one thread per plan: durations of the class's slots (fp64 cost model), ranks,
+//                 list scheduling, per-device memory peaks, score.  Per-plan state lives in a
+//                 workspace laid out [row][lane] per wavefront (coalesced whenever lanes agree on
+//                 the row); the ready list lives in LDS, [entry][lane].
+//
+// Build: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off (no fused multiply-add may be formed:
+// the scores must equal the reference's Python floats bit for bit).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "rpeg_lower.h"
+#include "rpeg_plan.h"
+
+using namespace rpeg;
+
+namespace {
+
+constexpr int WAVE = 64;
+constexpr int READY_CAP = 64;  // ready-list entries per plan (LDS); overflow sets RPEG_MASK_ERROR
+
+#define HIP_TRY(e, call)                                                                   \
+  do {                                                                                     \
+    hipError_t _s = (call);                                                                \
+    if (_s != hipSuccess) {                                                                \
+      (e)->err = std::string(#call) + ": " + hipGetErrorString(_s);                        \
+      return -2;                                                                           \
+    }                                                                                      \
+  } while (0)
+
+struct DevMem {
+  double* t;       // time rows, pre-offset by lane
+  double* r;       // rank rows
+  double* d;       // duration rows
+  uint8_t* deg;    // in-degree rows
+  uint16_t* ready; // LDS, pre-offset by lane
+  double* tr_start;
+  double* tr_finish;
+  __device__ double& time(int i) { return t[(size_t)i * WAVE]; }
+  __device__ double& rank(int i) { return r[(size_t)i * WAVE]; }
+  __device__ uint8_t& indeg(int i) { return deg[(size_t)i * WAVE]; }
+  __device__ double dur(int s) const { return d[(size_t)s * WAVE]; }
+  __device__ void set_dur(int s, double v) { d[(size_t)s * WAVE] = v; }
+  __device__ uint16_t& rd_node(int j) { return ready[j * WAVE]; }
+  __device__ void on_schedule(int v, double s, double f) {
+    if (tr_start) { tr_start[v] = s; tr_finish[v] = f; }
+  }
+};
+
+__host__ __device__ inline size_t wave_ws_bytes(uint32_t nodes, uint32_t slots) {
+  size_t b = (size_t)WAVE * (16ull * nodes + 8ull * slots + nodes);
+  return (b + 255) & ~size_t(255);
+}
+
+__global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
+                            const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig,
+                            double* makespan, double* peak, double* score, uint8_t* mask) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  PlanHead h = load_head(head, stride, i);
+  VPlan a[RPEG_MAX_V];
+  const int nv = (h.structure < P->n_struct) ? P->st[h.structure].n_vertex : 0;
+  for (int v = 0; v < RPEG_MAX_V; ++v)
+    if (v < nv) load_vertex(vert, stride, i, v, &a[v]);
+  if (nv == 0 || !plan_valid(*P, h, a)) {
+    sig[i] = SIG_INVALID;
+    const double nan = __builtin_nan("");
+    if (makespan) makespan[i] = nan;
+    if (peak) peak[i] = nan;
+    if (score) score[i] = nan;
+    if (mask) mask[i] = 0;
+    return;
+  }
+  sig[i] = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
+}
+
+__global__ __launch_bounds__(WAVE) void k_eval(const rpeg_problem_t* __restrict__ P, uint64_t n_sorted,
+                                               const int16_t* __restrict__ vert, const uint8_t* __restrict__ head,
+                                               uint64_t stride, const uint32_t* __restrict__ perm,
+                                               const uint32_t* __restrict__ cls_off, const uint8_t* __restrict__ pool,
+                                               uint8_t* __restrict__ ws, uint32_t ws_nodes, uint32_t ws_slots,
+                                               uint32_t flags, double* makespan, double* peak, double* score,
+                                               uint8_t* mask, double* tr_start, double* tr_finish) {
+  extern __shared__ uint16_t lds_ready[];
+  const int lane = threadIdx.x;
+  const uint64_t n_waves = (n_sorted + WAVE - 1) / WAVE;
+  uint8_t* base = ws + (size_t)blockIdx.x * wave_ws_bytes(ws_nodes, ws_slots);
+  DevMem mem;
+  mem.t = (double*)base + lane;
+  mem.r = (double*)base + (size_t)ws_nodes * WAVE + lane;
+  mem.d = (double*)base + 2 * (size_t)ws_nodes * WAVE + lane;
+  mem.deg = base + 8 * (2 * (size_t)ws_nodes + ws_slots) * WAVE + lane;
+  mem.ready = lds_ready + lane;
+  mem.tr_start = tr_start;
+  mem.tr_finish = tr_finish;
+  for (uint64_t w = blockIdx.x; w < n_waves; w += gridDim.x) {
+    const uint64_t t = w * WAVE + lane;
+    if (t >= n_sorted) continue;
+    const uint64_t i = perm[t];
+    const ClassView cv = class_view(pool + cls_off[t]);
+    PlanHead h = load_head(head, stride, i);
+    VPlan a[RPEG_MAX_V];
+    const int nv = P->st[h.structure].n_vertex;
+    for (int v = 0; v < RPEG_MAX_V; ++v)
+      if (v < nv) load_vertex(vert, stride, i, v, &a[v]);
+    PlanOut o = eval_plan(*P, cv, h, a, mem, READY_CAP, flags);
+    if (makespan) makespan[i] = o.makespan;
+    if (peak) peak[i] = o.peak;
+    if (score) score[i] = o.score;
+    if (mask) mask[i] = o.mask;
+  }
+}
+
+__global__ void k_op_time(const rpeg_problem_t* __restrict__ P, uint64_t n, int structure, int vertex,
+                          const int16_t* __restrict__ strat, uint64_t stride, double* time, double* peak) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const rpeg_vertex_t& vx = P->st[structure].vertex[vertex];
+  VPlan a;
+  a.dp = strat[0 * stride + i]; a.pp = strat[1 * stride + i]; a.tp = strat[2 * stride + i]; a.mb = strat[3 * stride + i];
+  a.o[0] = a.o[1] = a.o[2] = 0;
+  a.e[0] = strat[4 * stride + i]; a.e[1] = strat[5 * stride + i]; a.e[2] = strat[6 * stride + i];
+  bool zd = a.dp < 1 || a.pp < 1 || a.tp < 1 || a.mb < 1 || a.e[2] < 1;
+  if (zd) {
+    if (time) time[i] = __builtin_nan("");
+    if (peak) peak[i] = __builtin_nan("");
+    return;
+  }
+  if (time) {
+    double t = op_time(*P, vx, vx.unsplit, a, &zd);
+    time[i] = zd ? __builtin_nan("") : t;
+  }
+  if (peak) peak[i] = isolated_peak(vx, vertex_memory(*P, vx, a));
+}
+
+__global__ void k_exp(uint64_t n, const double* x, double* y) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = exp_libm(x[i]);
+}
+
+}  // namespace
+
+struct rpeg_engine_s {
+  rpeg_problem_t P;
+  rpeg_problem_t* dP = nullptr;
+  int device = 0;
+  std::string err;
+  // lowering classes
+  std::unordered_map<uint64_t, uint32_t> class_off;  // signature -> byte offset in the pool
+  std::vector<uint8_t> pool;
+  uint8_t* d_pool = nullptr;
+  size_t d_pool_cap = 0, d_pool_used = 0;
+  uint32_t max_nodes = 1, max_slots = 1;
+  // per-batch buffers
+  size_t cap_n = 0;
+  uint64_t* d_sig = nullptr;
+  uint64_t* h_sig = nullptr;
+  uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_perm = nullptr, *h_cls = nullptr;
+  uint8_t* d_ws = nullptr;
+  size_t ws_cap = 0;
+  // timing / stats
+  bool timing = false;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  double last_ms = -1.0;
+  uint64_t stats[5] = {0, 0, 0, 0, 0};
+  int n_cu = 256;
+};
+
+static int ensure_batch(rpeg_engine_t* e, size_t n) {
+  if (n <= e->cap_n) return 0;
+  size_t cap = std::max<size_t>(n, 4096);
+  if (e->d_sig) { hipFree(e->d_sig); hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_sig); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  e->cap_n = 0;
+  HIP_TRY(e, hipMalloc(&e->d_sig, cap * 8));
+  HIP_TRY(e, hipMalloc(&e->d_perm, cap * 4));
+  HIP_TRY(e, hipMalloc(&e->d_cls, cap * 4));
+  HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
+  HIP_TRY(e, hipHostMalloc(&e->h_perm, cap * 4));
+  HIP_TRY(e, hipHostMalloc(&e->h_cls, cap * 4));
+  e->cap_n = cap;
+  return 0;
+}
+
+static int ensure_pool(rpeg_engine_t* e, hipStream_t s) {
+  if (e->pool.size() > e->d_pool_cap) {
+    size_t cap = std::max<size_t>(e->pool.size() * 2, 1 << 20);
+    uint8_t* np = nullptr;
+    HIP_TRY(e, hipMalloc(&np, cap));
+    HIP_TRY(e, hipStreamSynchronize(s));
+    if (e->d_pool) hipFree(e->d_pool);
+    e->d_pool = np;
+    e->d_pool_cap = cap;
+    e->d_pool_used = 0;
+  }
+  if (e->pool.size() > e->d_pool_used) {
+    HIP_TRY(e, hipMemcpyAsync(e->d_pool + e->d_pool_used, e->pool.data() + e->d_pool_used,
+                              e->pool.size() - e->d_pool_used, hipMemcpyHostToDevice, s));
+    // the host vector may reallocate on the next insertion: finish the copy first
+    HIP_TRY(e, hipStreamSynchronize(s));
+    e->d_pool_used = e->pool.size();
+  }
+  return 0;
+}
+
+// returns the pool offset of the class of `sig`, lowering it on first sight; -1 on failure
+static int64_t class_offset(rpeg_engine_t* e, uint64_t sig, bool* is_new) {
+  auto it = e->class_off.find(sig);
+  if (it != e->class_off.end()) return it->second;
+  LoweredClass lc;
+  try {
+    lc = lower_class(e->P, sig);
+  } catch (const std::exception& ex) {
+    e->err = std::string("lowering failed: ") + ex.what();
+    return -1;
+  }
+  const ClassHdr* h = (const ClassHdr*)lc.blob.data();
+  e->max_nodes = std::max(e->max_nodes, h->n_nodes);
+  e->max_slots = std::max(e->max_slots, h->n_slots);
+  if (e->pool.size() + lc.blob.size() >= (1ull << 32)) { e->err = "class pool exceeds 4 GiB"; return -1; }
+  uint32_t off = (uint32_t)e->pool.size();
+  e->pool.insert(e->pool.end(), lc.blob.begin(), lc.blob.end());
+  e->class_off.emplace(sig, off);
+  if (is_new) *is_new = true;
+  return off;
+}
+
+static int ensure_ws(rpeg_engine_t* e, size_t bytes, hipStream_t s) {
+  if (bytes <= e->ws_cap) return 0;
+  HIP_TRY(e, hipStreamSynchronize(s));
+  if (e->d_ws) hipFree(e->d_ws);
+  e->d_ws = nullptr;
+  e->ws_cap = 0;
+  HIP_TRY(e, hipMalloc(&e->d_ws, bytes));
+  e->ws_cap = bytes;
+  return 0;
+}
+
+extern "C" {
+
+int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
+  if (!problem || !out) return -1;
+  *out = nullptr;
+  if (problem->abi_version != RPEG_ABI_VERSION) return -3;
+  if (problem->n_struct < 1 || problem->n_struct > RPEG_MAX_STRUCT || problem->n_split < 1 ||
+      problem->n_split > RPEG_MAX_SPLIT || problem->K_eval < 1)
+    return -3;
+  for (int s = 0; s < problem->n_struct; ++s) {
+    const rpeg_struct_t& st = problem->st[s];
+    if (st.n_vertex < 1 || st.n_vertex > RPEG_MAX_V || st.n_edge < 0 || st.n_edge > RPEG_MAX_E || st.n_pub < 0 ||
+        st.n_pub > RPEG_MAX_PUB || st.n_pair < 0 || st.n_pair > RPEG_MAX_PAIR || st.n_rel < 0 || st.n_rel > RPEG_MAX_REL)
+      return -3;
+  }
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count < 1) return -4;  // no GPU: there is no CPU path
+  rpeg_engine_t* e = new rpeg_engine_s();
+  e->P = *problem;
+  hipGetDevice(&e->device);
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, e->device) == hipSuccess) e->n_cu = prop.multiProcessorCount;
+  if (hipMalloc(&e->dP, sizeof(rpeg_problem_t)) != hipSuccess ||
+      hipMemcpy(e->dP, problem, sizeof(rpeg_problem_t), hipMemcpyHostToDevice) != hipSuccess ||
+      hipEventCreate(&e->ev0) != hipSuccess || hipEventCreate(&e->ev1) != hipSuccess) {
+    delete e;
+    return -2;
+  }
+  *out = e;
+  return 0;
+}
+
+void rpeg_engine_destroy(rpeg_engine_t* e) {
+  if (!e) return;
+  hipDeviceSynchronize();
+  if (e->dP) hipFree(e->dP);
+  if (e->d_pool) hipFree(e->d_pool);
+  if (e->d_sig) { hipFree(e->d_sig); hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_sig); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  if (e->d_ws) hipFree(e->d_ws);
+  if (e->ev0) hipEventDestroy(e->ev0);
+  if (e->ev1) hipEventDestroy(e->ev1);
+  delete e;
+}
+
+const char* rpeg_last_error(const rpeg_engine_t* e) { return e ? e->err.c_str() : "null engine"; }
+
+int rpeg_engine_set_timing(rpeg_engine_t* e, int32_t enabled) {
+  if (!e) return -1;
+  e->timing = enabled != 0;
+  return 0;
+}
+
+double rpeg_engine_last_kernel_ms(const rpeg_engine_t* e) { return e ? e->last_ms : -1.0; }
+
+int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n) {
+  if (!e || !out) return -1;
+  for (int i = 0; i < n && i < 5; ++i) out[i] = e->stats[i];
+  return 0;
+}
+
+int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                    double* peak, double* score, uint8_t* mask, void* stream) {
+  if (!e || !plans) return -1;
+  e->err.clear();
+  e->last_ms = -1.0;
+  if (n == 0) return 0;
+  if (n >= (1ull << 32)) { e->err = "at most 2^32-1 plans per call"; return -1; }
+  if (!plans->vert || !plans->head || plans->stride < n) { e->err = "bad plan tensors"; return -1; }
+  hipStream_t s = (hipStream_t)stream;
+  if (int rc = ensure_batch(e, n)) return rc;
+  const unsigned blk = 256;
+  hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + blk - 1) / blk)), dim3(blk), 0, s, e->dP, n, plans->vert,
+                     plans->head, plans->stride, e->d_sig, makespan, peak, score, mask);
+  HIP_TRY(e, hipGetLastError());
+  HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
+  HIP_TRY(e, hipStreamSynchronize(s));
+
+  // group plans by class: count, prefix, scatter (stable within a class)
+  std::unordered_map<uint64_t, uint32_t> local;  // signature -> dense id within this batch
+  std::vector<uint32_t> offs, counts;
+  std::vector<uint32_t> ids(n);
+  uint64_t n_new = 0;
+  uint64_t last_sig = SIG_INVALID;
+  uint32_t last_id = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    const uint64_t sg = e->h_sig[i];
+    if (sg == SIG_INVALID) { ids[i] = UINT32_MAX; continue; }
+    if (sg != last_sig) {
+      auto it = local.find(sg);
+      if (it == local.end()) {
+        bool is_new = false;
+        int64_t off = class_offset(e, sg, &is_new);
+        if (off < 0) return -5;
+        n_new += is_new;
+        it = local.emplace(sg, (uint32_t)offs.size()).first;
+        offs.push_back((uint32_t)off);
+        counts.push_back(0);
+      }
+      last_sig = sg;
+      last_id = it->second;
+    }
+    ids[i] = last_id;
+    ++counts[last_id];
+  }
+  std::vector<uint32_t> start(counts.size() + 1, 0);
+  for (size_t c = 0; c < counts.size(); ++c) start[c + 1] = start[c] + counts[c];
+  const uint64_t n_sorted = start.back();
+  std::vector<uint32_t> cursor(start.begin(), start.end() - 1);
+  for (uint64_t i = 0; i < n; ++i) {
+    if (ids[i] == UINT32_MAX) continue;
+    const uint32_t pos = cursor[ids[i]]++;
+    e->h_perm[pos] = (uint32_t)i;
+    e->h_cls[pos] = offs[ids[i]];
+  }
+  e->stats[0] = counts.size();
+  e->stats[1] = n_new;
+  if (n_sorted == 0) return 0;
+  if (int rc = ensure_pool(e, s)) return rc;
+  HIP_TRY(e, hipMemcpyAsync(e->d_perm, e->h_perm, n_sorted * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted * 4, hipMemcpyHostToDevice, s));
+
+  const uint64_t n_waves = (n_sorted + WAVE - 1) / WAVE;
+  const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * 16);
+  const size_t wsb = wave_ws_bytes(e->max_nodes, e->max_slots);
+  if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
+  const size_t lds = (size_t)READY_CAP * WAVE * sizeof(uint16_t);
+  e->stats[2] = n_waves;
+  e->stats[3] = lds;
+  e->stats[4] = wsb * grid;
+  if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
+  hipLaunchKernelGGL(k_eval, dim3(grid), dim3(WAVE), lds, s, e->dP, n_sorted, plans->vert, plans->head, plans->stride,
+                     e->d_perm, e->d_cls, e->d_pool, e->d_ws, e->max_nodes, e->max_slots, flags, makespan, peak, score,
+                     mask, (double*)nullptr, (double*)nullptr);
+  HIP_TRY(e, hipGetLastError());
+  if (e->timing) {
+    HIP_TRY(e, hipEventRecord(e->ev1, s));
+    HIP_TRY(e, hipEventSynchronize(e->ev1));
+    float ms = 0.f;
+    HIP_TRY(e, hipEventElapsedTime(&ms, e->ev0, e->ev1));
+    e->last_ms = ms;
+  }
+  return 0;
+}
+
+int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t vertex, const int16_t* strat,
+                       uint64_t stride, double* time, double* peak, void* stream) {
+  if (!e || !strat) return -1;
+  e->err.clear();
+  if (structure < 0 || structure >= e->P.n_struct || vertex < 0 || vertex >= e->P.st[structure].n_vertex || stride < n) {
+    e->err = "bad structure/vertex/stride";
+    return -1;
+  }
+  if (n == 0) return 0;
+  const unsigned blk = 256;
+  hipLaunchKernelGGL(k_op_time, dim3((unsigned)((n + blk - 1) / blk)), dim3(blk), 0, (hipStream_t)stream, e->dP, n,
+                     structure, vertex, strat, stride, time, peak);
+  HIP_TRY(e, hipGetLastError());
+  return 0;
+}
+
+int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* start, double* finish,
+                    int32_t* node_kind, int32_t* node_vertex, int32_t* node_step, int32_t cap) {
+  if (!e || !vert_fields || !head4 || !start || !finish) return -1;
+  e->err.clear();
+  PlanHead h = load_head(head4, 1, 0);
+  VPlan a[RPEG_MAX_V];
+  std::memset(a, 0, sizeof a);
+  if (h.structure >= e->P.n_struct) { e->err = "bad structure"; return -1; }
+  for (int v = 0; v < e->P.st[h.structure].n_vertex; ++v) load_vertex(vert_fields, 1, 0, v, &a[v]);
+  if (!plan_valid(e->P, h, a)) { e->err = "plan violates the integer validity rules"; return -6; }
+  const uint64_t sg = plan_signature(e->P, h.structure, h.split, h.tau0, h.tau1, a);
+  LoweredClass lc;
+  try { lc = lower_class(e->P, sg); } catch (const std::exception& ex) { e->err = ex.what(); return -5; }
+  const int n = (int)lc.nodes.size();
+  if (n > cap) { e->err = "trace arrays too small"; return -7; }
+  int64_t off = class_offset(e, sg, nullptr);
+  if (off < 0) return -5;
+  hipStream_t s = nullptr;
+  if (int rc = ensure_pool(e, s)) return rc;
+  if (int rc = ensure_batch(e, 1)) return rc;
+  if (int rc = ensure_ws(e, wave_ws_bytes(e->max_nodes, e->max_slots), s)) return rc;
+  int16_t* d_vert = nullptr;
+  uint8_t* d_head = nullptr;
+  double* d_tr = nullptr;
+  HIP_TRY(e, hipMalloc(&d_vert, RPEG_MAX_V * RPEG_FIELDS * 2));
+  HIP_TRY(e, hipMalloc(&d_head, 4));
+  HIP_TRY(e, hipMalloc(&d_tr, (size_t)n * 16));
+  HIP_TRY(e, hipMemcpy(d_vert, vert_fields, RPEG_MAX_V * RPEG_FIELDS * 2, hipMemcpyHostToDevice));
+  HIP_TRY(e, hipMemcpy(d_head, head4, 4, hipMemcpyHostToDevice));
+  const uint32_t zero = 0, o32 = (uint32_t)off;
+  HIP_TRY(e, hipMemcpy(e->d_perm, &zero, 4, hipMemcpyHostToDevice));
+  HIP_TRY(e, hipMemcpy(e->d_cls, &o32, 4, hipMemcpyHostToDevice));
+  hipLaunchKernelGGL(k_eval, dim3(1), dim3(WAVE), (size_t)READY_CAP * WAVE * 2, s, e->dP, (uint64_t)1, d_vert, d_head,
+                     (uint64_t)1, e->d_perm, e->d_cls, e->d_pool, e->d_ws, e->max_nodes, e->max_slots, 0u,
+                     (double*)nullptr, (double*)nullptr, (double*)nullptr, (uint8_t*)nullptr, d_tr, d_tr + n);
+  HIP_TRY(e, hipGetLastError());
+  HIP_TRY(e, hipMemcpy(start, d_tr, (size_t)n * 8, hipMemcpyDeviceToHost));
+  HIP_TRY(e, hipMemcpy(finish, d_tr + n, (size_t)n * 8, hipMemcpyDeviceToHost));
+  hipFree(d_vert); hipFree(d_head); hipFree(d_tr);
+  for (int i = 0; i < n; ++i) {
+    if (node_kind) node_kind[i] = lc.nodes[i].kind;
+    if (node_vertex) node_vertex[i] = lc.nodes[i].kind == 0 ? lc.nodes[i].vertex : lc.nodes[i].a1;
+    if (node_step) node_step[i] = lc.nodes[i].step;
+  }
+  return n;
+}
+
+int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream) {
+  if (!e || !x || !y) return -1;
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(k_exp, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, n, x, y);
+  HIP_TRY(e, hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,190 @@
+"""ctypes binding of librpeg_eval.so and the `Engine` host object.
+
+PyTorch is used only to own device buffers and to name the current HIP stream; every number is
+produced by the HIP kernels behind the C ABI (include/rpeg_eval.h).  There is no CPU fallback: a
+missing library or a missing GPU raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Dict, Optional
+
+import numpy as np
+
+from . import abi
+from .compile import compile_problem
+from .problem import EvalProblem, PlanBatch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "librpeg_eval.so")
+_lib = None
+
+EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
+           "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
+           "rpeg_engine_last_kernel_ms", "rpeg_device_exp")
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+def load_library(path: Optional[str] = None):
+    """Loads the in-tree shared library (built by rpeg_amd/build.py); raises if it is absent."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or _LIB_PATH
+    if not os.path.exists(p):
+        raise EngineError(f"{p} is missing: build it with `python -m rpeg_amd.build` (hipcc, gfx950)")
+    lib = C.CDLL(p)
+    vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int32
+    lib.rpeg_engine_create.restype = C.c_int
+    lib.rpeg_engine_create.argtypes = [vp, C.POINTER(vp)]
+    lib.rpeg_engine_destroy.restype = None
+    lib.rpeg_engine_destroy.argtypes = [vp]
+    lib.rpeg_last_error.restype = C.c_char_p
+    lib.rpeg_last_error.argtypes = [vp]
+    lib.rpeg_eval_batch.restype = C.c_int
+    lib.rpeg_eval_batch.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp]
+    lib.rpeg_op_time_batch.restype = C.c_int
+    lib.rpeg_op_time_batch.argtypes = [vp, u64, i32, i32, vp, u64, vp, vp, vp]
+    lib.rpeg_eval_trace.restype = C.c_int
+    lib.rpeg_eval_trace.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i32]
+    lib.rpeg_engine_stats.restype = C.c_int
+    lib.rpeg_engine_stats.argtypes = [vp, vp, i32]
+    lib.rpeg_engine_set_timing.restype = C.c_int
+    lib.rpeg_engine_set_timing.argtypes = [vp, i32]
+    lib.rpeg_engine_last_kernel_ms.restype = C.c_double
+    lib.rpeg_engine_last_kernel_ms.argtypes = [vp]
+    lib.rpeg_device_exp.restype = C.c_int
+    lib.rpeg_device_exp.argtypes = [vp, u64, vp, vp, vp]
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def _torch():
+    import torch
+    if not torch.cuda.is_available():
+        raise EngineError("no HIP device is visible; the evaluator has no CPU path")
+    return torch
+
+
+class DeviceBatch:
+    """Plan tensors resident in device memory (what rpeg_plan_soa_t points at)."""
+
+    def __init__(self, batch: PlanBatch, device="cuda:0"):
+        torch = _torch()
+        self.n = batch.n
+        self.vert = torch.from_numpy(np.ascontiguousarray(batch.vert)).to(device)
+        self.head = torch.from_numpy(np.ascontiguousarray(batch.head)).to(device)
+        self.soa = abi.PlanSoaT(self.vert.data_ptr(), self.head.data_ptr(), self.vert.shape[1])
+
+
+class Engine:
+    """One compiled problem on one GPU.  Not thread-safe; use one engine per host thread."""
+
+    def __init__(self, problem: EvalProblem, device: str = "cuda:0"):
+        torch = _torch()
+        self.lib = load_library()
+        self.problem = problem
+        self.device = torch.device(device)
+        self.P = compile_problem(problem)
+        self._h = C.c_void_p()
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_engine_create(C.addressof(self.P), C.byref(self._h))
+        if rc != 0:
+            raise EngineError(f"rpeg_engine_create failed with status {rc}")
+
+    def close(self):
+        if getattr(self, "_h", None) and self._h.value:
+            self.lib.rpeg_engine_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, rc: int, what: str):
+        if rc < 0:
+            raise EngineError(f"{what} failed ({rc}): {self.lib.rpeg_last_error(self._h).decode()}")
+
+    def set_timing(self, on: bool):
+        self.lib.rpeg_engine_set_timing(self._h, int(on))
+
+    def last_kernel_ms(self) -> float:
+        return float(self.lib.rpeg_engine_last_kernel_ms(self._h))
+
+    def stats(self) -> Dict[str, int]:
+        buf = (C.c_uint64 * 5)()
+        self.lib.rpeg_engine_stats(self._h, buf, 5)
+        return dict(classes=buf[0], classes_lowered=buf[1], wave_tasks=buf[2], lds_bytes=buf[3], workspace_bytes=buf[4])
+
+    def alloc_outputs(self, n: int):
+        torch = _torch()
+        return dict(makespan=torch.empty(n, dtype=torch.float64, device=self.device),
+                    peak=torch.empty(n, dtype=torch.float64, device=self.device),
+                    score=torch.empty(n, dtype=torch.float64, device=self.device),
+                    mask=torch.empty(n, dtype=torch.uint8, device=self.device))
+
+    def eval_device(self, dbatch: DeviceBatch, out=None, gate_stale: bool = True, n: Optional[int] = None):
+        """Evaluates plans already resident on the device into device outputs (no host copies of
+        plan data or results)."""
+        torch = _torch()
+        n = dbatch.n if n is None else n
+        out = out or self.alloc_outputs(n)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_eval_batch(self._h, n, C.addressof(dbatch.soa), abi.GATE_STALE if gate_stale else 0,
+                                          out["makespan"].data_ptr(), out["peak"].data_ptr(), out["score"].data_ptr(),
+                                          out["mask"].data_ptr(), stream)
+        self._check(rc, "rpeg_eval_batch")
+        return out
+
+    def eval(self, batch: PlanBatch, gate_stale: bool = True) -> Dict[str, np.ndarray]:
+        """Host convenience: upload, evaluate, download."""
+        out = self.eval_device(DeviceBatch(batch, self.device), gate_stale=gate_stale)
+        _torch().cuda.synchronize(self.device)
+        return {k: v.cpu().numpy() for k, v in out.items()}
+
+    def op_time(self, structure: int, vertex: int, strat: np.ndarray):
+        """time() and peak_bytes() of mock nodes: strat is int16 [7, n] = dp pp tp mb r_ext n_ext g_ext."""
+        torch = _torch()
+        strat = np.ascontiguousarray(strat, dtype=np.int16)
+        n = strat.shape[1]
+        d = torch.from_numpy(strat).to(self.device)
+        t = torch.empty(n, dtype=torch.float64, device=self.device)
+        p = torch.empty(n, dtype=torch.float64, device=self.device)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_op_time_batch(self._h, n, structure, vertex, d.data_ptr(), n, t.data_ptr(), p.data_ptr(), stream)
+        self._check(rc, "rpeg_op_time_batch")
+        torch.cuda.synchronize(self.device)
+        return t.cpu().numpy(), p.cpu().numpy()
+
+    def trace(self, batch: PlanBatch, i: int, cap: int = 4096):
+        """Start/finish of every lowered node of plan i, in the reference's node order."""
+        torch = _torch()
+        vert = np.ascontiguousarray(batch.vert[:, i], dtype=np.int16)
+        head = np.ascontiguousarray(batch.head[:, i], dtype=np.uint8)
+        start, finish = np.zeros(cap), np.zeros(cap)
+        kind, vertex, step = (np.zeros(cap, np.int32) for _ in range(3))
+        with torch.cuda.device(self.device):
+            n = self.lib.rpeg_eval_trace(self._h, vert.ctypes.data, head.ctypes.data, start.ctypes.data,
+                                         finish.ctypes.data, kind.ctypes.data, vertex.ctypes.data, step.ctypes.data, cap)
+        self._check(n, "rpeg_eval_trace")
+        return dict(start=start[:n], finish=finish[:n], kind=kind[:n], vertex=vertex[:n], step=step[:n])
+
+    def device_exp(self, x: np.ndarray) -> np.ndarray:
+        torch = _torch()
+        d = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float64)).to(self.device)
+        y = torch.empty_like(d)
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_device_exp(self._h, d.numel(), d.data_ptr(), y.data_ptr(),
+                                          torch.cuda.current_stream(self.device).cuda_stream)
+        self._check(rc, "rpeg_device_exp")
+        torch.cuda.synchronize(self.device)
+        return y.cpu().numpy()
