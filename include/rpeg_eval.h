@@ -162,12 +162,17 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
 int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t vertex,
                        const int16_t* strat, uint64_t stride, double* time, double* peak, void* stream);
 
-/* Start/finish time of every lowered node of ONE plan (host arrays of capacity cap), in the
-   reference's node order; what move_gen reads from Trace (moves.py:590-619).  Returns the node
-   count, or a negative status. */
+/* Start/finish time of every lowered node of ONE plan and the lowered graph itself (host arrays of
+   capacity cap nodes / cap edges), in the reference's node and edge order: what evaluate() returns
+   as (trace, lowered) (evaluate.py:290) and move_gen reads (moves.py:590-619).  vert_fields is one
+   plan's RPEG_MAX_V*RPEG_FIELDS int16 values (stride 1), head4 its 4 header bytes.  node_kind:
+   0 operator, 1 COMM, 2 RESHARD; node_vertex: the operator's vertex, or a transfer's destination
+   vertex; node_src: a transfer's source vertex; node_sub: quantile phase or -1; edges: (src,dst)
+   node index pairs.  Returns the node count, or a negative status. */
 int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4,
                     double* start, double* finish, int32_t* node_kind, int32_t* node_vertex,
-                    int32_t* node_step, int32_t cap);
+                    int32_t* node_step, int32_t* node_sub, int32_t* node_src, int32_t* edges,
+                    int32_t* n_edges, int32_t cap);
 
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] kernel-C dynamic LDS bytes, [4] workspace bytes. */

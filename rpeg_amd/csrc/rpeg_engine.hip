@@ -409,7 +409,8 @@ int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t 
 }
 
 int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* start, double* finish,
-                    int32_t* node_kind, int32_t* node_vertex, int32_t* node_step, int32_t cap) {
+                    int32_t* node_kind, int32_t* node_vertex, int32_t* node_step, int32_t* node_sub, int32_t* node_src,
+                    int32_t* edges, int32_t* n_edges, int32_t cap) {
   if (!e || !vert_fields || !head4 || !start || !finish) return -1;
   e->err.clear();
   PlanHead h = load_head(head4, 1, 0);
@@ -422,7 +423,7 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   LoweredClass lc;
   try { lc = lower_class(e->P, sg); } catch (const std::exception& ex) { e->err = ex.what(); return -5; }
   const int n = (int)lc.nodes.size();
-  if (n > cap) { e->err = "trace arrays too small"; return -7; }
+  if (n > cap || (edges && (int)lc.edges.size() > cap)) { e->err = "trace arrays too small"; return -7; }
   int64_t off = class_offset(e, sg, nullptr);
   if (off < 0) return -5;
   hipStream_t s = nullptr;
@@ -451,7 +452,12 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
     if (node_kind) node_kind[i] = lc.nodes[i].kind;
     if (node_vertex) node_vertex[i] = lc.nodes[i].kind == 0 ? lc.nodes[i].vertex : lc.nodes[i].a1;
     if (node_step) node_step[i] = lc.nodes[i].step;
+    if (node_sub) node_sub[i] = lc.nodes[i].sub;
+    if (node_src) node_src[i] = lc.nodes[i].kind == 0 ? lc.nodes[i].vertex : lc.nodes[i].a0;
   }
+  if (edges)
+    for (size_t j = 0; j < lc.edges.size(); ++j) { edges[2 * j] = lc.edges[j].first; edges[2 * j + 1] = lc.edges[j].second; }
+  if (n_edges) *n_edges = (int32_t)lc.edges.size();
   return n;
 }
 

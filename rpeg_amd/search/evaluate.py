@@ -1,0 +1,292 @@
+"""Drop-in evaluation calls: same names, arguments, return shapes and error behaviour as
+RPEG/search/evaluate.py, computed by the GPU engine.
+
+  evaluate(config, suite, workload, hw, K_eval, memory_policy)          -> (score, trace, lowered)
+  evaluate_cached(config, cache, suite, workload, hw, K_eval, policy)   -> (score, trace, feasible, miss)
+  _eval_worker((config, suite, workload, hw, K_eval[, policy]))         -> (score, trace, feasible)
+  evaluate_batch(configs, suite, workload, hw, K_eval, policy)          -> BatchResult   (new: the
+      batched form of Pool.map(_eval_worker, ...), RPEG/search/optimizer.py:793-798)
+
+The integer gates (`is_compatible`, `allocations_overlap`, `stale_publication_layout_valid`, the
+integer part of `is_valid`) are host code as in the reference.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from ..core.types import (Allocation, DeviceSpace, RPEG_TRANSFER_RESOURCE_POLICY, TransferResourcePolicy,
+                          packing_geometry, rectangular_node_layouts)
+from ..engine import abi
+from ..engine.problem import STRUCTURES, EvalProblem, PlanBatch
+from ..ir.plan import ExecutionPlan
+from ..ir.rpeg import RPEG
+from ..model.hardware import Hardware
+from ..model.memory import MemoryPolicy
+from ..model.models import ModelSuite
+from ..model.workload import Workload
+from .cache import EvalCache, config_hash
+
+_OOM_BETA = 40.0
+ABLATION_HARD_OOM = False
+
+
+@dataclass
+class Configuration:
+    rpeg: RPEG
+    plan: ExecutionPlan
+    device_space: DeviceSpace
+    intra_stage_fusion: bool = False
+    transfer_resource_policy: Optional[TransferResourcePolicy] = None
+
+
+def is_compatible(alloc: Allocation, pi: Tuple[int, int, int], device_space: DeviceSpace) -> bool:
+    """Placement feasibility under nested 3D parallelism with stage packing (evaluate.py:50-94)."""
+    dp, pp, tp = pi
+    if tp > device_space.G:
+        return False
+    geom = packing_geometry(dp, pp, tp, device_space.G)
+    if geom is None or alloc.extent[2] != geom[0]:
+        return False
+    if tuple(alloc.extent[:2]) not in rectangular_node_layouts(geom[1], device_space.R, device_space.N):
+        return False
+    bounds = (device_space.R, device_space.N, device_space.G)
+    return all(o >= 0 and o + e <= b for o, e, b in zip(alloc.origin, alloc.extent, bounds))
+
+
+def allocations_overlap(left: Allocation, right: Allocation) -> bool:
+    return all(left.origin[k] < right.origin[k] + right.extent[k] and right.origin[k] < left.origin[k] + left.extent[k]
+               for k in range(3))
+
+
+def stale_publication_layout_valid(config: Configuration) -> bool:
+    """Every publication with a positive staleness budget needs disjoint endpoints (evaluate.py:115-140)."""
+    for e in config.rpeg.pub_edges:
+        if int(config.rpeg.tau.get(e.src.kind.model, 0)) > 0 and \
+                allocations_overlap(config.plan.sigma[e.src], config.plan.sigma[e.dst]):
+            return False
+    return True
+
+
+# ----------------------------------------------------------------------------- engine plumbing
+_engines: Dict[tuple, object] = {}
+
+
+def _structure_of(rpeg: RPEG):
+    ids = tuple(v.id for v in rpeg.vertices)
+    for st in STRUCTURES.values():
+        # every shipped template has a distinct vertex-id tuple
+        if ids == _TEMPLATE_IDS[st.name]:
+            return st
+    raise ValueError(f"unsupported template graph with vertices {ids}")
+
+
+_TEMPLATE_IDS = {"ppo": ("g_pi", "i_ref", "i_R", "i_V", "t_pi", "t_V"), "grpo": ("g_pi", "i_ref", "i_R", "t_pi"),
+                 "dpo": ("i_pi", "i_ref", "t_pi"), "ac_share": ("g_ac", "i_ref", "i_R", "i_ac", "t_ac")}
+
+
+def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware, space: DeviceSpace, K_eval: int,
+                policy: MemoryPolicy):
+    from ..engine.runtime import Engine
+    st = _structure_of(rpeg)
+    key = (st.name, tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
+    eng = _engines.get(key)
+    if eng is None:
+        problem = EvalProblem(structures=(st,), suite=suite, workload=workload, hw=hw, device_space=space,
+                              K_eval=K_eval, memory_policy=policy)
+        eng = _engines[key] = Engine(problem)
+    return eng, st
+
+
+def _check_supported(config: Configuration):
+    if config.intra_stage_fusion:
+        raise NotImplementedError("intra_stage_fusion=True is not evaluated by this engine")
+    pol = config.transfer_resource_policy or RPEG_TRANSFER_RESOURCE_POLICY
+    if pol != RPEG_TRANSFER_RESOURCE_POLICY:
+        raise NotImplementedError("only the default transfer resource policy is evaluated by this engine")
+
+
+def _pack(configs: Sequence[Configuration], st, workload: Workload) -> PlanBatch:
+    batch = PlanBatch.empty(len(configs))
+    split = 1 if workload.gen_quantiles else 0
+    for i, cfg in enumerate(configs):
+        for v in cfg.rpeg.vertices:  # a missing vertex raises KeyError as lower() does (lower.py:447-451)
+            cfg.plan.sigma[v], cfg.plan.pi[v]
+        taus = [int(cfg.rpeg.tau[m]) for m in st.tau_models]
+        plan = cfg.plan
+        if any(v not in plan.mb for v in cfg.rpeg.vertices):
+            raise KeyError("plan.mb misses a template vertex")
+        batch.set_plan(i, 0, split, taus, cfg.rpeg, plan)
+    return batch
+
+
+@dataclass
+class BatchResult:
+    score: np.ndarray      # evaluate_cached semantics (0 where the stale-layout rule fails)
+    makespan: np.ndarray
+    peak: np.ndarray
+    mask: np.ndarray
+    feasible: np.ndarray   # memory-feasible and stale-layout valid
+
+
+def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload: Workload, hw: Hardware,
+                   K_eval: int, memory_policy: MemoryPolicy = MemoryPolicy(), gate_stale: bool = True) -> BatchResult:
+    """Scores many configurations of ONE template structure in one GPU launch."""
+    if not configs:
+        z = np.zeros(0)
+        return BatchResult(z, z, z, np.zeros(0, np.uint8), np.zeros(0, bool))
+    for c in configs:
+        _check_supported(c)
+    eng, st = _engine_for(configs[0].rpeg, suite, workload, hw, configs[0].device_space, K_eval, memory_policy)
+    out = eng.eval(_pack(configs, st, workload), gate_stale=gate_stale)
+    mask = out["mask"]
+    if np.any((mask & abi.MASK_VALID) == 0):
+        raise ValueError("a configuration violates the integer validity rules of is_valid")
+    if np.any(mask & abi.MASK_ERROR):
+        raise ZeroDivisionError("a configuration has a degenerate node duration or makespan")
+    feasible = ((mask & abi.MASK_MEM_OK) != 0) & ((mask & abi.MASK_STALE_OK) != 0)
+    score = out["score"].copy()
+    if ABLATION_HARD_OOM:
+        score[(mask & abi.MASK_MEM_OK) == 0] = 0.0
+    return BatchResult(score, out["makespan"], out["peak"], mask, feasible)
+
+
+# ----------------------------------------------------------------------------- trace objects
+@dataclass(frozen=True, eq=False)
+class ExecNode:
+    """Lowered node as the reference exposes it to its callers (lower.py:30-81), rebuilt from the
+    engine's per-node arrays."""
+    id: str
+    kind: str                       # "op" | "comm" | "reshard"
+    allocs: Tuple[Allocation, ...]
+    template_vertex: object = None  # operator nodes
+    k: Optional[int] = None
+    model: object = None
+    pi: Optional[Tuple[int, int, int]] = None
+    mb: Optional[int] = None
+
+    def __hash__(self):
+        return hash(self.id)
+
+    def __eq__(self, other):
+        return isinstance(other, ExecNode) and self.id == other.id
+
+
+@dataclass(frozen=True)
+class ExecEdge:
+    src: ExecNode
+    dst: ExecNode
+
+
+@dataclass(frozen=True)
+class ExecutableRPEG:
+    nodes: Tuple[ExecNode, ...]
+    edges: Tuple[ExecEdge, ...]
+    composite_operators: tuple = ()
+
+
+@dataclass(frozen=True)
+class Trace:
+    """Start/finish times per lowered node (mirror of RPEG/schedule/trace.py:18-51)."""
+    start: Dict[ExecNode, float]
+    finish: Dict[ExecNode, float]
+    reserved_allocations: Optional[dict] = None
+
+    def makespan(self) -> float:
+        return max(self.finish.values())
+
+    def throughput(self, W_step: float, K: int) -> float:
+        return K * W_step / self.makespan()
+
+
+def _trace_of(eng, st, config: Configuration, batch: PlanBatch):
+    tr = eng.trace(batch, 0)
+    verts = config.rpeg.vertices
+    nodes: List[ExecNode] = []
+    n_comm = n_reshard = 0
+    for kind, vertex, step, sub, src in zip(tr["kind"], tr["vertex"], tr["step"], tr["sub"], tr["src"]):
+        v = verts[vertex]
+        if kind == 0:
+            tag = "" if sub < 0 else f":{'g' if v.kind.role.value == 'GEN' else 'i'}{sub}"
+            nodes.append(ExecNode(id=f"{v.id}@{step}{tag}", kind="op", allocs=(config.plan.sigma[v],),
+                                  template_vertex=v, k=int(step), model=v.kind.model, pi=config.plan.pi[v],
+                                  mb=config.plan.mb[v]))
+        else:
+            if kind == 1:
+                n_comm += 1
+                name = f"comm{n_comm}"
+            else:
+                n_reshard += 1
+                name = f"reshard{n_reshard}"
+            nodes.append(ExecNode(id=name, kind="comm" if kind == 1 else "reshard",
+                                  allocs=(config.plan.sigma[verts[src]], config.plan.sigma[v])))
+    # dispatch order = order of start times is not recoverable from ties; keep the node order
+    start = {n: float(s) for n, s in zip(nodes, tr["start"])}
+    finish = {n: float(f) for n, f in zip(nodes, tr["finish"])}
+    edges = tuple(ExecEdge(nodes[a], nodes[b]) for a, b in tr["edges"])
+    return Trace(start=start, finish=finish), ExecutableRPEG(nodes=tuple(nodes), edges=edges)
+
+
+# ----------------------------------------------------------------------------- reference API
+def evaluate(config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
+             memory_policy: MemoryPolicy = MemoryPolicy()):
+    """unroll -> lower -> cost -> schedule -> score of one configuration (evaluate.py:235-290);
+    returns (score, trace, lowered)."""
+    _check_supported(config)
+    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy)
+    batch = _pack([config], st, workload)
+    trace, lowered = _trace_of(eng, st, config, batch)
+    score = trace.throughput(W_step=workload.B * workload.K * (workload.S + workload.T), K=K_eval)
+    return score, trace, lowered
+
+
+def evaluation_cache_key(config: Configuration, memory_policy: MemoryPolicy = MemoryPolicy()) -> str:
+    """Same key text as evaluate.py:301-326."""
+    pol = config.transfer_resource_policy or RPEG_TRANSFER_RESOURCE_POLICY
+    return (f"{config_hash(config.rpeg, config.plan)}:mem:"
+            f"fusion={int(config.intra_stage_fusion)}:"
+            f"transfer={','.join(pol.to_dict().values())}:"
+            f"{memory_policy.optimizer_stage}:"
+            f"{int(memory_policy.activation_checkpointing)}:"
+            f"{memory_policy.runtime_overhead_fraction:.12g}:"
+            f"{memory_policy.worker_overhead_bytes:.12g}:"
+            f"activation_cache={memory_policy.semantic_activation_cache_bytes:.12g}:"
+            f"groups={memory_policy.max_worker_groups_per_gpu}")
+
+
+def _score_one(config, suite, workload, hw, K_eval, memory_policy, gate_stale):
+    _check_supported(config)
+    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy)
+    batch = _pack([config], st, workload)
+    res = evaluate_batch([config], suite, workload, hw, K_eval, memory_policy, gate_stale=gate_stale)
+    trace, _ = _trace_of(eng, st, config, batch)
+    return float(res.score[0]), trace, res
+
+
+def evaluate_cached(config: Configuration, cache: EvalCache, suite: ModelSuite, workload: Workload, hw: Hardware,
+                    K_eval: int, memory_policy: MemoryPolicy = MemoryPolicy()):
+    """Cache lookup, then evaluation with the soft OOM penalty; a plan whose positive-lag
+    publication endpoints intersect scores 0 and is infeasible (evaluate.py:329-403).
+    Returns (score, trace, feasible, miss)."""
+    h = evaluation_cache_key(config, memory_policy)
+    if h in cache:
+        score, trace, feasible = cache.get(h)
+        return score, trace, feasible, False
+    score, trace, res = _score_one(config, suite, workload, hw, K_eval, memory_policy, gate_stale=True)
+    feasible = bool(res.feasible[0])
+    cache.put(h, score, trace, feasible)
+    return score, trace, feasible, True
+
+
+def _eval_worker(args):
+    """Pool target of the reference (evaluate.py:406-442): no cache, no stale-layout gate."""
+    if len(args) == 5:
+        config, suite, workload, hw, K_eval = args
+        memory_policy = MemoryPolicy()
+    else:
+        config, suite, workload, hw, K_eval, memory_policy = args
+    score, trace, res = _score_one(config, suite, workload, hw, K_eval, memory_policy, gate_stale=False)
+    return score, trace, bool(res.mask[0] & abi.MASK_MEM_OK)

@@ -1,0 +1,75 @@
+"""The host build of the kernels' arithmetic (oracle/cpu_port.cpp compiles rpeg_amd/csrc/*.h with
+g++) against the reference vectors and the Python oracle: this checks the code the GPU runs, on the
+CPU, including the class lowering and the heap-free scheduler."""
+
+import numpy as np
+import pytest
+
+from oracle import rpeg_oracle as oracle
+from oracle.cpu_port import CpuPort, exp_libm
+from rpeg_amd.engine import abi
+from tests.helpers import load_golden, oracle_eval, seeded_batch
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_port_matches_reference_vectors(c):
+    gold = load_golden(c)
+    cfg, batch = seeded_batch(c, gold["n"])
+    out = CpuPort(cfg.problem).eval(batch)
+    for i, want in enumerate(gold["plans"]):
+        assert float(out["makespan"][i]).hex() == want["makespan"], i
+        assert float(out["peak"][i]).hex() == want["peak"], i
+        assert float(out["score"][i]).hex() == want["score"], i
+        assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], i
+        assert out["mask"][i] & abi.MASK_VALID and not out["mask"][i] & abi.MASK_ERROR
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_port_matches_oracle_beyond_fixtures(c):
+    cfg, batch = seeded_batch(c, 48, start=100_000)
+    out = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE)
+    for i in range(48):
+        rpeg, plan, wl = batch.configuration(cfg.problem, i)
+        p = cfg.problem
+        want = oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy,
+                                    check_stale=True)
+        assert out["makespan"][i] == want["makespan"] and out["peak"][i] == want["peak"]
+        assert out["score"][i] == want["score"]
+        assert bool(out["mask"][i] & abi.MASK_STALE_OK) == want["stale_ok"]
+
+
+def test_port_lowering_equals_oracle_lowering():
+    for c in (1, 2, 3, 4):
+        cfg, batch = seeded_batch(c, 40)
+        p = cfg.problem
+        port = CpuPort(p)
+        for i in range(40):
+            rpeg, plan, wl = batch.configuration(p, i)
+            nodes, edges = oracle.lower(rpeg, plan, p.suite, p.K_eval, wl)
+            low = port.lower(batch, i)
+            kinds = {oracle.OP: 0, oracle.COMM: 1, oracle.RESHARD: 2}
+            assert [kinds[n.kind] for n in nodes] == list(low["kind"])
+            idx = {n.id: j for j, n in enumerate(nodes)}
+            assert [(idx[a.id], idx[b.id]) for a, b in edges] == [tuple(e) for e in low["edges"]]
+            cost = oracle.CostModel(p.hw, p.suite, wl)
+            assert [cost.time(n) for n in nodes] == list(low["dur"])
+
+
+def test_exp_equals_libm():
+    import math
+    rng = np.random.default_rng(7)
+    x = np.concatenate([-28.0 * rng.random(200_000), -np.logspace(-12, 1.5, 2000), [0.0, -0.0, -40.0, -64.0]])
+    y = exp_libm(x)
+    for a, b in zip(x.tolist(), y.tolist()):
+        assert math.exp(a) == b
+
+
+def test_invalid_plans_are_masked():
+    cfg, batch = seeded_batch(2, 8)
+    batch.vert[0, 1] = 3          # dp = 3 does not divide B
+    batch.vert[3, 2] = 5          # mb violates the microbatch rule
+    batch.head[1, 3] = 7          # split index out of range
+    batch.vert[7, 4] = 99         # extent outside the mesh
+    out = CpuPort(cfg.problem).eval(batch)
+    assert list(out["mask"][1:5] & abi.MASK_VALID) == [0, 0, 0, 0]
+    assert out["mask"][0] & abi.MASK_VALID and np.all(np.isnan(out["score"][1:5]))

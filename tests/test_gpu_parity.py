@@ -1,0 +1,220 @@
+"""GPU parity tests: every call goes through the C ABI (librpeg_eval.so) on a real MI355X.
+
+Bars: feasibility masks, ranking and best plan bit-exact; makespan, peak and score bit-exact
+(stricter than the 1e-12 relative the workload description allows)."""
+
+import math
+
+import numpy as np
+import pytest
+
+from oracle import rpeg_oracle as oracle
+from oracle.cpu_port import CpuPort
+from rpeg_amd import configs
+from rpeg_amd.engine import abi
+from rpeg_amd.engine.problem import PlanBatch
+from tests.helpers import load_golden, seeded_batch
+
+pytestmark = pytest.mark.gpu
+
+_engines = {}
+
+
+def engine(c):
+    from rpeg_amd.engine.runtime import Engine
+    if c not in _engines:
+        _engines[c] = Engine(configs.config(c).problem)
+    return _engines[c]
+
+
+def same_bits(a, b):
+    return np.array_equal(np.asarray(a, np.float64).view(np.uint64), np.asarray(b, np.float64).view(np.uint64))
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_reference_vectors(c):
+    gold = load_golden(c)
+    cfg, batch = seeded_batch(c, gold["n"])
+    out = engine(c).eval(batch, gate_stale=False)
+    for i, want in enumerate(gold["plans"]):
+        assert float(out["makespan"][i]).hex() == want["makespan"], i
+        assert float(out["peak"][i]).hex() == want["peak"], i
+        assert float(out["score"][i]).hex() == want["score"], i
+        assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], i
+        assert out["mask"][i] & abi.MASK_VALID and not out["mask"][i] & abi.MASK_ERROR
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_python_oracle_beyond_fixtures(c):
+    cfg, batch = seeded_batch(c, 40, start=200_000)
+    p = cfg.problem
+    out = engine(c).eval(batch, gate_stale=True)
+    for i in range(40):
+        rpeg, plan, wl = batch.configuration(p, i)
+        want = oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy,
+                                    check_stale=True)
+        assert out["makespan"][i] == want["makespan"] and out["peak"][i] == want["peak"], i
+        assert out["score"][i] == want["score"], i
+        assert bool(out["mask"][i] & abi.MASK_STALE_OK) == want["stale_ok"], i
+        assert bool(out["mask"][i] & abi.MASK_MEM_OK) == (not want["peak"] > want["cap"]), i
+
+
+@pytest.mark.parametrize("c,n", [(1, 4096), (2, 65536), (3, 65536), (4, 262144)])
+def test_full_candidate_sets_rank_and_argmax(c, n):
+    """Whole seeded sets: masks, every score, the ranking and the best plan equal the host build of
+    the same arithmetic, which the CPU suite ties to the reference vectors."""
+    cfg, batch = seeded_batch(c, n)
+    out = engine(c).eval(batch, gate_stale=True)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    assert np.array_equal(out["mask"], ref["mask"])
+    assert same_bits(out["makespan"], ref["makespan"])
+    assert same_bits(out["peak"], ref["peak"])
+    assert same_bits(out["score"], ref["score"])
+    assert np.array_equal(np.argsort(-out["score"], kind="stable"), np.argsort(-ref["score"], kind="stable"))
+    assert int(np.argmax(out["score"])) == int(np.argmax(ref["score"]))
+    # size-independent properties
+    assert np.all(out["makespan"] > 0) and np.all(out["peak"] > 0)
+    feasible = (out["mask"] & abi.MASK_MEM_OK) != 0
+    stale_ok = (out["mask"] & abi.MASK_STALE_OK) != 0
+    raw = cfg.problem.K_eval * cfg.problem.workload.B * cfg.problem.workload.K * \
+        (cfg.problem.workload.S + cfg.problem.workload.T) / out["makespan"]
+    assert same_bits(out["score"][feasible & stale_ok], raw[feasible & stale_ok])
+    assert np.all(out["score"][~stale_ok] == 0.0)
+    assert np.all(out["score"][~feasible & stale_ok] < raw[~feasible & stale_ok])
+
+
+def test_config4_is_mostly_infeasible():
+    cfg, batch = seeded_batch(4, 262144)
+    out = engine(4).eval(batch)
+    frac = 1.0 - np.mean((out["mask"] & abi.MASK_MEM_OK) != 0)
+    assert 0.6 < frac < 0.85
+
+
+def test_permutation_duplicates_and_stride():
+    from rpeg_amd.engine.runtime import DeviceBatch
+    import torch
+    cfg, batch = seeded_batch(2, 5000)
+    eng = engine(2)
+    base = eng.eval(batch)
+    perm = np.random.default_rng(0).permutation(5000)
+    shuffled = eng.eval(batch.take(perm))
+    for k in ("makespan", "peak", "score", "mask"):
+        assert np.array_equal(shuffled[k], base[k][perm]), k
+    dup = eng.eval(batch.take(np.repeat(np.arange(100), 7)))
+    assert same_bits(dup["score"], np.repeat(base["score"][:100], 7))
+    # stride larger than n: evaluate the first 1000 plans of the 5000-plan tensors
+    db = DeviceBatch(batch)
+    out = eng.eval_device(db, n=1000)
+    torch.cuda.synchronize()
+    assert same_bits(out["score"].cpu().numpy(), base["score"][:1000])
+
+
+def test_empty_single_and_invalid():
+    cfg, batch = seeded_batch(2, 8)
+    eng = engine(2)
+    assert eng.eval(batch.slice(0, 0))["score"].shape == (0,)
+    one = eng.eval(batch.slice(3, 4))
+    assert same_bits(one["score"], eng.eval(batch)["score"][3:4])
+    batch.vert[0, 1] = 3
+    batch.vert[3, 2] = 5
+    batch.head[1, 3] = 7
+    batch.vert[7, 4] = 99
+    out = eng.eval(batch)
+    assert list(out["mask"][1:5]) == [0, 0, 0, 0] and np.all(np.isnan(out["score"][1:5]))
+    assert out["mask"][0] & abi.MASK_VALID and out["mask"][5] & abi.MASK_VALID
+    allbad = PlanBatch.empty(3)
+    assert list(eng.eval(allbad)["mask"]) == [0, 0, 0]
+
+
+def test_mixed_structures_config3():
+    cfg, batch = seeded_batch(3, 2000, start=500_000)
+    out = engine(3).eval(batch)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    assert set(np.unique(batch.head[0])) == {0, 1}
+    assert same_bits(out["score"], ref["score"]) and np.array_equal(out["mask"], ref["mask"])
+
+
+@pytest.mark.parametrize("c", [1, 3, 4])
+def test_op_time_batch_is_the_candidate_directory_arithmetic(c):
+    from rpeg_amd.search.candidates import strategy_space
+    p = configs.config(c).problem
+    eng = engine(c)
+    rpeg = p.template(0)
+    sp = p.device_space
+    cost = oracle.CostModel(p.hw, p.suite, p.workload)
+    mm = oracle.make_mem_model(rpeg, p.suite, p.workload, p.hw, p.memory_policy)
+    from rpeg_amd.core.types import Allocation
+    for vi, v in enumerate(rpeg.vertices):
+        space = strategy_space(p.suite.specs[v.kind.model].L, p.workload.B, sp.R, sp.N, sp.G)
+        pick = np.linspace(0, len(space) - 1, 60).astype(int)
+        strat = np.zeros((7, len(pick)), np.int16)
+        for j, s in enumerate(pick):
+            dp, pp, tp, er, en, eg = space[s]
+            mb = 1 if pp == 1 else max(m for m in (1, 2, 4, 8, 16, 32, 64) if (p.workload.B // dp) % m == 0)
+            strat[:, j] = (dp, pp, tp, mb, er, en, eg)
+        t, pk = eng.op_time(0, vi, strat)
+        for j in range(len(pick)):
+            dp, pp, tp, mb, er, en, eg = (int(x) for x in strat[:, j])
+            node = oracle.XNode("_approx", oracle.OP, (Allocation((0, 0, 0), (er, en, eg)),), tpl=v, k=0,
+                                model=v.kind.model, pi=(dp, pp, tp), mb=mb)
+            assert t[j] == cost.time(node), (v.id, j)
+            assert pk[j] == float(mm.peak_bytes(node)), (v.id, j)
+
+
+@pytest.mark.parametrize("c", [1, 2, 4])
+def test_trace_equals_oracle_schedule(c):
+    cfg, batch = seeded_batch(c, 12)
+    p = cfg.problem
+    eng = engine(c)
+    for i in range(12):
+        rpeg, plan, wl = batch.configuration(p, i)
+        nodes, edges = oracle.lower(rpeg, plan, p.suite, p.K_eval, wl)
+        cost = oracle.CostModel(p.hw, p.suite, wl)
+        start, finish, _ = oracle.schedule(nodes, edges, cost, p.device_space)
+        tr = eng.trace(batch, i)
+        assert [start[n.id] for n in nodes] == list(tr["start"])
+        assert [finish[n.id] for n in nodes] == list(tr["finish"])
+        idx = {n.id: j for j, n in enumerate(nodes)}
+        assert [(idx[a.id], idx[b.id]) for a, b in edges] == [tuple(e) for e in tr["edges"]]
+
+
+def test_device_exp_equals_host_libm():
+    rng = np.random.default_rng(11)
+    x = np.concatenate([-28.0 * rng.random(1_000_000), -np.logspace(-12, 1.5, 5000), [0.0, -40.0, -64.0]])
+    y = engine(4).device_exp(x)
+    want = np.array([math.exp(v) for v in x.tolist()])
+    assert same_bits(y, want)
+
+
+def test_drop_in_calls():
+    from rpeg_amd.search.evaluate import Configuration, _eval_worker, evaluate, evaluate_batch, evaluate_cached
+    from rpeg_amd.search.cache import EvalCache
+    cfg, batch = seeded_batch(1, 6)
+    p = cfg.problem
+    cache = EvalCache()
+    cfgs = []
+    for i in range(6):
+        rpeg, plan, wl = batch.configuration(p, i)
+        want = oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy,
+                                    check_stale=True, want_trace=True)
+        conf = Configuration(rpeg, plan, p.device_space)
+        score, trace, lowered = evaluate(conf, p.suite, wl, p.hw, p.K_eval)
+        assert score == want["raw"] and trace.makespan() == want["makespan"]
+        assert [n.id for n in lowered.nodes] == [n.id for n in want["nodes"]]
+        assert {n.id: t for n, t in trace.finish.items()} == want["finish"]
+        s2, tr2, feasible, miss = evaluate_cached(conf, cache, p.suite, wl, p.hw, p.K_eval)
+        assert miss and s2 == want["score"] and feasible == want["feasible"]
+        s3, _, _, miss2 = evaluate_cached(conf, cache, p.suite, wl, p.hw, p.K_eval)
+        assert not miss2 and s3 == s2
+        worker = oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy,
+                                      check_stale=False)
+        s4, _, f4 = _eval_worker((conf, p.suite, wl, p.hw, p.K_eval))
+        assert s4 == worker["score"] and f4 == worker["feasible"]
+        if wl == batch.configuration(p, 0)[2]:
+            cfgs.append((conf, want["score"]))
+    wl0 = batch.configuration(p, 0)[2]
+    res = evaluate_batch([c for c, _ in cfgs], p.suite, wl0, p.hw, p.K_eval)
+    assert list(res.score) == [s for _, s in cfgs]
+    bad = Configuration(cfgs[0][0].rpeg, cfgs[0][0].plan, p.device_space, intra_stage_fusion=True)
+    with pytest.raises(NotImplementedError):
+        evaluate(bad, p.suite, wl0, p.hw, p.K_eval)
