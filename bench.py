@@ -1,0 +1,153 @@
+#!/usr/bin/env python3
+"""Benchmark of the batched plan evaluator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu]
+
+A step is one pass of the hot path (signature kernel, class grouping, evaluation kernel) over the
+whole seeded candidate set of the configuration (config 2: 65,536 GRPO plans), with the plan
+tensors already resident in HBM and the results left in HBM.  Prints one JSON line.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+FP64_PEAK_TFLOPS = 78.6     # MI355X vector FP64, published
+# algorithmic bytes per plan: int16 plan fields (10 per vertex) + 4 header bytes in, 3 doubles + 1 mask byte out
+ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
+# algorithmic fp64 operations per plan (cost model + scheduler + memory model of the fully split DAG)
+ALG_FLOPS = {1: 3.7e3, 2: 2.5e3, 3: 6.0e3, 4: 0.83e3, 5: 3.7e3}
+
+
+def cpu_baseline(cfg, batch, seconds=12.0):
+    """The Python oracle (restatement of the reference's pure-Python path) on one core, on the first
+    plans of the same candidate set, for about `seconds`."""
+    from oracle import rpeg_oracle as oracle
+    p = cfg.problem
+    t0 = time.perf_counter()
+    done = 0
+    while done < batch.n and time.perf_counter() - t0 < seconds:
+        rpeg, plan, wl = batch.configuration(p, done)
+        oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy)
+        done += 1
+    dt = time.perf_counter() - t0
+    return dict(value=done / dt, unit="plan evals/s", cores=1, kind="port",
+                sample=f"first {done} plans of the same seeded set, Python oracle, 1 process, {dt:.1f} s")
+
+
+def cxx_port(cfg, batch, threads):
+    from oracle.cpu_port import CpuPort
+    port = CpuPort(cfg.problem)
+    n = min(batch.n, 65536)
+    sub = batch.slice(0, n)
+    port.eval(sub.slice(0, 256), threads=threads)
+    t0 = time.perf_counter()
+    port.eval(sub, threads=threads)
+    dt = time.perf_counter() - t0
+    return dict(value=n / dt, unit="plan evals/s", cores=threads,
+                sample=f"first {n} plans, host build of the kernels' arithmetic (OpenMP), lowering included")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every box of this build has one MI355X and the path needs no "
+                 "second one (plans are independent; see DESIGN.md for how it would shard). Use --gpus 1.")
+
+    import torch
+    from rpeg_amd import configs
+    from rpeg_amd.engine import abi
+    from rpeg_amd.engine.runtime import DeviceBatch, Engine
+    from rpeg_amd.search import candidates
+
+    c = args.config
+    cfg = configs.config(c)
+    n = cfg.n_plans if c != 5 else 64 * 6 * 256
+    batch = candidates.generate(cfg.problem, n, cfg.tau_choices, seed=42, tag=c)
+    eng = Engine(cfg.problem, "cuda:0")
+    db = DeviceBatch(batch, "cuda:0")
+    out = eng.alloc_outputs(n)
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eng.eval_device(db, out)
+    torch.cuda.synchronize()
+    first_call_ms = (time.perf_counter() - t0) * 1e3
+    for _ in range(args.warmup):
+        eng.eval_device(db, out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        eng.eval_device(db, out)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = n * args.steps / dt
+
+    # cold steps: every class of the batch is lowered again inside the step
+    cold_steps = max(1, min(args.steps, 5))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(cold_steps):
+        eng.reset_classes()
+        eng.eval_device(db, out)
+    torch.cuda.synchronize()
+    cold_ms = (time.perf_counter() - t0) / cold_steps * 1e3
+
+    # dominant kernel (k_eval) duration: HIP events on the launch stream, recorded by the library
+    eng.set_timing(True)
+    k_ms = []
+    for _ in range(args.steps):
+        eng.eval_device(db, out)
+        k_ms.append(eng.last_kernel_ms())
+    eng.set_timing(False)
+    kernel_ms = sum(k_ms) / len(k_ms)
+    stats = eng.stats()
+
+    mask = out["mask"].cpu().numpy()
+    score = out["score"].cpu().numpy()
+    valid = (mask & abi.MASK_VALID) != 0
+    alg_bytes = ALG_BYTES[c] * n
+    achieved_gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    achieved_tflops = ALG_FLOPS[c] * n / (kernel_ms * 1e-3) / 1e12
+    line = {
+        "metric": "cost-model plan evals/sec on 1 MI355X",
+        "value": value, "unit": "plan evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": cfg.name, "n_plans": n, "seed": 42, "K_eval": cfg.problem.K_eval,
+                   "device_mesh": [cfg.problem.device_space.R, cfg.problem.device_space.N, cfg.problem.device_space.G],
+                   "classes": stats["classes"], "inputs": "resident in HBM", "outputs": "left in HBM"},
+        "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "k_eval", "kernel_ms": kernel_ms, "algorithmic_bytes_per_plan": ALG_BYTES[c]},
+        "fp64_valu": {"achieved": achieved_tflops, "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
+                      "frac": achieved_tflops / FP64_PEAK_TFLOPS, "algorithmic_flops_per_plan": ALG_FLOPS[c]},
+        "kernel_only_evals_per_s": n / (kernel_ms * 1e-3),
+        "first_call_ms": first_call_ms, "cold_ms_per_step": cold_ms, "cold_evals_per_s": n / (cold_ms * 1e-3),
+        "feasible_fraction": float(((mask & abi.MASK_MEM_OK) != 0)[valid].mean()),
+        "best_plan": int(score.argmax()), "best_score": float(score.max()),
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(cfg, batch)
+        line["cpu_port_cxx"] = cxx_port(cfg, batch, threads=min(16, os.cpu_count() or 1))
+        line["host_cores"] = os.cpu_count()
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -178,6 +178,10 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
    by this call, [2] wave tasks, [3] kernel-C dynamic LDS bytes, [4] workspace bytes. */
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
 
+/* Forgets every lowered class, so that the next rpeg_eval_batch lowers all the classes of its batch
+   again (used to measure a cold call). */
+int rpeg_engine_reset_classes(rpeg_engine_t* e);
+
 /* Kernel time of the dominant kernel in the last rpeg_eval_batch call, measured with HIP events on
    the launch stream (milliseconds); negative when timing was not enabled. */
 int rpeg_engine_set_timing(rpeg_engine_t* e, int32_t enabled);

@@ -61,15 +61,7 @@ struct NodeRec {
                         // too when dp differs across the transfer.  0 otherwise.
 };
 
-// bit (u*8 + v) set when dp of vertex u differs from dp of vertex v
-RPEG_HD uint64_t dp_differs(const VPlan* a, int nv) {
-  uint64_t m = 0;
-  for (int u = 0; u < nv; ++u)
-    for (int v = 0; v < nv; ++v)
-      if (a[u].dp != a[v].dp) m |= 1ull << (u * 8 + v);
-  return m;
-}
-
+// dpne: bit (u*8 + v) set when dp of vertex u differs from dp of vertex v (PlanMasks::dpne)
 RPEG_HD unsigned blocked_mask(const NodeRec& r, uint64_t dpne) {
   unsigned b = r.blocked;
   if (r.cond) {
@@ -187,7 +179,9 @@ RPEG_HD double list_schedule(const ClassView& c, MEM& mem, const uint8_t* ovl, u
   double makespan = 0.0;
   int done = 0;
   // every iteration either schedules a node or raises one node's key; the bound guards a broken class
+  long guard_iters = 0;
   for (long guard = 0; done < n && guard < (long)n * n + 64; ++guard) {
+    ++guard_iters;
     if (n_ready == 0) { *error = true; return 0.0; }  // cycle (scheduler.py:548-550)
     int bj = 0;
     int bv = mem.rd_node(0);
@@ -242,6 +236,9 @@ RPEG_HD double list_schedule(const ClassView& c, MEM& mem, const uint8_t* ovl, u
       mem.time(w) = t;
     }
   }
+#ifdef RPEG_COUNT_ITERS
+  RPEG_COUNT_ITERS(n, guard_iters);
+#endif
   if (done != n) *error = true;
   return makespan;
 }

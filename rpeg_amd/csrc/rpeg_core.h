@@ -445,106 +445,105 @@ RPEG_HD double isolated_peak(const rpeg_vertex_t& vx, const VMem& m) {
   return m.mem_w + m.x2;
 }
 
+// Pair relations of one plan packed 8 bits per vertex: bit (8*u + v) of the word.
+struct PlanMasks {
+  uint64_t ovl;  // allocations of u and v intersect (u == v included)
+  uint64_t eq;   // allocations of u and v are identical
+  uint64_t dpne; // dp of u differs from dp of v
+};
+RPEG_HD unsigned mask_row(uint64_t m, int v) { return (unsigned)(m >> (8 * v)) & 0xFFu; }
+
+// Plan-independent vertex sets of one structure (bit v = vertex v).
+struct StructMasks {
+  uint8_t same_model[RPEG_MAX_V];   // vertices invoking the same model as v
+  uint8_t train_same[RPEG_MAX_V];   // TRAIN vertices of v's model
+  uint8_t before[RPEG_MAX_V];       // vertices that precede order[i] in first-appearance order
+  uint8_t train, trainable;         // TRAIN vertices; vertices of trainable models
+};
+RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) {
+  StructMasks m;
+  m.train = m.trainable = 0;
+  unsigned seen = 0;
+  for (int i = 0; i < RPEG_MAX_V; ++i) { m.same_model[i] = m.train_same[i] = m.before[i] = 0; }
+  for (int v = 0; v < st.n_vertex; ++v) {
+    if (st.vertex[v].role == RPEG_ROLE_TRAIN) m.train |= (uint8_t)(1u << v);
+    if (st.trainable[st.vertex[v].model]) m.trainable |= (uint8_t)(1u << v);
+    for (int w = 0; w < st.n_vertex; ++w)
+      if (st.vertex[w].model == st.vertex[v].model) {
+        m.same_model[v] |= (uint8_t)(1u << w);
+        if (st.vertex[w].role == RPEG_ROLE_TRAIN) m.train_same[v] |= (uint8_t)(1u << w);
+      }
+  }
+  for (int i = 0; i < st.n_vertex; ++i) { m.before[i] = (uint8_t)seen; seen |= 1u << order[i]; }
+  return m;
+}
+
 // Largest per-device peak (memory.py:608-841, worker-liveness model).  A device's peak depends
 // only on the set of vertices whose allocation contains it, and grows with that set; boxes have
 // the Helly property, so the maximum over devices is the maximum over the maximal cliques of the
 // pairwise-overlap graph.  `order` lists the vertices in order of first appearance among the
 // lowered operator nodes (it fixes the insertion order of the reference's dicts and hence the
-// order of its float sums); ovl[v] is the bit set of vertices whose allocation intersects v's.
-RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const VPlan* a, const VMem* vm,
-                               const uint8_t* order, const uint8_t* ovl) {
+// order of its float sums).  VM provides w_shard(v) (as double), mem_w(v), opt(v), extra(v).
+template <class VM>
+RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
+                               const PlanMasks& pm, const VM& vm) {
   const int nv = st.n_vertex;
+  const StructMasks sm = struct_masks(st, order);
   const unsigned full = (1u << nv) - 1u;
   double best = -1.0;
   for (unsigned M = 1; M <= full; ++M) {
     bool clique = true, maximal = true;
-    for (int v = 0; v < nv; ++v)
-      if ((M >> v) & 1u) { if (M & ~(unsigned)ovl[v]) { clique = false; break; } }
-    if (!clique) continue;
-    for (int v = 0; v < nv; ++v)
-      if (!((M >> v) & 1u) && !(M & ~(unsigned)ovl[v])) { maximal = false; break; }
-    if (!maximal) continue;
-    // persistent state: optimizer shards, then serving shards, then frozen weights
+    for (int v = 0; v < nv; ++v) {
+      const bool in = (M >> v) & 1u;
+      const bool fits = (M & ~mask_row(pm.ovl, v)) == 0;   // every member of M intersects v
+      if (in && !fits) clique = false;
+      if (!in && fits) maximal = false;
+    }
+    if (!clique || !maximal) continue;
     double persistent = 0.0;
     int groups = 0;
     for (int i = 0; i < nv; ++i) {  // distinct (model, allocation) worker keys
-      int v = order[i];
+      const int v = order[i];
       if (!((M >> v) & 1u)) continue;
-      bool dup = false;
-      for (int j = 0; j < i; ++j) {
-        int w = order[j];
-        if (((M >> w) & 1u) && st.vertex[w].model == st.vertex[v].model && alloc_equal(a[w], a[v])) dup = true;
-      }
-      if (!dup) ++groups;
+      if ((mask_row(pm.eq, v) & M & sm.same_model[v] & sm.before[i]) == 0) ++groups;
     }
-    for (int i = 0; i < nv; ++i) {
-      int v = order[i];
-      if (!((M >> v) & 1u)) continue;
-      if (st.vertex[v].role == RPEG_ROLE_TRAIN && st.trainable[st.vertex[v].model]) persistent += vm[v].opt;
+    for (int i = 0; i < nv; ++i) {  // optimizer shards of the training vertices
+      const int v = order[i];
+      if (((M & sm.train & sm.trainable) >> v) & 1u) persistent += vm.opt(v);
     }
-    unsigned serving = 0;  // vertices whose worker key is a serving shard
+    unsigned serving = 0;           // serving shards: one per worker key that is not a training worker
     for (int i = 0; i < nv; ++i) {
-      int v = order[i];
-      if (!((M >> v) & 1u)) continue;
-      const rpeg_vertex_t& vx = st.vertex[v];
-      if (!st.trainable[vx.model] || vx.role == RPEG_ROLE_TRAIN) continue;
-      bool is_train_key = false;
-      for (int w = 0; w < nv; ++w)
-        if (((M >> w) & 1u) && st.vertex[w].role == RPEG_ROLE_TRAIN && st.vertex[w].model == vx.model &&
-            alloc_equal(a[w], a[v]))
-          is_train_key = true;
-      if (is_train_key) continue;
+      const int v = order[i];
+      if (!(((M & sm.trainable & ~(unsigned)sm.train) >> v) & 1u)) continue;
+      const unsigned same_key = mask_row(pm.eq, v) & M & sm.same_model[v];
+      if (same_key & sm.train_same[v]) continue;
+      const bool first = (same_key & serving) == 0;
       serving |= 1u << v;
-      // one entry per worker key, inserted at its first vertex, holding the largest shard
-      bool first = true;
-      for (int j = 0; j < i; ++j) {
-        int w = order[j];
-        if (((serving >> w) & 1u) && st.vertex[w].model == vx.model && alloc_equal(a[w], a[v])) first = false;
-      }
       if (!first) continue;
-      int64_t ws = vm[v].w_shard;
-      for (int j = i + 1; j < nv; ++j) {
-        int w = order[j];
-        if (!((M >> w) & 1u)) continue;
-        const rpeg_vertex_t& wx = st.vertex[w];
-        if (wx.model == vx.model && wx.role != RPEG_ROLE_TRAIN && alloc_equal(a[w], a[v]) && vm[w].w_shard > ws)
-          ws = vm[w].w_shard;
-      }
-      persistent += (double)(P.model[vx.model].sb * ws);
+      double ws = 0.0;
+      for (int w = 0; w < nv; ++w)
+        if (((same_key & ~(unsigned)sm.train) >> w) & 1u) ws = dmax(ws, vm.w_shard(w));
+      persistent += (double)P.model[st.vertex[v].model].sb * ws;
     }
-    for (int i = 0; i < nv; ++i) {
-      int v = order[i];
-      if (!((M >> v) & 1u)) continue;
-      const rpeg_vertex_t& vx = st.vertex[v];
-      if (st.trainable[vx.model]) continue;
-      bool first = true;
-      for (int j = 0; j < i; ++j) {
-        int w = order[j];
-        if (((M >> w) & 1u) && st.vertex[w].model == vx.model) first = false;
-      }
-      if (!first) continue;
-      double wb = dmax(0.0, vm[v].mem_w);
-      for (int j = i + 1; j < nv; ++j) {
-        int w = order[j];
-        if (((M >> w) & 1u) && st.vertex[w].model == vx.model) wb = dmax(wb, vm[w].mem_w);
-      }
+    for (int i = 0; i < nv; ++i) {  // frozen weights: one entry per model, its largest shard
+      const int v = order[i];
+      if (!(((M & ~(unsigned)sm.trainable) >> v) & 1u)) continue;
+      const unsigned same = M & sm.same_model[v];
+      if (same & sm.before[i]) continue;
+      double wb = 0.0;
+      for (int w = 0; w < nv; ++w)
+        if ((same >> w) & 1u) wb = dmax(wb, vm.mem_w(w));
       persistent += wb;
     }
     double top = 0.0;
     for (int i = 0; i < nv; ++i) {
-      int v = order[i];
+      const int v = order[i];
       if (!((M >> v) & 1u)) continue;
-      const rpeg_vertex_t& vx = st.vertex[v];
-      bool resident = !st.trainable[vx.model];
-      if (!resident) {  // worker key present among the serving shards of this device
-        for (int w = 0; w < nv; ++w)
-          if (((serving >> w) & 1u) && st.vertex[w].model == vx.model && alloc_equal(a[w], a[v])) resident = true;
-      }
-      double c = resident ? vm[v].extra : vm[v].mem_w + vm[v].extra;
+      const bool resident = !((sm.trainable >> v) & 1u) || (mask_row(pm.eq, v) & serving & sm.same_model[v]) != 0;
+      const double c = resident ? vm.extra(v) : vm.mem_w(v) + vm.extra(v);
       top = dmax(top, c);
     }
-    double overhead = (double)groups * P.group_overhead;
-    double peak = overhead + persistent + top;
+    double peak = (double)groups * P.group_overhead + persistent + top;
     if (P.max_groups > 0 && groups > P.max_groups) peak = __builtin_inf();  // memory.py:699-704
     if (peak > best) best = peak;
   }

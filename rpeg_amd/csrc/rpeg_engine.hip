@@ -22,6 +22,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "rpeg_kernel_eval.h"
 #include "rpeg_lower.h"
 #include "rpeg_plan.h"
 
@@ -30,7 +31,8 @@ using namespace rpeg;
 namespace {
 
 constexpr int WAVE = 64;
-constexpr int READY_CAP = 64;  // ready-list entries per plan (LDS); overflow sets RPEG_MASK_ERROR
+constexpr int READY_CAP = 64;
+constexpr uint32_t IDLE_LANE = 0xFFFFFFFFu;  // padding lane of a partly filled wavefront  // ready-list entries per plan (LDS); overflow sets RPEG_MASK_ERROR
 
 #define HIP_TRY(e, call)                                                                   \
   do {                                                                                     \
@@ -87,10 +89,17 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
   sig[i] = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
 }
 
-__global__ __launch_bounds__(WAVE) void k_eval(const rpeg_problem_t* __restrict__ P, uint64_t n_sorted,
+__global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
+  extern __shared__ uint8_t ke_lds[];
+  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) ke_eval_wave(L, w, ke_lds);
+}
+
+// Generic single-wavefront kernel over the host/device-shared scheduler template; used for the
+// per-node trace of one plan.
+__global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __restrict__ P, uint64_t n_sorted,
                                                const int16_t* __restrict__ vert, const uint8_t* __restrict__ head,
                                                uint64_t stride, const uint32_t* __restrict__ perm,
-                                               const uint32_t* __restrict__ cls_off, const uint8_t* __restrict__ pool,
+                                               const uint32_t* __restrict__ wave_cls, const uint8_t* __restrict__ pool,
                                                uint8_t* __restrict__ ws, uint32_t ws_nodes, uint32_t ws_slots,
                                                uint32_t flags, double* makespan, double* peak, double* score,
                                                uint8_t* mask, double* tr_start, double* tr_finish) {
@@ -107,10 +116,10 @@ __global__ __launch_bounds__(WAVE) void k_eval(const rpeg_problem_t* __restrict_
   mem.tr_start = tr_start;
   mem.tr_finish = tr_finish;
   for (uint64_t w = blockIdx.x; w < n_waves; w += gridDim.x) {
-    const uint64_t t = w * WAVE + lane;
-    if (t >= n_sorted) continue;
-    const uint64_t i = perm[t];
-    const ClassView cv = class_view(pool + cls_off[t]);
+    // every wavefront works on one class: the class tables are addressed uniformly (scalar loads)
+    const ClassView cv = class_view(pool + wave_cls[w]);
+    const uint64_t i = perm[w * WAVE + lane];
+    if (i == IDLE_LANE) continue;
     PlanHead h = load_head(head, stride, i);
     VPlan a[RPEG_MAX_V];
     const int nv = P->st[h.structure].n_vertex;
@@ -163,9 +172,13 @@ struct rpeg_engine_s {
   std::vector<uint8_t> pool;
   uint8_t* d_pool = nullptr;
   size_t d_pool_cap = 0, d_pool_used = 0;
-  uint32_t max_nodes = 1, max_slots = 1;
+  uint32_t max_nodes = 1, max_slots = 1, max_cls_bytes = 16;
+  bool lds_attr_set = false;
+  bool prof_on = false;
+  unsigned long long* d_prof = nullptr;
+  uint64_t prof_waves = 0;
   // per-batch buffers
-  size_t cap_n = 0;
+  size_t cap_n = 0, cap_perm = 0;
   uint64_t* d_sig = nullptr;
   uint64_t* h_sig = nullptr;
   uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_perm = nullptr, *h_cls = nullptr;
@@ -182,15 +195,25 @@ struct rpeg_engine_s {
 static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (n <= e->cap_n) return 0;
   size_t cap = std::max<size_t>(n, 4096);
-  if (e->d_sig) { hipFree(e->d_sig); hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_sig); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); }
   e->cap_n = 0;
   HIP_TRY(e, hipMalloc(&e->d_sig, cap * 8));
-  HIP_TRY(e, hipMalloc(&e->d_perm, cap * 4));
-  HIP_TRY(e, hipMalloc(&e->d_cls, cap * 4));
   HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
-  HIP_TRY(e, hipHostMalloc(&e->h_perm, cap * 4));
-  HIP_TRY(e, hipHostMalloc(&e->h_cls, cap * 4));
   e->cap_n = cap;
+  return 0;
+}
+
+// permutation (one entry per lane, classes padded to wavefronts) and class offset per wavefront
+static int ensure_perm(rpeg_engine_t* e, size_t lanes) {
+  if (lanes <= e->cap_perm) return 0;
+  size_t cap = std::max<size_t>(lanes + lanes / 4, 8192);
+  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  e->cap_perm = 0;
+  HIP_TRY(e, hipMalloc(&e->d_perm, cap * 4));
+  HIP_TRY(e, hipMalloc(&e->d_cls, (cap / WAVE + 1) * 4));
+  HIP_TRY(e, hipHostMalloc(&e->h_perm, cap * 4));
+  HIP_TRY(e, hipHostMalloc(&e->h_cls, (cap / WAVE + 1) * 4));
+  e->cap_perm = cap;
   return 0;
 }
 
@@ -229,6 +252,7 @@ static int64_t class_offset(rpeg_engine_t* e, uint64_t sig, bool* is_new) {
   const ClassHdr* h = (const ClassHdr*)lc.blob.data();
   e->max_nodes = std::max(e->max_nodes, h->n_nodes);
   e->max_slots = std::max(e->max_slots, h->n_slots);
+  e->max_cls_bytes = std::max(e->max_cls_bytes, h->n_nodes * 8u + h->n_succ * 2u);
   if (e->pool.size() + lc.blob.size() >= (1ull << 32)) { e->err = "class pool exceeds 4 GiB"; return -1; }
   uint32_t off = (uint32_t)e->pool.size();
   e->pool.insert(e->pool.end(), lc.blob.begin(), lc.blob.end());
@@ -285,7 +309,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   hipDeviceSynchronize();
   if (e->dP) hipFree(e->dP);
   if (e->d_pool) hipFree(e->d_pool);
-  if (e->d_sig) { hipFree(e->d_sig); hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_sig); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); }
+  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
   if (e->ev1) hipEventDestroy(e->ev1);
@@ -301,6 +326,28 @@ int rpeg_engine_set_timing(rpeg_engine_t* e, int32_t enabled) {
 }
 
 double rpeg_engine_last_kernel_ms(const rpeg_engine_t* e) { return e ? e->last_ms : -1.0; }
+
+// Phase clocks of the last batch (development aid): 8 counters of the 100 MHz wall clock per wavefront.
+int rpeg_engine_profile(rpeg_engine_t* e, int32_t enable, unsigned long long* out, uint64_t cap_waves) {
+  if (!e) return -1;
+  e->prof_on = enable != 0;
+  if (out && e->d_prof) {
+    uint64_t nw = std::min<uint64_t>(cap_waves, e->prof_waves);
+    hipDeviceSynchronize();
+    hipMemcpy(out, e->d_prof, nw * 64, hipMemcpyDeviceToHost);
+    return (int)nw;
+  }
+  return 0;
+}
+
+int rpeg_engine_reset_classes(rpeg_engine_t* e) {
+  if (!e) return -1;
+  hipDeviceSynchronize();
+  e->class_off.clear();
+  e->pool.clear();
+  e->d_pool_used = 0;
+  return 0;
+}
 
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n) {
   if (!e || !out) return -1;
@@ -352,35 +399,59 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
     ids[i] = last_id;
     ++counts[last_id];
   }
+  // every class starts on a wavefront boundary; the lanes left over are idle
   std::vector<uint32_t> start(counts.size() + 1, 0);
-  for (size_t c = 0; c < counts.size(); ++c) start[c + 1] = start[c] + counts[c];
+  for (size_t c = 0; c < counts.size(); ++c) start[c + 1] = start[c] + (counts[c] + WAVE - 1) / WAVE * WAVE;
   const uint64_t n_sorted = start.back();
-  std::vector<uint32_t> cursor(start.begin(), start.end() - 1);
-  for (uint64_t i = 0; i < n; ++i) {
-    if (ids[i] == UINT32_MAX) continue;
-    const uint32_t pos = cursor[ids[i]]++;
-    e->h_perm[pos] = (uint32_t)i;
-    e->h_cls[pos] = offs[ids[i]];
-  }
   e->stats[0] = counts.size();
   e->stats[1] = n_new;
   if (n_sorted == 0) return 0;
+  if (int rc = ensure_perm(e, n_sorted)) return rc;
+  std::fill(e->h_perm, e->h_perm + n_sorted, IDLE_LANE);
+  std::vector<uint32_t> cursor(start.begin(), start.end() - 1);
+  for (uint64_t i = 0; i < n; ++i) {
+    if (ids[i] == UINT32_MAX) continue;
+    e->h_perm[cursor[ids[i]]++] = (uint32_t)i;
+  }
+  for (size_t c = 0; c < counts.size(); ++c)
+    for (uint32_t w = start[c] / WAVE; w < start[c + 1] / WAVE; ++w) e->h_cls[w] = offs[c];
   if (int rc = ensure_pool(e, s)) return rc;
   HIP_TRY(e, hipMemcpyAsync(e->d_perm, e->h_perm, n_sorted * 4, hipMemcpyHostToDevice, s));
-  HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted / WAVE * 4, hipMemcpyHostToDevice, s));
 
-  const uint64_t n_waves = (n_sorted + WAVE - 1) / WAVE;
+  const uint64_t n_waves = n_sorted / WAVE;
   const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * 16);
-  const size_t wsb = wave_ws_bytes(e->max_nodes, e->max_slots);
+  const size_t wsb = ke_ws_bytes(e->max_nodes, e->max_slots);
   if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
-  const size_t lds = (size_t)READY_CAP * WAVE * sizeof(uint16_t);
+  EvalLaunch L;
+  L.P = e->dP; L.vert = plans->vert; L.head = plans->head; L.stride = plans->stride;
+  L.perm = e->d_perm; L.wave_cls = e->d_cls; L.pool = e->d_pool; L.ws = e->d_ws;
+  L.n_waves = n_waves; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
+  L.cls_bytes = (e->max_cls_bytes + 15u) & ~15u;
+  // ready-list capacity (a multiple of the scan's batch of 8); classes with more than 4095 nodes or
+  // tie-break keys above 15 cannot be packed into a ready entry
+  if (e->max_nodes > 4095) { e->err = "class with more than 4095 nodes"; return -8; }
+  L.rcap = 32;
+  L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
+  L.prof = nullptr;
+  if (e->prof_on) {
+    if (e->d_prof) hipFree(e->d_prof);
+    HIP_TRY(e, hipMalloc(&e->d_prof, n_waves * 64));
+    HIP_TRY(e, hipMemsetAsync(e->d_prof, 0, n_waves * 64, s));
+    e->prof_waves = n_waves;
+    L.prof = e->d_prof;
+  }
+  const size_t lds = ke_lds_bytes(L.cls_bytes, L.rcap);
+  if (lds > 160 * 1024) { e->err = "class tables exceed the LDS"; return -8; }
+  if (lds > 64 * 1024 && !e->lds_attr_set) {
+    HIP_TRY(e, hipFuncSetAttribute((const void*)k_eval, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    e->lds_attr_set = true;
+  }
   e->stats[2] = n_waves;
   e->stats[3] = lds;
   e->stats[4] = wsb * grid;
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
-  hipLaunchKernelGGL(k_eval, dim3(grid), dim3(WAVE), lds, s, e->dP, n_sorted, plans->vert, plans->head, plans->stride,
-                     e->d_perm, e->d_cls, e->d_pool, e->d_ws, e->max_nodes, e->max_slots, flags, makespan, peak, score,
-                     mask, (double*)nullptr, (double*)nullptr);
+  hipLaunchKernelGGL(k_eval, dim3(grid), dim3(WAVE), lds, s, L);
   HIP_TRY(e, hipGetLastError());
   if (e->timing) {
     HIP_TRY(e, hipEventRecord(e->ev1, s));
@@ -428,7 +499,7 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   if (off < 0) return -5;
   hipStream_t s = nullptr;
   if (int rc = ensure_pool(e, s)) return rc;
-  if (int rc = ensure_batch(e, 1)) return rc;
+  if (int rc = ensure_perm(e, WAVE)) return rc;
   if (int rc = ensure_ws(e, wave_ws_bytes(e->max_nodes, e->max_slots), s)) return rc;
   int16_t* d_vert = nullptr;
   uint8_t* d_head = nullptr;
@@ -438,10 +509,12 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   HIP_TRY(e, hipMalloc(&d_tr, (size_t)n * 16));
   HIP_TRY(e, hipMemcpy(d_vert, vert_fields, RPEG_MAX_V * RPEG_FIELDS * 2, hipMemcpyHostToDevice));
   HIP_TRY(e, hipMemcpy(d_head, head4, 4, hipMemcpyHostToDevice));
-  const uint32_t zero = 0, o32 = (uint32_t)off;
-  HIP_TRY(e, hipMemcpy(e->d_perm, &zero, 4, hipMemcpyHostToDevice));
+  uint32_t lanes[WAVE];
+  for (int l = 0; l < WAVE; ++l) lanes[l] = l == 0 ? 0u : IDLE_LANE;
+  const uint32_t o32 = (uint32_t)off;
+  HIP_TRY(e, hipMemcpy(e->d_perm, lanes, sizeof lanes, hipMemcpyHostToDevice));
   HIP_TRY(e, hipMemcpy(e->d_cls, &o32, 4, hipMemcpyHostToDevice));
-  hipLaunchKernelGGL(k_eval, dim3(1), dim3(WAVE), (size_t)READY_CAP * WAVE * 2, s, e->dP, (uint64_t)1, d_vert, d_head,
+  hipLaunchKernelGGL(k_eval_generic, dim3(1), dim3(WAVE), (size_t)READY_CAP * WAVE * 2, s, e->dP, (uint64_t)WAVE, d_vert, d_head,
                      (uint64_t)1, e->d_perm, e->d_cls, e->d_pool, e->d_ws, e->max_nodes, e->max_slots, 0u,
                      (double*)nullptr, (double*)nullptr, (double*)nullptr, (uint8_t*)nullptr, d_tr, d_tr + n);
   HIP_TRY(e, hipGetLastError());

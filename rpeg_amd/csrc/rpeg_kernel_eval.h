@@ -1,0 +1,364 @@
+// rpeg_kernel_eval.h - the batch evaluation kernel (device only).
+//
+// One wavefront evaluates up to 64 plans of ONE lowering class, one plan per lane.
+//
+// Memory placement, chosen for the latency of the list scheduler's dependent accesses:
+//   LDS   class tables (node records, successor lists): read with per-lane node indices
+//         plan fields [field][lane] int16, aliased with ...
+//         ... the ready list [entry][lane]: key (est), rank, node|tie.  The arg-min scan, the
+//         stale-key update and the removal never leave LDS.
+//   HBM   per-plan arrays in a per-wavefront workspace laid out [row][lane] (a row is 512
+//         contiguous bytes, so accesses coalesce whenever lanes agree on the row): durations per
+//         slot, rank / ready-time / remaining in-degree per node.  A scheduling step issues all of
+//         its loads (duration of the dispatched node; ready-time, in-degree and rank of up to four
+//         successors) before it waits, i.e. one memory round trip per dispatched node.
+#ifndef RPEG_KERNEL_EVAL_H
+#define RPEG_KERNEL_EVAL_H
+
+#include "rpeg_plan.h"
+
+namespace rpeg {
+
+constexpr int KE_WAVE = 64;
+constexpr uint32_t KE_IDLE = 0xFFFFFFFFu;
+
+struct EvalLaunch {              // uniform launch parameters
+  const rpeg_problem_t* P;
+  const int16_t* vert;
+  const uint8_t* head;
+  uint64_t stride;
+  const uint32_t* perm;          // lane -> plan index, KE_IDLE for padding lanes
+  const uint32_t* wave_cls;      // wavefront -> class blob offset
+  const uint8_t* pool;
+  uint8_t* ws;
+  uint64_t n_waves;
+  uint32_t ws_nodes, ws_slots;   // workspace row counts (maxima over the engine's classes)
+  uint32_t cls_bytes;            // LDS bytes reserved for class tables
+  uint32_t rcap;                 // ready-list capacity per plan
+  uint32_t flags;
+  double* makespan;
+  double* peak;
+  double* score;
+  uint8_t* mask;
+  unsigned long long* prof;      // optional per-wavefront phase clocks (8 per wavefront), or null
+};
+
+__host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
+  size_t lane = (16ull * nodes + 8ull * slots + nodes + 63) & ~size_t(63);
+  return (size_t)KE_WAVE * lane;
+}
+__host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap) {
+  size_t ready = (size_t)rcap * KE_WAVE * 20;
+  size_t plan = (size_t)RPEG_MAX_V * RPEG_FIELDS * KE_WAVE * 2 + (size_t)RPEG_MAX_V * 4 * KE_WAVE * 8;
+  return cls_bytes + (ready > plan ? ready : plan);
+}
+
+#if defined(__HIPCC__)
+
+__device__ inline VPlan ke_vplan(const int16_t* pl, int v) {
+  const int16_t* p = pl + v * RPEG_FIELDS * KE_WAVE;
+  VPlan a;
+  a.dp = p[0 * KE_WAVE]; a.pp = p[1 * KE_WAVE]; a.tp = p[2 * KE_WAVE]; a.mb = p[3 * KE_WAVE];
+  a.o[0] = p[4 * KE_WAVE]; a.o[1] = p[5 * KE_WAVE]; a.o[2] = p[6 * KE_WAVE];
+  a.e[0] = p[7 * KE_WAVE]; a.e[1] = p[8 * KE_WAVE]; a.e[2] = p[9 * KE_WAVE];
+  return a;
+}
+
+__device__ inline double ke_slot_duration(const rpeg_problem_t& P, const rpeg_struct_t& st, int split,
+                                          const SlotDesc sd, const int16_t* pl, bool* zero_div) {
+  switch (sd.type) {
+    case SLOT_OP_UNSPLIT:
+      return op_time(P, st.vertex[sd.a], st.vertex[sd.a].unsplit, ke_vplan(pl, sd.a), zero_div);
+    case SLOT_OP_SUB:
+      return op_time(P, st.vertex[sd.a], st.vertex[sd.a].sub[split][sd.q], ke_vplan(pl, sd.a), zero_div);
+    case SLOT_COMM_DATA: {
+      const rpeg_edge_t& e = st.edge[sd.a];
+      int64_t payload = sd.q == 0xFF ? e.full_bytes : e.sub_bytes[split][sd.q];
+      return comm_time(P, ke_vplan(pl, e.src), ke_vplan(pl, e.dst), payload, e.is_weight != 0);
+    }
+    case SLOT_COMM_PUB: {
+      const rpeg_pub_t& p = st.pub[sd.a];
+      VPlan s = ke_vplan(pl, p.src), d = ke_vplan(pl, p.dst);
+      return comm_time(P, s, d, pub_payload(P, s, d, p.model), true);
+    }
+    default:
+      return reshard_time(P, ke_vplan(pl, sd.a), sd.b);
+  }
+}
+
+struct KeVMem {  // per-vertex memory quantities in LDS, [vertex*4 + field][lane]
+  const double* p;
+  __device__ double w_shard(int v) const { return p[(v * 4 + 0) * KE_WAVE]; }
+  __device__ double mem_w(int v) const { return p[(v * 4 + 1) * KE_WAVE]; }
+  __device__ double opt(int v) const { return p[(v * 4 + 2) * KE_WAVE]; }
+  __device__ double extra(int v) const { return p[(v * 4 + 3) * KE_WAVE]; }
+};
+
+// max of last_fin over the vertices of a bit set
+__device__ inline double ke_dev_max(unsigned m, const double (&lf)[RPEG_MAX_V]) {
+  double d = 0.0;
+#pragma unroll
+  for (int x = 0; x < RPEG_MAX_V; ++x) d = ((m >> x) & 1u) && lf[x] > d ? lf[x] : d;
+  return d;
+}
+
+#define KE_STAMP(k) do { if (L.prof && lane == first_lane) L.prof[w * 8 + (k)] = wall_clock64(); } while (0)
+
+__device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* lds) {
+  const int lane = threadIdx.x;
+  int first_lane = 0;
+  const rpeg_problem_t& P = *L.P;
+  const ClassView cv = class_view(L.pool + L.wave_cls[w]);   // uniform
+  const int n = (int)cv.h->n_nodes, n_slots = (int)cv.h->n_slots, n_succ_all = (int)cv.h->n_succ;
+
+  // ---- LDS carve-up
+  uint64_t* l_node = (uint64_t*)lds;                                  // NodeRec[n]
+  uint16_t* l_succ = (uint16_t*)(lds + (size_t)n * 8);                // uint16[n_succ]
+  uint8_t* dyn = lds + L.cls_bytes;
+  int16_t* l_plan = (int16_t*)dyn + lane;                             // [60][64], aliased with the ready list
+  double* l_vm = (double*)(dyn + (size_t)RPEG_MAX_V * RPEG_FIELDS * KE_WAVE * 2) + lane;  // [24][64], aliased too
+  double* r_key = (double*)dyn + lane;                                // [rcap][64]
+  double* r_rank = (double*)dyn + (size_t)L.rcap * KE_WAVE + lane;    // [rcap][64]
+  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * KE_WAVE * 16) + lane;  // [rcap][64] node | tie << 16
+
+  __syncthreads();  // the previous task of this wavefront is done with LDS
+  for (int i = lane; i < n; i += KE_WAVE) l_node[i] = ((const uint64_t*)cv.node)[i];
+  for (int i = lane; i < n_succ_all; i += KE_WAVE) l_succ[i] = cv.succ[i];
+  __syncthreads();
+
+  const uint64_t pi = L.perm[w * KE_WAVE + lane];
+  if (pi == KE_IDLE) return;
+  first_lane = __builtin_ctzll(__ballot(1));
+  KE_STAMP(0);
+
+  // ---- workspace rows of this lane
+  uint8_t* base = L.ws + (size_t)blockIdx.x * ke_ws_bytes(L.ws_nodes, L.ws_slots);
+  // per-lane contiguous block: time[nodes] rank[nodes] dur[slots] deg[nodes]
+  const size_t lane_bytes = ke_ws_bytes(L.ws_nodes, L.ws_slots) / KE_WAVE;
+  uint8_t* lbase = base + (size_t)lane * lane_bytes;
+  double* g_time = (double*)lbase;
+  double* g_rank = g_time + L.ws_nodes;
+  double* g_dur = g_rank + L.ws_nodes;
+  uint8_t* g_deg = (uint8_t*)(g_dur + L.ws_slots);
+
+  // ---- plan fields -> LDS
+  const PlanHead h = load_head(L.head, L.stride, pi);
+  const rpeg_struct_t& st = P.st[cv.h->structure];   // uniform (the class fixes the structure)
+  const int nv = st.n_vertex;
+  for (int f = 0; f < nv * RPEG_FIELDS; ++f) l_plan[f * KE_WAVE] = L.vert[(uint64_t)f * L.stride + pi];
+
+  VPlan a[RPEG_MAX_V];
+#pragma unroll
+  for (int v = 0; v < RPEG_MAX_V; ++v)
+    if (v < nv) a[v] = ke_vplan(l_plan, v);
+
+  // ---- per-plan relations
+  const PlanMasks pm = plan_masks(a, nv);
+  const uint64_t dpne = pm.dpne;
+
+  KE_STAMP(1);
+  // ---- durations of the class's slots
+  bool err = cv.h->error != 0, zero_div = false;
+  const int split = (int)cv.h->split;
+  for (int s = 0; s < n_slots; ++s) g_dur[s] = ke_slot_duration(P, st, split, cv.slot[s], l_plan, &zero_div);
+  err = err || zero_div;
+
+  KE_STAMP(2);
+  // ---- memory model and gates (plan fields in LDS are dead after this point)
+#pragma unroll
+  for (int v = 0; v < RPEG_MAX_V; ++v)
+    if (v < nv) {
+      const VMem m = vertex_memory(P, st.vertex[v], a[v]);
+      l_vm[(v * 4 + 0) * KE_WAVE] = (double)m.w_shard;
+      l_vm[(v * 4 + 1) * KE_WAVE] = m.mem_w;
+      l_vm[(v * 4 + 2) * KE_WAVE] = m.opt;
+      l_vm[(v * 4 + 3) * KE_WAVE] = m.extra;
+    }
+  const KeVMem kvm{l_vm};
+  const double peak = device_peak_max(P, st, cv.h->vorder, pm, kvm);
+  const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
+  const bool mem_ok = !(peak > P.cap);
+
+  KE_STAMP(3);
+  // ---- ranks: reverse topological pass, then chain inheritance (scheduler.py:71-100, 367-378)
+  for (int i = n - 1; i >= 0; --i) {
+    const int v = cv.topo[i];
+    const NodeRec nr = cv.node[v];
+    double best = 0.0;
+    for (int j = 0; j < nr.n_succ; ++j) {
+      const double r = g_rank[cv.succ[nr.succ_begin + j]];
+      best = r > best ? r : best;
+    }
+    g_rank[v] = g_dur[nr.slot] + best;
+  }
+  for (unsigned g = 0; g < cv.h->n_groups; ++g) {
+    const GroupRec gr = cv.group[g];
+    double top = g_rank[cv.gmember[gr.begin]];
+    for (int j = 1; j < gr.count; ++j) {
+      const double r = g_rank[cv.gmember[gr.begin + j]];
+      top = r > top ? r : top;
+    }
+    for (int j = 0; j < gr.count; ++j) g_rank[cv.gmember[gr.begin + j]] = top;
+  }
+  for (int v = 0; v < n; ++v) {
+    g_deg[v] = cv.node[v].indeg;
+    g_time[v] = 0.0;
+  }
+
+  KE_STAMP(4);
+  // ---- list scheduling
+  double lf[RPEG_MAX_V];
+#pragma unroll
+  for (int x = 0; x < RPEG_MAX_V; ++x) lf[x] = 0.0;
+  int n_ready = 0, done = 0;
+  uint32_t tie = 0;
+  const int rcap = (int)L.rcap;
+  for (unsigned i = 0; i < cv.h->n_init && !err; ++i) {
+    const int v = cv.init[i];
+    if (n_ready >= rcap) { err = true; break; }
+    r_key[n_ready * KE_WAVE] = 0.0;
+    r_rank[n_ready * KE_WAVE] = g_rank[v];
+    r_nt[n_ready * KE_WAVE] = (uint32_t)v | ((uint32_t)cv.node[v].ptkey << 12) | (tie++ << 16);
+    ++n_ready;
+  }
+  double makespan = 0.0;
+  const long guard_max = (long)n * n + 64;
+  long guard_total = 0;
+  for (long guard = 0; !err && done < n && guard < guard_max; ++guard) {
+    ++guard_total;
+    if (n_ready == 0 || tie >= 0xFFF0u) { err = true; break; }
+    // arg-min of (est, comm_prio*8+topo_idx, -rank, tie) over the ready list, eight entries per
+    // batch of LDS loads (entries past n_ready are in bounds and ignored)
+    int bj = 0;
+    double bk = __builtin_inf(), br = 0.0;
+    uint32_t bm = 0;
+    for (int j0 = 0; j0 < n_ready; j0 += 8) {
+      double k[8], r[8];
+      uint32_t m[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        k[u] = r_key[(j0 + u) * KE_WAVE];
+        r[u] = r_rank[(j0 + u) * KE_WAVE];
+        m[u] = r_nt[(j0 + u) * KE_WAVE];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (j0 + u >= n_ready) continue;
+        bool better = k[u] < bk;
+        if (k[u] == bk) {
+          const unsigned pa = (m[u] >> 12) & 15u, pb = (bm >> 12) & 15u;
+          better = pa != pb ? pa < pb : (r[u] > br || (r[u] == br && (m[u] >> 16) < (bm >> 16)));
+        }
+        if (better) { bj = j0 + u; bk = k[u]; br = r[u]; bm = m[u]; }
+      }
+    }
+    const int bv = (int)(bm & 0xFFFu);
+    const uint64_t nbits = l_node[bv];
+    NodeRec nr;
+    __builtin_memcpy(&nr, &nbits, 8);
+    const unsigned blocked = blocked_mask(nr, dpne);
+    const double dev = ke_dev_max(blocked, lf);
+    const double est = dev > bk ? dev : bk;
+    if (est > bk) {  // stale key: same entry, corrected est, fresh tie (scheduler.py:437-443)
+      r_key[bj * KE_WAVE] = est;
+      r_nt[bj * KE_WAVE] = (bm & 0xFFFFu) | (tie++ << 16);
+      continue;
+    }
+    // dispatch bv: issue every load of this step before using any of them
+    const double d = g_dur[nr.slot];
+    int wv[4];
+    double wt[4], wr[4];
+    uint8_t wd[4];
+    const int ns = nr.n_succ;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      wv[j] = j < ns ? (int)l_succ[nr.succ_begin + j] : 0;
+      if (j < ns) {
+        wt[j] = g_time[wv[j]];
+        wd[j] = g_deg[wv[j]];
+        wr[j] = g_rank[wv[j]];
+      }
+    }
+    // remove the entry: the last entry takes its place (order is carried by the tie field)
+    --n_ready;
+    if (bj != n_ready) {
+      r_key[bj * KE_WAVE] = r_key[n_ready * KE_WAVE];
+      r_rank[bj * KE_WAVE] = r_rank[n_ready * KE_WAVE];
+      r_nt[bj * KE_WAVE] = r_nt[n_ready * KE_WAVE];
+    }
+    const double fin = est + d;
+    makespan = fin > makespan ? fin : makespan;
+    ++done;
+    unsigned touched = 0;
+#pragma unroll
+    for (int x = 0; x < RPEG_MAX_V; ++x)
+      if ((blocked >> x) & 1u) touched |= mask_row(pm.ovl, x);
+#pragma unroll
+    for (int x = 0; x < RPEG_MAX_V; ++x)
+      if (((touched >> x) & 1u) && fin > lf[x]) lf[x] = fin;
+    for (int j0 = 0; j0 < ns; j0 += 4) {
+      if (j0 > 0) {  // rare: more than four successors
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          wv[j] = j0 + j < ns ? (int)l_succ[nr.succ_begin + j0 + j] : 0;
+          if (j0 + j < ns) {
+            wt[j] = g_time[wv[j]];
+            wd[j] = g_deg[wv[j]];
+            wr[j] = g_rank[wv[j]];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j0 + j >= ns) break;
+        const int wn = wv[j];
+        double t = fin > wt[j] ? fin : wt[j];
+        const uint8_t left = (uint8_t)(wd[j] - 1);
+        if (left == 0) {
+          uint64_t wb = l_node[wn];
+          NodeRec wrc;
+          __builtin_memcpy(&wrc, &wb, 8);
+          const double d2 = ke_dev_max(blocked_mask(wrc, dpne), lf);
+          t = d2 > t ? d2 : t;
+          if (n_ready >= rcap) { err = true; break; }
+          r_key[n_ready * KE_WAVE] = t;
+          r_rank[n_ready * KE_WAVE] = wr[j];
+          r_nt[n_ready * KE_WAVE] = (uint32_t)wn | ((uint32_t)wrc.ptkey << 12) | (tie++ << 16);
+          ++n_ready;
+        } else {
+          g_time[wn] = t;
+          g_deg[wn] = left;
+        }
+      }
+    }
+  }
+  if (done != n) err = true;
+  KE_STAMP(5);
+  if (L.prof) atomicMax(&L.prof[w * 8 + 7], ((unsigned long long)n << 32) | (unsigned long long)guard_total);
+
+  // ---- outputs
+  uint8_t mask = RPEG_MASK_VALID;
+  if (stale_ok) mask |= RPEG_MASK_STALE_OK;
+  if (mem_ok) mask |= RPEG_MASK_MEM_OK;
+  double out_makespan, out_score;
+  if (err || makespan == 0.0) {
+    out_makespan = out_score = __builtin_nan("");
+    mask |= RPEG_MASK_ERROR;
+  } else {
+    double score = P.score_num / makespan;
+    if (!mem_ok) score = score * oom_penalty(peak, P.cap);
+    if ((L.flags & RPEG_GATE_STALE) && !stale_ok) score = 0.0;
+    out_makespan = makespan;
+    out_score = score;
+  }
+  if (L.makespan) L.makespan[pi] = out_makespan;
+  if (L.peak) L.peak[pi] = peak;
+  if (L.score) L.score[pi] = out_score;
+  if (L.mask) L.mask[pi] = mask;
+  KE_STAMP(6);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace rpeg
+#endif

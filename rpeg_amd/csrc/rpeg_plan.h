@@ -41,23 +41,45 @@ RPEG_HD bool plan_valid(const rpeg_problem_t& P, const PlanHead& h, const VPlan*
 }
 
 // evaluate.py:115-140
-RPEG_HD bool stale_layout_ok(const rpeg_struct_t& st, const PlanHead& h, const VPlan* a) {
+RPEG_HD bool stale_layout_ok(const rpeg_struct_t& st, const PlanHead& h, uint64_t ovl) {
   for (int p = 0; p < st.n_pub; ++p) {
     int tau = st.pub[p].tau_slot == 0 ? h.tau0 : h.tau1;
     if (tau <= 0) continue;
-    if (!alloc_disjoint(a[st.pub[p].src], a[st.pub[p].dst])) return false;
+    if ((ovl >> (8 * st.pub[p].src + st.pub[p].dst)) & 1ull) return false;
   }
   return true;
 }
 
-RPEG_HD void overlap_rows(const rpeg_struct_t& st, const VPlan* a, uint8_t* ovl) {
-  for (int v = 0; v < st.n_vertex; ++v) {
-    unsigned m = 0;
-    for (int w = 0; w < st.n_vertex; ++w)
-      if (!alloc_disjoint(a[v], a[w])) m |= 1u << w;
-    ovl[v] = (uint8_t)m;
+// Pair relations of one plan.  The loops run over the compile-time vertex bound so that `a` is only
+// ever indexed statically (register-resident on the device).
+RPEG_HD PlanMasks plan_masks(const VPlan* a, int nv) {
+  PlanMasks m;
+  m.ovl = m.eq = m.dpne = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+#endif
+  for (int u = 0; u < RPEG_MAX_V; ++u) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+#endif
+    for (int v = 0; v < RPEG_MAX_V; ++v) {
+      if (u >= nv || v >= nv) continue;
+      const uint64_t bit = 1ull << (8 * u + v);
+      if (!alloc_disjoint(a[u], a[v])) m.ovl |= bit;
+      if (alloc_equal(a[u], a[v])) m.eq |= bit;
+      if (a[u].dp != a[v].dp) m.dpne |= bit;
+    }
   }
+  return m;
 }
+
+struct VMemArray {   // host-side accessor over an array of VMem
+  const VMem* vm;
+  RPEG_HD double w_shard(int v) const { return (double)vm[v].w_shard; }
+  RPEG_HD double mem_w(int v) const { return vm[v].mem_w; }
+  RPEG_HD double opt(int v) const { return vm[v].opt; }
+  RPEG_HD double extra(int v) const { return vm[v].extra; }
+};
 
 // Everything after the class is known.  MEM additionally provides set_dur(slot, value).
 template <class MEM>
@@ -66,16 +88,18 @@ RPEG_HD PlanOut eval_plan(const rpeg_problem_t& P, const ClassView& c, const Pla
   const rpeg_struct_t& st = P.st[h.structure];
   PlanOut out;
   bool err = c.h->error != 0, zero_div = false;
+  const PlanMasks pm = plan_masks(a, st.n_vertex);
   uint8_t ovl[RPEG_MAX_V];
-  overlap_rows(st, a, ovl);
+  for (int v = 0; v < RPEG_MAX_V; ++v) ovl[v] = (uint8_t)mask_row(pm.ovl, v);
   for (unsigned s = 0; s < c.h->n_slots; ++s) mem.set_dur(s, slot_duration(P, st, h.split, c.slot[s], a, &zero_div));
   err = err || zero_div;
   double makespan = 0.0;
-  if (!err) makespan = list_schedule(c, mem, ovl, dp_differs(a, st.n_vertex), st.n_vertex, ready_cap, &err);
+  if (!err) makespan = list_schedule(c, mem, ovl, pm.dpne, st.n_vertex, ready_cap, &err);
   VMem vm[RPEG_MAX_V];
   for (int v = 0; v < st.n_vertex; ++v) vm[v] = vertex_memory(P, st.vertex[v], a[v]);
-  const double peak = device_peak_max(P, st, a, vm, c.h->vorder, ovl);
-  const bool stale_ok = stale_layout_ok(st, h, a);
+  const VMemArray vma{vm};
+  const double peak = device_peak_max(P, st, c.h->vorder, pm, vma);
+  const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
   const bool mem_ok = !(peak > P.cap);
   uint8_t mask = RPEG_MASK_VALID;
   if (stale_ok) mask |= RPEG_MASK_STALE_OK;

@@ -22,7 +22,7 @@ _lib = None
 
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
-           "rpeg_engine_last_kernel_ms", "rpeg_device_exp")
+           "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes")
 
 
 class EngineError(RuntimeError):
@@ -57,6 +57,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_set_timing.argtypes = [vp, i32]
     lib.rpeg_engine_last_kernel_ms.restype = C.c_double
     lib.rpeg_engine_last_kernel_ms.argtypes = [vp]
+    lib.rpeg_engine_reset_classes.restype = C.c_int
+    lib.rpeg_engine_reset_classes.argtypes = [vp]
     lib.rpeg_device_exp.restype = C.c_int
     lib.rpeg_device_exp.argtypes = [vp, u64, vp, vp, vp]
     if path is None:
@@ -114,6 +116,9 @@ class Engine:
 
     def set_timing(self, on: bool):
         self.lib.rpeg_engine_set_timing(self._h, int(on))
+
+    def reset_classes(self):
+        self.lib.rpeg_engine_reset_classes(self._h)
 
     def last_kernel_ms(self) -> float:
         return float(self.lib.rpeg_engine_last_kernel_ms(self._h))
