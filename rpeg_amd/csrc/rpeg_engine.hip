@@ -400,21 +400,30 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
     ++counts[last_id];
   }
   // every class starts on a wavefront boundary; the lanes left over are idle
-  std::vector<uint32_t> start(counts.size() + 1, 0);
-  for (size_t c = 0; c < counts.size(); ++c) start[c + 1] = start[c] + (counts[c] + WAVE - 1) / WAVE * WAVE;
+  // classes with the largest graphs first: their wavefronts run longest and should not start last
+  std::vector<uint32_t> order(counts.size());
+  for (size_t c = 0; c < counts.size(); ++c) order[c] = (uint32_t)c;
+  std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+    return ((const ClassHdr*)(e->pool.data() + offs[a]))->n_nodes > ((const ClassHdr*)(e->pool.data() + offs[b]))->n_nodes;
+  });
+  std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0);
+  for (size_t k = 0; k < order.size(); ++k) {
+    first[order[k]] = start[k];
+    start[k + 1] = start[k] + (counts[order[k]] + WAVE - 1) / WAVE * WAVE;
+  }
   const uint64_t n_sorted = start.back();
   e->stats[0] = counts.size();
   e->stats[1] = n_new;
   if (n_sorted == 0) return 0;
   if (int rc = ensure_perm(e, n_sorted)) return rc;
   std::fill(e->h_perm, e->h_perm + n_sorted, IDLE_LANE);
-  std::vector<uint32_t> cursor(start.begin(), start.end() - 1);
+  std::vector<uint32_t> cursor(first);
   for (uint64_t i = 0; i < n; ++i) {
     if (ids[i] == UINT32_MAX) continue;
     e->h_perm[cursor[ids[i]]++] = (uint32_t)i;
   }
-  for (size_t c = 0; c < counts.size(); ++c)
-    for (uint32_t w = start[c] / WAVE; w < start[c + 1] / WAVE; ++w) e->h_cls[w] = offs[c];
+  for (size_t k = 0; k < order.size(); ++k)
+    for (uint32_t w = start[k] / WAVE; w < start[k + 1] / WAVE; ++w) e->h_cls[w] = offs[order[k]];
   if (int rc = ensure_pool(e, s)) return rc;
   HIP_TRY(e, hipMemcpyAsync(e->d_perm, e->h_perm, n_sorted * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted / WAVE * 4, hipMemcpyHostToDevice, s));
