@@ -61,6 +61,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
+                    help="also run one device-to-device copy of this size (reference dispatch for scaling "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every box of this build has one MI355X and the path needs no "
@@ -115,6 +118,12 @@ def main():
     eng.set_timing(False)
     kernel_ms = sum(k_ms) / len(k_ms)
     stats = eng.stats()
+
+    if args.copy_probe:
+        src = torch.ones(args.copy_probe << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     mask = out["mask"].cpu().numpy()
     score = out["score"].cpu().numpy()
