@@ -21,6 +21,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 FP64_PEAK_TFLOPS = 78.6     # MI355X vector FP64, published
 # algorithmic bytes per plan: int16 plan fields (10 per vertex) + 4 header bytes in, 3 doubles + 1 mask byte out
 ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
+# HBM bytes per launch of k_eval measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB
+# copy (profiles/k_eval_cfg2_grpo_65536.md); None where no counter run exists
+MEASURED_TRAFFIC = {2: 706.5e6}
 # algorithmic fp64 operations per plan (cost model + scheduler + memory model of the fully split DAG)
 ALG_FLOPS = {1: 3.7e3, 2: 2.5e3, 3: 6.0e3, 4: 0.83e3, 5: 3.7e3}
 
@@ -125,6 +128,13 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
 
+    # the same step when the caller hands over host buffers: H2D of the plan tensors, D2H of the results
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        eng.eval(batch)
+    pcie_ms = (time.perf_counter() - t0) / 3 * 1e3
+
     mask = out["mask"].cpu().numpy()
     score = out["score"].cpu().numpy()
     valid = (mask & abi.MASK_VALID) != 0
@@ -140,11 +150,12 @@ def main():
                    "device_mesh": [cfg.problem.device_space.R, cfg.problem.device_space.N, cfg.problem.device_space.G],
                    "classes": stats["classes"], "inputs": "resident in HBM", "outputs": "left in HBM"},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(c),
                      "kernel": "k_eval", "kernel_ms": kernel_ms, "algorithmic_bytes_per_plan": ALG_BYTES[c]},
         "fp64_valu": {"achieved": achieved_tflops, "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
                       "frac": achieved_tflops / FP64_PEAK_TFLOPS, "algorithmic_flops_per_plan": ALG_FLOPS[c]},
         "kernel_only_evals_per_s": n / (kernel_ms * 1e-3),
+        "pcie_inclusive_ms_per_step": pcie_ms, "pcie_inclusive_evals_per_s": n / (pcie_ms * 1e-3),
         "first_call_ms": first_call_ms, "cold_ms_per_step": cold_ms, "cold_evals_per_s": n / (cold_ms * 1e-3),
         "feasible_fraction": float(((mask & abi.MASK_MEM_OK) != 0)[valid].mean()),
         "best_plan": int(score.argmax()), "best_score": float(score.max()),
