@@ -155,6 +155,16 @@ const char* rpeg_last_error(const rpeg_engine_t* e);
 int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
                     double* makespan, double* peak, double* score, uint8_t* mask, void* stream);
 
+/* rpeg_eval_batch plus the critical-chain mass of every plan: what move_gen derives from (trace,
+   lowered) of the current plan to bias its choice of vertex (_critical_chain and _critical_mass,
+   RPEG/search/moves.py:590-642).  mass[i*RPEG_MAX_V + v] = summed finish - start of the operator nodes
+   of vertex v on the chain that follows, from the first node of largest finish time backwards, the
+   first predecessor of largest finish time; summed from the sink backwards (the reference sums in the
+   iteration order of a set of string-hashed nodes, which differs between processes).  Device array of
+   n*RPEG_MAX_V doubles. */
+int rpeg_eval_batch_mass(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
+                         double* makespan, double* peak, double* score, uint8_t* mask, double* mass, void* stream);
+
 /* Single-node durations and isolated peaks: the batched form of the candidate-directory loop
    (RPEG/search/moves.py:532-549): for strategy i, time = NodeCostModel.time(mock node) and
    peak = NodeMemoryModel.peak_bytes(mock node) of vertex `vertex` of structure `structure` placed at
@@ -173,6 +183,48 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
                     double* start, double* finish, int32_t* node_kind, int32_t* node_vertex,
                     int32_t* node_step, int32_t* node_sub, int32_t* node_src, int32_t* edges,
                     int32_t* n_edges, int32_t cap);
+
+/* Batched simulated annealing: n_chains independent Metropolis-Hastings chains of n_steps steps.  One
+   step of a chain is one iteration of the inner loop of optimize() (RPEG/search/optimizer.py:702-930):
+   with probability alpha_pair*min(1,T/T_init) a donor/receiver proposal (multi_move_pair,
+   moves.py:845-950), else up to K_x single-vertex proposals (move_gen, moves.py:645-825); the
+   candidates of ALL chains are evaluated in one rpeg_eval_batch_mass launch (the reference maps
+   _eval_worker over one chain's candidates, optimizer.py:793-798); best of K, one acceptance test,
+   restart from the chain's best elite plan at T_warm after stag_window consecutive rejections
+   (optimizer.py:632-694, 932-936).  Draws come from a counter-based generator keyed by (seed, chain,
+   step), not from MT19937.  Chain c uses staleness variant c % n_variants.  Host memory throughout. */
+typedef struct rpeg_sa_params_s {
+  int32_t n_chains, n_steps, K_x, T_max, K_elite, stag_window, restart_attempts;
+  int32_t gate_candidates;    /* 1: apply the stale-layout gate to candidates too (evaluate_cached);
+                                 0: as _eval_worker, which the reference uses for candidates        */
+  int32_t geometric_cooling;  /* OptimizerConfig.geometric_cooling (optimizer.py:77)                 */
+  int32_t structure, split, n_variants;
+  uint8_t tau[8][2];          /* staleness of the (up to 2) trainable models per variant             */
+  double T_init, T_warm, T_min, T_cool, alpha_pair, score_eps;
+  uint64_t seed;
+  int32_t dir_n[RPEG_MAX_V];  /* candidate directory (moves.py:464-551): entries per vertex ...      */
+  const int16_t* dir[RPEG_MAX_V]; /* ... rows of dp pp tp r_ext n_ext mb, ascending by time          */
+} rpeg_sa_params_t;
+
+typedef struct rpeg_sa_result_s {   /* per-chain arrays of n_chains elements, any may be NULL */
+  int16_t* best_plan;      /* [RPEG_MAX_V*RPEG_FIELDS] per chain: best feasible plan, else best plan   */
+  double* best_score;
+  int32_t* best_step;      /* step at which it was first seen (-1: the start plan)                    */
+  double* best_time;       /* seconds from the start of the run until then                            */
+  uint8_t* best_feasible;  /* 1 when best_* describe a memory-feasible plan                           */
+  int16_t* cur_plan;
+  double* cur_score;
+  int32_t* restarts;
+  int64_t* n_eval;
+  uint8_t* dead;           /* chain stopped: no valid restart found                                   */
+  uint8_t* log;            /* [n_chains][n_steps]: kind (0 single, 1 pair) | candidates << 1 |
+                              verdict << 4 (0 none, 1 rejected, 2 accepted) | restart << 6            */
+  double wall_s, eval_s;   /* whole run / time inside the batched evaluations                         */
+  int64_t n_launch, n_plans;
+} rpeg_sa_result_t;
+
+int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* params, const int16_t* base_plan,
+                rpeg_sa_result_t* result, void* stream);
 
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] kernel-C dynamic LDS bytes, [4] workspace bytes. */

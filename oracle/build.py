@@ -13,7 +13,7 @@ OUT = os.path.join(HERE, "_build", "libcpu_port.so")
 def build(force: bool = False) -> str:
     src = os.path.join(HERE, "cpu_port.cpp")
     deps = [src] + [os.path.join(HERE, "..", "rpeg_amd", "csrc", f) for f in
-                    ("rpeg_core.h", "rpeg_class.h", "rpeg_lower.h", "rpeg_plan.h", "rpeg_exp_table.inc")]
+                    ("rpeg_core.h", "rpeg_class.h", "rpeg_lower.h", "rpeg_plan.h", "rpeg_sa.h", "rpeg_exp_table.inc")]
     deps.append(os.path.join(HERE, "..", "include", "rpeg_eval.h"))
     if not force and os.path.exists(OUT) and all(os.path.getmtime(OUT) >= os.path.getmtime(d) for d in deps):
         return OUT

@@ -14,6 +14,7 @@
 
 #include "../rpeg_amd/csrc/rpeg_lower.h"
 #include "../rpeg_amd/csrc/rpeg_plan.h"
+#include "../rpeg_amd/csrc/rpeg_sa.h"
 
 using namespace rpeg;
 
@@ -66,7 +67,7 @@ long port_n_classes(void* h) { return (long)((Port*)h)->classes.size(); }
 // host arrays, same layout as the device tensors; returns 0 or -1
 int port_eval(void* h, uint64_t n, const int16_t* vert, const uint8_t* head, uint64_t stride, uint32_t flags,
               double* makespan, double* peak, double* score, uint8_t* mask, uint64_t* sig_out, int32_t* max_ready,
-              int threads) {
+              int threads, double* mass) {
   Port* e = (Port*)h;
   int rc = 0;
   int mr = 0;
@@ -89,8 +90,19 @@ int port_eval(void* h, uint64_t n, const int16_t* vert, const uint8_t* head, uin
         ClassView cv = class_view(lc->blob.data());
         HostMem mem;
         mem.fit(cv.h);
+        std::vector<double> ts, tf;
+        if (mass) {
+          ts.assign(cv.h->n_nodes, 0.0); tf.assign(cv.h->n_nodes, 0.0);
+          mem.trace_start = &ts; mem.trace_finish = &tf;
+        }
         o = eval_plan(e->P, cv, ph, a, mem, (int)cv.h->n_nodes + 1, flags);
         if (mem.max_ready > mr) mr = mem.max_ready;
+        if (mass) {
+          double m[RPEG_MAX_V];
+          if (o.mask & RPEG_MASK_ERROR) for (double& x : m) x = NAN;
+          else critical_mass(cv, [&](int k) { return tf[k]; }, [&](int k) { return ts[k]; }, m);
+          for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = m[x];
+        }
       } catch (const std::exception& ex) {
 #pragma omp critical
         { e->err = ex.what(); rc = -1; }
@@ -103,6 +115,8 @@ int port_eval(void* h, uint64_t n, const int16_t* vert, const uint8_t* head, uin
     if (score) score[i] = o.score;
     if (mask) mask[i] = o.mask;
     if (sig_out) sig_out[i] = sig;
+    if (mass && sig == SIG_INVALID)
+      for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = NAN;
   }
   if (max_ready) *max_ready = mr;
   return rc;
@@ -151,6 +165,111 @@ int port_op_time(void* h, uint64_t n, int structure, int vertex, const int16_t* 
     peak[i] = isolated_peak(st.vertex[vertex], vertex_memory(e->P, st.vertex[vertex], a));
   }
   return 0;
+}
+
+// ---- simulated annealing: the host logic of rpeg_sa.h with this CPU evaluator behind it
+namespace {
+struct CpuSaBackend : SaBackend {
+  Port* e;
+  uint8_t head_of[8][4];
+  int threads = 1;
+  int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override {
+    const size_t V = RPEG_MAX_V * RPEG_FIELDS;
+    std::vector<int16_t> vert(V * n);
+    std::vector<uint8_t> head(4 * (size_t)n), mask(n);
+    std::vector<double> score(n), mass((size_t)n * RPEG_MAX_V);
+    for (int i = 0; i < n; ++i) {
+      const int16_t* f = &plans[i].f[0][0];
+      for (size_t x = 0; x < V; ++x) vert[x * n + i] = f[x];
+      for (int x = 0; x < 4; ++x) head[(size_t)x * n + i] = head_of[variant[i]][x];
+    }
+    int rc = port_eval(e, n, vert.data(), head.data(), n, 0u, nullptr, nullptr, score.data(), mask.data(), nullptr,
+                       nullptr, threads, mass.data());
+    for (int i = 0; i < n; ++i) {
+      out[i].score = score[i];
+      out[i].mask = mask[i];
+      for (int x = 0; x < RPEG_MAX_V; ++x) out[i].mass[x] = mass[(size_t)i * RPEG_MAX_V + x];
+    }
+    return rc;
+  }
+};
+
+void sa_context(Port* e, const rpeg_sa_params_t* prm, SaContext& cx) {
+  cx.init(e->P, prm->structure);
+  for (int v = 0; v < cx.nv; ++v) cx.set_directory(v, prm->dir[v], prm->dir_n[v]);
+}
+}  // namespace
+
+int port_sa_run(void* h, const rpeg_sa_params_t* prm, const int16_t* base_plan, rpeg_sa_result_t* res, int threads) {
+  Port* e = (Port*)h;
+  SaContext cx;
+  sa_context(e, prm, cx);
+  SaSettings st;
+  st.n_chains = prm->n_chains; st.n_steps = prm->n_steps; st.K_x = prm->K_x; st.T_max = prm->T_max;
+  st.K_elite = prm->K_elite; st.stag_window = prm->stag_window; st.restart_attempts = prm->restart_attempts;
+  st.gate_candidates = prm->gate_candidates; st.geometric_cooling = prm->geometric_cooling;
+  st.n_variants = prm->n_variants; st.T_init = prm->T_init; st.T_warm = prm->T_warm; st.T_min = prm->T_min;
+  st.T_cool = prm->T_cool; st.alpha_pair = prm->alpha_pair; st.score_eps = prm->score_eps; st.seed = prm->seed;
+  CpuSaBackend be;
+  be.e = e; be.threads = threads;
+  for (int k = 0; k < prm->n_variants; ++k) {
+    be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
+    be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];
+  }
+  SaRun run(cx, st, be);
+  SaPlan base;
+  if (base_plan) std::memcpy(&base, base_plan, sizeof base);
+  if (int rc = run.run(base_plan ? &base : nullptr)) return rc;
+  const size_t V = RPEG_MAX_V * RPEG_FIELDS;
+  for (int c = 0; c < st.n_chains; ++c) {
+    const SaChain& ch = run.chains[c];
+    const bool feas = ch.has_feasible;
+    const SaEntry& b = feas ? ch.best_feasible : ch.best;
+    if (res->best_plan) std::memcpy(res->best_plan + c * V, &b.plan, V * 2);
+    if (res->best_score) res->best_score[c] = feas ? ch.best_feasible_score : (ch.has_best ? ch.best_score : NAN);
+    if (res->best_step) res->best_step[c] = feas ? ch.best_feasible_step : ch.best_step;
+    if (res->best_time) res->best_time[c] = feas ? ch.best_feasible_time : -1.0;
+    if (res->best_feasible) res->best_feasible[c] = feas;
+    if (res->cur_plan) std::memcpy(res->cur_plan + c * V, &ch.cur.plan, V * 2);
+    if (res->cur_score) res->cur_score[c] = ch.score;
+    if (res->restarts) res->restarts[c] = ch.restarts;
+    if (res->n_eval) res->n_eval[c] = ch.n_eval;
+    if (res->dead) res->dead[c] = ch.dead;
+  }
+  if (res->log) std::memcpy(res->log, run.log.data(), run.log.size());
+  res->wall_s = run.now();
+  return 0;
+}
+
+// single proposals with the stream (seed, a, b, c): what = 0 move_gen, 1 pair, 2 region sample of vertex `v`
+// in racks [r_lo, r_hi).  Returns the number of plans (or rows) written; *draws = words consumed (in: words
+// to skip).
+int port_sa_propose(void* h, const rpeg_sa_params_t* prm, int what, uint64_t seed, uint64_t a, uint64_t b, uint64_t c,
+                    const int16_t* plan, const double* mass, double T, int v, int r_lo, int r_hi, int16_t* out,
+                    int64_t* draws, int32_t* fallback) {
+  Port* e = (Port*)h;
+  SaContext cx;
+  sa_context(e, prm, cx);
+  SaRng rng(seed, a, b, c);
+  if (draws) rng.k = (uint64_t)*draws;   // continue a stream
+  SaPlan cur;
+  if (plan) std::memcpy(&cur, plan, sizeof cur);
+  int n = 0;
+  int fb = 0;
+  if (what == 0) {
+    std::vector<SaPlan> o(prm->K_x);
+    n = sa_move_gen(rng, cx, cur, mass, prm->K_x, prm->T_max, T, prm->T_init, o.data(), &fb);
+    std::memcpy(out, o.data(), sizeof(SaPlan) * n);
+  } else if (what == 1) {
+    SaPlan o;
+    n = sa_move_pair(rng, cx, cur, &o) ? 1 : 0;
+    if (n) std::memcpy(out, &o, sizeof o);
+  } else {
+    n = sa_sample_region(rng, cx, v, r_lo, r_hi, out) ? 1 : 0;
+  }
+  if (draws) *draws = (int64_t)rng.k;
+  if (fallback) *fallback = fb;
+  return n;
 }
 
 void port_exp(uint64_t n, const double* x, double* y) {

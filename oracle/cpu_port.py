@@ -28,7 +28,13 @@ def lib():
         _lib.port_n_classes.argtypes = [C.c_void_p]
         _lib.port_eval.restype = C.c_int
         _lib.port_eval.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint32] + \
-            [C.c_void_p] * 6 + [C.c_int]
+            [C.c_void_p] * 6 + [C.c_int, C.c_void_p]
+        _lib.port_sa_run.restype = C.c_int
+        _lib.port_sa_run.argtypes = [C.c_void_p] * 4 + [C.c_int]
+        _lib.port_sa_propose.restype = C.c_int
+        _lib.port_sa_propose.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_uint64,
+                                         C.c_uint64, C.c_void_p, C.c_void_p, C.c_double, C.c_int, C.c_int, C.c_int,
+                                         C.c_void_p, C.c_void_p, C.c_void_p]
         _lib.port_lower.restype = C.c_int
         _lib.port_lower.argtypes = [C.c_void_p] * 9 + [C.c_int32, C.c_void_p]
         _lib.port_op_time.restype = C.c_int
@@ -52,16 +58,19 @@ class CpuPort:
     def n_classes(self):
         return lib().port_n_classes(self.h)
 
-    def eval(self, batch, flags=0, threads=1):
+    def eval(self, batch, flags=0, threads=1, want_mass=False):
         n = batch.n
         vert = np.ascontiguousarray(batch.vert)
         head = np.ascontiguousarray(batch.head)
         out = dict(makespan=np.empty(n), peak=np.empty(n), score=np.empty(n), mask=np.empty(n, np.uint8),
                    sig=np.empty(n, np.uint64))
         mr = C.c_int32(0)
+        if want_mass:
+            out["mass"] = np.empty((n, abi.MAX_V))
         rc = lib().port_eval(self.h, n, vert.ctypes.data, head.ctypes.data, n, flags,
                              out["makespan"].ctypes.data, out["peak"].ctypes.data, out["score"].ctypes.data,
-                             out["mask"].ctypes.data, out["sig"].ctypes.data, C.addressof(mr), threads)
+                             out["mask"].ctypes.data, out["sig"].ctypes.data, C.addressof(mr), threads,
+                             out["mass"].ctypes.data if want_mass else None)
         if rc != 0:
             raise RuntimeError(lib().port_error(self.h).decode())
         out["max_ready"] = mr.value
@@ -80,6 +89,59 @@ class CpuPort:
             raise RuntimeError(f"port_lower failed ({n}): {lib().port_error(self.h).decode()}")
         return dict(kind=kind[:n], vertex=vertex[:n], step=step[:n], sub=sub[:n], dur=dur[:n],
                     edges=edges[:2 * ne.value].reshape(-1, 2))
+
+    @staticmethod
+    def _set_directory(params, directory):
+        keep = []
+        for v in range(abi.MAX_V):
+            if v < len(directory):
+                a = np.ascontiguousarray(directory[v], dtype=np.int16).reshape(-1, 6)
+                keep.append(a)
+                params.dir_n[v] = a.shape[0]
+                params.dir[v] = a.ctypes.data
+            else:
+                params.dir_n[v] = 0
+                params.dir[v] = None
+        return keep
+
+    def sa_run(self, params, directory, base_plan=None, threads=1):
+        """The host annealing logic of rpeg_amd/csrc/rpeg_sa.h over this CPU evaluator."""
+        keep = self._set_directory(params, directory)
+        nc, ns = params.n_chains, params.n_steps
+        W = abi.MAX_V * abi.FIELDS
+        out = dict(best_plan=np.zeros((nc, W), np.int16), best_score=np.zeros(nc), best_step=np.zeros(nc, np.int32),
+                   best_time=np.zeros(nc), best_feasible=np.zeros(nc, np.uint8), cur_plan=np.zeros((nc, W), np.int16),
+                   cur_score=np.zeros(nc), restarts=np.zeros(nc, np.int32), n_eval=np.zeros(nc, np.int64),
+                   dead=np.zeros(nc, np.uint8), log=np.zeros((nc, max(ns, 1)), np.uint8))
+        res = abi.SaResultT()
+        for k, a in out.items():
+            setattr(res, k, a.ctypes.data)
+        base = None if base_plan is None else np.ascontiguousarray(base_plan, dtype=np.int16).reshape(W)
+        rc = lib().port_sa_run(self.h, C.addressof(params), base.ctypes.data if base is not None else None,
+                               C.addressof(res), threads)
+        if rc != 0:
+            raise RuntimeError(f"port_sa_run failed ({rc}): {lib().port_error(self.h).decode()}")
+        del keep
+        out["log"] = out["log"][:, :ns]
+        out["wall_s"] = res.wall_s
+        return out
+
+    def sa_propose(self, params, directory, what, stream, plan=None, mass=None, T=0.0, v=0, r_lo=0, r_hi=0, skip=0):
+        """One proposal with generator stream (seed, a, b, c): what = 0 move_gen, 1 donor/receiver pair,
+        2 region sample.  Returns (rows [n, MAX_V*10] or [n, 10], words drawn so far, fallback count)."""
+        keep = self._set_directory(params, directory)
+        W = abi.MAX_V * abi.FIELDS
+        out = np.zeros((max(params.K_x, 1), W), np.int16)
+        draws, fb = C.c_int64(skip), C.c_int32(0)
+        p = None if plan is None else np.ascontiguousarray(plan, dtype=np.int16).reshape(W)
+        m = None if mass is None else np.ascontiguousarray(mass, dtype=np.float64)
+        n = lib().port_sa_propose(self.h, C.addressof(params), what, *[int(x) for x in stream],
+                                  p.ctypes.data if p is not None else None, m.ctypes.data if m is not None else None,
+                                  float(T), v, r_lo, r_hi, out.ctypes.data, C.addressof(draws), C.addressof(fb))
+        del keep
+        if what == 2:
+            return out.reshape(-1)[:10 * n].reshape(n, 10), draws.value, fb.value
+        return out[:n], draws.value, fb.value
 
     def op_time(self, structure, vertex, strat):
         strat = np.ascontiguousarray(strat, dtype=np.int16)

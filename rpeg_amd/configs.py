@@ -24,6 +24,12 @@ SPEC_70B = ModelSpec(L=80, d=8192, d_ff=28672, V=128256)
 
 # memory_per_gpu that makes about 70 % of config 4's seeded candidates infeasible
 CFG4_MEMORY_PER_GPU = 1.03e11
+# Config 5 does not state its hardware block.  With the README's 1.03e11 B per device no plan of its
+# models fits at T = 16384 (the actor's generation stage alone needs 3.8e11 B whatever the strategy), the
+# candidate directory (RPEG/search/moves.py:532-541) is empty for four of the six vertices and the
+# reference's move_gen raises on the empty range.  8.0e11 is the smallest round figure at which every
+# vertex keeps at least 40 memory-feasible strategies.
+CFG5_MEMORY_PER_GPU = 8.0e11
 
 
 def readme_hardware(memory_per_gpu: float = 1.03e11) -> Hardware:
@@ -83,5 +89,5 @@ def config(i: int) -> BenchConfig:
                             Model.CRITIC: SPEC_7B, Model.AC_SHARE: SPEC_70B})
         wl = Workload(B=512, K=4, S=1024, T=16384, gen_quantiles=((0.5, 2048), (0.9, 8192), (1.0, 16384)))
         return _cfg("cfg5_ppo_sa_4x32x4", (PPO,), suite, wl, DeviceSpace(4, 32, 4), 5, 64 * 2000 * 6,
-                    {"ppo": ((0, 1), (0,))})
+                    {"ppo": ((0, 1), (0,))}, hw=readme_hardware(CFG5_MEMORY_PER_GPU))
     raise ValueError(f"no benchmark configuration {i}")

@@ -76,6 +76,7 @@ struct GroupRec { uint16_t begin, count; };  // sub-node chains that share the c
 struct ClassHdr {
   uint32_t n_nodes, n_slots, n_succ, n_init, n_groups, n_gmembers;
   uint32_t off_node, off_succ, off_init, off_topo, off_slot, off_group, off_gmember;  // byte offsets in the blob
+  uint32_t off_pbeg, off_pred;       // predecessor lists in edge order: pred[pbeg[v] .. pbeg[v+1])
   uint32_t bytes;
   uint32_t structure, split, error;  // error != 0: the reference would raise for this class
   uint8_t vorder[8];                 // vertices by first appearance among the lowered operator nodes
@@ -90,6 +91,8 @@ struct ClassView {
   const SlotDesc* slot;
   const GroupRec* group;
   const uint16_t* gmember;
+  const uint16_t* pbeg;
+  const uint16_t* pred;
 };
 
 RPEG_HD ClassView class_view(const uint8_t* blob) {
@@ -102,6 +105,8 @@ RPEG_HD ClassView class_view(const uint8_t* blob) {
   v.slot = (const SlotDesc*)(blob + v.h->off_slot);
   v.group = (const GroupRec*)(blob + v.h->off_group);
   v.gmember = (const uint16_t*)(blob + v.h->off_gmember);
+  v.pbeg = (const uint16_t*)(blob + v.h->off_pbeg);
+  v.pred = (const uint16_t*)(blob + v.h->off_pred);
   return v;
 }
 
@@ -241,6 +246,41 @@ RPEG_HD double list_schedule(const ClassView& c, MEM& mem, const uint8_t* ovl, u
 #endif
   if (done != n) *error = true;
   return makespan;
+}
+
+// Critical-chain mass per template vertex (RPEG/search/moves.py:590-642): from the first node of
+// largest finish time follow, at every node, the first predecessor (in edge order) of largest finish
+// time; a vertex's mass is the sum of finish - start over its operator nodes on that chain, added from
+// the sink backwards.  fin(i) / start(i) give the times of node i.
+template <class Fin, class Start>
+RPEG_HD void critical_mass(const ClassView& c, Fin fin, Start start, double (&mass)[RPEG_MAX_V]) {
+  for (int x = 0; x < RPEG_MAX_V; ++x) mass[x] = 0.0;
+  const int n = (int)c.h->n_nodes;
+  int cur = 0;
+  double best = fin(0);
+  for (int i = 1; i < n; ++i) {
+    const double f = fin(i);
+    if (f > best) { best = f; cur = i; }
+  }
+  for (int hops = 0; hops <= n; ++hops) {   // a chain visits a node at most once
+    const SlotDesc sd = c.slot[c.node[cur].slot];
+    if (sd.type <= SLOT_OP_SUB) {
+      const double d = best - start(cur);
+      for (int x = 0; x < RPEG_MAX_V; ++x)
+        if (x == (int)sd.a) mass[x] += d;
+    }
+    const int pb = c.pbeg[cur], pe = c.pbeg[cur + 1];
+    if (pb == pe) break;
+    int nx = c.pred[pb];
+    double bf = fin(nx);
+    for (int j = pb + 1; j < pe; ++j) {
+      const int q = c.pred[j];
+      const double f = fin(q);
+      if (f > bf) { bf = f; nx = q; }
+    }
+    cur = nx;
+    best = bf;
+  }
 }
 
 }  // namespace rpeg

@@ -25,6 +25,7 @@
 #include "rpeg_kernel_eval.h"
 #include "rpeg_lower.h"
 #include "rpeg_plan.h"
+#include "rpeg_sa.h"
 
 using namespace rpeg;
 
@@ -69,7 +70,7 @@ __host__ __device__ inline size_t wave_ws_bytes(uint32_t nodes, uint32_t slots) 
 
 __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
                             const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig,
-                            double* makespan, double* peak, double* score, uint8_t* mask) {
+                            double* makespan, double* peak, double* score, uint8_t* mask, double* mass) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   PlanHead h = load_head(head, stride, i);
@@ -84,6 +85,8 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
     if (peak) peak[i] = nan;
     if (score) score[i] = nan;
     if (mask) mask[i] = 0;
+    if (mass)
+      for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
     return;
   }
   sig[i] = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
@@ -272,6 +275,9 @@ static int ensure_ws(rpeg_engine_t* e, size_t bytes, hipStream_t s) {
   return 0;
 }
 
+static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                           double* peak, double* score, uint8_t* mask, double* mass, void* stream);
+
 extern "C" {
 
 int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
@@ -357,6 +363,18 @@ int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n) {
 
 int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                     double* peak, double* score, uint8_t* mask, void* stream) {
+  return eval_batch_impl(e, n, plans, flags, makespan, peak, score, mask, nullptr, stream);
+}
+
+int rpeg_eval_batch_mass(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                         double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
+  return eval_batch_impl(e, n, plans, flags, makespan, peak, score, mask, mass, stream);
+}
+
+}  // extern "C"
+
+static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                           double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
   if (!e || !plans) return -1;
   e->err.clear();
   e->last_ms = -1.0;
@@ -367,7 +385,7 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
   if (int rc = ensure_batch(e, n)) return rc;
   const unsigned blk = 256;
   hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + blk - 1) / blk)), dim3(blk), 0, s, e->dP, n, plans->vert,
-                     plans->head, plans->stride, e->d_sig, makespan, peak, score, mask);
+                     plans->head, plans->stride, e->d_sig, makespan, peak, score, mask, mass);
   HIP_TRY(e, hipGetLastError());
   HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
   HIP_TRY(e, hipStreamSynchronize(s));
@@ -442,6 +460,7 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
   if (e->max_nodes > 4095) { e->err = "class with more than 4095 nodes"; return -8; }
   L.rcap = 32;
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
+  L.mass = mass;
   L.prof = nullptr;
   if (e->prof_on) {
     if (e->d_prof) hipFree(e->d_prof);
@@ -471,6 +490,8 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
   }
   return 0;
 }
+
+extern "C" {
 
 int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t vertex, const int16_t* strat,
                        uint64_t stride, double* time, double* peak, void* stream) {
@@ -541,6 +562,143 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
     for (size_t j = 0; j < lc.edges.size(); ++j) { edges[2 * j] = lc.edges[j].first; edges[2 * j + 1] = lc.edges[j].second; }
   if (n_edges) *n_edges = (int32_t)lc.edges.size();
   return n;
+}
+
+}  // extern "C"
+
+// Evaluates the candidates of a simulated-annealing step on the GPU: plans are staged through pinned
+// host memory into structure-of-arrays device tensors, scored by the batch kernel (with critical-chain
+// masses) and read back in one synchronisation.
+namespace {
+struct GpuSaBackend : SaBackend {
+  rpeg_engine_t* e;
+  hipStream_t s;
+  int cap = 0;
+  uint8_t head_of[8][4];
+  int16_t *h_vert = nullptr, *d_vert = nullptr;
+  uint8_t *h_head = nullptr, *d_head = nullptr, *h_mask = nullptr, *d_mask = nullptr;
+  double *h_score = nullptr, *d_score = nullptr, *h_mass = nullptr, *d_mass = nullptr;
+  double eval_s = 0.0;
+  long n_launch = 0, n_plans = 0;
+  int rc_alloc = 0;
+
+  GpuSaBackend(rpeg_engine_t* eng, hipStream_t st, int capacity) : e(eng), s(st), cap(capacity) {
+    const size_t V = RPEG_MAX_V * RPEG_FIELDS;
+    bool ok = hipHostMalloc(&h_vert, V * cap * 2) == hipSuccess && hipMalloc(&d_vert, V * cap * 2) == hipSuccess &&
+              hipHostMalloc(&h_head, 4 * (size_t)cap) == hipSuccess && hipMalloc(&d_head, 4 * (size_t)cap) == hipSuccess &&
+              hipHostMalloc(&h_mask, cap) == hipSuccess && hipMalloc(&d_mask, cap) == hipSuccess &&
+              hipHostMalloc(&h_score, 8 * (size_t)cap) == hipSuccess && hipMalloc(&d_score, 8 * (size_t)cap) == hipSuccess &&
+              hipHostMalloc(&h_mass, 8 * (size_t)cap * RPEG_MAX_V) == hipSuccess &&
+              hipMalloc(&d_mass, 8 * (size_t)cap * RPEG_MAX_V) == hipSuccess;
+    if (!ok) { rc_alloc = -2; e->err = "out of memory for the annealing buffers"; }
+    else std::memset(h_vert, 0, V * cap * 2);
+  }
+  ~GpuSaBackend() override {
+    hipStreamSynchronize(s);
+    if (h_vert) hipHostFree(h_vert);
+    if (d_vert) hipFree(d_vert);
+    if (h_head) hipHostFree(h_head);
+    if (d_head) hipFree(d_head);
+    if (h_mask) hipHostFree(h_mask);
+    if (d_mask) hipFree(d_mask);
+    if (h_score) hipHostFree(h_score);
+    if (d_score) hipFree(d_score);
+    if (h_mass) hipHostFree(h_mass);
+    if (d_mass) hipFree(d_mass);
+  }
+
+  int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override {
+    if (n > cap) { e->err = "annealing batch exceeds its buffers"; return -1; }
+    const auto t0 = std::chrono::steady_clock::now();
+    const size_t V = RPEG_MAX_V * RPEG_FIELDS;
+    for (int i = 0; i < n; ++i) {
+      const int16_t* f = &plans[i].f[0][0];
+      for (size_t x = 0; x < V; ++x) h_vert[x * cap + i] = f[x];
+      for (int x = 0; x < 4; ++x) h_head[(size_t)x * cap + i] = head_of[variant[i]][x];
+    }
+    // rows are `cap` apart: copy the used prefix of every row in one strided copy
+    HIP_TRY(e, hipMemcpy2DAsync(d_vert, (size_t)cap * 2, h_vert, (size_t)cap * 2, (size_t)n * 2, V, hipMemcpyHostToDevice, s));
+    HIP_TRY(e, hipMemcpy2DAsync(d_head, cap, h_head, cap, n, 4, hipMemcpyHostToDevice, s));
+    rpeg_plan_soa_t soa{d_vert, d_head, (uint64_t)cap};
+    if (int rc = eval_batch_impl(e, (uint64_t)n, &soa, 0u, nullptr, nullptr, d_score, d_mask, d_mass, s)) return rc;
+    HIP_TRY(e, hipMemcpyAsync(h_score, d_score, 8 * (size_t)n, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipMemcpyAsync(h_mask, d_mask, n, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipMemcpyAsync(h_mass, d_mass, 8 * (size_t)n * RPEG_MAX_V, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipStreamSynchronize(s));
+    for (int i = 0; i < n; ++i) {
+      out[i].score = h_score[i];
+      out[i].mask = h_mask[i];
+      for (int x = 0; x < RPEG_MAX_V; ++x) out[i].mass[x] = h_mass[(size_t)i * RPEG_MAX_V + x];
+    }
+    eval_s += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    ++n_launch;
+    n_plans += n;
+    return 0;
+  }
+};
+}  // namespace
+
+extern "C" {
+
+int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* base_plan, rpeg_sa_result_t* res,
+                void* stream) {
+  if (!e || !prm || !res) return -1;
+  e->err.clear();
+  if (prm->structure < 0 || prm->structure >= e->P.n_struct || prm->split < 0 || prm->split >= e->P.n_split ||
+      prm->n_variants < 1 || prm->n_variants > 8 || prm->n_chains < 1 || prm->n_steps < 0 || prm->K_x < 1 ||
+      prm->K_x > 16 || prm->restart_attempts < 1 || prm->T_max < 0 || !(prm->T_init > 0.0)) {
+    e->err = "bad annealing parameters";
+    return -1;
+  }
+  SaContext cx;
+  cx.init(e->P, prm->structure);
+  for (int v = 0; v < cx.nv; ++v) {
+    if (prm->dir_n[v] < 0 || (prm->dir_n[v] > 0 && !prm->dir[v])) { e->err = "bad candidate directory"; return -1; }
+    if (const char* msg = cx.set_directory(v, prm->dir[v], prm->dir_n[v])) { e->err = msg; return -1; }
+  }
+  SaSettings st;
+  st.n_chains = prm->n_chains; st.n_steps = prm->n_steps; st.K_x = prm->K_x; st.T_max = prm->T_max;
+  st.K_elite = prm->K_elite; st.stag_window = prm->stag_window; st.restart_attempts = prm->restart_attempts;
+  st.gate_candidates = prm->gate_candidates; st.geometric_cooling = prm->geometric_cooling;
+  st.n_variants = prm->n_variants; st.T_init = prm->T_init; st.T_warm = prm->T_warm; st.T_min = prm->T_min;
+  st.T_cool = prm->T_cool; st.alpha_pair = prm->alpha_pair; st.score_eps = prm->score_eps; st.seed = prm->seed;
+  const int cap = prm->n_chains * std::max(prm->K_x, prm->restart_attempts);
+  GpuSaBackend be(e, (hipStream_t)stream, cap);
+  if (be.rc_alloc) return be.rc_alloc;
+  for (int k = 0; k < prm->n_variants; ++k) {
+    be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
+    be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];
+  }
+  SaRun run(cx, st, be);
+  SaPlan base;
+  if (base_plan) std::memcpy(&base, base_plan, sizeof base);
+  const bool was_timing = e->timing;
+  e->timing = false;
+  const int rc = run.run(base_plan ? &base : nullptr);
+  e->timing = was_timing;
+  if (rc) return rc;
+  const size_t V = RPEG_MAX_V * RPEG_FIELDS;
+  for (int c = 0; c < st.n_chains; ++c) {
+    const SaChain& ch = run.chains[c];
+    const bool feas = ch.has_feasible;
+    const SaEntry& b = feas ? ch.best_feasible : ch.best;
+    if (res->best_plan) std::memcpy(res->best_plan + c * V, &b.plan, V * 2);
+    if (res->best_score) res->best_score[c] = feas ? ch.best_feasible_score : (ch.has_best ? ch.best_score : __builtin_nan(""));
+    if (res->best_step) res->best_step[c] = feas ? ch.best_feasible_step : ch.best_step;
+    if (res->best_time) res->best_time[c] = feas ? ch.best_feasible_time : -1.0;
+    if (res->best_feasible) res->best_feasible[c] = feas;
+    if (res->cur_plan) std::memcpy(res->cur_plan + c * V, &ch.cur.plan, V * 2);
+    if (res->cur_score) res->cur_score[c] = ch.score;
+    if (res->restarts) res->restarts[c] = ch.restarts;
+    if (res->n_eval) res->n_eval[c] = ch.n_eval;
+    if (res->dead) res->dead[c] = ch.dead;
+  }
+  if (res->log) std::memcpy(res->log, run.log.data(), run.log.size());
+  res->wall_s = run.now();
+  res->eval_s = be.eval_s;
+  res->n_launch = be.n_launch;
+  res->n_plans = be.n_plans;
+  return 0;
 }
 
 int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream) {

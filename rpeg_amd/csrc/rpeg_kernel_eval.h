@@ -40,6 +40,7 @@ struct EvalLaunch {              // uniform launch parameters
   double* peak;
   double* score;
   uint8_t* mask;
+  double* mass;                  // optional critical-chain mass, [plan][RPEG_MAX_V], or null
   unsigned long long* prof;      // optional per-wavefront phase clocks (8 per wavefront), or null
 };
 
@@ -289,6 +290,10 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     const double fin = est + d;
     makespan = fin > makespan ? fin : makespan;
     ++done;
+    if (L.mass) {  // keep the trace: a dispatched node needs neither its ready time nor its rank again
+      g_time[bv] = fin;
+      g_rank[bv] = est;
+    }
     unsigned touched = 0;
 #pragma unroll
     for (int x = 0; x < RPEG_MAX_V; ++x)
@@ -355,6 +360,17 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   if (L.peak) L.peak[pi] = peak;
   if (L.score) L.score[pi] = out_score;
   if (L.mask) L.mask[pi] = mask;
+  if (L.mass) {
+    double m[RPEG_MAX_V];
+    if (err) {
+#pragma unroll
+      for (int x = 0; x < RPEG_MAX_V; ++x) m[x] = __builtin_nan("");
+    } else {
+      critical_mass(cv, [&](int i) { return g_time[i]; }, [&](int i) { return g_rank[i]; }, m);
+    }
+#pragma unroll
+    for (int x = 0; x < RPEG_MAX_V; ++x) L.mass[pi * RPEG_MAX_V + x] = m[x];
+  }
   KE_STAMP(6);
 }
 

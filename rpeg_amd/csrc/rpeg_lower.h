@@ -312,6 +312,13 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
     groups.push_back(GroupRec{(uint16_t)gmember.size(), (uint16_t)kv.second.size()});
     for (int i : kv.second) gmember.push_back((uint16_t)i);
   }
+  std::vector<uint16_t> pbeg(n + 1, 0), pred(out.edges.size(), 0);
+  {
+    for (auto& ed : out.edges) ++pbeg[ed.second + 1];
+    for (int i = 0; i < n; ++i) pbeg[i + 1] = (uint16_t)(pbeg[i + 1] + pbeg[i]);
+    std::vector<uint16_t> cur(pbeg.begin(), pbeg.end() - 1);
+    for (auto& ed : out.edges) pred[cur[ed.second]++] = (uint16_t)ed.first;
+  }
   ClassHdr h{};
   h.n_nodes = n; h.n_slots = (uint32_t)slots.size(); h.n_succ = (uint32_t)succ.size(); h.n_init = (uint32_t)init.size();
   h.n_groups = (uint32_t)groups.size(); h.n_gmembers = (uint32_t)gmember.size();
@@ -326,6 +333,8 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   h.off_slot = (uint32_t)off; off = align8(off + slots.size() * sizeof(SlotDesc));
   h.off_group = (uint32_t)off; off = align8(off + groups.size() * sizeof(GroupRec));
   h.off_gmember = (uint32_t)off; off = align8(off + gmember.size() * 2);
+  h.off_pbeg = (uint32_t)off; off = align8(off + pbeg.size() * 2);
+  h.off_pred = (uint32_t)off; off = align8(off + pred.size() * 2);
   h.bytes = (uint32_t)off;
   out.blob.assign(off, 0);
   std::memcpy(out.blob.data(), &h, sizeof h);
@@ -336,6 +345,8 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   if (!slots.empty()) std::memcpy(out.blob.data() + h.off_slot, slots.data(), slots.size() * sizeof(SlotDesc));
   if (!groups.empty()) std::memcpy(out.blob.data() + h.off_group, groups.data(), groups.size() * sizeof(GroupRec));
   if (!gmember.empty()) std::memcpy(out.blob.data() + h.off_gmember, gmember.data(), gmember.size() * 2);
+  std::memcpy(out.blob.data() + h.off_pbeg, pbeg.data(), pbeg.size() * 2);
+  if (!pred.empty()) std::memcpy(out.blob.data() + h.off_pred, pred.data(), pred.size() * 2);
   return out;
 }
 

@@ -1,0 +1,553 @@
+// rpeg_sa.h - host side of the batched simulated annealing: proposal kernels, restarts, elites and the
+// Metropolis-Hastings step for a population of independent chains (host only, C++17).
+//
+// The proposals are integer work of a few hundred instructions per chain and step; they run on the
+// host.  Every candidate of every chain of a step is evaluated in ONE batched call of the backend
+// (the GPU evaluator), which is where the time goes.
+//
+// Follows RPEG/search/moves.py (strategy space :97-176, samplers :180-278, candidate directory lookup
+// :554-586, single-vertex kernel move_gen :645-825, donor/receiver kernel multi_move_pair :845-950)
+// and RPEG/search/optimizer.py (elites :158-198, restarts :201-362, chain loop :690-946).  The
+// reference draws from Python's MT19937; here every draw is word k of a counter-based stream keyed by
+// (seed, chain, step, purpose), so a trajectory can be replayed anywhere.
+#ifndef RPEG_SA_H
+#define RPEG_SA_H
+
+#include <algorithm>
+#include <array>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <set>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "rpeg_core.h"
+
+namespace rpeg {
+
+// ------------------------------------------------------------------------------------- generator
+struct SaRng {
+  uint64_t h, k = 0;
+  static uint64_t mix(uint64_t x) {
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+  }
+  SaRng(uint64_t seed, uint64_t a, uint64_t b, uint64_t c) {
+    const uint64_t g = 0x9E3779B97F4A7C15ull;
+    h = mix(seed + g * (0x5Aull + 1));
+    h = mix(h + g * (a + 1));
+    h = mix(h + g * (b + 1));
+    h = mix(h + g * (c + 1));
+  }
+  uint64_t word() { return mix(h + 0x9E3779B97F4A7C15ull * ++k); }
+  double random() { return (double)(word() >> 11) * (1.0 / 9007199254740992.0); }
+  int below(int n) { return (int)(((word() >> 32) * (uint64_t)n) >> 32); }
+  // random.choices(population, weights, k=1): bisect of random()*total in the running sums
+  int weighted(const double* w, int n) {
+    double cum[RPEG_MAX_V];
+    double acc = 0.0;
+    for (int i = 0; i < n; ++i) { acc = i == 0 ? w[0] : acc + w[i]; cum[i] = acc; }
+    const double x = random() * (cum[n - 1] + 0.0);
+    int lo = 0, hi = n - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi) / 2;
+      if (x < cum[mid]) hi = mid; else lo = mid + 1;
+    }
+    return lo;
+  }
+};
+
+// ------------------------------------------------------------------------------------- plans
+enum { SA_DP = 0, SA_PP, SA_TP, SA_MB, SA_OR, SA_ON, SA_OG, SA_ER, SA_EN, SA_EG };
+
+struct SaPlan { int16_t f[RPEG_MAX_V][RPEG_FIELDS]; };
+
+struct SaEval {          // what one evaluation returns
+  double score;          // throughput times the soft memory penalty, without the stale-layout gate
+  double mass[RPEG_MAX_V];
+  uint8_t mask;          // RPEG_MASK_*
+};
+
+struct SaEntry { SaPlan plan; SaEval ev; };
+
+struct SaBackend {
+  virtual ~SaBackend() {}
+  // evaluates n plans; variant[i] selects the staleness variant of plan i
+  virtual int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) = 0;
+};
+
+struct SaSettings {
+  int n_chains = 64, n_steps = 2000, K_x = 6, T_max = 50, K_elite = 3, stag_window = 20, restart_attempts = 50;
+  int gate_candidates = 0, geometric_cooling = 0, n_variants = 1;
+  double T_init = 0.30, T_warm = 0.05, T_min = 0.01, T_cool = 1.0, alpha_pair = 0.28, score_eps = 1e-4;
+  uint64_t seed = 42;
+};
+
+struct SaContext {
+  int nv = 0, R = 1, N = 1, G = 1, B = 1;
+  int L[RPEG_MAX_V] = {0};
+  std::vector<int> tps, dps;
+  std::vector<int> pps[RPEG_MAX_V];
+  std::vector<std::array<int16_t, 6>> dir[RPEG_MAX_V];       // dp pp tp r_ext n_ext mb, ascending by time
+  std::unordered_map<uint64_t, int> dir_index[RPEG_MAX_V];
+
+  static uint64_t key6(int dp, int pp, int tp, int re, int ne, int mb) {
+    return (uint64_t)dp | (uint64_t)pp << 10 | (uint64_t)tp << 20 | (uint64_t)re << 30 | (uint64_t)ne << 40 |
+           (uint64_t)mb << 50;
+  }
+
+  // moves.py:97-137
+  void init(const rpeg_problem_t& P, int structure) {
+    const rpeg_struct_t& st = P.st[structure];
+    nv = st.n_vertex; R = P.R; N = P.N; G = P.G; B = P.B;
+    const int total = R * N * G;
+    tps.clear(); dps.clear();
+    for (int t = 1; t <= G; ++t) if (G % t == 0) tps.push_back(t);
+    for (int d = 1; d <= total; ++d) if (B % d == 0) dps.push_back(d);
+    for (int v = 0; v < nv; ++v) {
+      L[v] = P.model[st.vertex[v].model].L;
+      pps[v].clear();
+      for (int d = 1; d <= total; ++d) if (L[v] % d == 0 && (d == 1 || d % 2 == 0)) pps[v].push_back(d);
+    }
+  }
+
+  // returns an error text or null
+  const char* set_directory(int v, const int16_t* rows, int n) {
+    dir[v].assign(n, {});
+    dir_index[v].clear();
+    for (int j = 0; j < n; ++j) {
+      for (int x = 0; x < 6; ++x) {
+        if (rows[j * 6 + x] < 0 || rows[j * 6 + x] >= 1024) return "directory field outside 0..1023";
+        dir[v][j][x] = rows[j * 6 + x];
+      }
+      const int16_t* r = rows + j * 6;
+      dir_index[v][key6(r[0], r[1], r[2], r[3], r[4], r[5])] = j;   // a later duplicate wins, as dict does
+    }
+    return nullptr;
+  }
+};
+
+// moves.py:148-176 (ablations off)
+inline void sa_valid_mb(int pp, int dp, int B, std::vector<int>& out) {
+  out.clear();
+  const int local = B / dp;
+  if (local < 8 && dp > 1) return;
+  if (pp == 1) { out.push_back(1); return; }
+  const int max_mb = local / 8;
+  for (int mb = pp; mb <= std::min(max_mb, local); ++mb)
+    if (local % mb == 0) out.push_back(mb);
+}
+
+// moves.py:685-694: three draws, also when only one origin exists
+inline void sa_sample_origin(SaRng& rng, const SaContext& cx, int re, int ne, int ge, int16_t* o) {
+  o[0] = (int16_t)(rng.below(cx.R / re) * re);
+  o[1] = (int16_t)(rng.below(cx.N / ne) * ne);
+  o[2] = (int16_t)(rng.below(cx.G / ge) * ge);
+}
+
+// moves.py:645-825 without intra-stage fusion.  Writes up to K_x plans, returns their number.
+inline int sa_move_gen(SaRng& rng, const SaContext& cx, const SaPlan& plan, const double* mass, int K_x, int T_max,
+                       double T, double T_init, SaPlan* out, int* fallback = nullptr) {
+  int v;
+  if (rng.random() >= 0.4) {
+    double w[RPEG_MAX_V];
+    for (int x = 0; x < cx.nv; ++x) w[x] = mass[x] + 1e-6;
+    v = rng.weighted(w, cx.nv);
+  } else {
+    v = rng.below(cx.nv);
+  }
+  const auto& tab = cx.dir[v];
+  const int len = (int)tab.size();
+  const double frac = std::min(1.0, T / T_init);
+  const int w = std::max(5, (int)((double)len * frac));
+  const int16_t* cur = plan.f[v];
+  int j_star;
+  {
+    auto it = cx.dir_index[v].find(SaContext::key6(cur[SA_DP], cur[SA_PP], cur[SA_TP], cur[SA_ER], cur[SA_EN], cur[SA_MB]));
+    if (it != cx.dir_index[v].end()) j_star = it->second;
+    else { j_star = len / 2; if (fallback) ++*fallback; }
+  }
+  const int low = std::max(0, j_star - w), high = std::min(len - 1, j_star + w);
+
+  int n_out = 0;
+  std::array<int16_t, 7> seen[64];
+  int n_seen = 0;
+  auto add = [&](int dp, int pp, int tp, int mb, const int16_t* o, int re, int ne, int ge) {
+    SaPlan& q = out[n_out++];
+    q = plan;
+    int16_t* r = q.f[v];
+    r[SA_DP] = (int16_t)dp; r[SA_PP] = (int16_t)pp; r[SA_TP] = (int16_t)tp; r[SA_MB] = (int16_t)mb;
+    r[SA_OR] = o[0]; r[SA_ON] = o[1]; r[SA_OG] = o[2];
+    r[SA_ER] = (int16_t)re; r[SA_EN] = (int16_t)ne; r[SA_EG] = (int16_t)ge;
+    seen[n_seen++] = {(int16_t)dp, (int16_t)pp, (int16_t)tp, o[0], o[1], o[2], (int16_t)mb};
+  };
+
+  for (int t = 0; t < std::min(5, T_max); ++t) {   // placement only, best effort
+    int16_t o[3];
+    sa_sample_origin(rng, cx, cur[SA_ER], cur[SA_EN], cur[SA_EG], o);
+    if (o[0] != cur[SA_OR] || o[1] != cur[SA_ON] || o[2] != cur[SA_OG]) {
+      add(cur[SA_DP], cur[SA_PP], cur[SA_TP], cur[SA_MB], o, cur[SA_ER], cur[SA_EN], cur[SA_EG]);
+      break;
+    }
+  }
+  for (int t = 0; t < T_max; ++t) {                // strategy changes from the window around j_star
+    if (n_out >= K_x || high < low || n_seen >= 64) break;
+    const int j = low + rng.below(high - low + 1);
+    if (j == j_star) continue;
+    const auto& e = tab[j];
+    int ge, nodes;
+    if (!packing_geometry(e[0], e[1], e[2], cx.G, &ge, &nodes)) continue;
+    int16_t o[3];
+    sa_sample_origin(rng, cx, e[3], e[4], ge, o);
+    const std::array<int16_t, 7> key = {e[0], e[1], e[2], o[0], o[1], o[2], e[5]};
+    bool dup = false;
+    for (int s = 0; s < n_seen; ++s) dup = dup || seen[s] == key;
+    if (dup) continue;
+    add(e[0], e[1], e[2], e[5], o, e[3], e[4], ge);
+  }
+  return n_out;
+}
+
+// moves.py:180-278: a random (allocation, strategy, mb) of vertex v within racks [r_lo, r_hi)
+inline bool sa_sample_region(SaRng& rng, const SaContext& cx, int v, int r_lo, int r_hi, int16_t* row) {
+  const int R_eff = r_hi - r_lo;
+  const int tp = cx.tps[rng.below((int)cx.tps.size())];
+  if (cx.pps[v].empty()) return false;
+  const int pp = cx.pps[v][rng.below((int)cx.pps[v].size())];
+  const int s = std::min(pp, cx.G / tp);
+  if (pp % s != 0) return false;
+  int dcand[1024];
+  int nd = 0;
+  for (int d : cx.dps) {
+    int ge, nodes;
+    if (packing_geometry(d, pp, tp, cx.G, &ge, &nodes) && nodes <= R_eff * cx.N && nd < 1024) dcand[nd++] = d;
+  }
+  if (nd == 0) return false;
+  const int dp = dcand[rng.below(nd)];
+  int ge, need;
+  packing_geometry(dp, pp, tp, cx.G, &ge, &need);
+  int lay[64][2];
+  int nl = 0;
+  for (int re = 1; re <= std::min(R_eff, need); ++re)
+    if (need % re == 0 && need / re <= cx.N && nl < 64) { lay[nl][0] = re; lay[nl][1] = need / re; ++nl; }
+  if (nl == 0) return false;
+  const int li = rng.below(nl);
+  const int re = lay[li][0], ne = lay[li][1];
+  if (R_eff / re == 0) return false;
+  const int r_o = r_lo + rng.below(R_eff / re) * re;
+  const int n_o = rng.below(cx.N / ne) * ne;
+  const int g_o = rng.below(cx.G / ge) * ge;
+  std::vector<int> mbs;
+  sa_valid_mb(pp, dp, cx.B, mbs);
+  if (mbs.empty()) return false;
+  const int mb = mbs[rng.below((int)mbs.size())];
+  row[SA_DP] = (int16_t)dp; row[SA_PP] = (int16_t)pp; row[SA_TP] = (int16_t)tp; row[SA_MB] = (int16_t)mb;
+  row[SA_OR] = (int16_t)r_o; row[SA_ON] = (int16_t)n_o; row[SA_OG] = (int16_t)g_o;
+  row[SA_ER] = (int16_t)re; row[SA_EN] = (int16_t)ne; row[SA_EG] = (int16_t)ge;
+  return true;
+}
+
+inline bool sa_boxes_overlap(const int16_t* a, const int16_t* b) {
+  for (int x = 0; x < 3; ++x)
+    if (a[SA_OR + x] + a[SA_ER + x] <= b[SA_OR + x] || b[SA_OR + x] + b[SA_ER + x] <= a[SA_OR + x]) return false;
+  return true;
+}
+
+// moves.py:845-950 without intra-stage fusion
+inline bool sa_move_pair(SaRng& rng, const SaContext& cx, const SaPlan& plan, SaPlan* out, int max_retries = 100) {
+  double w[RPEG_MAX_V], sum = 0.0;
+  for (int v = 0; v < cx.nv; ++v) {
+    w[v] = (double)(plan.f[v][SA_ER] * plan.f[v][SA_EN] * plan.f[v][SA_EG]);
+    sum = v == 0 ? w[0] : sum + w[v];
+  }
+  if (sum == 0.0) return false;
+  const int vd = rng.weighted(w, cx.nv);
+  int ov[RPEG_MAX_V], n_ov = 0;
+  for (int v = 0; v < cx.nv; ++v)
+    if (v != vd && sa_boxes_overlap(plan.f[v], plan.f[vd])) ov[n_ov++] = v;
+  if (n_ov == 0) return false;
+  const int vr = ov[rng.below(n_ov)];
+
+  const int d_lo = plan.f[vd][SA_OR], d_ext = plan.f[vd][SA_ER];
+  int new_lo, new_ext;
+  if (d_ext > 1) {
+    new_ext = 1 + rng.below(d_ext - 1);
+    new_lo = d_lo + rng.below(d_ext - new_ext + 1);
+  } else {
+    new_lo = d_lo; new_ext = 1;
+  }
+  int16_t donor[RPEG_FIELDS], recv[RPEG_FIELDS];
+  bool ok = false;
+  for (int t = 0; t < max_retries && !ok; ++t) ok = sa_sample_region(rng, cx, vd, new_lo, new_lo + new_ext, donor);
+  if (!ok) return false;
+
+  int recv_lo = 0, recv_hi = cx.R;
+  if (new_ext < d_ext) {   // some racks were freed
+    const int freed_min = new_lo > d_lo ? d_lo : new_lo + new_ext;
+    const int freed_max = new_lo + new_ext < d_lo + d_ext ? d_lo + d_ext - 1 : new_lo - 1;
+    const int r_o = plan.f[vr][SA_OR], r_e = plan.f[vr][SA_ER];
+    recv_lo = std::min(r_o, freed_min);
+    recv_hi = std::max(r_o + r_e - 1, freed_max) + 1;
+  }
+  ok = false;
+  for (int t = 0; t < max_retries && !ok; ++t) ok = sa_sample_region(rng, cx, vr, recv_lo, recv_hi, recv);
+  if (!ok) return false;
+  *out = plan;
+  std::memcpy(out->f[vd], donor, sizeof donor);
+  std::memcpy(out->f[vr], recv, sizeof recv);
+  return true;
+}
+
+// optimizer.py:201-256 without fusion; false where the reference raises
+inline bool sa_sample_all(SaRng& rng, const SaContext& cx, SaPlan* out) {
+  std::memset(out, 0, sizeof *out);
+  for (int v = 0; v < cx.nv; ++v) {
+    bool ok = false;
+    for (int t = 0; t < 100 && !ok; ++t) ok = sa_sample_region(rng, cx, v, 0, cx.R, out->f[v]);
+    if (!ok) return false;
+  }
+  return true;
+}
+
+// ------------------------------------------------------------------------------------- chains
+struct SaChain {
+  SaEntry cur;
+  double score = 0.0, T = 0.0;
+  int rej = 0, restarts = 0;
+  bool dead = false;
+  std::vector<SaEntry> elite;                       // descending by score
+  std::set<std::vector<int16_t>> seen;
+  bool has_best = false, has_feasible = false;
+  SaEntry best, best_feasible;
+  double best_score = -INFINITY, best_feasible_score = -INFINITY;
+  int best_step = -1, best_feasible_step = -1;
+  double best_feasible_time = 0.0;
+  long n_eval = 0;
+};
+
+struct SaRun {
+  const SaContext& cx;
+  const SaSettings& p;
+  SaBackend& be;
+  std::vector<SaChain> chains;
+  std::vector<uint8_t> log;     // [chain][step]: kind | n_candidates << 1 | verdict << 4 | restart << 6
+  std::chrono::steady_clock::time_point t0;
+  std::string err;
+
+  SaRun(const SaContext& c, const SaSettings& s, SaBackend& b) : cx(c), p(s), be(b) {}
+
+  double now() const { return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count(); }
+  uint8_t variant(int chain) const { return (uint8_t)(chain % p.n_variants); }
+
+  static bool full_ok(uint8_t m) {   // is_valid (evaluate.py:143-232) of a plan the samplers built
+    return (m & RPEG_MASK_VALID) && (m & RPEG_MASK_STALE_OK) && (m & RPEG_MASK_MEM_OK) && !(m & RPEG_MASK_ERROR);
+  }
+  static double gated(const SaEval& e) { return (e.mask & RPEG_MASK_STALE_OK) ? e.score : 0.0; }
+
+  std::vector<int16_t> fingerprint(const SaPlan& q) const {   // optimizer.py:158-172: pi, origin, mb
+    std::vector<int16_t> fp;
+    for (int v = 0; v < cx.nv; ++v)
+      for (int x : {SA_DP, SA_PP, SA_TP, SA_OR, SA_ON, SA_OG, SA_MB}) fp.push_back(q.f[v][x]);
+    return fp;
+  }
+
+  void elite_insert(SaChain& ch, const SaEntry& e) {          // optimizer.py:175-198
+    auto fp = fingerprint(e.plan);
+    if (ch.seen.count(fp)) return;
+    if ((int)ch.elite.size() >= p.K_elite && e.ev.score <= ch.elite.back().ev.score) return;
+    ch.elite.push_back(e);
+    std::stable_sort(ch.elite.begin(), ch.elite.end(),
+                     [](const SaEntry& a, const SaEntry& b) { return a.ev.score > b.ev.score; });
+    if ((int)ch.elite.size() > p.K_elite) ch.elite.resize(p.K_elite);
+    ch.seen.insert(fp);
+  }
+
+  void note(SaChain& ch, const SaEntry& e, double score, int step, bool feasible) {   // optimizer.py:676-686, 846-861
+    if (feasible) elite_insert(ch, e);
+    if (!ch.has_best || score > ch.best_score * (1.0 + p.score_eps)) {
+      ch.has_best = true; ch.best = e; ch.best_score = score; ch.best_step = step;
+    }
+    if (feasible && score > ch.best_feasible_score) {
+      ch.has_feasible = true; ch.best_feasible = e; ch.best_feasible_score = score; ch.best_feasible_step = step;
+      ch.best_feasible_time = now();
+    }
+  }
+
+  void enter(SaChain& ch, const SaEntry& e, int step, double T) {   // optimizer.py:666-694
+    ch.cur = e;
+    ch.score = gated(e.ev);
+    const bool feasible = (e.ev.mask & RPEG_MASK_MEM_OK) && (e.ev.mask & RPEG_MASK_STALE_OK);
+    note(ch, e, ch.score, step, feasible);
+    ch.T = T;
+    ch.rej = 0;
+  }
+
+  // optimizer.py:259-289 for every chain of `who`: the first valid one of restart_attempts random plans
+  // (found = 1), else the first attempt as it is (found = 2), else nothing (found = 0: the sampler failed)
+  int random_restart(const std::vector<int>& who, int step, std::vector<int>& found, std::vector<SaEntry>& entry) {
+    found.assign(who.size(), 0);
+    entry.assign(who.size(), SaEntry{});
+    std::vector<SaPlan> plans;
+    std::vector<uint8_t> var;
+    std::vector<int> first(who.size() + 1, 0);
+    for (size_t i = 0; i < who.size(); ++i) {
+      for (int a = 0; a < p.restart_attempts; ++a) {
+        SaRng rng(p.seed, (uint64_t)who[i], (uint64_t)(step + 1), (uint64_t)(1 + a));
+        SaPlan q;
+        if (!sa_sample_all(rng, cx, &q)) break;
+        plans.push_back(q);
+        var.push_back(variant(who[i]));
+      }
+      first[i + 1] = (int)plans.size();
+    }
+    std::vector<SaEval> ev(plans.size());
+    if (!plans.empty())
+      if (int rc = be.evaluate((int)plans.size(), plans.data(), var.data(), ev.data())) return rc;
+    for (size_t i = 0; i < who.size(); ++i) {
+      SaChain& ch = chains[who[i]];
+      // a sampler failure ends the restart where the reference raises; attempts before it still count
+      for (int j = first[i]; j < first[i + 1]; ++j) {
+        ++ch.n_eval;
+        if (full_ok(ev[j].mask)) { found[i] = 1; entry[i].plan = plans[j]; entry[i].ev = ev[j]; break; }
+      }
+      if (!found[i] && first[i + 1] > first[i] && (ev[first[i]].mask & RPEG_MASK_VALID) &&
+          !(ev[first[i]].mask & RPEG_MASK_ERROR)) {
+        found[i] = 2; entry[i].plan = plans[first[i]]; entry[i].ev = ev[first[i]];
+      }
+    }
+    return 0;
+  }
+
+  int run(const SaPlan* base_plan) {
+    t0 = std::chrono::steady_clock::now();
+    chains.assign(p.n_chains, SaChain{});
+    log.assign((size_t)p.n_chains * p.n_steps, 0);
+    // ---- start: the base plan if valid, else a valid random plan, else the base plan as it is (the soft
+    // memory penalty guides the search, optimizer.py:612-616), else the first random plan as it is
+    {
+      std::vector<int> need;
+      std::vector<SaEntry> base(p.n_chains);
+      if (base_plan) {
+        std::vector<SaPlan> plans(p.n_chains, *base_plan);
+        std::vector<uint8_t> var(p.n_chains);
+        std::vector<SaEval> ev(p.n_chains);
+        for (int c = 0; c < p.n_chains; ++c) var[c] = variant(c);
+        if (int rc = be.evaluate(p.n_chains, plans.data(), var.data(), ev.data())) return rc;
+        for (int c = 0; c < p.n_chains; ++c) {
+          ++chains[c].n_eval;
+          base[c].plan = *base_plan; base[c].ev = ev[c];
+          if (full_ok(ev[c].mask)) enter(chains[c], base[c], -1, p.T_init); else need.push_back(c);
+        }
+      } else {
+        for (int c = 0; c < p.n_chains; ++c) need.push_back(c);
+      }
+      std::vector<int> found;
+      std::vector<SaEntry> entry;
+      if (int rc = random_restart(need, -1, found, entry)) return rc;
+      for (size_t i = 0; i < need.size(); ++i) {
+        SaChain& ch = chains[need[i]];
+        if (found[i] == 1) enter(ch, entry[i], -1, p.T_init);
+        else if (base_plan && !(base[need[i]].ev.mask & RPEG_MASK_ERROR) && (base[need[i]].ev.mask & RPEG_MASK_VALID))
+          enter(ch, base[need[i]], -1, p.T_init);
+        else if (found[i] == 2) enter(ch, entry[i], -1, p.T_init);
+        else ch.dead = true;
+      }
+    }
+
+    std::vector<SaPlan> cand((size_t)p.n_chains * p.K_x);
+    std::vector<uint8_t> var((size_t)p.n_chains * p.K_x);
+    std::vector<SaEval> ev((size_t)p.n_chains * p.K_x);
+    std::vector<int> first(p.n_chains + 1), kind(p.n_chains);
+    std::vector<SaRng> rngs;
+    for (int step = 0; step < p.n_steps; ++step) {
+      // ---- proposals of every live chain
+      rngs.clear();
+      int total = 0;
+      for (int c = 0; c < p.n_chains; ++c) {
+        SaChain& ch = chains[c];
+        rngs.emplace_back(p.seed, (uint64_t)c, (uint64_t)(step + 1), 0);
+        first[c] = total;
+        kind[c] = -1;
+        if (ch.dead) continue;
+        SaRng& rng = rngs.back();
+        const double frac = std::min(1.0, ch.T / p.T_init);
+        if (rng.random() < p.alpha_pair * frac) {
+          kind[c] = 1;
+          if (sa_move_pair(rng, cx, ch.cur.plan, &cand[total])) total += 1;
+          else { ch.T = std::max(p.T_min, ch.T * p.T_cool); kind[c] = 2; }   // optimizer.py:737-740
+        } else {
+          kind[c] = 0;
+          total += sa_move_gen(rng, cx, ch.cur.plan, ch.cur.ev.mass, p.K_x, p.T_max, ch.T, p.T_init, &cand[total]);
+        }
+        for (int j = first[c]; j < total; ++j) var[j] = variant(c);
+      }
+      first[p.n_chains] = total;
+      if (total > 0)
+        if (int rc = be.evaluate(total, cand.data(), var.data(), ev.data())) return rc;
+
+      // ---- best of K, one Metropolis-Hastings step, stagnation
+      std::vector<int> random_who;
+      for (int c = 0; c < p.n_chains; ++c) {
+        SaChain& ch = chains[c];
+        if (ch.dead || kind[c] < 0) continue;
+        uint8_t& lg = log[(size_t)c * p.n_steps + step];
+        if (kind[c] == 2) { lg = 1; continue; }
+        const int nc = first[c + 1] - first[c];
+        lg = (uint8_t)(kind[c] | nc << 1);
+        bool restart = false;
+        if (nc == 0) {
+          restart = true;   // "chain stuck" (optimizer.py:767-769)
+        } else {
+          int bi = -1;
+          double bs = -INFINITY;
+          for (int j = first[c]; j < first[c + 1]; ++j) {
+            ++ch.n_eval;
+            SaEntry e; e.plan = cand[j]; e.ev = ev[j];
+            const bool stale_ok = (ev[j].mask & RPEG_MASK_STALE_OK) != 0;
+            double s = p.gate_candidates ? gated(ev[j]) : ev[j].score;
+            if (ev[j].mask & RPEG_MASK_ERROR) s = -INFINITY;
+            const bool feas = (ev[j].mask & RPEG_MASK_MEM_OK) && !(ev[j].mask & RPEG_MASK_ERROR) &&
+                              (stale_ok || !p.gate_candidates);
+            if (!(ev[j].mask & RPEG_MASK_ERROR)) note(ch, e, s, step, feas);
+            if (s > bs) { bs = s; bi = j; }
+          }
+          if (bi >= 0) {
+            const double delta = (bs - ch.score) / (std::fabs(ch.score) + 1e-12);
+            if (std::fabs(delta) >= 1e-6) {
+              const double prob = delta >= 0.0 ? 1.0 : exp_libm(delta / ch.T);
+              const bool acc = rngs[c].random() < prob;
+              if (acc) { ch.cur.plan = cand[bi]; ch.cur.ev = ev[bi]; ch.score = bs; ch.rej = 0; }
+              else ++ch.rej;
+              lg |= (uint8_t)((acc ? 2 : 1) << 4);
+            }
+          }
+          if (p.geometric_cooling) ch.T = std::max(p.T_min, ch.T * p.T_cool);
+          if (p.stag_window > 0 && ch.rej >= p.stag_window) restart = true;
+        }
+        if (restart) {
+          lg |= 1 << 6;
+          ++ch.restarts;
+          if (!ch.elite.empty() && full_ok(ch.elite[0].ev.mask)) enter(ch, ch.elite[0], step, p.T_warm);
+          else random_who.push_back(c);
+        }
+      }
+      if (!random_who.empty()) {
+        std::vector<int> found;
+        std::vector<SaEntry> entry;
+        if (int rc = random_restart(random_who, step, found, entry)) return rc;
+        for (size_t i = 0; i < random_who.size(); ++i) {
+          SaChain& ch = chains[random_who[i]];
+          if (found[i] == 1) enter(ch, entry[i], step, p.T_warm);
+          else { ch.T = p.T_warm; ch.rej = 0; }   // no valid restart: go on from the current plan
+        }
+      }
+    }
+    return 0;
+  }
+};
+
+}  // namespace rpeg
+#endif

@@ -79,3 +79,23 @@ class ProblemT(C.Structure):
 
 class PlanSoaT(C.Structure):
     _fields_ = [("vert", C.c_void_p), ("head", C.c_void_p), ("stride", C.c_uint64)]
+
+
+class SaParamsT(C.Structure):
+    _fields_ = [("n_chains", C.c_int32), ("n_steps", C.c_int32), ("K_x", C.c_int32), ("T_max", C.c_int32),
+                ("K_elite", C.c_int32), ("stag_window", C.c_int32), ("restart_attempts", C.c_int32),
+                ("gate_candidates", C.c_int32), ("geometric_cooling", C.c_int32),
+                ("structure", C.c_int32), ("split", C.c_int32), ("n_variants", C.c_int32),
+                ("tau", (C.c_uint8 * 2) * 8),
+                ("T_init", C.c_double), ("T_warm", C.c_double), ("T_min", C.c_double), ("T_cool", C.c_double),
+                ("alpha_pair", C.c_double), ("score_eps", C.c_double),
+                ("seed", C.c_uint64),
+                ("dir_n", C.c_int32 * MAX_V), ("dir", C.c_void_p * MAX_V)]
+
+
+class SaResultT(C.Structure):
+    _fields_ = [("best_plan", C.c_void_p), ("best_score", C.c_void_p), ("best_step", C.c_void_p),
+                ("best_time", C.c_void_p), ("best_feasible", C.c_void_p), ("cur_plan", C.c_void_p),
+                ("cur_score", C.c_void_p), ("restarts", C.c_void_p), ("n_eval", C.c_void_p), ("dead", C.c_void_p),
+                ("log", C.c_void_p), ("wall_s", C.c_double), ("eval_s", C.c_double),
+                ("n_launch", C.c_int64), ("n_plans", C.c_int64)]

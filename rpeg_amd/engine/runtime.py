@@ -22,7 +22,8 @@ _lib = None
 
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
-           "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes")
+           "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
+           "rpeg_sa_run")
 
 
 class EngineError(RuntimeError):
@@ -47,6 +48,10 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_last_error.argtypes = [vp]
     lib.rpeg_eval_batch.restype = C.c_int
     lib.rpeg_eval_batch.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp]
+    lib.rpeg_eval_batch_mass.restype = C.c_int
+    lib.rpeg_eval_batch_mass.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp, vp]
+    lib.rpeg_sa_run.restype = C.c_int
+    lib.rpeg_sa_run.argtypes = [vp, vp, vp, vp, vp]
     lib.rpeg_op_time_batch.restype = C.c_int
     lib.rpeg_op_time_batch.argtypes = [vp, u64, i32, i32, vp, u64, vp, vp, vp]
     lib.rpeg_eval_trace.restype = C.c_int
@@ -154,6 +159,57 @@ class Engine:
         out = self.eval_device(DeviceBatch(batch, self.device), gate_stale=gate_stale)
         _torch().cuda.synchronize(self.device)
         return {k: v.cpu().numpy() for k, v in out.items()}
+
+    def eval_mass(self, batch: PlanBatch, gate_stale: bool = False) -> Dict[str, np.ndarray]:
+        """`eval` plus the critical-chain mass per template vertex, float64 [n, MAX_V]."""
+        torch = _torch()
+        db = DeviceBatch(batch, self.device)
+        out = self.alloc_outputs(db.n)
+        out["mass"] = torch.empty((db.n, abi.MAX_V), dtype=torch.float64, device=self.device)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_eval_batch_mass(self._h, db.n, C.addressof(db.soa), abi.GATE_STALE if gate_stale else 0,
+                                               out["makespan"].data_ptr(), out["peak"].data_ptr(),
+                                               out["score"].data_ptr(), out["mask"].data_ptr(),
+                                               out["mass"].data_ptr(), stream)
+        self._check(rc, "rpeg_eval_batch_mass")
+        torch.cuda.synchronize(self.device)
+        return {k: v.cpu().numpy() for k, v in out.items()}
+
+    def sa_run(self, params: "abi.SaParamsT", directory, base_plan: Optional[np.ndarray] = None) -> Dict[str, object]:
+        """Runs the batched simulated annealing (rpeg_sa_run).  `directory` is a list of int16 arrays
+        [n_v, 6] (dp pp tp r_ext n_ext mb, ascending by time), one per template vertex."""
+        torch = _torch()
+        keep = []
+        for v in range(abi.MAX_V):
+            if v < len(directory):
+                a = np.ascontiguousarray(directory[v], dtype=np.int16).reshape(-1, 6)
+                keep.append(a)
+                params.dir_n[v] = a.shape[0]
+                params.dir[v] = a.ctypes.data
+            else:
+                params.dir_n[v] = 0
+                params.dir[v] = None
+        nc, ns = params.n_chains, params.n_steps
+        W = abi.MAX_V * abi.FIELDS
+        out = dict(best_plan=np.zeros((nc, W), np.int16), best_score=np.zeros(nc), best_step=np.zeros(nc, np.int32),
+                   best_time=np.zeros(nc), best_feasible=np.zeros(nc, np.uint8), cur_plan=np.zeros((nc, W), np.int16),
+                   cur_score=np.zeros(nc), restarts=np.zeros(nc, np.int32), n_eval=np.zeros(nc, np.int64),
+                   dead=np.zeros(nc, np.uint8), log=np.zeros((nc, max(ns, 1)), np.uint8))
+        res = abi.SaResultT()
+        for k, a in out.items():
+            setattr(res, k, a.ctypes.data)
+        base = None
+        if base_plan is not None:
+            base = np.ascontiguousarray(base_plan, dtype=np.int16).reshape(W)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_sa_run(self._h, C.addressof(params), base.ctypes.data if base is not None else None,
+                                      C.addressof(res), stream)
+        self._check(rc, "rpeg_sa_run")
+        out["log"] = out["log"][:, :ns]
+        out.update(wall_s=res.wall_s, eval_s=res.eval_s, n_launch=res.n_launch, n_plans=res.n_plans)
+        return out
 
     def op_time(self, structure: int, vertex: int, strat: np.ndarray):
         """time() and peak_bytes() of mock nodes: strat is int16 [7, n] = dp pp tp mb r_ext n_ext g_ext."""

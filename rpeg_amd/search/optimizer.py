@@ -1,0 +1,204 @@
+"""Batched simulated annealing on the GPU evaluator.
+
+`OptimizerConfig` mirrors RPEG/search/optimizer.py:33-128 (same fields, same derived I_max and
+T_cool).  The reference runs ONE chain at a time and maps `_eval_worker` over the K_x candidates of
+its current step (optimizer.py:793-798); here a population of independent chains advances in
+lock-step and the candidates of all chains of a step are scored in one launch (rpeg_sa_run).  The
+neighbourhood (move_gen, multi_move_pair), the best-of-K proposal, the acceptance rule, the elite
+list and the stagnation restarts are the reference's; the random numbers are a counter-based stream
+instead of MT19937, so a run is reproducible but not draw-for-draw equal to a reference run.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Dict, FrozenSet, List, Optional, Sequence, Set, Tuple
+
+import numpy as np
+
+from ..core.types import Allocation, Model
+from ..engine import abi
+from ..engine.problem import EvalProblem, FIELDS_PER_VERTEX
+from ..ir.plan import ExecutionPlan
+from ..model.hardware import Hardware
+from ..model.memory import MemoryPolicy
+from ..model.models import ModelSuite
+from ..model.workload import Workload
+from .cache import EvalCache
+from .evaluate import Configuration, _check_supported, _engine_for, _structure_of
+from .moves import build_candidate_directory, directory_arrays
+
+DEFAULT_T_CAND: Dict[Model, Set[int]] = {Model.ACTOR: {0, 1}, Model.CRITIC: {0, 1}, Model.AC_SHARE: {0, 1}}
+
+
+@dataclass
+class OptimizerConfig:
+    """RPEG/search/optimizer.py:33-128.  Fields that steer parts this engine does not run (structural
+    outer loop budgets, utilisation objective, ablations) are kept so that existing call sites
+    construct it unchanged; they are ignored unless noted."""
+    K_x: int = 6
+    T_max: int = 50
+    E_max: int = 5000
+    E_struct: int = 400
+    T_cand: Optional[Dict[Model, Set[int]]] = None
+    structural_candidates: Optional[FrozenSet[str]] = None
+    lambda_ac: float = 0.15
+    score_eps: float = 1e-4
+    T_init: float = 0.30
+    T_warm: float = 0.05
+    T_min: float = 0.01
+    K_elite: int = 3
+    alpha_pair: float = 0.28
+    stag_window: int = 20
+    max_throughput_loss: float = 0.0
+    I_max: int = 0
+    R_max: int = 10000
+    T_cool: float = 0.0
+    algorithm: str = "ppo"
+    deadline: Optional[float] = None
+    deadline_per_struct: Optional[float] = None
+    fixed_mb: bool = False
+    uniform_vertex: bool = False
+    no_polish: bool = False
+    hard_oom: bool = False
+    geometric_cooling: bool = False
+    memory_optimizer_stage: int = 2
+    memory_activation_checkpointing: bool = True
+    memory_runtime_overhead_fraction: float = 0.0
+    memory_worker_overhead_bytes: float = 0.0
+    memory_semantic_activation_cache_bytes: float = 0.0
+    memory_max_worker_groups_per_gpu: int = 0
+
+    def __post_init__(self) -> None:
+        allowed = frozenset({"separate", "fused", "ac_share"})
+        if self.structural_candidates is not None:
+            unknown = self.structural_candidates - allowed
+            if unknown:
+                raise ValueError("unknown structural_candidates: " + ", ".join(sorted(unknown)))
+            if not self.structural_candidates:
+                raise ValueError("structural_candidates must not be empty")
+        self.memory_policy()
+        if self.I_max <= 0:
+            self.I_max = int(self.E_struct / ((self.K_x + 1) / 2) * 0.5)
+        self.T_cool = (self.T_min / self.T_init) ** (1.0 / (0.7 * self.I_max))
+
+    def memory_policy(self) -> MemoryPolicy:
+        return MemoryPolicy(optimizer_stage=self.memory_optimizer_stage,
+                            activation_checkpointing=self.memory_activation_checkpointing,
+                            runtime_overhead_fraction=self.memory_runtime_overhead_fraction,
+                            worker_overhead_bytes=self.memory_worker_overhead_bytes,
+                            semantic_activation_cache_bytes=self.memory_semantic_activation_cache_bytes,
+                            max_worker_groups_per_gpu=self.memory_max_worker_groups_per_gpu)
+
+
+@dataclass
+class ChainResult:
+    """Outcome of `optimize_chains` (arrays are indexed by chain)."""
+    best_plan: np.ndarray          # int16 [n_chains, MAX_V*10]
+    best_score: np.ndarray
+    best_step: np.ndarray
+    best_time: np.ndarray          # seconds from the start of the run to the first sight of best_plan
+    best_feasible: np.ndarray
+    cur_plan: np.ndarray
+    cur_score: np.ndarray
+    restarts: np.ndarray
+    n_eval: np.ndarray
+    dead: np.ndarray
+    log: np.ndarray
+    variants: List[Tuple[int, ...]]
+    wall_s: float = 0.0
+    eval_s: float = 0.0
+    n_launch: int = 0
+    n_plans: int = 0
+
+    def argbest(self) -> int:
+        """Chain holding the best feasible plan (lowest chain index among equals); falls back to the
+        best infeasible one as optimize() does (optimizer.py:946)."""
+        feas = self.best_feasible.astype(bool)
+        pool = np.flatnonzero(feas) if feas.any() else np.flatnonzero(~np.isnan(self.best_score))
+        if pool.size == 0:
+            raise RuntimeError("no chain holds a plan")
+        return int(pool[np.argmax(self.best_score[pool])])
+
+
+def sa_params(opt: OptimizerConfig, n_chains: int, n_steps: int, variants: Sequence[Sequence[int]], structure: int = 0,
+              split: int = 1, seed: int = 42, restart_attempts: int = 50, gate_candidates: bool = False) -> abi.SaParamsT:
+    p = abi.SaParamsT()
+    p.n_chains, p.n_steps, p.K_x, p.T_max, p.K_elite = n_chains, n_steps, opt.K_x, opt.T_max, opt.K_elite
+    p.stag_window, p.restart_attempts = opt.stag_window, restart_attempts
+    p.gate_candidates, p.geometric_cooling = int(gate_candidates), int(opt.geometric_cooling)
+    p.structure, p.split, p.n_variants = structure, split, len(variants)
+    if not 1 <= len(variants) <= 8:
+        raise ValueError("between 1 and 8 staleness variants")
+    for k, taus in enumerate(variants):
+        for t in range(2):
+            p.tau[k][t] = int(taus[t]) if t < len(taus) else 0
+    p.T_init, p.T_warm, p.T_min, p.T_cool = opt.T_init, opt.T_warm, opt.T_min, opt.T_cool
+    p.alpha_pair, p.score_eps, p.seed = opt.alpha_pair, opt.score_eps, seed
+    return p
+
+
+def plan_row(rpeg, plan: ExecutionPlan) -> np.ndarray:
+    row = np.zeros(abi.MAX_V * FIELDS_PER_VERTEX, np.int16)
+    for slot, v in enumerate(rpeg.vertices):
+        a = plan.sigma[v]
+        row[slot * FIELDS_PER_VERTEX:(slot + 1) * FIELDS_PER_VERTEX] = [*plan.pi[v], plan.mb[v], *a.origin, *a.extent]
+    return row
+
+
+def row_plan(rpeg, row: np.ndarray) -> ExecutionPlan:
+    sigma, pi, mb = {}, {}, {}
+    for slot, v in enumerate(rpeg.vertices):
+        f = [int(x) for x in row[slot * FIELDS_PER_VERTEX:(slot + 1) * FIELDS_PER_VERTEX]]
+        pi[v], mb[v] = (f[0], f[1], f[2]), f[3]
+        sigma[v] = Allocation(origin=(f[4], f[5], f[6]), extent=(f[7], f[8], f[9]))
+    return ExecutionPlan(sigma=sigma, pi=pi, mb=mb)
+
+
+def optimize_chains(problem: EvalProblem, opt: OptimizerConfig, n_chains: int, n_steps: int,
+                    variants: Sequence[Sequence[int]], seed: int = 42, base_plan: Optional[ExecutionPlan] = None,
+                    engine=None, structure: int = 0, directory=None, gate_candidates: bool = False) -> ChainResult:
+    """Runs `n_chains` chains of `n_steps` steps on the GPU.  Chain c anneals under staleness variant
+    variants[c % len(variants)] (one staleness value per trainable model of the structure)."""
+    from ..engine.runtime import Engine
+    eng = engine or Engine(problem)
+    rpeg0 = problem.template(structure, ())
+    if directory is None:
+        table, _ = build_candidate_directory(rpeg0, problem.suite, problem.device_space, problem.workload, eng, structure)
+        directory = directory_arrays(rpeg0, table)
+    split = 1 if problem.workload.gen_quantiles else 0
+    params = sa_params(opt, n_chains, n_steps, variants, structure, split, seed, gate_candidates=gate_candidates)
+    base = plan_row(rpeg0, base_plan) if base_plan is not None else None
+    out = eng.sa_run(params, directory, base)
+    return ChainResult(variants=[tuple(int(t) for t in v) for v in variants], **out)
+
+
+def _iter_staleness(tau_models, t_cand) -> List[Tuple[int, ...]]:
+    """RPEG/search/inter_model.py:43-62 in the order of the structure's trainable models."""
+    import itertools
+    return [tuple(c) for c in itertools.product(*[sorted(t_cand[m]) for m in tau_models])]
+
+
+def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
+             opt_config: OptimizerConfig, cache: Optional[EvalCache] = None, n_chains: int = 64, seed: int = 42) -> Configuration:
+    """Drop-in for optimize() (RPEG/search/optimizer.py:365-946) on the template of `base_config`.
+
+    The structural outer loop is replaced by running all staleness variants of T_cand side by side
+    (chain c uses variant c mod n); every chain runs the number of iterations the reference's
+    per-structure budget is calibrated for (2 * I_max = E_struct / ((K_x+1)/2), optimizer.py:121-125).
+    AC-share and intra-stage-fusion structures are not entered: the returned configuration keeps the
+    template of `base_config` with the staleness of the winning chain.  `cache` is accepted for
+    signature compatibility; results do not depend on it."""
+    _check_supported(base_config)
+    policy = opt_config.memory_policy()
+    eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy)
+    t_cand = opt_config.T_cand if opt_config.T_cand is not None else DEFAULT_T_CAND
+    variants = _iter_staleness(st.tau_models, t_cand)
+    res = optimize_chains(eng.problem, opt_config, n_chains, max(1, 2 * opt_config.I_max), variants, seed,
+                          base_config.plan, eng)
+    c = res.argbest()
+    tau = {m: res.variants[c % len(variants)][i] for i, m in enumerate(st.tau_models)}
+    rpeg = st.build(suite, workload, tau=tau)
+    return Configuration(rpeg, row_plan(rpeg, res.best_plan[c]), base_config.device_space,
+                         intra_stage_fusion=False, transfer_resource_policy=base_config.transfer_resource_policy)

@@ -132,11 +132,12 @@ def node_vectors(lowered, cost, mm, limit):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--ref", default="/root/reference")
+    ap.add_argument("--configs", default="1,2,3,4,5")
     args = ap.parse_args()
     mods = load_reference(args.ref)
     from rpeg_amd import configs
     from rpeg_amd.search import candidates
-    for c in range(1, 6):
+    for c in (int(x) for x in args.configs.split(",")):
         cfg = configs.config(c)
         n = N_PLANS[c]
         batch = candidates.generate(cfg.problem, n, cfg.tau_choices, seed=42, tag=c)

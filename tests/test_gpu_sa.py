@@ -1,0 +1,113 @@
+"""GPU tests of the annealing path through the C ABI: critical-chain masses, the candidate directory,
+and whole populations of chains (rpeg_sa_run) against the same host logic over the CPU build of the
+evaluator, which the CPU suite ties to the Python restatement and the reference's vectors."""
+
+import json
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+from oracle.cpu_port import CpuPort
+from rpeg_amd import configs
+from rpeg_amd.engine import abi
+from rpeg_amd.search.moves import build_candidate_directory, directory_arrays
+from rpeg_amd.search.optimizer import OptimizerConfig, optimize_chains, sa_params
+from tests.helpers import GOLDEN, seeded_batch
+
+pytestmark = pytest.mark.gpu
+
+_engines = {}
+
+
+def engine(c):
+    from rpeg_amd.engine.runtime import Engine
+    if c not in _engines:
+        _engines[c] = Engine(configs.config(c).problem)
+    return _engines[c]
+
+
+def same_bits(a, b):
+    return np.array_equal(np.asarray(a, np.float64).view(np.uint64), np.asarray(b, np.float64).view(np.uint64))
+
+
+@pytest.mark.parametrize("c,n", [(1, 4096), (2, 16384), (3, 16384), (4, 16384), (5, 4096)])
+def test_critical_mass_bit_exact(c, n):
+    cfg, batch = seeded_batch(c, n)
+    got = engine(c).eval_mass(batch)
+    ref = CpuPort(cfg.problem).eval(batch, threads=16, want_mass=True)
+    assert np.array_equal(got["mask"], ref["mask"])
+    assert same_bits(got["score"], ref["score"])
+    assert same_bits(got["mass"], ref["mass"])
+    # the mass output must not disturb the plain outputs
+    plain = engine(c).eval(batch, gate_stale=False)
+    assert same_bits(plain["score"], got["score"]) and same_bits(plain["makespan"], got["makespan"])
+
+
+@pytest.mark.parametrize("c", [1, 5])
+def test_candidate_directory_matches_reference(c):
+    with open(os.path.join(GOLDEN, "ref_sa.json")) as f:
+        g = json.load(f)["configs"][str(c)]["directory"]
+    p = configs.config(c).problem
+    rpeg0 = p.template(0, ())
+    table, index = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, engine(c))
+    for v in rpeg0.vertices:
+        want = g[v.id]
+        assert len(table[v]) == want["n"]
+        keys = ",".join(str(x) for e in table[v] for x in e[:6])
+        times = ",".join(e[6].hex() for e in table[v])
+        assert zlib.crc32(keys.encode()) == want["key_crc"], v.id
+        assert zlib.crc32(times.encode()) == want["time_crc"], v.id
+        assert all(index[v][e[:6]] == j for j, e in enumerate(table[v]))
+
+
+def _variants(p):
+    n_tau = len(p.structures[0].tau_models)
+    return [(0,) * n_tau, (1,) + (0,) * (n_tau - 1)]
+
+
+@pytest.mark.parametrize("c,n_chains,n_steps,kw", [
+    (1, 64, 200, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
+    (2, 32, 100, dict(T_init=0.30, T_min=0.01, T_warm=0.05, stag_window=5, geometric_cooling=True)),
+    (5, 64, 60, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
+])
+def test_chains_equal_host_replay(c, n_chains, n_steps, kw):
+    """Same counter-based draws, GPU evaluator against CPU evaluator: every decision of every chain,
+    the final plans, the best plans and their scores are identical."""
+    p = configs.config(c).problem
+    eng = engine(c)
+    opt = OptimizerConfig(**kw)
+    rpeg0 = p.template(0, ())
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, eng)
+    arrays = directory_arrays(rpeg0, table)
+    got = optimize_chains(p, opt, n_chains, n_steps, _variants(p), seed=42, engine=eng, directory=arrays)
+    split = 1 if p.workload.gen_quantiles else 0
+    ref = CpuPort(p).sa_run(sa_params(opt, n_chains, n_steps, _variants(p), 0, split, 42), arrays, threads=16)
+    assert np.array_equal(got.log, ref["log"])
+    assert np.array_equal(got.cur_plan, ref["cur_plan"]) and same_bits(got.cur_score, ref["cur_score"])
+    assert np.array_equal(got.best_plan, ref["best_plan"]) and same_bits(got.best_score, ref["best_score"])
+    assert np.array_equal(got.best_step, ref["best_step"]) and np.array_equal(got.best_feasible, ref["best_feasible"])
+    assert np.array_equal(got.restarts, ref["restarts"]) and np.array_equal(got.n_eval, ref["n_eval"])
+    assert np.array_equal(got.dead, ref["dead"])
+    live = ~got.dead.astype(bool)
+    assert live.any()
+    assert ((got.log >> 4) & 3 == 2).sum() > 0, "no accepted move in the whole population"
+    assert got.n_launch >= n_steps
+
+
+def test_base_plan_start_and_gate():
+    p = configs.config(1).problem
+    eng = engine(1)
+    cfg, batch = seeded_batch(1, 64)
+    out = eng.eval(batch, gate_stale=True)
+    ok = np.flatnonzero((out["mask"] & 7) == 7)
+    assert ok.size
+    rpeg, plan, _ = batch.configuration(p, int(ok[0]))
+    opt = OptimizerConfig(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)
+    res = optimize_chains(p, opt, 8, 50, [(0, 0)], seed=7, base_plan=plan, engine=eng, gate_candidates=True)
+    assert not res.dead.any() and res.best_feasible.all()
+    # a chain never reports a best feasible score below that of its valid start
+    assert (res.best_score >= out["score"][ok[0]]).all()
+    c = res.argbest()
+    assert res.best_score[c] == res.best_score.max()

@@ -1,0 +1,149 @@
+"""The shipped annealing host logic (rpeg_amd/csrc/rpeg_sa.h) and the critical-chain mass of the shared
+scheduler code, run through the CPU build of the kernels' headers:
+
+* its proposal kernels against the vectors written by the reference's own move_gen / multi_move_pair /
+  sample_expl_in_region (same counter-based draws),
+* its critical-chain masses against the Python restatement,
+* a whole population of chains against the Python restatement of the chain loop: identical
+  trajectories, step by step.
+"""
+
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import rpeg_oracle as O
+from oracle import sa_oracle as S
+from oracle.cpu_port import CpuPort
+from rpeg_amd import configs
+from rpeg_amd.core.types import Allocation
+from rpeg_amd.engine import abi
+from rpeg_amd.engine.problem import PlanBatch
+from rpeg_amd.ir.plan import ExecutionPlan
+from rpeg_amd.search.optimizer import OptimizerConfig, plan_row, row_plan, sa_params
+from tests.helpers import GOLDEN, seeded_batch
+
+
+def _directory(p, rpeg0):
+    cost = O.CostModel(p.hw, p.suite, p.workload, p.memory_policy.optimizer_stage, p.memory_policy.activation_checkpointing)
+    mem = O.make_mem_model(rpeg0, p.suite, p.workload, p.hw, p.memory_policy)
+    table, index = S.build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, cost, mem)
+    arrays = [np.asarray([c[:6] for c in table[v]], np.int16).reshape(-1, 6) for v in rpeg0.vertices]
+    return table, index, arrays
+
+
+def _rows6(rows, nv):
+    return [[int(x) for x in rows[v * 10:(v + 1) * 10]] for v in range(nv)]
+
+
+@pytest.mark.parametrize("c", [1, 5])
+def test_cxx_proposals_match_reference_vectors(c):
+    with open(os.path.join(GOLDEN, "ref_sa.json")) as f:
+        cases = json.load(f)["configs"][str(c)]["cases"]
+    cfg, batch = seeded_batch(c, len(cases))
+    p = cfg.problem
+    sp = p.device_space
+    rpeg0 = p.template(0, ())
+    nv = len(rpeg0.vertices)
+    _, _, arrays = _directory(p, rpeg0)
+    port = CpuPort(p)
+    for rec in cases:
+        i = rec["i"]
+        mg = rec["move_gen"]
+        opt = OptimizerConfig(T_init=mg["T_init"], T_min=min(0.01, mg["T_init"]))
+        params = sa_params(opt, 1, 1, [(0, 0)])
+        _, plan_m, _ = batch.configuration(p, i)
+        row = plan_row(rpeg0, ExecutionPlan(sigma={v: plan_m.sigma[u] for v, u in zip(rpeg0.vertices, plan_m.sigma)},
+                                            pi={v: plan_m.pi[u] for v, u in zip(rpeg0.vertices, plan_m.pi)},
+                                            mb={v: plan_m.mb[u] for v, u in zip(rpeg0.vertices, plan_m.mb)}))
+        mass = np.zeros(abi.MAX_V)
+        mass[:nv] = [float.fromhex(x) for x in rec["mass"]]
+        out, draws, fb = port.sa_propose(params, arrays, 0, (42, c, i, 1), plan=row, mass=mass, T=mg["T"])
+        assert [_rows6(r, nv) for r in out] == mg["plans"], i
+        assert draws == mg["n_draws"] and fb == mg["fallback"], i
+        out, draws, _ = port.sa_propose(params, arrays, 1, (42, c, i, 2), plan=row)
+        assert ([_rows6(r, nv) for r in out] or [None])[0] == rec["pair"]["plan"], i
+        assert draws == rec["pair"]["n_draws"], i
+        draws, rows = 0, []
+        for v in range(nv):
+            lo = i % sp.R
+            hi = min(sp.R, lo + 1 + (i // 3) % sp.R)
+            out, draws, _ = port.sa_propose(params, arrays, 2, (42, c, i, 3), v=v, r_lo=lo, r_hi=hi, skip=draws)
+            rows.append([int(x) for x in out[0]] if len(out) else None)
+        assert rows == rec["sample"]["rows"], i
+        assert draws == rec["sample"]["n_draws"], i
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_critical_mass_matches_restatement(c):
+    n = 40
+    cfg, batch = seeded_batch(c, n)
+    p = cfg.problem
+    got = CpuPort(p).eval(batch, want_mass=True)
+    for i in range(n):
+        rpeg, plan, wl = batch.configuration(p, i)
+        r = O.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy,
+                            check_stale=False, want_trace=True)
+        chain = S.critical_chain(r["nodes"], r["edges"], r["finish"])
+        mass = S.critical_mass(chain, rpeg, r["start"], r["finish"])
+        want = [mass[v] for v in rpeg.vertices]
+        assert [x.hex() for x in got["mass"][i, :len(want)]] == [x.hex() for x in want], i
+        assert not got["mass"][i, len(want):].any()
+
+
+def _log_byte(entry):
+    step, kind, nc, acc = entry
+    b = (1 if kind == "pair" else 0) | nc << 1
+    if acc is not None:
+        b |= (2 if acc else 1) << 4
+    return b
+
+
+@pytest.mark.parametrize("c,n_chains,n_steps,kw", [
+    (1, 6, 40, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=4)),
+    (5, 4, 12, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
+    (2, 3, 25, dict(T_init=0.30, T_min=0.01, T_warm=0.05, stag_window=3, geometric_cooling=True)),
+])
+def test_chain_trajectories_match_restatement(c, n_chains, n_steps, kw):
+    cfg = configs.config(c)
+    p = cfg.problem
+    opt = OptimizerConfig(**kw)
+    n_tau = len(p.structures[0].tau_models)
+    variants = [(0,) * n_tau, (1,) + (0,) * (n_tau - 1)]
+    rpeg0 = p.template(0, ())
+    _, _, arrays = _directory(p, rpeg0)
+    split = 1 if p.workload.gen_quantiles else 0
+    params = sa_params(opt, n_chains, n_steps, variants, 0, split, 42)
+    got = CpuPort(p).sa_run(params, arrays, threads=4)
+    sp = S.SaParams(K_x=opt.K_x, T_max=opt.T_max, T_init=opt.T_init, T_warm=opt.T_warm, T_min=opt.T_min,
+                    K_elite=opt.K_elite, alpha_pair=opt.alpha_pair, stag_window=opt.stag_window,
+                    score_eps=opt.score_eps, E_struct=opt.E_struct, geometric_cooling=opt.geometric_cooling, seed=42)
+    assert sp.T_cool == opt.T_cool
+    rpegs = [p.template(0, v) for v in variants]
+    table, index, _ = _directory(p, rpegs[0])
+    nv = len(rpeg0.vertices)
+    for cid in range(n_chains):
+        rpeg = rpegs[cid % len(variants)]
+        tabs = ({v: table[v0] for v, v0 in zip(rpeg.vertices, rpegs[0].vertices)},
+                {v: index[v0] for v, v0 in zip(rpeg.vertices, rpegs[0].vertices)})
+        ev = S.oracle_evaluator(rpeg, p.device_space, p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+        ch = S.run_chains(lambda _c: rpeg, ExecutionPlan, Allocation, p.device_space, p.suite, p.workload,
+                          lambda _c: ev, tabs, 1, n_steps, sp, first_chain=cid)[0]
+        assert bool(got["dead"][cid]) == ch.dead, cid
+        if ch.dead:
+            continue
+        want_log = np.zeros(n_steps, np.uint8)
+        for e in ch.log:
+            want_log[e[0]] = _log_byte(e)
+        assert [int(x) & 0x3F for x in got["log"][cid]] == [int(x) for x in want_log], cid
+        assert _rows6(got["cur_plan"][cid], nv) == _rows6(plan_row(rpeg, ch.cur.plan), nv), cid
+        assert got["cur_score"][cid].hex() == float(ch.score).hex(), cid
+        assert got["restarts"][cid] == ch.r and got["n_eval"][cid] == ch.n_eval, cid
+        feas = ch.best_feasible is not None
+        assert bool(got["best_feasible"][cid]) == feas, cid
+        best = ch.best_feasible if feas else ch.best
+        assert _rows6(got["best_plan"][cid], nv) == _rows6(plan_row(rpeg, best.plan), nv), cid
+        assert got["best_score"][cid].hex() == float(ch.best_feasible_score if feas else ch.best_score).hex(), cid
+        assert got["best_step"][cid] == (ch.best_feasible_step if feas else ch.best_step), cid
