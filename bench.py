@@ -2,6 +2,7 @@
 """Benchmark of the batched plan evaluator on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu]
+    python bench.py --config 5 [--chains 64] [--sa-steps 2000]      (batched simulated annealing)
 
 A step is one pass of the hot path (signature kernel, class grouping, evaluation kernel) over the
 whole seeded candidate set of the configuration (config 2: 65,536 GRPO plans), with the plan
@@ -57,6 +58,73 @@ def cxx_port(cfg, batch, threads):
                 sample=f"first {n} plans, host build of the kernels' arithmetic (OpenMP), lowering included")
 
 
+def bench_sa(args):
+    """Config 5: 64 chains x 2000 steps of batched simulated annealing.  Prints one JSON line whose value
+    is the wall-clock of the whole run (directory build excluded and reported beside it)."""
+    import zlib
+    import torch
+    from rpeg_amd import configs
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.search.moves import build_candidate_directory, directory_arrays
+    from rpeg_amd.search.optimizer import OptimizerConfig, optimize_chains, sa_params
+
+    cfg = configs.config(5)
+    p = cfg.problem
+    opt = OptimizerConfig(K_x=6, T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)
+    variants = [(0, 0), (1, 0)]          # actor staleness {0, 1}, critic {0}; chains alternate
+    eng = Engine(p, "cuda:0")
+    rpeg0 = p.template(0, ())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, eng)
+    arrays = directory_arrays(rpeg0, table)
+    dir_s = time.perf_counter() - t0
+    runs = []
+    for rep in range(max(1, args.steps if args.steps < 20 else 2)):   # first run lowers every class it meets
+        res = optimize_chains(p, opt, args.chains, args.sa_steps, variants, seed=42, engine=eng, directory=arrays)
+        runs.append(res)
+    cold, warm = runs[0], runs[-1]
+    c = cold.argbest()
+    assert all((r.best_plan == cold.best_plan).all() and (r.best_score == cold.best_score).all() for r in runs)
+    line = {
+        "metric": "SA wall-clock, 64 chains x 2000 steps, to best plan", "value": cold.wall_s, "unit": "s",
+        "n_gpus": 1, "steps": args.sa_steps, "warmup": 0, "ms_per_step": cold.wall_s / max(1, args.sa_steps) * 1e3,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": cfg.name, "chains": args.chains, "steps_per_chain": args.sa_steps, "K_x": opt.K_x,
+                   "T_init": opt.T_init, "T_min": opt.T_min, "T_warm": opt.T_warm, "stag_window": opt.stag_window,
+                   "seed": 42, "staleness_variants": variants, "memory_per_gpu": p.hw.memory_per_gpu},
+        "time_to_best_s": float(cold.best_time[c]), "best_chain": c, "best_step": int(cold.best_step[c]),
+        "best_score": float(cold.best_score[c]), "best_feasible": bool(cold.best_feasible[c]),
+        "best_plan_crc": zlib.crc32(cold.best_plan[c].tobytes()),
+        "plans_evaluated": int(cold.n_plans), "launches": int(cold.n_launch),
+        "evals_per_s": cold.n_plans / cold.wall_s, "eval_share_of_wall": cold.eval_s / cold.wall_s,
+        "warm_wall_s": warm.wall_s, "warm_time_to_best_s": float(warm.best_time[c]),
+        "directory_s": dir_s, "directory_sizes": [int(a.shape[0]) for a in arrays],
+        "accept_rate": float((((cold.log >> 4) & 3) == 2).sum() / max(1, (((cold.log >> 4) & 3) != 0).sum())),
+        "restarts": int(cold.restarts.sum()), "dead_chains": int(cold.dead.sum()),
+        "feasible_chains": int(cold.best_feasible.sum()),
+    }
+    if not args.no_cpu:
+        # the same host logic over the CPU build of the evaluator, all host cores, on a bounded number of steps
+        from oracle.cpu_port import CpuPort
+        threads = min(16, os.cpu_count() or 1)
+        steps = max(1, min(args.sa_steps, 40))
+        split = 1 if p.workload.gen_quantiles else 0
+        t0 = time.perf_counter()
+        ref = CpuPort(p).sa_run(sa_params(opt, args.chains, steps, variants, 0, split, 42), arrays, threads=threads)
+        dt = time.perf_counter() - t0
+        same = bool((ref["log"] == cold.log[:, :steps]).all())
+        n_ev = int(ref["n_eval"].sum())
+        line["cpu_baseline"] = dict(value=dt / steps * args.sa_steps, unit="s", cores=threads, kind="port",
+                                    sample=f"first {steps} steps of the same {args.chains} chains over the host build "
+                                           f"of the evaluator ({dt:.1f} s, {n_ev} evaluations), scaled to "
+                                           f"{args.sa_steps} steps; same decisions as the GPU run: {same}")
+        line["host_cores"] = os.cpu_count()
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,10 +135,15 @@ def main():
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="also run one device-to-device copy of this size (reference dispatch for scaling "
                          "FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--chains", type=int, default=64)
+    ap.add_argument("--sa-steps", type=int, default=2000)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every box of this build has one MI355X and the path needs no "
                  "second one (plans are independent; see DESIGN.md for how it would shard). Use --gpus 1.")
+
+    if args.config == 5:
+        return bench_sa(args)
 
     import torch
     from rpeg_amd import configs
@@ -80,7 +153,7 @@ def main():
 
     c = args.config
     cfg = configs.config(c)
-    n = cfg.n_plans if c != 5 else 64 * 6 * 256
+    n = cfg.n_plans
     batch = candidates.generate(cfg.problem, n, cfg.tau_choices, seed=42, tag=c)
     eng = Engine(cfg.problem, "cuda:0")
     db = DeviceBatch(batch, "cuda:0")
