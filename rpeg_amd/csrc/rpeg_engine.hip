@@ -92,9 +92,10 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
   sig[i] = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
 }
 
+template <int LS>
 __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
   extern __shared__ uint8_t ke_lds[];
-  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) ke_eval_wave(L, w, ke_lds);
+  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) ke_eval_wave<LS>(L, w, ke_lds);
 }
 
 // Generic single-wavefront kernel over the host/device-shared scheduler template; used for the
@@ -176,7 +177,8 @@ struct rpeg_engine_s {
   uint8_t* d_pool = nullptr;
   size_t d_pool_cap = 0, d_pool_used = 0;
   uint32_t max_nodes = 1, max_slots = 1, max_cls_bytes = 16;
-  bool lds_attr_set = false;
+  bool lds_attr_set[5] = {false, false, false, false, false};
+  int state_lanes = -1;   // -1: chosen per batch; 0: per-plan state in HBM; 8/16/32/64: in LDS, that many plans per wavefront
   bool prof_on = false;
   unsigned long long* d_prof = nullptr;
   uint64_t prof_waves = 0;
@@ -191,7 +193,7 @@ struct rpeg_engine_s {
   bool timing = false;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   double last_ms = -1.0;
-  uint64_t stats[5] = {0, 0, 0, 0, 0};
+  uint64_t stats[6] = {0, 0, 0, 0, 0, 0};
   int n_cu = 256;
 };
 
@@ -346,6 +348,16 @@ int rpeg_engine_profile(rpeg_engine_t* e, int32_t enable, unsigned long long* ou
   return 0;
 }
 
+int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
+  if (!e) return -1;
+  if (lanes != -1 && lanes != 0 && lanes != 8 && lanes != 16 && lanes != 32 && lanes != 64) {
+    e->err = "state lanes must be -1, 0, 8, 16, 32 or 64";
+    return -1;
+  }
+  e->state_lanes = lanes;
+  return 0;
+}
+
 int rpeg_engine_reset_classes(rpeg_engine_t* e) {
   if (!e) return -1;
   hipDeviceSynchronize();
@@ -357,7 +369,7 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
 
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n) {
   if (!e || !out) return -1;
-  for (int i = 0; i < n && i < 5; ++i) out[i] = e->stats[i];
+  for (int i = 0; i < n && i < 6; ++i) out[i] = e->stats[i];
   return 0;
 }
 
@@ -417,6 +429,29 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     ids[i] = last_id;
     ++counts[last_id];
   }
+  // Plans per wavefront and where their scheduler state lives.  A full batch keeps 64 plans per wavefront
+  // with the state in the HBM workspace; a batch too small to fill the chip that way is spread over more
+  // wavefronts of fewer plans whose state fits in LDS, which shortens every scheduler step.
+  int ls = e->state_lanes;
+  {
+    auto waves_for = [&](uint32_t per) { uint64_t t = 0; for (uint32_t c : counts) t += (c + per - 1) / per; return t; };
+    auto fits = [&](int l) {
+      return ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, 32, (uint32_t)l, e->max_nodes, e->max_slots) <= 160 * 1024;
+    };
+    if (ls < 0) {
+      ls = 0;
+      if (waves_for(WAVE) < (uint64_t)e->n_cu * 2)   // under two wavefronts per compute unit
+        for (int l : {8, 16, 32, 64}) {              // fewest plans per wavefront that still gives each its own SIMD
+          if (!fits(l)) break;
+          ls = l;
+          if (waves_for((uint32_t)l) <= (uint64_t)e->n_cu * 4) break;
+        }
+    } else if (ls > 0 && !fits(ls)) {
+      e->err = "per-plan state of this problem does not fit in LDS with that many plans per wavefront";
+      return -8;
+    }
+  }
+  const uint32_t lpw = ls ? (uint32_t)ls : (uint32_t)WAVE;   // plans per wavefront
   // every class starts on a wavefront boundary; the lanes left over are idle
   // classes with the largest graphs first: their wavefronts run longest and should not start last
   std::vector<uint32_t> order(counts.size());
@@ -424,32 +459,42 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
     return ((const ClassHdr*)(e->pool.data() + offs[a]))->n_nodes > ((const ClassHdr*)(e->pool.data() + offs[b]))->n_nodes;
   });
-  std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0);
+  // start[k]: first wavefront of the k-th class in launch order
+  std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0), clpw(counts.size(), lpw);
+  {
+    static const char* hn = getenv("RPEG_HEAVY_NODES");
+    static const char* hl = getenv("RPEG_HEAVY_LPW");
+    if (hn && hl && !ls)
+      for (size_t c = 0; c < counts.size(); ++c)
+        if (((const ClassHdr*)(e->pool.data() + offs[c]))->n_nodes >= (uint32_t)atoi(hn)) clpw[c] = (uint32_t)atoi(hl);
+  }
   for (size_t k = 0; k < order.size(); ++k) {
     first[order[k]] = start[k];
-    start[k + 1] = start[k] + (counts[order[k]] + WAVE - 1) / WAVE * WAVE;
+    start[k + 1] = start[k] + (counts[order[k]] + clpw[order[k]] - 1) / clpw[order[k]];
   }
-  const uint64_t n_sorted = start.back();
+  const uint64_t n_sorted = (uint64_t)start.back() * WAVE;
   e->stats[0] = counts.size();
   e->stats[1] = n_new;
   if (n_sorted == 0) return 0;
   if (int rc = ensure_perm(e, n_sorted)) return rc;
   std::fill(e->h_perm, e->h_perm + n_sorted, IDLE_LANE);
-  std::vector<uint32_t> cursor(first);
+  std::vector<uint32_t> cursor(counts.size(), 0);   // plans of the class placed so far
   for (uint64_t i = 0; i < n; ++i) {
     if (ids[i] == UINT32_MAX) continue;
-    e->h_perm[cursor[ids[i]]++] = (uint32_t)i;
+    const uint32_t k = cursor[ids[i]]++, cl = clpw[ids[i]];
+    e->h_perm[(size_t)(first[ids[i]] + k / cl) * WAVE + k % cl] = (uint32_t)i;
   }
   for (size_t k = 0; k < order.size(); ++k)
-    for (uint32_t w = start[k] / WAVE; w < start[k + 1] / WAVE; ++w) e->h_cls[w] = offs[order[k]];
+    for (uint32_t w = start[k]; w < start[k + 1]; ++w) e->h_cls[w] = offs[order[k]];
   if (int rc = ensure_pool(e, s)) return rc;
   HIP_TRY(e, hipMemcpyAsync(e->d_perm, e->h_perm, n_sorted * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted / WAVE * 4, hipMemcpyHostToDevice, s));
 
   const uint64_t n_waves = n_sorted / WAVE;
   const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * 16);
-  const size_t wsb = ke_ws_bytes(e->max_nodes, e->max_slots);
-  if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
+  const size_t wsb = ls ? 0 : ke_ws_bytes(e->max_nodes, e->max_slots);
+  if (!ls)
+    if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
   EvalLaunch L;
   L.P = e->dP; L.vert = plans->vert; L.head = plans->head; L.stride = plans->stride;
   L.perm = e->d_perm; L.wave_cls = e->d_cls; L.pool = e->d_pool; L.ws = e->d_ws;
@@ -469,17 +514,27 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     e->prof_waves = n_waves;
     L.prof = e->d_prof;
   }
-  const size_t lds = ke_lds_bytes(L.cls_bytes, L.rcap);
+  const size_t lds = ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots);
   if (lds > 160 * 1024) { e->err = "class tables exceed the LDS"; return -8; }
-  if (lds > 64 * 1024 && !e->lds_attr_set) {
-    HIP_TRY(e, hipFuncSetAttribute((const void*)k_eval, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    e->lds_attr_set = true;
+  const void* kfn = ls == 0 ? (const void*)k_eval<0> : ls == 8 ? (const void*)k_eval<8> : ls == 16 ? (const void*)k_eval<16>
+                  : ls == 32 ? (const void*)k_eval<32> : (const void*)k_eval<64>;
+  const int ki = ls == 0 ? 0 : ls == 8 ? 1 : ls == 16 ? 2 : ls == 32 ? 3 : 4;
+  if (lds > 64 * 1024 && !e->lds_attr_set[ki]) {
+    HIP_TRY(e, hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    e->lds_attr_set[ki] = true;
   }
   e->stats[2] = n_waves;
   e->stats[3] = lds;
   e->stats[4] = wsb * grid;
+  e->stats[5] = (uint64_t)ls;
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
-  hipLaunchKernelGGL(k_eval, dim3(grid), dim3(WAVE), lds, s, L);
+  switch (ls) {
+    case 0: hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds, s, L); break;
+    case 8: hipLaunchKernelGGL(k_eval<8>, dim3(grid), dim3(WAVE), lds, s, L); break;
+    case 16: hipLaunchKernelGGL(k_eval<16>, dim3(grid), dim3(WAVE), lds, s, L); break;
+    case 32: hipLaunchKernelGGL(k_eval<32>, dim3(grid), dim3(WAVE), lds, s, L); break;
+    default: hipLaunchKernelGGL(k_eval<64>, dim3(grid), dim3(WAVE), lds, s, L); break;
+  }
   HIP_TRY(e, hipGetLastError());
   if (e->timing) {
     HIP_TRY(e, hipEventRecord(e->ev1, s));

@@ -48,51 +48,62 @@ __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
   size_t lane = (16ull * nodes + 8ull * slots + nodes + 63) & ~size_t(63);
   return (size_t)KE_WAVE * lane;
 }
-__host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap) {
-  size_t ready = (size_t)rcap * KE_WAVE * 20;
-  size_t plan = (size_t)RPEG_MAX_V * RPEG_FIELDS * KE_WAVE * 2 + (size_t)RPEG_MAX_V * 4 * KE_WAVE * 8;
-  return cls_bytes + (ready > plan ? ready : plan);
+// Dynamic LDS of one wavefront.  ls = 0: the per-plan state lives in the HBM workspace and all 64 lanes
+// carry plans.  ls > 0: only the first `ls` lanes carry plans and their state (ready time, rank,
+// in-degree per node, duration per slot) lives in LDS too, interleaved by lane.
+__host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls) {
+  const size_t rw = ls ? ls : KE_WAVE;
+  size_t ready = (size_t)rcap * rw * 20;
+  size_t plan = (size_t)RPEG_MAX_V * RPEG_FIELDS * rw * 2 + (size_t)RPEG_MAX_V * 4 * rw * 8;
+  return ((ready > plan ? ready : plan) + 15) & ~size_t(15);
+}
+__host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap, uint32_t ls = 0, uint32_t nodes = 0,
+                                               uint32_t slots = 0) {
+  return cls_bytes + ke_dyn_bytes(rcap, ls) + (size_t)ls * ((16ull * nodes + 8ull * slots + nodes + 15) & ~15ull);
 }
 
 #if defined(__HIPCC__)
 
+template <int RW>
 __device__ inline VPlan ke_vplan(const int16_t* pl, int v) {
-  const int16_t* p = pl + v * RPEG_FIELDS * KE_WAVE;
+  const int16_t* p = pl + v * RPEG_FIELDS * RW;
   VPlan a;
-  a.dp = p[0 * KE_WAVE]; a.pp = p[1 * KE_WAVE]; a.tp = p[2 * KE_WAVE]; a.mb = p[3 * KE_WAVE];
-  a.o[0] = p[4 * KE_WAVE]; a.o[1] = p[5 * KE_WAVE]; a.o[2] = p[6 * KE_WAVE];
-  a.e[0] = p[7 * KE_WAVE]; a.e[1] = p[8 * KE_WAVE]; a.e[2] = p[9 * KE_WAVE];
+  a.dp = p[0 * RW]; a.pp = p[1 * RW]; a.tp = p[2 * RW]; a.mb = p[3 * RW];
+  a.o[0] = p[4 * RW]; a.o[1] = p[5 * RW]; a.o[2] = p[6 * RW];
+  a.e[0] = p[7 * RW]; a.e[1] = p[8 * RW]; a.e[2] = p[9 * RW];
   return a;
 }
 
+template <int RW>
 __device__ inline double ke_slot_duration(const rpeg_problem_t& P, const rpeg_struct_t& st, int split,
                                           const SlotDesc sd, const int16_t* pl, bool* zero_div) {
   switch (sd.type) {
     case SLOT_OP_UNSPLIT:
-      return op_time(P, st.vertex[sd.a], st.vertex[sd.a].unsplit, ke_vplan(pl, sd.a), zero_div);
+      return op_time(P, st.vertex[sd.a], st.vertex[sd.a].unsplit, ke_vplan<RW>(pl, sd.a), zero_div);
     case SLOT_OP_SUB:
-      return op_time(P, st.vertex[sd.a], st.vertex[sd.a].sub[split][sd.q], ke_vplan(pl, sd.a), zero_div);
+      return op_time(P, st.vertex[sd.a], st.vertex[sd.a].sub[split][sd.q], ke_vplan<RW>(pl, sd.a), zero_div);
     case SLOT_COMM_DATA: {
       const rpeg_edge_t& e = st.edge[sd.a];
       int64_t payload = sd.q == 0xFF ? e.full_bytes : e.sub_bytes[split][sd.q];
-      return comm_time(P, ke_vplan(pl, e.src), ke_vplan(pl, e.dst), payload, e.is_weight != 0);
+      return comm_time(P, ke_vplan<RW>(pl, e.src), ke_vplan<RW>(pl, e.dst), payload, e.is_weight != 0);
     }
     case SLOT_COMM_PUB: {
       const rpeg_pub_t& p = st.pub[sd.a];
-      VPlan s = ke_vplan(pl, p.src), d = ke_vplan(pl, p.dst);
+      VPlan s = ke_vplan<RW>(pl, p.src), d = ke_vplan<RW>(pl, p.dst);
       return comm_time(P, s, d, pub_payload(P, s, d, p.model), true);
     }
     default:
-      return reshard_time(P, ke_vplan(pl, sd.a), sd.b);
+      return reshard_time(P, ke_vplan<RW>(pl, sd.a), sd.b);
   }
 }
 
+template <int RW>
 struct KeVMem {  // per-vertex memory quantities in LDS, [vertex*4 + field][lane]
   const double* p;
-  __device__ double w_shard(int v) const { return p[(v * 4 + 0) * KE_WAVE]; }
-  __device__ double mem_w(int v) const { return p[(v * 4 + 1) * KE_WAVE]; }
-  __device__ double opt(int v) const { return p[(v * 4 + 2) * KE_WAVE]; }
-  __device__ double extra(int v) const { return p[(v * 4 + 3) * KE_WAVE]; }
+  __device__ double w_shard(int v) const { return p[(v * 4 + 0) * RW]; }
+  __device__ double mem_w(int v) const { return p[(v * 4 + 1) * RW]; }
+  __device__ double opt(int v) const { return p[(v * 4 + 2) * RW]; }
+  __device__ double extra(int v) const { return p[(v * 4 + 3) * RW]; }
 };
 
 // max of last_fin over the vertices of a bit set
@@ -105,7 +116,12 @@ __device__ inline double ke_dev_max(unsigned m, const double (&lf)[RPEG_MAX_V]) 
 
 #define KE_STAMP(k) do { if (L.prof && lane == first_lane) L.prof[w * 8 + (k)] = wall_clock64(); } while (0)
 
+// LS = 0: 64 plans per wavefront, per-plan state in the HBM workspace.  LS > 0: LS plans per wavefront
+// (lanes LS..63 only help to stage the class tables), per-plan state in LDS.
+template <int LS>
 __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* lds) {
+  constexpr int RW = LS ? LS : KE_WAVE;   // lane stride of the per-lane LDS arrays
+  constexpr int SS = LS ? LS : 1;         // element stride of the per-plan state arrays
   const int lane = threadIdx.x;
   int first_lane = 0;
   const rpeg_problem_t& P = *L.P;
@@ -117,41 +133,51 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   uint16_t* l_succ = (uint16_t*)(lds + (size_t)n * 8);                // uint16[n_succ]
   uint8_t* dyn = lds + L.cls_bytes;
   int16_t* l_plan = (int16_t*)dyn + lane;                             // [60][64], aliased with the ready list
-  double* l_vm = (double*)(dyn + (size_t)RPEG_MAX_V * RPEG_FIELDS * KE_WAVE * 2) + lane;  // [24][64], aliased too
-  double* r_key = (double*)dyn + lane;                                // [rcap][64]
-  double* r_rank = (double*)dyn + (size_t)L.rcap * KE_WAVE + lane;    // [rcap][64]
-  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * KE_WAVE * 16) + lane;  // [rcap][64] node | tie << 16
+  double* l_vm = (double*)(dyn + (size_t)RPEG_MAX_V * RPEG_FIELDS * RW * 2) + lane;  // [24][RW], aliased too
+  double* r_key = (double*)dyn + lane;                                // [rcap][RW]
+  double* r_rank = (double*)dyn + (size_t)L.rcap * RW + lane;         // [rcap][RW]
+  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * RW * 16) + lane;  // [rcap][RW] node | tie << 16
 
   __syncthreads();  // the previous task of this wavefront is done with LDS
   for (int i = lane; i < n; i += KE_WAVE) l_node[i] = ((const uint64_t*)cv.node)[i];
   for (int i = lane; i < n_succ_all; i += KE_WAVE) l_succ[i] = cv.succ[i];
   __syncthreads();
 
+  if (LS && lane >= LS) return;
   const uint64_t pi = L.perm[w * KE_WAVE + lane];
   if (pi == KE_IDLE) return;
   first_lane = __builtin_ctzll(__ballot(1));
   KE_STAMP(0);
 
   // ---- workspace rows of this lane
-  uint8_t* base = L.ws + (size_t)blockIdx.x * ke_ws_bytes(L.ws_nodes, L.ws_slots);
-  // per-lane contiguous block: time[nodes] rank[nodes] dur[slots] deg[nodes]
-  const size_t lane_bytes = ke_ws_bytes(L.ws_nodes, L.ws_slots) / KE_WAVE;
-  uint8_t* lbase = base + (size_t)lane * lane_bytes;
-  double* g_time = (double*)lbase;
-  double* g_rank = g_time + L.ws_nodes;
-  double* g_dur = g_rank + L.ws_nodes;
-  uint8_t* g_deg = (uint8_t*)(g_dur + L.ws_slots);
+  double *g_time, *g_rank, *g_dur;
+  uint8_t* g_deg;
+  if (LS) {  // LDS, [row][lane]: time[nodes] rank[nodes] dur[slots] deg[nodes]
+    uint8_t* sbase = dyn + ke_dyn_bytes(L.rcap, LS);
+    g_time = (double*)sbase + lane;
+    g_rank = g_time + (size_t)L.ws_nodes * LS;
+    g_dur = g_rank + (size_t)L.ws_nodes * LS;
+    g_deg = (uint8_t*)((double*)sbase + (2 * (size_t)L.ws_nodes + L.ws_slots) * LS) + lane;
+  } else {   // HBM, one contiguous block per lane: time[nodes] rank[nodes] dur[slots] deg[nodes]
+    uint8_t* base = L.ws + (size_t)blockIdx.x * ke_ws_bytes(L.ws_nodes, L.ws_slots);
+    const size_t lane_bytes = ke_ws_bytes(L.ws_nodes, L.ws_slots) / KE_WAVE;
+    uint8_t* lbase = base + (size_t)lane * lane_bytes;
+    g_time = (double*)lbase;
+    g_rank = g_time + L.ws_nodes;
+    g_dur = g_rank + L.ws_nodes;
+    g_deg = (uint8_t*)(g_dur + L.ws_slots);
+  }
 
   // ---- plan fields -> LDS
   const PlanHead h = load_head(L.head, L.stride, pi);
   const rpeg_struct_t& st = P.st[cv.h->structure];   // uniform (the class fixes the structure)
   const int nv = st.n_vertex;
-  for (int f = 0; f < nv * RPEG_FIELDS; ++f) l_plan[f * KE_WAVE] = L.vert[(uint64_t)f * L.stride + pi];
+  for (int f = 0; f < nv * RPEG_FIELDS; ++f) l_plan[f * RW] = L.vert[(uint64_t)f * L.stride + pi];
 
   VPlan a[RPEG_MAX_V];
 #pragma unroll
   for (int v = 0; v < RPEG_MAX_V; ++v)
-    if (v < nv) a[v] = ke_vplan(l_plan, v);
+    if (v < nv) a[v] = ke_vplan<RW>(l_plan, v);
 
   // ---- per-plan relations
   const PlanMasks pm = plan_masks(a, nv);
@@ -161,7 +187,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   // ---- durations of the class's slots
   bool err = cv.h->error != 0, zero_div = false;
   const int split = (int)cv.h->split;
-  for (int s = 0; s < n_slots; ++s) g_dur[s] = ke_slot_duration(P, st, split, cv.slot[s], l_plan, &zero_div);
+  for (int s = 0; s < n_slots; ++s) g_dur[(s) * SS] = ke_slot_duration<RW>(P, st, split, cv.slot[s], l_plan, &zero_div);
   err = err || zero_div;
 
   KE_STAMP(2);
@@ -170,12 +196,12 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   for (int v = 0; v < RPEG_MAX_V; ++v)
     if (v < nv) {
       const VMem m = vertex_memory(P, st.vertex[v], a[v]);
-      l_vm[(v * 4 + 0) * KE_WAVE] = (double)m.w_shard;
-      l_vm[(v * 4 + 1) * KE_WAVE] = m.mem_w;
-      l_vm[(v * 4 + 2) * KE_WAVE] = m.opt;
-      l_vm[(v * 4 + 3) * KE_WAVE] = m.extra;
+      l_vm[(v * 4 + 0) * RW] = (double)m.w_shard;
+      l_vm[(v * 4 + 1) * RW] = m.mem_w;
+      l_vm[(v * 4 + 2) * RW] = m.opt;
+      l_vm[(v * 4 + 3) * RW] = m.extra;
     }
-  const KeVMem kvm{l_vm};
+  const KeVMem<RW> kvm{l_vm};
   const double peak = device_peak_max(P, st, cv.h->vorder, pm, kvm);
   const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
   const bool mem_ok = !(peak > P.cap);
@@ -187,23 +213,23 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     const NodeRec nr = cv.node[v];
     double best = 0.0;
     for (int j = 0; j < nr.n_succ; ++j) {
-      const double r = g_rank[cv.succ[nr.succ_begin + j]];
+      const double r = g_rank[(cv.succ[nr.succ_begin + j]) * SS];
       best = r > best ? r : best;
     }
-    g_rank[v] = g_dur[nr.slot] + best;
+    g_rank[(v) * SS] = g_dur[(nr.slot) * SS] + best;
   }
   for (unsigned g = 0; g < cv.h->n_groups; ++g) {
     const GroupRec gr = cv.group[g];
-    double top = g_rank[cv.gmember[gr.begin]];
+    double top = g_rank[(cv.gmember[gr.begin]) * SS];
     for (int j = 1; j < gr.count; ++j) {
-      const double r = g_rank[cv.gmember[gr.begin + j]];
+      const double r = g_rank[(cv.gmember[gr.begin + j]) * SS];
       top = r > top ? r : top;
     }
-    for (int j = 0; j < gr.count; ++j) g_rank[cv.gmember[gr.begin + j]] = top;
+    for (int j = 0; j < gr.count; ++j) g_rank[(cv.gmember[gr.begin + j]) * SS] = top;
   }
   for (int v = 0; v < n; ++v) {
-    g_deg[v] = cv.node[v].indeg;
-    g_time[v] = 0.0;
+    g_deg[(v) * SS] = cv.node[v].indeg;
+    g_time[(v) * SS] = 0.0;
   }
 
   KE_STAMP(4);
@@ -217,9 +243,9 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   for (unsigned i = 0; i < cv.h->n_init && !err; ++i) {
     const int v = cv.init[i];
     if (n_ready >= rcap) { err = true; break; }
-    r_key[n_ready * KE_WAVE] = 0.0;
-    r_rank[n_ready * KE_WAVE] = g_rank[v];
-    r_nt[n_ready * KE_WAVE] = (uint32_t)v | ((uint32_t)cv.node[v].ptkey << 12) | (tie++ << 16);
+    r_key[n_ready * RW] = 0.0;
+    r_rank[n_ready * RW] = g_rank[(v) * SS];
+    r_nt[n_ready * RW] = (uint32_t)v | ((uint32_t)cv.node[v].ptkey << 12) | (tie++ << 16);
     ++n_ready;
   }
   double makespan = 0.0;
@@ -238,9 +264,9 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
       uint32_t m[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        k[u] = r_key[(j0 + u) * KE_WAVE];
-        r[u] = r_rank[(j0 + u) * KE_WAVE];
-        m[u] = r_nt[(j0 + u) * KE_WAVE];
+        k[u] = r_key[(j0 + u) * RW];
+        r[u] = r_rank[(j0 + u) * RW];
+        m[u] = r_nt[(j0 + u) * RW];
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -261,12 +287,12 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     const double dev = ke_dev_max(blocked, lf);
     const double est = dev > bk ? dev : bk;
     if (est > bk) {  // stale key: same entry, corrected est, fresh tie (scheduler.py:437-443)
-      r_key[bj * KE_WAVE] = est;
-      r_nt[bj * KE_WAVE] = (bm & 0xFFFFu) | (tie++ << 16);
+      r_key[bj * RW] = est;
+      r_nt[bj * RW] = (bm & 0xFFFFu) | (tie++ << 16);
       continue;
     }
     // dispatch bv: issue every load of this step before using any of them
-    const double d = g_dur[nr.slot];
+    const double d = g_dur[(nr.slot) * SS];
     int wv[4];
     double wt[4], wr[4];
     uint8_t wd[4];
@@ -275,24 +301,24 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     for (int j = 0; j < 4; ++j) {
       wv[j] = j < ns ? (int)l_succ[nr.succ_begin + j] : 0;
       if (j < ns) {
-        wt[j] = g_time[wv[j]];
-        wd[j] = g_deg[wv[j]];
-        wr[j] = g_rank[wv[j]];
+        wt[j] = g_time[(wv[j]) * SS];
+        wd[j] = g_deg[(wv[j]) * SS];
+        wr[j] = g_rank[(wv[j]) * SS];
       }
     }
     // remove the entry: the last entry takes its place (order is carried by the tie field)
     --n_ready;
     if (bj != n_ready) {
-      r_key[bj * KE_WAVE] = r_key[n_ready * KE_WAVE];
-      r_rank[bj * KE_WAVE] = r_rank[n_ready * KE_WAVE];
-      r_nt[bj * KE_WAVE] = r_nt[n_ready * KE_WAVE];
+      r_key[bj * RW] = r_key[n_ready * RW];
+      r_rank[bj * RW] = r_rank[n_ready * RW];
+      r_nt[bj * RW] = r_nt[n_ready * RW];
     }
     const double fin = est + d;
     makespan = fin > makespan ? fin : makespan;
     ++done;
     if (L.mass) {  // keep the trace: a dispatched node needs neither its ready time nor its rank again
-      g_time[bv] = fin;
-      g_rank[bv] = est;
+      g_time[(bv) * SS] = fin;
+      g_rank[(bv) * SS] = est;
     }
     unsigned touched = 0;
 #pragma unroll
@@ -307,9 +333,9 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         for (int j = 0; j < 4; ++j) {
           wv[j] = j0 + j < ns ? (int)l_succ[nr.succ_begin + j0 + j] : 0;
           if (j0 + j < ns) {
-            wt[j] = g_time[wv[j]];
-            wd[j] = g_deg[wv[j]];
-            wr[j] = g_rank[wv[j]];
+            wt[j] = g_time[(wv[j]) * SS];
+            wd[j] = g_deg[(wv[j]) * SS];
+            wr[j] = g_rank[(wv[j]) * SS];
           }
         }
       }
@@ -326,13 +352,13 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
           const double d2 = ke_dev_max(blocked_mask(wrc, dpne), lf);
           t = d2 > t ? d2 : t;
           if (n_ready >= rcap) { err = true; break; }
-          r_key[n_ready * KE_WAVE] = t;
-          r_rank[n_ready * KE_WAVE] = wr[j];
-          r_nt[n_ready * KE_WAVE] = (uint32_t)wn | ((uint32_t)wrc.ptkey << 12) | (tie++ << 16);
+          r_key[n_ready * RW] = t;
+          r_rank[n_ready * RW] = wr[j];
+          r_nt[n_ready * RW] = (uint32_t)wn | ((uint32_t)wrc.ptkey << 12) | (tie++ << 16);
           ++n_ready;
         } else {
-          g_time[wn] = t;
-          g_deg[wn] = left;
+          g_time[(wn) * SS] = t;
+          g_deg[(wn) * SS] = left;
         }
       }
     }
@@ -366,7 +392,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
 #pragma unroll
       for (int x = 0; x < RPEG_MAX_V; ++x) m[x] = __builtin_nan("");
     } else {
-      critical_mass(cv, [&](int i) { return g_time[i]; }, [&](int i) { return g_rank[i]; }, m);
+      critical_mass(cv, [&](int i) { return g_time[(i) * SS]; }, [&](int i) { return g_rank[(i) * SS]; }, m);
     }
 #pragma unroll
     for (int x = 0; x < RPEG_MAX_V; ++x) L.mass[pi * RPEG_MAX_V + x] = m[x];

@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run")
+           "rpeg_sa_run", "rpeg_engine_set_state_lanes")
 
 
 class EngineError(RuntimeError):
@@ -62,6 +62,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_set_timing.argtypes = [vp, i32]
     lib.rpeg_engine_last_kernel_ms.restype = C.c_double
     lib.rpeg_engine_last_kernel_ms.argtypes = [vp]
+    lib.rpeg_engine_set_state_lanes.restype = C.c_int
+    lib.rpeg_engine_set_state_lanes.argtypes = [vp, i32]
     lib.rpeg_engine_reset_classes.restype = C.c_int
     lib.rpeg_engine_reset_classes.argtypes = [vp]
     lib.rpeg_device_exp.restype = C.c_int
@@ -122,6 +124,10 @@ class Engine:
     def set_timing(self, on: bool):
         self.lib.rpeg_engine_set_timing(self._h, int(on))
 
+    def set_state_lanes(self, lanes: int):
+        """-1 automatic; 0 scheduler state in HBM (64 plans per wavefront); 8/16/32/64 state in LDS."""
+        self._check(self.lib.rpeg_engine_set_state_lanes(self._h, int(lanes)), "rpeg_engine_set_state_lanes")
+
     def reset_classes(self):
         self.lib.rpeg_engine_reset_classes(self._h)
 
@@ -129,9 +135,10 @@ class Engine:
         return float(self.lib.rpeg_engine_last_kernel_ms(self._h))
 
     def stats(self) -> Dict[str, int]:
-        buf = (C.c_uint64 * 5)()
-        self.lib.rpeg_engine_stats(self._h, buf, 5)
-        return dict(classes=buf[0], classes_lowered=buf[1], wave_tasks=buf[2], lds_bytes=buf[3], workspace_bytes=buf[4])
+        buf = (C.c_uint64 * 6)()
+        self.lib.rpeg_engine_stats(self._h, buf, 6)
+        return dict(classes=buf[0], classes_lowered=buf[1], wave_tasks=buf[2], lds_bytes=buf[3], workspace_bytes=buf[4],
+                    state_lanes=buf[5])
 
     def alloc_outputs(self, n: int):
         torch = _torch()
