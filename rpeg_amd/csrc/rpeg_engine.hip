@@ -68,9 +68,27 @@ __host__ __device__ inline size_t wave_ws_bytes(uint32_t nodes, uint32_t slots) 
   return (b + 255) & ~size_t(255);
 }
 
+constexpr uint32_t CID_INVALID = 0xFFFFFFFFu, CID_UNKNOWN = 0xFFFFFFFEu;
+
+__host__ __device__ inline uint64_t sig_hash(uint64_t x) {
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+
+__global__ void k_fill_u32(uint32_t* p, uint64_t n, uint32_t v) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// Integer validity gate, class signature, class id (open-addressing table of the classes lowered so far)
+// and the per-class plan count.  count[n_classes] counts the plans of classes not lowered yet.
 __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
                             const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig,
-                            double* makespan, double* peak, double* score, uint8_t* mask, double* mass) {
+                            double* makespan, double* peak, double* score, uint8_t* mask, double* mass,
+                            const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval, uint32_t hmask,
+                            uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
+                            uint32_t n_classes) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   PlanHead h = load_head(head, stride, i);
@@ -87,9 +105,50 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
     if (mask) mask[i] = 0;
     if (mass)
       for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
+    cid[i] = CID_INVALID;
     return;
   }
-  sig[i] = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
+  const uint64_t sg = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
+  sig[i] = sg;
+  uint32_t c = CID_UNKNOWN;
+  for (uint32_t slot = (uint32_t)sig_hash(sg) & hmask, probes = 0; probes <= hmask; slot = (slot + 1) & hmask, ++probes) {
+    const uint64_t key = hkey[slot];
+    if (key == sg) { c = hval[slot]; break; }
+    if (key == SIG_INVALID) break;
+  }
+  cid[i] = c;
+  // arrival index within the class: one atomic per distinct class of the wavefront, not per plan
+  const uint32_t key = c == CID_UNKNOWN ? n_classes : c;
+  const int lane = (int)(threadIdx.x & (WAVE - 1));
+  bool pending = true;
+  uint32_t k = 0;
+  for (int guard = 0; guard < WAVE; ++guard) {
+    const unsigned long long am = __ballot(pending);
+    if (!am) break;
+    const int leader = __ffsll(am) - 1;
+    const uint32_t k0 = (uint32_t)__shfl((int)key, leader);
+    const unsigned long long same = __ballot(pending && key == k0);
+    uint32_t base = 0;
+    if (lane == leader) base = atomicAdd(&count[k0], (uint32_t)__popcll(same));
+    base = (uint32_t)__shfl((int)base, leader);
+    if (pending && key == k0) {
+      k = base + (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
+      pending = false;
+    }
+  }
+  kidx[i] = k;
+}
+
+// perm[(first wavefront of the class + k / lanes) * 64 + k % lanes] = plan, k = arrival order within the class
+__global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const uint32_t* __restrict__ kidx,
+                          const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
+                          uint32_t* __restrict__ perm) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t c = cid[i];
+  if (c >= CID_UNKNOWN) return;
+  const uint32_t k = kidx[i], l = clpw[c];
+  perm[(uint64_t)(cfirst[c] + k / l) * WAVE + k % l] = (uint32_t)i;
 }
 
 template <int LS>
@@ -173,6 +232,15 @@ struct rpeg_engine_s {
   std::string err;
   // lowering classes
   std::unordered_map<uint64_t, uint32_t> class_off;  // signature -> byte offset in the pool
+  std::vector<uint64_t> cls_sig;                     // class id -> signature / pool offset / node count
+  std::vector<uint32_t> cls_off, cls_nodes;
+  uint64_t* d_hkey = nullptr;                        // device table signature -> class id
+  uint32_t* d_hval = nullptr;
+  uint32_t hcap = 0, tables_for = 0;                 // table capacity; class count the device tables reflect
+  uint32_t ccap = 0;                                 // capacity of the per-class device arrays
+  uint32_t *d_ccount = nullptr, *d_cfirst = nullptr, *d_clpw = nullptr;
+  uint32_t *h_ccount = nullptr, *h_cfirst = nullptr, *h_clpw = nullptr;
+  uint32_t *d_cid = nullptr, *d_kidx = nullptr;   // per plan: class id, arrival index within the class
   std::vector<uint8_t> pool;
   uint8_t* d_pool = nullptr;
   size_t d_pool_cap = 0, d_pool_used = 0;
@@ -200,11 +268,56 @@ struct rpeg_engine_s {
 static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (n <= e->cap_n) return 0;
   size_t cap = std::max<size_t>(n, 4096);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); }
   e->cap_n = 0;
   HIP_TRY(e, hipMalloc(&e->d_sig, cap * 8));
   HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
+  HIP_TRY(e, hipMalloc(&e->d_cid, cap * 4));
+  HIP_TRY(e, hipMalloc(&e->d_kidx, cap * 4));
   e->cap_n = cap;
+  return 0;
+}
+
+// device copies of the class tables: signature -> class id, and room for the per-class counters
+static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
+  const uint32_t ncls = (uint32_t)e->cls_sig.size();
+  if (e->d_hkey && e->tables_for == ncls) return 0;
+  HIP_TRY(e, hipStreamSynchronize(s));
+  uint32_t hcap = 1024;
+  while (hcap < 4 * ncls) hcap *= 2;
+  if (hcap != e->hcap) {
+    if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
+    e->d_hkey = nullptr; e->hcap = 0;
+    HIP_TRY(e, hipMalloc(&e->d_hkey, (size_t)hcap * 8));
+    HIP_TRY(e, hipMalloc(&e->d_hval, (size_t)hcap * 4));
+    e->hcap = hcap;
+  }
+  std::vector<uint64_t> hk(hcap, SIG_INVALID);
+  std::vector<uint32_t> hv(hcap, 0);
+  for (uint32_t c = 0; c < ncls; ++c) {
+    uint32_t slot = (uint32_t)sig_hash(e->cls_sig[c]) & (hcap - 1);
+    while (hk[slot] != SIG_INVALID) slot = (slot + 1) & (hcap - 1);
+    hk[slot] = e->cls_sig[c];
+    hv[slot] = c;
+  }
+  HIP_TRY(e, hipMemcpy(e->d_hkey, hk.data(), (size_t)hcap * 8, hipMemcpyHostToDevice));
+  HIP_TRY(e, hipMemcpy(e->d_hval, hv.data(), (size_t)hcap * 4, hipMemcpyHostToDevice));
+  if (ncls + 1 > e->ccap) {
+    const uint32_t cap = std::max<uint32_t>(2 * (ncls + 1), 4096);
+    if (e->d_ccount) {
+      hipFree(e->d_ccount); hipFree(e->d_cfirst); hipFree(e->d_clpw);
+      hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
+    }
+    e->d_ccount = nullptr; e->ccap = 0;
+    HIP_TRY(e, hipMalloc(&e->d_ccount, (size_t)cap * 4));
+    HIP_TRY(e, hipMalloc(&e->d_cfirst, (size_t)cap * 4));
+    HIP_TRY(e, hipMalloc(&e->d_clpw, (size_t)cap * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (size_t)cap * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_cfirst, (size_t)cap * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_clpw, (size_t)cap * 4));
+    e->ccap = cap;
+  }
+  e->tables_for = ncls;
   return 0;
 }
 
@@ -262,6 +375,9 @@ static int64_t class_offset(rpeg_engine_t* e, uint64_t sig, bool* is_new) {
   uint32_t off = (uint32_t)e->pool.size();
   e->pool.insert(e->pool.end(), lc.blob.begin(), lc.blob.end());
   e->class_off.emplace(sig, off);
+  e->cls_sig.push_back(sig);
+  e->cls_off.push_back(off);
+  e->cls_nodes.push_back(h->n_nodes);
   if (is_new) *is_new = true;
   return off;
 }
@@ -317,7 +433,12 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   hipDeviceSynchronize();
   if (e->dP) hipFree(e->dP);
   if (e->d_pool) hipFree(e->d_pool);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); }
+  if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
+  if (e->d_ccount) {
+    hipFree(e->d_ccount); hipFree(e->d_cfirst); hipFree(e->d_clpw);
+    hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
+  }
   if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
@@ -362,6 +483,10 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
   if (!e) return -1;
   hipDeviceSynchronize();
   e->class_off.clear();
+  e->cls_sig.clear();
+  e->cls_off.clear();
+  e->cls_nodes.clear();
+  e->tables_for = 0xFFFFFFFFu;
   e->pool.clear();
   e->d_pool_used = 0;
   return 0;
@@ -396,39 +521,39 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   hipStream_t s = (hipStream_t)stream;
   if (int rc = ensure_batch(e, n)) return rc;
   const unsigned blk = 256;
-  hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + blk - 1) / blk)), dim3(blk), 0, s, e->dP, n, plans->vert,
-                     plans->head, plans->stride, e->d_sig, makespan, peak, score, mask, mass);
-  HIP_TRY(e, hipGetLastError());
-  HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
-  HIP_TRY(e, hipStreamSynchronize(s));
-
-  // group plans by class: count, prefix, scatter (stable within a class)
-  std::unordered_map<uint64_t, uint32_t> local;  // signature -> dense id within this batch
-  std::vector<uint32_t> offs, counts;
-  std::vector<uint32_t> ids(n);
+  const unsigned nblk = (unsigned)((n + blk - 1) / blk);
+  // classes of the batch: every plan looks its class id up on the device and counts itself; only the
+  // per-class counts come back.  Plans of classes not lowered yet make the call take the slow round:
+  // their signatures are read back, the classes are lowered on the host, the tables are rebuilt.
   uint64_t n_new = 0;
-  uint64_t last_sig = SIG_INVALID;
-  uint32_t last_id = 0;
-  for (uint64_t i = 0; i < n; ++i) {
-    const uint64_t sg = e->h_sig[i];
-    if (sg == SIG_INVALID) { ids[i] = UINT32_MAX; continue; }
-    if (sg != last_sig) {
-      auto it = local.find(sg);
-      if (it == local.end()) {
-        bool is_new = false;
-        int64_t off = class_offset(e, sg, &is_new);
-        if (off < 0) return -5;
-        n_new += is_new;
-        it = local.emplace(sg, (uint32_t)offs.size()).first;
-        offs.push_back((uint32_t)off);
-        counts.push_back(0);
-      }
+  uint32_t ncls = 0;
+  for (int round = 0;; ++round) {
+    if (int rc = ensure_class_tables(e, s)) return rc;
+    ncls = (uint32_t)e->cls_sig.size();
+    hipLaunchKernelGGL(k_fill_u32, dim3((ncls + 1 + blk - 1) / blk), dim3(blk), 0, s, e->d_ccount, (uint64_t)ncls + 1, 0u);
+    hipLaunchKernelGGL(k_signature, dim3(nblk), dim3(blk), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
+                       e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
+                       e->d_kidx, e->d_ccount, ncls);
+    HIP_TRY(e, hipGetLastError());
+    HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, ((size_t)ncls + 1) * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipStreamSynchronize(s));
+    if (e->h_ccount[ncls] == 0) break;
+    if (round >= 2) { e->err = "class table did not converge"; return -5; }
+    HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipStreamSynchronize(s));
+    uint64_t last_sig = SIG_INVALID;
+    for (uint64_t i = 0; i < n; ++i) {
+      const uint64_t sg = e->h_sig[i];
+      if (sg == SIG_INVALID || sg == last_sig) continue;
       last_sig = sg;
-      last_id = it->second;
+      bool is_new = false;
+      if (class_offset(e, sg, &is_new) < 0) return -5;
+      n_new += is_new;
     }
-    ids[i] = last_id;
-    ++counts[last_id];
   }
+  std::vector<uint32_t> offs, counts, cids;   // the classes present in this batch
+  for (uint32_t c = 0; c < ncls; ++c)
+    if (e->h_ccount[c]) { cids.push_back(c); offs.push_back(e->cls_off[c]); counts.push_back(e->h_ccount[c]); }
   // Plans per wavefront and where their scheduler state lives.  A full batch keeps 64 plans per wavefront
   // with the state in the HBM workspace; a batch too small to fill the chip that way is spread over more
   // wavefronts of fewer plans whose state fits in LDS, which shortens every scheduler step.
@@ -461,12 +586,22 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   });
   // start[k]: first wavefront of the k-th class in launch order
   std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0), clpw(counts.size(), lpw);
-  {
-    static const char* hn = getenv("RPEG_HEAVY_NODES");
-    static const char* hl = getenv("RPEG_HEAVY_LPW");
-    if (hn && hl && !ls)
+  if (!ls && !order.empty()) {
+    // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
+    // classes with the largest graphs (within a tenth of the largest) get eight plans per wavefront, so
+    // that fewer plans wait for the slowest one, unless they are a large share of the batch or the batch
+    // is many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest).
+    static const char* hl = getenv("RPEG_HEAVY_LPW");   // development override
+    const uint32_t heavy_lpw = hl ? (uint32_t)atoi(hl) : 8u;
+    const uint32_t top = e->cls_nodes[cids[order[0]]];
+    uint64_t heavy_plans = 0;
+    for (size_t c = 0; c < counts.size(); ++c)
+      if (10ull * e->cls_nodes[cids[c]] >= 9ull * top) heavy_plans += counts[c];
+    uint64_t waves64 = 0;
+    for (uint32_t c : counts) waves64 += (c + WAVE - 1) / WAVE;
+    if (heavy_plans * 4 <= n && waves64 <= (uint64_t)e->n_cu * 16 && heavy_lpw >= 1 && heavy_lpw <= WAVE)
       for (size_t c = 0; c < counts.size(); ++c)
-        if (((const ClassHdr*)(e->pool.data() + offs[c]))->n_nodes >= (uint32_t)atoi(hn)) clpw[c] = (uint32_t)atoi(hl);
+        if (10ull * e->cls_nodes[cids[c]] >= 9ull * top) clpw[c] = heavy_lpw;
   }
   for (size_t k = 0; k < order.size(); ++k) {
     first[order[k]] = start[k];
@@ -477,18 +612,19 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   e->stats[1] = n_new;
   if (n_sorted == 0) return 0;
   if (int rc = ensure_perm(e, n_sorted)) return rc;
-  std::fill(e->h_perm, e->h_perm + n_sorted, IDLE_LANE);
-  std::vector<uint32_t> cursor(counts.size(), 0);   // plans of the class placed so far
-  for (uint64_t i = 0; i < n; ++i) {
-    if (ids[i] == UINT32_MAX) continue;
-    const uint32_t k = cursor[ids[i]]++, cl = clpw[ids[i]];
-    e->h_perm[(size_t)(first[ids[i]] + k / cl) * WAVE + k % cl] = (uint32_t)i;
+  for (size_t c = 0; c < counts.size(); ++c) {
+    e->h_cfirst[cids[c]] = first[c];
+    e->h_clpw[cids[c]] = clpw[c];
   }
   for (size_t k = 0; k < order.size(); ++k)
     for (uint32_t w = start[k]; w < start[k + 1]; ++w) e->h_cls[w] = offs[order[k]];
   if (int rc = ensure_pool(e, s)) return rc;
-  HIP_TRY(e, hipMemcpyAsync(e->d_perm, e->h_perm, n_sorted * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_cfirst, e->h_cfirst, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_clpw, e->h_clpw, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted / WAVE * 4, hipMemcpyHostToDevice, s));
+  hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
+  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_perm);
+  HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_sorted / WAVE;
   const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * 16);

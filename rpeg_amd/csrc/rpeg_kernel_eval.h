@@ -53,7 +53,8 @@ __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
 // in-degree per node, duration per slot) lives in LDS too, interleaved by lane.
 __host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls) {
   const size_t rw = ls ? ls : KE_WAVE;
-  size_t ready = (size_t)rcap * rw * 20;
+  // ready list (key, rank, meta) with eight entries of slack for the batched list shifts
+  size_t ready = (size_t)(rcap + 8) * rw * 20;
   size_t plan = (size_t)RPEG_MAX_V * RPEG_FIELDS * rw * 2 + (size_t)RPEG_MAX_V * 4 * rw * 8;
   return ((ready > plan ? ready : plan) + 15) & ~size_t(15);
 }
@@ -134,9 +135,9 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   uint8_t* dyn = lds + L.cls_bytes;
   int16_t* l_plan = (int16_t*)dyn + lane;                             // [60][64], aliased with the ready list
   double* l_vm = (double*)(dyn + (size_t)RPEG_MAX_V * RPEG_FIELDS * RW * 2) + lane;  // [24][RW], aliased too
-  double* r_key = (double*)dyn + lane;                                // [rcap][RW]
-  double* r_rank = (double*)dyn + (size_t)L.rcap * RW + lane;         // [rcap][RW]
-  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * RW * 16) + lane;  // [rcap][RW] node | tie << 16
+  double* r_key = (double*)dyn + lane;                                // [rcap+8][RW]
+  double* r_rank = (double*)dyn + (size_t)(L.rcap + 8) * RW + lane;   // [rcap+8][RW]
+  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)(L.rcap + 8) * RW * 16) + lane;  // [rcap+8][RW] node | prio << 12 | x << 16 | y << 19
 
   __syncthreads();  // the previous task of this wavefront is done with LDS
   for (int i = lane; i < n; i += KE_WAVE) l_node[i] = ((const uint64_t*)cv.node)[i];
@@ -233,33 +234,92 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   }
 
   KE_STAMP(4);
-  // ---- list scheduling
+  // ---- list scheduling (scheduler.py:399-546 with the lazy heap replaced by a position-ordered list)
+  //
+  // The reference pops the minimum of (est, comm_prio, topo_idx, -rank, tie) from a heap whose keys may
+  // be stale: a popped entry whose true est (device availability included) exceeds its key is pushed
+  // back with the true est and a fresh tie.  Here the ready list is kept sorted by the part of the key
+  // that never changes while an entry waits: (comm_prio*8+topo_idx ascending, rank descending, push
+  // order); a new entry goes behind every entry that is not after it.
+  //
+  // While no two waiting entries agree in (prio, rank), a fresh tie cannot change the order, and the
+  // next node the heap dispatches is simply the first entry of minimum TRUE est; the entries the heap
+  // would have popped and pushed back on the way are those whose (key, position) precedes the winner's
+  // (true est, position): their keys are raised to their true est.  Every plan of the wavefront then
+  // dispatches one node per iteration, in lock step.  A plan whose list holds two entries of equal
+  // (prio, rank) takes the heap's own steps instead (pop by key; push back behind its equals, or
+  // dispatch) until the pair is gone.
   double lf[RPEG_MAX_V];
 #pragma unroll
   for (int x = 0; x < RPEG_MAX_V; ++x) lf[x] = 0.0;
   int n_ready = 0, done = 0;
-  uint32_t tie = 0;
   const int rcap = (int)L.rcap;
-  for (unsigned i = 0; i < cv.h->n_init && !err; ++i) {
-    const int v = cv.init[i];
-    if (n_ready >= rcap) { err = true; break; }
-    r_key[n_ready * RW] = 0.0;
-    r_rank[n_ready * RW] = g_rank[(v) * SS];
-    r_nt[n_ready * RW] = (uint32_t)v | ((uint32_t)cv.node[v].ptkey << 12) | (tie++ << 16);
-    ++n_ready;
+  const double inf = __builtin_inf();
+  for (int j = 0; j < rcap + 8; ++j) {   // entries past n_ready never win a scan
+    r_key[j * RW] = inf;
+    r_nt[j * RW] = 0;
   }
-  double makespan = 0.0;
-  const long guard_max = (long)n * n + 64;
-  long guard_total = 0;
-  for (long guard = 0; !err && done < n && guard < guard_max; ++guard) {
-    ++guard_total;
-    if (n_ready == 0 || tie >= 0xFFF0u) { err = true; break; }
-    // arg-min of (est, comm_prio*8+topo_idx, -rank, tie) over the ready list, eight entries per
-    // batch of LDS loads (entries past n_ready are in bounds and ignored)
-    int bj = 0;
-    double bk = __builtin_inf(), br = 0.0;
-    uint32_t bm = 0;
+  // meta: node | prio << 12 | x << 16 | y << 19, with x, y the (one or two) vertices whose devices the node reserves
+  auto make_meta = [&](int v, const NodeRec& r) -> uint32_t {
+    const unsigned blk = blocked_mask(r, dpne);
+    const unsigned x = (unsigned)__builtin_ctz(blk | 0x100u);
+    const unsigned rest = blk & (blk - 1u);
+    const unsigned y = rest ? (unsigned)__builtin_ctz(rest) : x;
+    if (rest & (rest - 1u)) err = true;   // more than two reserved vertices cannot be packed
+    return (uint32_t)v | ((uint32_t)r.ptkey << 12) | (x << 16) | (y << 19);
+  };
+  auto push = [&](uint32_t meta, double key, double rank) {
+    const unsigned pt = (meta >> 12) & 15u;
+    int pos = 0;
     for (int j0 = 0; j0 < n_ready; j0 += 8) {
+      double r[8];
+      uint32_t m[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        r[u] = r_rank[(j0 + u) * RW];
+        m[u] = r_nt[(j0 + u) * RW];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const unsigned pu = (m[u] >> 12) & 15u;
+        const bool after = pu > pt || (pu == pt && r[u] < rank);
+        pos += (j0 + u < n_ready && !after) ? 1 : 0;
+      }
+    }
+    for (int j1 = n_ready; j1 > pos; j1 -= 8) {   // entries [pos, n_ready) move one up, eight per round trip
+      double k[8], r[8];
+      uint32_t m[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int src = j1 - 1 - u < 0 ? 0 : j1 - 1 - u;
+        k[u] = r_key[src * RW];
+        r[u] = r_rank[src * RW];
+        m[u] = r_nt[src * RW];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int src = j1 - 1 - u;
+        if (src < pos) continue;
+        r_key[(src + 1) * RW] = k[u];
+        r_rank[(src + 1) * RW] = r[u];
+        r_nt[(src + 1) * RW] = m[u];
+      }
+    }
+    r_key[pos * RW] = key;
+    r_rank[pos * RW] = rank;
+    r_nt[pos * RW] = meta;
+    ++n_ready;
+  };
+  // Up to four pushes at once, with the result of pushing them one after the other: a stable merge in
+  // which a new entry goes behind the waiting entries and the earlier new entries that are not after it.
+  // The list is read and written once, from the top down (entries only move up).
+  auto push_many = [&](int cnt, const uint32_t (&nm)[4], const double (&nk)[4], const double (&nr)[4]) {
+    unsigned npt[4];
+    int c[4] = {0, 0, 0, 0};   // waiting entries not after new entry q
+#pragma unroll
+    for (int q = 0; q < 4; ++q) npt[q] = (nm[q] >> 12) & 15u;
+    for (int j1 = (n_ready + 7) & ~7; j1 > 0; j1 -= 8) {
+      const int j0 = j1 - 8;
       double k[8], r[8];
       uint32_t m[8];
 #pragma unroll
@@ -271,26 +331,98 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         if (j0 + u >= n_ready) continue;
-        bool better = k[u] < bk;
-        if (k[u] == bk) {
-          const unsigned pa = (m[u] >> 12) & 15u, pb = (bm >> 12) & 15u;
-          better = pa != pb ? pa < pb : (r[u] > br || (r[u] == br && (m[u] >> 16) < (bm >> 16)));
+        const unsigned pu = (m[u] >> 12) & 15u;
+        int up = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const bool after = pu > npt[q] || (pu == npt[q] && r[u] < nr[q]);   // the waiting entry is after new entry q
+          up += (q < cnt && after) ? 1 : 0;
+          c[q] += after ? 0 : 1;
         }
-        if (better) { bj = j0 + u; bk = k[u]; br = r[u]; bm = m[u]; }
+        if (up) {
+          r_key[(j0 + u + up) * RW] = k[u];
+          r_rank[(j0 + u + up) * RW] = r[u];
+          r_nt[(j0 + u + up) * RW] = m[u];
+        }
       }
     }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (q >= cnt) break;
+      int idx = c[q];
+#pragma unroll
+      for (int o = 0; o < 4; ++o) {
+        if (o == q || o >= cnt) continue;
+        const bool o_after = npt[o] > npt[q] || (npt[o] == npt[q] && nr[o] < nr[q]);     // o strictly after q
+        const bool o_before = npt[o] < npt[q] || (npt[o] == npt[q] && nr[o] > nr[q]);    // o strictly before q
+        idx += (o < q ? !o_after : o_before) ? 1 : 0;
+      }
+      r_key[idx * RW] = nk[q];
+      r_rank[idx * RW] = nr[q];
+      r_nt[idx * RW] = nm[q];
+    }
+    n_ready += cnt;
+  };
+  for (unsigned i = 0; i < cv.h->n_init && !err; ++i) {
+    const int v = cv.init[i];
+    if (n_ready >= rcap - 1) { err = true; break; }
+    push(make_meta(v, cv.node[v]), 0.0, g_rank[(v) * SS]);
+  }
+  double makespan = 0.0;
+  const long guard_max = (long)n * n + 64;
+  long guard_total = 0;
+  for (long guard = 0; !err && done < n && guard < guard_max; ++guard) {
+    ++guard_total;
+    if (n_ready == 0) { err = true; break; }
+    // The heap's pops up to the next dispatch: first entry of minimum key; while that key is stale, raise
+    // it to the true est and move the entry behind its equals (scheduler.py:437-443).  This inner loop is
+    // short; the dispatch below then runs once per node for all plans of the wavefront together.
+    int bj = 0;
+    double est = 0.0;
+    for (long inner = 0; inner < guard_max; ++inner) {
+      double bk = inf;
+      bj = 0;
+      for (int j0 = 0; j0 < n_ready; j0 += 8) {
+        double k[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) k[u] = r_key[(j0 + u) * RW];
+        const bool c01 = k[1] < k[0], c23 = k[3] < k[2], c45 = k[5] < k[4], c67 = k[7] < k[6];
+        const double a0 = c01 ? k[1] : k[0], a1 = c23 ? k[3] : k[2], a2 = c45 ? k[5] : k[4], a3 = c67 ? k[7] : k[6];
+        const int i0 = c01 ? 1 : 0, i1 = c23 ? 3 : 2, i2 = c45 ? 5 : 4, i3 = c67 ? 7 : 6;
+        const bool d0 = a1 < a0, d1 = a3 < a2;
+        const double b0 = d0 ? a1 : a0, b1 = d1 ? a3 : a2;
+        const int x0 = d0 ? i1 : i0, x1 = d1 ? i3 : i2;
+        const bool e0 = b1 < b0;
+        const double c = e0 ? b1 : b0;
+        if (c < bk) { bk = c; bj = j0 + (e0 ? x1 : x0); }
+      }
+      const uint32_t m0 = r_nt[bj * RW];
+      const double my_rank = r_rank[bj * RW];
+      const uint32_t m1 = r_nt[(bj + 1) * RW];
+      const double r1 = r_rank[(bj + 1) * RW];
+      const double dv = ke_dev_max((1u << ((m0 >> 16) & 7u)) | (1u << ((m0 >> 19) & 7u)), lf);
+      est = dv > bk ? dv : bk;
+      if (!(est > bk)) break;
+      ++guard_total;
+      r_key[bj * RW] = est;
+      if (bj + 1 < n_ready && ((m1 ^ m0) & 0xF000u) == 0 && r1 == my_rank) {
+        while (bj + 1 < n_ready) {
+          const uint32_t m2 = r_nt[(bj + 1) * RW];
+          const double r2 = r_rank[(bj + 1) * RW];
+          if (((m2 ^ m0) & 0xF000u) != 0 || r2 != my_rank) break;
+          const double k2 = r_key[(bj + 1) * RW];
+          r_key[bj * RW] = k2; r_rank[bj * RW] = r2; r_nt[bj * RW] = m2;
+          ++bj;
+          r_key[bj * RW] = est; r_rank[bj * RW] = my_rank; r_nt[bj * RW] = m0;
+        }
+      }
+    }
+    const uint32_t bm = r_nt[bj * RW];
     const int bv = (int)(bm & 0xFFFu);
+    const unsigned blocked = (1u << ((bm >> 16) & 7u)) | (1u << ((bm >> 19) & 7u));
     const uint64_t nbits = l_node[bv];
     NodeRec nr;
     __builtin_memcpy(&nr, &nbits, 8);
-    const unsigned blocked = blocked_mask(nr, dpne);
-    const double dev = ke_dev_max(blocked, lf);
-    const double est = dev > bk ? dev : bk;
-    if (est > bk) {  // stale key: same entry, corrected est, fresh tie (scheduler.py:437-443)
-      r_key[bj * RW] = est;
-      r_nt[bj * RW] = (bm & 0xFFFFu) | (tie++ << 16);
-      continue;
-    }
     // dispatch bv: issue every load of this step before using any of them
     const double d = g_dur[(nr.slot) * SS];
     int wv[4];
@@ -306,13 +438,26 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         wr[j] = g_rank[(wv[j]) * SS];
       }
     }
-    // remove the entry: the last entry takes its place (order is carried by the tie field)
+    // remove the entry, keeping the order
     --n_ready;
-    if (bj != n_ready) {
-      r_key[bj * RW] = r_key[n_ready * RW];
-      r_rank[bj * RW] = r_rank[n_ready * RW];
-      r_nt[bj * RW] = r_nt[n_ready * RW];
+    for (int j0 = bj; j0 < n_ready; j0 += 8) {    // entries (bj, n_ready] move one down, eight per round trip
+      double k[8], r[8];
+      uint32_t m[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        k[u] = r_key[(j0 + 1 + u) * RW];
+        r[u] = r_rank[(j0 + 1 + u) * RW];
+        m[u] = r_nt[(j0 + 1 + u) * RW];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (j0 + u >= n_ready) continue;
+        r_key[(j0 + u) * RW] = k[u];
+        r_rank[(j0 + u) * RW] = r[u];
+        r_nt[(j0 + u) * RW] = m[u];
+      }
     }
+    r_key[n_ready * RW] = inf;
     const double fin = est + d;
     makespan = fin > makespan ? fin : makespan;
     ++done;
@@ -339,6 +484,10 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
           }
         }
       }
+      // successors that become ready are collected in successor order and pushed together
+      uint32_t nm[4] = {0, 0, 0, 0};
+      double nk[4] = {0.0, 0.0, 0.0, 0.0}, nrk[4] = {0.0, 0.0, 0.0, 0.0};
+      int cnt = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (j0 + j >= ns) break;
@@ -351,16 +500,18 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
           __builtin_memcpy(&wrc, &wb, 8);
           const double d2 = ke_dev_max(blocked_mask(wrc, dpne), lf);
           t = d2 > t ? d2 : t;
-          if (n_ready >= rcap) { err = true; break; }
-          r_key[n_ready * RW] = t;
-          r_rank[n_ready * RW] = wr[j];
-          r_nt[n_ready * RW] = (uint32_t)wn | ((uint32_t)wrc.ptkey << 12) | (tie++ << 16);
-          ++n_ready;
+          const uint32_t meta = make_meta(wn, wrc);
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (q == cnt) { nm[q] = meta; nk[q] = t; nrk[q] = wr[j]; }
+          ++cnt;
         } else {
           g_time[(wn) * SS] = t;
           g_deg[(wn) * SS] = left;
         }
       }
+      if (n_ready + cnt >= rcap) { err = true; break; }
+      if (cnt) push_many(cnt, nm, nk, nrk);
     }
   }
   if (done != n) err = true;
