@@ -117,12 +117,14 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
     if (key == SIG_INVALID) break;
   }
   cid[i] = c;
-  // arrival index within the class: one atomic per distinct class of the wavefront, not per plan
+  // arrival index within the class.  The plans of the (up to four) first classes met in a wavefront share
+  // one atomic per class: batches of few classes would otherwise serialise on a handful of counters.  The
+  // rest (many classes, few plans each) add themselves one by one.
   const uint32_t key = c == CID_UNKNOWN ? n_classes : c;
   const int lane = (int)(threadIdx.x & (WAVE - 1));
   bool pending = true;
   uint32_t k = 0;
-  for (int guard = 0; guard < WAVE; ++guard) {
+  for (int round = 0; round < 4; ++round) {
     const unsigned long long am = __ballot(pending);
     if (!am) break;
     const int leader = __ffsll(am) - 1;
@@ -136,6 +138,7 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
       pending = false;
     }
   }
+  if (pending) k = atomicAdd(&count[key], 1u);
   kidx[i] = k;
 }
 
@@ -591,8 +594,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     // classes with the largest graphs (within a tenth of the largest) get eight plans per wavefront, so
     // that fewer plans wait for the slowest one, unless they are a large share of the batch or the batch
     // is many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest).
-    static const char* hl = getenv("RPEG_HEAVY_LPW");   // development override
-    const uint32_t heavy_lpw = hl ? (uint32_t)atoi(hl) : 8u;
+    const uint32_t heavy_lpw = 8u;
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t heavy_plans = 0;
     for (size_t c = 0; c < counts.size(); ++c)

@@ -15,6 +15,8 @@
 #ifndef RPEG_KERNEL_EVAL_H
 #define RPEG_KERNEL_EVAL_H
 
+#include <type_traits>
+
 #include "rpeg_plan.h"
 
 namespace rpeg {
@@ -313,11 +315,13 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   // Up to four pushes at once, with the result of pushing them one after the other: a stable merge in
   // which a new entry goes behind the waiting entries and the earlier new entries that are not after it.
   // The list is read and written once, from the top down (entries only move up).
-  auto push_many = [&](int cnt, const uint32_t (&nm)[4], const double (&nk)[4], const double (&nr)[4]) {
-    unsigned npt[4];
-    int c[4] = {0, 0, 0, 0};   // waiting entries not after new entry q
+  // NQ: the largest number of new entries of any plan of the wavefront (compile-time loop bound)
+  auto push_many = [&](auto nq_tag, int cnt, const uint32_t (&nm)[4], const double (&nk)[4], const double (&nr)[4]) {
+    constexpr int NQ = decltype(nq_tag)::value;
+    unsigned npt[NQ];
+    int c[NQ];                 // waiting entries not after new entry q
 #pragma unroll
-    for (int q = 0; q < 4; ++q) npt[q] = (nm[q] >> 12) & 15u;
+    for (int q = 0; q < NQ; ++q) { npt[q] = (nm[q] >> 12) & 15u; c[q] = 0; }
     for (int j1 = (n_ready + 7) & ~7; j1 > 0; j1 -= 8) {
       const int j0 = j1 - 8;
       double k[8], r[8];
@@ -334,7 +338,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         const unsigned pu = (m[u] >> 12) & 15u;
         int up = 0;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < NQ; ++q) {
           const bool after = pu > npt[q] || (pu == npt[q] && r[u] < nr[q]);   // the waiting entry is after new entry q
           up += (q < cnt && after) ? 1 : 0;
           c[q] += after ? 0 : 1;
@@ -347,11 +351,11 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
       }
     }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < NQ; ++q) {
       if (q >= cnt) break;
       int idx = c[q];
 #pragma unroll
-      for (int o = 0; o < 4; ++o) {
+      for (int o = 0; o < NQ; ++o) {
         if (o == q || o >= cnt) continue;
         const bool o_after = npt[o] > npt[q] || (npt[o] == npt[q] && nr[o] < nr[q]);     // o strictly after q
         const bool o_before = npt[o] < npt[q] || (npt[o] == npt[q] && nr[o] > nr[q]);    // o strictly before q
@@ -511,7 +515,14 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         }
       }
       if (n_ready + cnt >= rcap) { err = true; break; }
-      if (cnt) push_many(cnt, nm, nk, nrk);
+      // the widest push of the wavefront selects the code: most dispatches release one or two successors
+      if (__ballot(cnt > 2)) {
+        if (cnt) push_many(std::integral_constant<int, 4>{}, cnt, nm, nk, nrk);
+      } else if (__ballot(cnt > 1)) {
+        if (cnt) push_many(std::integral_constant<int, 2>{}, cnt, nm, nk, nrk);
+      } else if (cnt) {
+        push_many(std::integral_constant<int, 1>{}, cnt, nm, nk, nrk);
+      }
     }
   }
   if (done != n) err = true;

@@ -218,3 +218,39 @@ def test_drop_in_calls():
     bad = Configuration(cfgs[0][0].rpeg, cfgs[0][0].plan, p.device_space, intra_stage_fusion=True)
     with pytest.raises(NotImplementedError):
         evaluate(bad, p.suite, wl0, p.hw, p.K_eval)
+
+
+@pytest.mark.parametrize("c,n", [(1, 2048), (2, 8192), (5, 1024)])
+def test_every_state_layout_gives_the_same_bits(c, n):
+    """Scheduler state in the HBM workspace (64 plans per wavefront) or in LDS (8/16/32/64 plans per
+    wavefront), and the per-batch automatic choice: identical outputs."""
+    from rpeg_amd.engine.runtime import Engine, EngineError
+    cfg, batch = seeded_batch(c, n)
+    eng = Engine(cfg.problem)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    seen = set()
+    for lanes in (0, 8, 16, 32, 64, -1):
+        eng.set_state_lanes(lanes)
+        try:
+            out = eng.eval(batch, gate_stale=True)
+        except EngineError as ex:
+            assert lanes > 0 and "does not fit in LDS" in str(ex)   # the largest class is too big for that many plans
+            continue
+        seen.add(eng.stats()["state_lanes"])
+        assert np.array_equal(out["mask"], ref["mask"]), lanes
+        assert same_bits(out["makespan"], ref["makespan"]) and same_bits(out["score"], ref["score"]), lanes
+        assert same_bits(out["peak"], ref["peak"]), lanes
+    assert 0 in seen and 8 in seen
+    with pytest.raises(EngineError):
+        eng.set_state_lanes(12)
+
+
+def test_small_batches_pick_the_latency_layout():
+    cfg, batch = seeded_batch(2, 512)
+    eng = engine(2)
+    eng.set_state_lanes(-1)
+    eng.eval(batch)
+    assert eng.stats()["state_lanes"] > 0
+    cfg, batch = seeded_batch(2, 65536)
+    eng.eval(batch)
+    assert eng.stats()["state_lanes"] == 0
