@@ -591,19 +591,20 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0), clpw(counts.size(), lpw);
   if (!ls && !order.empty()) {
     // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
-    // classes with the largest graphs (within a tenth of the largest) get eight plans per wavefront, so
+    // classes with the largest graphs (at least seven tenths of the largest) get eight plans per wavefront, so
     // that fewer plans wait for the slowest one, unless they are a large share of the batch or the batch
     // is many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest).
     const uint32_t heavy_lpw = 8u;
+    const uint64_t hfrac = 7ull;   // tenths of the largest node count
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t heavy_plans = 0;
     for (size_t c = 0; c < counts.size(); ++c)
-      if (10ull * e->cls_nodes[cids[c]] >= 9ull * top) heavy_plans += counts[c];
+      if (10ull * e->cls_nodes[cids[c]] >= hfrac * top) heavy_plans += counts[c];
     uint64_t waves64 = 0;
     for (uint32_t c : counts) waves64 += (c + WAVE - 1) / WAVE;
     if (heavy_plans * 4 <= n && waves64 <= (uint64_t)e->n_cu * 16 && heavy_lpw >= 1 && heavy_lpw <= WAVE)
       for (size_t c = 0; c < counts.size(); ++c)
-        if (10ull * e->cls_nodes[cids[c]] >= 9ull * top) clpw[c] = heavy_lpw;
+        if (10ull * e->cls_nodes[cids[c]] >= hfrac * top) clpw[c] = heavy_lpw;
   }
   for (size_t k = 0; k < order.size(); ++k) {
     first[order[k]] = start[k];

@@ -55,8 +55,8 @@ __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
 // in-degree per node, duration per slot) lives in LDS too, interleaved by lane.
 __host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls) {
   const size_t rw = ls ? ls : KE_WAVE;
-  // ready list (key, rank, meta) with eight entries of slack for the batched list shifts
-  size_t ready = (size_t)(rcap + 8) * rw * 20;
+  // ready list: key (8 bytes) and meta (4 bytes) per entry
+  size_t ready = (size_t)rcap * rw * 12;
   size_t plan = (size_t)RPEG_MAX_V * RPEG_FIELDS * rw * 2 + (size_t)RPEG_MAX_V * 4 * rw * 8;
   return ((ready > plan ? ready : plan) + 15) & ~size_t(15);
 }
@@ -137,9 +137,8 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   uint8_t* dyn = lds + L.cls_bytes;
   int16_t* l_plan = (int16_t*)dyn + lane;                             // [60][64], aliased with the ready list
   double* l_vm = (double*)(dyn + (size_t)RPEG_MAX_V * RPEG_FIELDS * RW * 2) + lane;  // [24][RW], aliased too
-  double* r_key = (double*)dyn + lane;                                // [rcap+8][RW]
-  double* r_rank = (double*)dyn + (size_t)(L.rcap + 8) * RW + lane;   // [rcap+8][RW]
-  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)(L.rcap + 8) * RW * 16) + lane;  // [rcap+8][RW] node | prio << 12 | x << 16 | y << 19
+  double* r_key = (double*)dyn + lane;                                       // [rcap][RW]
+  uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * RW * 8) + lane;        // [rcap][RW] meta, see below
 
   __syncthreads();  // the previous task of this wavefront is done with LDS
   for (int i = lane; i < n; i += KE_WAVE) l_node[i] = ((const uint64_t*)cv.node)[i];
@@ -242,26 +241,28 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   // be stale: a popped entry whose true est (device availability included) exceeds its key is pushed
   // back with the true est and a fresh tie.  Here the ready list is kept sorted by the part of the key
   // that never changes while an entry waits: (comm_prio*8+topo_idx ascending, rank descending, push
-  // order); a new entry goes behind every entry that is not after it.
+  // order).  A new entry goes behind every entry that is not after it; an entry pushed back (fresh tie)
+  // moves behind the entries that agree with it in (prio, rank).  The heap's pop is then the FIRST entry
+  // of minimum key: one load, one compare and three selects per entry.
   //
-  // While no two waiting entries agree in (prio, rank), a fresh tie cannot change the order, and the
-  // next node the heap dispatches is simply the first entry of minimum TRUE est; the entries the heap
-  // would have popped and pushed back on the way are those whose (key, position) precedes the winner's
-  // (true est, position): their keys are raised to their true est.  Every plan of the wavefront then
-  // dispatches one node per iteration, in lock step.  A plan whose list holds two entries of equal
-  // (prio, rank) takes the heap's own steps instead (pop by key; push back behind its equals, or
-  // dispatch) until the pair is gone.
+  // An entry is its key (8 bytes) and a meta word: node | prio << 12 | x << 16 | y << 19 | same << 22,
+  // x and y the (one or two) vertices whose devices the node reserves, `same` set when the entry agrees
+  // in (prio, rank) with the entry before it.  Ranks stay in the per-plan state and are read only when
+  // entries are inserted.
+  //
+  // Each outer iteration first takes the heap's pops up to the next dispatch (a short inner loop: pop,
+  // and if the key is stale push back), then dispatches one node for all plans of the wavefront together.
   double lf[RPEG_MAX_V];
 #pragma unroll
   for (int x = 0; x < RPEG_MAX_V; ++x) lf[x] = 0.0;
   int n_ready = 0, done = 0;
-  const int rcap = (int)L.rcap;
+  const int rcap = (int)L.rcap;   // a multiple of eight
   const double inf = __builtin_inf();
-  for (int j = 0; j < rcap + 8; ++j) {   // entries past n_ready never win a scan
+  constexpr uint32_t SAME = 1u << 22;
+  for (int j = 0; j < rcap; ++j) {   // entries past n_ready never win a scan
     r_key[j * RW] = inf;
     r_nt[j * RW] = 0;
   }
-  // meta: node | prio << 12 | x << 16 | y << 19, with x, y the (one or two) vertices whose devices the node reserves
   auto make_meta = [&](int v, const NodeRec& r) -> uint32_t {
     const unsigned blk = blocked_mask(r, dpne);
     const unsigned x = (unsigned)__builtin_ctz(blk | 0x100u);
@@ -270,58 +271,18 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     if (rest & (rest - 1u)) err = true;   // more than two reserved vertices cannot be packed
     return (uint32_t)v | ((uint32_t)r.ptkey << 12) | (x << 16) | (y << 19);
   };
-  auto push = [&](uint32_t meta, double key, double rank) {
-    const unsigned pt = (meta >> 12) & 15u;
-    int pos = 0;
-    for (int j0 = 0; j0 < n_ready; j0 += 8) {
-      double r[8];
-      uint32_t m[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        r[u] = r_rank[(j0 + u) * RW];
-        m[u] = r_nt[(j0 + u) * RW];
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const unsigned pu = (m[u] >> 12) & 15u;
-        const bool after = pu > pt || (pu == pt && r[u] < rank);
-        pos += (j0 + u < n_ready && !after) ? 1 : 0;
-      }
-    }
-    for (int j1 = n_ready; j1 > pos; j1 -= 8) {   // entries [pos, n_ready) move one up, eight per round trip
-      double k[8], r[8];
-      uint32_t m[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int src = j1 - 1 - u < 0 ? 0 : j1 - 1 - u;
-        k[u] = r_key[src * RW];
-        r[u] = r_rank[src * RW];
-        m[u] = r_nt[src * RW];
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int src = j1 - 1 - u;
-        if (src < pos) continue;
-        r_key[(src + 1) * RW] = k[u];
-        r_rank[(src + 1) * RW] = r[u];
-        r_nt[(src + 1) * RW] = m[u];
-      }
-    }
-    r_key[pos * RW] = key;
-    r_rank[pos * RW] = rank;
-    r_nt[pos * RW] = meta;
-    ++n_ready;
-  };
-  // Up to four pushes at once, with the result of pushing them one after the other: a stable merge in
+  // Up to NQ pushes at once, with the result of pushing them one after the other: a stable merge in
   // which a new entry goes behind the waiting entries and the earlier new entries that are not after it.
-  // The list is read and written once, from the top down (entries only move up).
-  // NQ: the largest number of new entries of any plan of the wavefront (compile-time loop bound)
+  // The list is read and written once, from the top down (entries only move up).  NQ bounds the number
+  // of new entries of any plan of the wavefront.  A waiting entry keeps its `same` flag: no new entry
+  // can land between two entries that agree.
   auto push_many = [&](auto nq_tag, int cnt, const uint32_t (&nm)[4], const double (&nk)[4], const double (&nr)[4]) {
     constexpr int NQ = decltype(nq_tag)::value;
     unsigned npt[NQ];
     int c[NQ];                 // waiting entries not after new entry q
+    bool eq[NQ];               // a waiting entry agrees with new entry q in (prio, rank)
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) { npt[q] = (nm[q] >> 12) & 15u; c[q] = 0; }
+    for (int q = 0; q < NQ; ++q) { npt[q] = (nm[q] >> 12) & 15u; c[q] = 0; eq[q] = false; }
     for (int j1 = (n_ready + 7) & ~7; j1 > 0; j1 -= 8) {
       const int j0 = j1 - 8;
       double k[8], r[8];
@@ -329,9 +290,10 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         k[u] = r_key[(j0 + u) * RW];
-        r[u] = r_rank[(j0 + u) * RW];
         m[u] = r_nt[(j0 + u) * RW];
       }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) r[u] = g_rank[((int)(m[u] & 0xFFFu)) * SS];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         if (j0 + u >= n_ready) continue;
@@ -342,10 +304,10 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
           const bool after = pu > npt[q] || (pu == npt[q] && r[u] < nr[q]);   // the waiting entry is after new entry q
           up += (q < cnt && after) ? 1 : 0;
           c[q] += after ? 0 : 1;
+          eq[q] = eq[q] || (pu == npt[q] && r[u] == nr[q]);
         }
         if (up) {
           r_key[(j0 + u + up) * RW] = k[u];
-          r_rank[(j0 + u + up) * RW] = r[u];
           r_nt[(j0 + u + up) * RW] = m[u];
         }
       }
@@ -354,23 +316,26 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     for (int q = 0; q < NQ; ++q) {
       if (q >= cnt) break;
       int idx = c[q];
+      bool same = eq[q];
 #pragma unroll
       for (int o = 0; o < NQ; ++o) {
         if (o == q || o >= cnt) continue;
         const bool o_after = npt[o] > npt[q] || (npt[o] == npt[q] && nr[o] < nr[q]);     // o strictly after q
         const bool o_before = npt[o] < npt[q] || (npt[o] == npt[q] && nr[o] > nr[q]);    // o strictly before q
         idx += (o < q ? !o_after : o_before) ? 1 : 0;
+        same = same || (o < q && npt[o] == npt[q] && nr[o] == nr[q]);
       }
       r_key[idx * RW] = nk[q];
-      r_rank[idx * RW] = nr[q];
-      r_nt[idx * RW] = nm[q];
+      r_nt[idx * RW] = nm[q] | (same ? SAME : 0u);
     }
     n_ready += cnt;
   };
   for (unsigned i = 0; i < cv.h->n_init && !err; ++i) {
     const int v = cv.init[i];
     if (n_ready >= rcap - 1) { err = true; break; }
-    push(make_meta(v, cv.node[v]), 0.0, g_rank[(v) * SS]);
+    const uint32_t nm[4] = {make_meta(v, cv.node[v]), 0u, 0u, 0u};
+    const double nk[4] = {0.0, 0.0, 0.0, 0.0}, nrk[4] = {g_rank[(v) * SS], 0.0, 0.0, 0.0};
+    push_many(std::integral_constant<int, 1>{}, 1, nm, nk, nrk);
   }
   double makespan = 0.0;
   const long guard_max = (long)n * n + 64;
@@ -378,9 +343,6 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   for (long guard = 0; !err && done < n && guard < guard_max; ++guard) {
     ++guard_total;
     if (n_ready == 0) { err = true; break; }
-    // The heap's pops up to the next dispatch: first entry of minimum key; while that key is stale, raise
-    // it to the true est and move the entry behind its equals (scheduler.py:437-443).  This inner loop is
-    // short; the dispatch below then runs once per node for all plans of the wavefront together.
     int bj = 0;
     double est = 0.0;
     for (long inner = 0; inner < guard_max; ++inner) {
@@ -401,23 +363,27 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         if (c < bk) { bk = c; bj = j0 + (e0 ? x1 : x0); }
       }
       const uint32_t m0 = r_nt[bj * RW];
-      const double my_rank = r_rank[bj * RW];
-      const uint32_t m1 = r_nt[(bj + 1) * RW];
-      const double r1 = r_rank[(bj + 1) * RW];
+      const uint32_t m1 = r_nt[(bj + 1 < rcap ? bj + 1 : bj) * RW];
       const double dv = ke_dev_max((1u << ((m0 >> 16) & 7u)) | (1u << ((m0 >> 19) & 7u)), lf);
       est = dv > bk ? dv : bk;
       if (!(est > bk)) break;
       ++guard_total;
-      r_key[bj * RW] = est;
-      if (bj + 1 < n_ready && ((m1 ^ m0) & 0xF000u) == 0 && r1 == my_rank) {
-        while (bj + 1 < n_ready) {
-          const uint32_t m2 = r_nt[(bj + 1) * RW];
-          const double r2 = r_rank[(bj + 1) * RW];
-          if (((m2 ^ m0) & 0xF000u) != 0 || r2 != my_rank) break;
+      r_key[bj * RW] = est;   // scheduler.py:437-443
+      if (bj + 1 < n_ready && (m1 & SAME)) {
+        // behind its equals: the next entry takes this place (and this entry's relation to the entry before)
+        uint32_t mine = m0;
+        uint32_t nxt = m1;
+        while (true) {
           const double k2 = r_key[(bj + 1) * RW];
-          r_key[bj * RW] = k2; r_rank[bj * RW] = r2; r_nt[bj * RW] = m2;
+          r_key[bj * RW] = k2;
+          r_nt[bj * RW] = (nxt & ~SAME) | (mine & SAME);
           ++bj;
-          r_key[bj * RW] = est; r_rank[bj * RW] = my_rank; r_nt[bj * RW] = m0;
+          mine |= SAME;
+          r_key[bj * RW] = est;
+          r_nt[bj * RW] = mine;
+          if (bj + 1 >= n_ready) break;
+          nxt = r_nt[(bj + 1) * RW];
+          if (!(nxt & SAME)) break;
         }
       }
     }
@@ -445,19 +411,20 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     // remove the entry, keeping the order
     --n_ready;
     for (int j0 = bj; j0 < n_ready; j0 += 8) {    // entries (bj, n_ready] move one down, eight per round trip
-      double k[8], r[8];
+      double k[8];
       uint32_t m[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        k[u] = r_key[(j0 + 1 + u) * RW];
-        r[u] = r_rank[(j0 + 1 + u) * RW];
-        m[u] = r_nt[(j0 + 1 + u) * RW];
+        const int src = j0 + 1 + u < rcap ? j0 + 1 + u : rcap - 1;
+        k[u] = r_key[src * RW];
+        m[u] = r_nt[src * RW];
       }
+      // the entry that follows the removed one agrees with its new neighbour only if both did
+      if (j0 == bj) m[0] &= ~SAME | (bm & SAME);
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         if (j0 + u >= n_ready) continue;
         r_key[(j0 + u) * RW] = k[u];
-        r_rank[(j0 + u) * RW] = r[u];
         r_nt[(j0 + u) * RW] = m[u];
       }
     }
