@@ -24,7 +24,7 @@ FP64_PEAK_TFLOPS = 78.6     # MI355X vector FP64, published
 ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
 # HBM bytes per launch of k_eval measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB
 # copy (profiles/k_eval_cfg2_grpo_65536.md); None where no counter run exists
-MEASURED_TRAFFIC = {2: 706.5e6}
+MEASURED_TRAFFIC = {2: 718.6e6}
 # algorithmic fp64 operations per plan (cost model + scheduler + memory model of the fully split DAG)
 ALG_FLOPS = {1: 3.7e3, 2: 2.5e3, 3: 6.0e3, 4: 0.83e3, 5: 3.7e3}
 
