@@ -178,9 +178,11 @@ int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t 
    plan's RPEG_MAX_V*RPEG_FIELDS int16 values (stride 1), head4 its 4 header bytes.  node_kind:
    0 operator, 1 COMM, 2 RESHARD; node_vertex: the operator's vertex, or a transfer's destination
    vertex; node_src: a transfer's source vertex; node_sub: quantile phase or -1; edges: (src,dst)
-   node index pairs.  Returns the node count, or a negative status. */
+   node index pairs; dispatch_index (may be NULL): position of the node in the scheduler's dispatch order,
+   the insertion order of the reference's Trace.start (scheduler.py:517-518).  Returns the node count, or
+   a negative status. */
 int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4,
-                    double* start, double* finish, int32_t* node_kind, int32_t* node_vertex,
+                    double* start, double* finish, int32_t* dispatch_index, int32_t* node_kind, int32_t* node_vertex,
                     int32_t* node_step, int32_t* node_sub, int32_t* node_src, int32_t* edges,
                     int32_t* n_edges, int32_t cap);
 

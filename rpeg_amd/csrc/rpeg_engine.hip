@@ -52,6 +52,8 @@ struct DevMem {
   uint16_t* ready; // LDS, pre-offset by lane
   double* tr_start;
   double* tr_finish;
+  int32_t* tr_seq;   // dispatch index per node
+  int32_t seq;
   __device__ double& time(int i) { return t[(size_t)i * WAVE]; }
   __device__ double& rank(int i) { return r[(size_t)i * WAVE]; }
   __device__ uint8_t& indeg(int i) { return deg[(size_t)i * WAVE]; }
@@ -59,7 +61,7 @@ struct DevMem {
   __device__ void set_dur(int s, double v) { d[(size_t)s * WAVE] = v; }
   __device__ uint16_t& rd_node(int j) { return ready[j * WAVE]; }
   __device__ void on_schedule(int v, double s, double f) {
-    if (tr_start) { tr_start[v] = s; tr_finish[v] = f; }
+    if (tr_start) { tr_start[v] = s; tr_finish[v] = f; tr_seq[v] = seq++; }
   }
 };
 
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
                                                const uint32_t* __restrict__ wave_cls, const uint8_t* __restrict__ pool,
                                                uint8_t* __restrict__ ws, uint32_t ws_nodes, uint32_t ws_slots,
                                                uint32_t flags, double* makespan, double* peak, double* score,
-                                               uint8_t* mask, double* tr_start, double* tr_finish) {
+                                               uint8_t* mask, double* tr_start, double* tr_finish, int32_t* tr_seq) {
   extern __shared__ uint16_t lds_ready[];
   const int lane = threadIdx.x;
   const uint64_t n_waves = (n_sorted + WAVE - 1) / WAVE;
@@ -181,6 +183,8 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
   mem.ready = lds_ready + lane;
   mem.tr_start = tr_start;
   mem.tr_finish = tr_finish;
+  mem.tr_seq = tr_seq;
+  mem.seq = 0;
   for (uint64_t w = blockIdx.x; w < n_waves; w += gridDim.x) {
     // every wavefront works on one class: the class tables are addressed uniformly (scalar loads)
     const ClassView cv = class_view(pool + wave_cls[w]);
@@ -704,7 +708,7 @@ int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t 
 }
 
 int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* start, double* finish,
-                    int32_t* node_kind, int32_t* node_vertex, int32_t* node_step, int32_t* node_sub, int32_t* node_src,
+                    int32_t* dispatch_index, int32_t* node_kind, int32_t* node_vertex, int32_t* node_step, int32_t* node_sub, int32_t* node_src,
                     int32_t* edges, int32_t* n_edges, int32_t cap) {
   if (!e || !vert_fields || !head4 || !start || !finish) return -1;
   e->err.clear();
@@ -730,7 +734,7 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   double* d_tr = nullptr;
   HIP_TRY(e, hipMalloc(&d_vert, RPEG_MAX_V * RPEG_FIELDS * 2));
   HIP_TRY(e, hipMalloc(&d_head, 4));
-  HIP_TRY(e, hipMalloc(&d_tr, (size_t)n * 16));
+  HIP_TRY(e, hipMalloc(&d_tr, (size_t)n * 20));
   HIP_TRY(e, hipMemcpy(d_vert, vert_fields, RPEG_MAX_V * RPEG_FIELDS * 2, hipMemcpyHostToDevice));
   HIP_TRY(e, hipMemcpy(d_head, head4, 4, hipMemcpyHostToDevice));
   uint32_t lanes[WAVE];
@@ -740,10 +744,12 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   HIP_TRY(e, hipMemcpy(e->d_cls, &o32, 4, hipMemcpyHostToDevice));
   hipLaunchKernelGGL(k_eval_generic, dim3(1), dim3(WAVE), (size_t)READY_CAP * WAVE * 2, s, e->dP, (uint64_t)WAVE, d_vert, d_head,
                      (uint64_t)1, e->d_perm, e->d_cls, e->d_pool, e->d_ws, e->max_nodes, e->max_slots, 0u,
-                     (double*)nullptr, (double*)nullptr, (double*)nullptr, (uint8_t*)nullptr, d_tr, d_tr + n);
+                     (double*)nullptr, (double*)nullptr, (double*)nullptr, (uint8_t*)nullptr, d_tr, d_tr + n,
+                     (int32_t*)(d_tr + 2 * (size_t)n));
   HIP_TRY(e, hipGetLastError());
   HIP_TRY(e, hipMemcpy(start, d_tr, (size_t)n * 8, hipMemcpyDeviceToHost));
   HIP_TRY(e, hipMemcpy(finish, d_tr + n, (size_t)n * 8, hipMemcpyDeviceToHost));
+  if (dispatch_index) HIP_TRY(e, hipMemcpy(dispatch_index, d_tr + 2 * (size_t)n, (size_t)n * 4, hipMemcpyDeviceToHost));
   hipFree(d_vert); hipFree(d_head); hipFree(d_tr);
   for (int i = 0; i < n; ++i) {
     if (node_kind) node_kind[i] = lc.nodes[i].kind;

@@ -223,9 +223,10 @@ def _trace_of(eng, st, config: Configuration, batch: PlanBatch):
                 name = f"reshard{n_reshard}"
             nodes.append(ExecNode(id=name, kind="comm" if kind == 1 else "reshard",
                                   allocs=(config.plan.sigma[verts[src]], config.plan.sigma[v])))
-    # dispatch order = order of start times is not recoverable from ties; keep the node order
-    start = {n: float(s) for n, s in zip(nodes, tr["start"])}
-    finish = {n: float(f) for n, f in zip(nodes, tr["finish"])}
+    # Trace.start / Trace.finish are filled in dispatch order (scheduler.py:517-518)
+    by_dispatch = sorted(range(len(nodes)), key=lambda i: int(tr["order"][i]))
+    start = {nodes[i]: float(tr["start"][i]) for i in by_dispatch}
+    finish = {nodes[i]: float(tr["finish"][i]) for i in by_dispatch}
     edges = tuple(ExecEdge(nodes[a], nodes[b]) for a, b in tr["edges"])
     return Trace(start=start, finish=finish), ExecutableRPEG(nodes=tuple(nodes), edges=edges)
 

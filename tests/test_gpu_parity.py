@@ -254,3 +254,28 @@ def test_small_batches_pick_the_latency_layout():
     cfg, batch = seeded_batch(2, 65536)
     eng.eval(batch)
     assert eng.stats()["state_lanes"] == 0
+
+
+@pytest.mark.parametrize("c", [1, 2, 4])
+def test_execution_schedule_artifact_equals_reference(c):
+    """evaluate()'s trace is filled in dispatch order, so the schedule section of a plan artifact
+    (ir/serialize.py:244-274) lists the nodes as the reference does, with the same times."""
+    import json, os, zlib
+    from rpeg_amd.ir import serialize as ser
+    from rpeg_amd.search.evaluate import Configuration, evaluate
+    from tests.helpers import GOLDEN
+    with open(os.path.join(GOLDEN, "ref_plans.json")) as f:
+        recs = json.load(f)[str(c)]
+    cfg, batch = seeded_batch(c, 3)
+    p = cfg.problem
+    for rec in recs:
+        rpeg, plan, wl = batch.configuration(p, rec["i"])
+        config = Configuration(rpeg, plan, p.device_space)
+        score, trace, lowered = evaluate(config, p.suite, wl, p.hw, p.K_eval, p.memory_policy)
+        got = ser.execution_schedule_to_dict(trace, horizon=p.K_eval)
+        want = rec["schedule"]
+        assert got["policy"] == want["policy"] and got["horizon"] == want["horizon"]
+        assert got["predicted_makespan_s"].hex() == want["makespan"] and len(got["nodes"]) == want["n"]
+        assert zlib.crc32(",".join(n["node_id"] for n in got["nodes"]).encode()) == want["order_crc"]
+        assert [[n["node_id"], n["dispatch_index"], n["predicted_start_s"].hex(), n["predicted_finish_s"].hex()]
+                for n in got["nodes"][:6]] == want["head"]
