@@ -582,3 +582,62 @@ def run_chains(rpeg_of_chain, plan_type, alloc_type, space, suite, workload, eva
                     continue
                 _enter(ch, nxt, step, p.T_warm, p)
     return chains
+
+
+# ----------------------------------------------------------------------------- polish
+def polish(rpeg, plan, space, suite, workload, evaluate, table, index, T_min, T_init, max_rounds=50):
+    """optimizer.py:949-1188 without fusion, AC-share penalty and utilisation weighting: greedy
+    coordinate descent.  Vertices in id order; for each, every strategy of the directory window
+    [j*-w, j*+w] (w = max(5, int(n*T_min/T_init))) placed at origin (0,0,0) is evaluated (as
+    `_eval_worker` scores it, memory-infeasible candidates dropped) and the best strict
+    improvement is taken; passes repeat until one brings no improvement.
+
+    `evaluate(plan)` returns an Evaluated.  Returns (plan, score, rounds, distinct plans evaluated)."""
+    Alloc = type(next(iter(plan.sigma.values())))
+    seen = {}                                             # the evaluation cache: every plan is scored once
+
+    def key(q):
+        return tuple((tuple(q.pi[v]), q.mb[v], tuple(q.sigma[v].origin), tuple(q.sigma[v].extent)) for v in rpeg.vertices)
+
+    def cached(q):
+        k = key(q)
+        if k not in seen:
+            seen[k] = evaluate(q)
+        return seen[k]
+    cur = cached(plan)
+    score = cur.gated                                     # evaluate_cached (optimizer.py:1044)
+    rounds = 0
+    w_frac = T_min / T_init
+    order = sorted(rpeg.vertices, key=lambda v: v.id)
+    for round_idx in range(max_rounds):
+        rounds = round_idx + 1
+        improved = False
+        for v in order:
+            best_s, best_plan = score, None
+            tab = table[v]
+            n = len(tab)
+            w = max(5, int(n * w_frac))
+            dp, pp, tp = plan.pi[v]
+            r_ext, n_ext, _ = plan.sigma[v].extent
+            j_star = index[v].get((dp, pp, tp, r_ext, n_ext, plan.mb[v]), n // 2)
+            cands = []
+            for j in range(max(0, j_star - w), min(n - 1, j_star + w) + 1):
+                if j == j_star:
+                    continue
+                d2, p2, t2, re2, ne2, mb2 = tab[j][:6]
+                g_ext = O.packing_geometry(d2, p2, t2, space.G)[0]
+                cands.append(_new_plan(plan, {v: (Alloc((0, 0, 0), (re2, ne2, g_ext)), (d2, p2, t2), mb2)}))
+            # cache hits are merged before fresh results (optimizer.py:1151-1166): equal scores resolve that way
+            hits = [c for c in cands if key(c) in seen]
+            fresh = [c for c in cands if key(c) not in seen]
+            for cand in hits + fresh:
+                ev = cached(cand)
+                if not ev.mem_ok:
+                    continue
+                if ev.score > best_s:
+                    best_s, best_plan = ev.score, cand
+            if best_plan is not None:
+                plan, score, improved = best_plan, best_s, True
+        if not improved:
+            break
+    return plan, score, rounds, len(seen)

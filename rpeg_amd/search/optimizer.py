@@ -17,7 +17,7 @@ from typing import Dict, FrozenSet, List, Optional, Sequence, Set, Tuple
 
 import numpy as np
 
-from ..core.types import Allocation, Model
+from ..core.types import Allocation, Model, packing_geometry
 from ..engine import abi
 from ..engine.problem import EvalProblem, FIELDS_PER_VERTEX
 from ..ir.plan import ExecutionPlan
@@ -26,7 +26,8 @@ from ..model.memory import MemoryPolicy
 from ..model.models import ModelSuite
 from ..model.workload import Workload
 from .cache import EvalCache
-from .evaluate import Configuration, _check_supported, _engine_for, _structure_of
+from .evaluate import (Configuration, _check_supported, _engine_for, _structure_of, evaluate_batch, evaluate_cached,
+                       evaluation_cache_key)
 from .moves import build_candidate_directory, directory_arrays
 
 DEFAULT_T_CAND: Dict[Model, Set[int]] = {Model.ACTOR: {0, 1}, Model.CRITIC: {0, 1}, Model.AC_SHARE: {0, 1}}
@@ -202,3 +203,73 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
     rpeg = st.build(suite, workload, tau=tau)
     return Configuration(rpeg, row_plan(rpeg, res.best_plan[c]), base_config.device_space,
                          intra_stage_fusion=False, transfer_resource_policy=base_config.transfer_resource_policy)
+
+
+def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
+           opt_config: OptimizerConfig, cache: EvalCache, table, index, ac_share: bool = False,
+           max_rounds: int = 50) -> Configuration:
+    """Drop-in for polish() (RPEG/search/optimizer.py:949-1188): deterministic greedy coordinate descent on
+    the plan returned by optimize().  Vertices in id order; for each, every strategy of the directory window
+    around the current one, placed at origin (0,0,0), is scored in ONE batched launch (the reference maps
+    `_eval_worker` over them, optimizer.py:1138-1148); the best strict improvement among the memory-feasible
+    ones is applied; passes repeat until one brings no improvement.  Cache hits are merged before fresh
+    results, as in the reference, so equal scores resolve the same way."""
+    _check_supported(best_config)
+    if opt_config.max_throughput_loss > 0.0:
+        raise NotImplementedError("the utilisation-weighted objective needs per-candidate traces")
+    policy = opt_config.memory_policy()
+    config, rpeg = best_config, best_config.rpeg
+    G = config.device_space.G
+
+    def _score(raw: float) -> float:
+        return raw * (1.0 - opt_config.lambda_ac) if ac_share and opt_config.lambda_ac != 0.0 else raw
+
+    vertices = sorted(rpeg.vertices, key=lambda v: v.id)
+    w_frac = opt_config.T_min / opt_config.T_init
+    raw, _trace, _feasible, _miss = evaluate_cached(config, cache, suite, workload, hw, K_eval, policy)
+    score = _score(raw)
+    for _round in range(max_rounds):
+        improved = False
+        for v in vertices:
+            best_score, best = score, None
+            v_table = table[v]
+            n = len(v_table)
+            w = max(5, int(n * w_frac))
+            dp_c, pp_c, tp_c = config.plan.pi[v]
+            r_ext_c, n_ext_c, _g = config.plan.sigma[v].extent
+            j_star = index[v].get((dp_c, pp_c, tp_c, r_ext_c, n_ext_c, config.plan.mb[v]), n // 2)
+            cands = []
+            for j in range(max(0, j_star - w), min(n - 1, j_star + w) + 1):
+                if j == j_star:
+                    continue
+                dp, pp, tp, r_ext, n_ext, mb = v_table[j][:6]
+                geom = packing_geometry(dp, pp, tp, G)
+                if geom is None:
+                    continue
+                plan = ExecutionPlan(sigma={**config.plan.sigma, v: Allocation(origin=(0, 0, 0), extent=(r_ext, n_ext, geom[0]))},
+                                     pi={**config.plan.pi, v: (dp, pp, tp)}, mb={**config.plan.mb, v: mb})
+                cands.append(Configuration(rpeg, plan, config.device_space, intra_stage_fusion=False,
+                                           transfer_resource_policy=config.transfer_resource_policy))
+            hits, misses = [], []
+            for nb in cands:
+                h = evaluation_cache_key(nb, policy)
+                if h in cache:
+                    s, t, f = cache.get(h)
+                    hits.append((nb, s, f))
+                else:
+                    misses.append((nb, h))
+            fresh = []
+            if misses:
+                res = evaluate_batch([nb for nb, _ in misses], suite, workload, hw, K_eval, policy, gate_stale=False)
+                for (nb, h), s, m in zip(misses, res.score, res.mask):
+                    f = bool(m & abi.MASK_MEM_OK)
+                    cache.put(h, float(s), None, f)
+                    fresh.append((nb, float(s), f))
+            for nb, s, f in hits + fresh:
+                if f and _score(s) > best_score:
+                    best_score, best = _score(s), nb
+            if best is not None:
+                config, score, improved = best, best_score, True
+        if not improved:
+            break
+    return config

@@ -111,3 +111,34 @@ def test_base_plan_start_and_gate():
     assert (res.best_score >= out["score"][ok[0]]).all()
     c = res.argbest()
     assert res.best_score[c] == res.best_score.max()
+
+
+def test_polish_equals_reference():
+    """The drop-in polish() on the GPU evaluator against what the reference's own polish() returned for the
+    same start plans (tests/golden/make_golden_polish.py): same final plan, same score."""
+    from rpeg_amd.ir.plan import ExecutionPlan
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration, evaluate_cached
+    from rpeg_amd.search.optimizer import plan_row, polish
+    with open(os.path.join(GOLDEN, "ref_polish.json")) as f:
+        g = json.load(f)
+    cfg, batch = seeded_batch(1, 64)
+    p = cfg.problem
+    rpeg0 = p.template(0, ())
+    table, index = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, engine(1))
+    opt = OptimizerConfig(K_x=1, T_init=g["T_init"], T_min=g["T_min"])
+    nv = len(rpeg0.vertices)
+    for case in g["cases"]:
+        _, plan_m, _ = batch.configuration(p, case["i"])
+        by_id = {v.id: v for v in rpeg0.vertices}
+        plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
+                             pi={by_id[v.id]: x for v, x in plan_m.pi.items()},
+                             mb={by_id[v.id]: x for v, x in plan_m.mb.items()})
+        start = Configuration(rpeg0, plan, p.device_space)
+        cache = EvalCache()
+        out = polish(start, p.suite, p.workload, p.hw, p.K_eval, opt, cache, table, index)
+        rows = plan_row(rpeg0, out.plan)
+        assert [[int(x) for x in rows[v * 10:(v + 1) * 10]] for v in range(nv)] == case["plan"], case["i"]
+        score, _, feasible, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+        assert float(score).hex() == case["final_score"] and feasible == case["final_feasible"]
+        assert cache.misses - 1 == case["evaluations"]

@@ -134,3 +134,32 @@ def test_counter_rng_choices_is_cpython_bisect():
         r = S.CounterRng(1)
         r.random = lambda u=u: u
         assert r.choices(pop, weights=w, k=1) == Fixed(u).choices(pop, weights=w, k=1)
+
+
+def test_polish_and_optimizer_config_match_reference():
+    """The reference's own polish() (run unmodified by tests/golden/make_golden_polish.py) and the derived
+    fields of its OptimizerConfig."""
+    from rpeg_amd.search.optimizer import OptimizerConfig
+    with open(os.path.join(GOLDEN, "ref_polish.json")) as f:
+        g = json.load(f)
+    oc = g["optimizer_config"]
+    for name, cfg in (("default", OptimizerConfig()),
+                      ("cfg5", OptimizerConfig(K_x=6, T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
+                      ("e800", OptimizerConfig(E_struct=800, K_x=4))):
+        assert [cfg.I_max, cfg.T_cool.hex()] == oc[name]
+    cfg, batch, rpeg0, cost, mem = _world(1, 64)
+    p = cfg.problem
+    table, index = S.build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, cost, mem)
+    ev = S.oracle_evaluator(rpeg0, p.device_space, p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+    for case in g["cases"]:
+        _, plan_m, _ = batch.configuration(p, case["i"])
+        by_id = {v.id: v for v in rpeg0.vertices}
+        plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
+                             pi={by_id[v.id]: x for v, x in plan_m.pi.items()},
+                             mb={by_id[v.id]: x for v, x in plan_m.mb.items()})
+        assert ev(plan).gated.hex() == case["start_score"]
+        out, score, rounds, n_eval = S.polish(rpeg0, plan, p.device_space, p.suite, p.workload, ev, table, index,
+                                              g["T_min"], g["T_init"])
+        assert _rows(rpeg0, out) == case["plan"], case["i"]
+        assert score.hex() == case["final_score"], case["i"]
+        assert n_eval - 1 == case["evaluations"], case["i"]
