@@ -18,7 +18,10 @@ reference calls on Python's `random` module (`random`, `choice`, `choices`, `ran
 reference draws from MT19937; here the generator is counter based (`CounterRng`), so a chain's
 trajectory is a pure function of (seed, chain, step).  The proposal functions are pinned against
 the reference by handing the reference's own functions the same generator object
-(tests/golden/make_golden_sa.py): same draws in the same order give the same proposals.
+(tests/golden/make_golden_sa.py): same draws in the same order give the same proposals.  The
+chain loop is pinned the same way: `serial_chain` reproduces, evaluation by evaluation, what the
+reference's own optimize() does on that generator (tests/golden/make_golden_optimize.py), and
+`polish` what its polish() returns (tests/golden/make_golden_polish.py).
 
 Differences from the reference, all deliberate:
 
@@ -494,6 +497,25 @@ def _enter(ch, ev, step, T, p):
     ch.T, ch.rej = T, 0
 
 
+def propose(rng, rpeg, cur, space, suite, workload, table, index, p, T):
+    """Kernel selection and proposals of one iteration (optimizer.py:726-765).  Returns (kind, plans);
+    plans is None when the donor/receiver kernel failed to sample."""
+    frac = min(1.0, T / p.T_init)
+    if rng.random() < p.alpha_pair * frac:
+        nb = multi_move_pair(rng, rpeg, cur.plan, space, suite, workload)
+        return "pair", (None if nb is None else [nb])
+    return "single", move_gen(rng, rpeg, cur.plan, space, cur.mass, table, index, p.K_x, p.T_max, T, p.T_init)
+
+
+def mh_accept(rng, best_s, score_curr, T):
+    """One Metropolis-Hastings test (optimizer.py:881-895): None below the noise threshold (no draw)."""
+    delta = (best_s - score_curr) / (abs(score_curr) + 1e-12)
+    if abs(delta) < 1e-6:
+        return None
+    prob = 1.0 if delta >= 0.0 else math.exp(delta / T)
+    return rng.random() < prob
+
+
 def run_chains(rpeg_of_chain, plan_type, alloc_type, space, suite, workload, evaluate_of_chain, tables,
                n_chains, n_steps, params, base_plan=None, first_chain=0):
     """`n_chains` independent chains of `n_steps` Metropolis-Hastings steps each.
@@ -531,19 +553,11 @@ def run_chains(rpeg_of_chain, plan_type, alloc_type, space, suite, workload, eva
             rpeg, evaluate = rpeg_of_chain(ch.id), evaluate_of_chain(ch.id)
             rng = CounterRng(p.seed, ch.id, step + 1, 0)
             restart = False
-            frac = min(1.0, ch.T / p.T_init)
-            if rng.random() < p.alpha_pair * frac:
-                kind = "pair"
-                nb = multi_move_pair(rng, rpeg, ch.cur.plan, space, suite, workload)
-                if nb is None:
-                    ch.T = max(p.T_min, ch.T * p.T_cool)            # optimizer.py:737-740
-                    ch.log.append((step, "pair", 0, None))
-                    continue
-                cands = [nb]
-            else:
-                kind = "single"
-                cands = move_gen(rng, rpeg, ch.cur.plan, space, ch.cur.mass, table, index, p.K_x, p.T_max,
-                                 ch.T, p.T_init)
+            kind, cands = propose(rng, rpeg, ch.cur, space, suite, workload, table, index, p, ch.T)
+            if cands is None:
+                ch.T = max(p.T_min, ch.T * p.T_cool)                # optimizer.py:737-740
+                ch.log.append((step, "pair", 0, None))
+                continue
             accepted = None
             if not cands:
                 restart = True                                       # "chain stuck" (optimizer.py:767-769)
@@ -557,14 +571,11 @@ def run_chains(rpeg_of_chain, plan_type, alloc_type, space, suite, workload, eva
                     _note(ch, ev, s, step, p, feas)
                     if s > best_s:
                         best_ev, best_s = ev, s
-                delta = (best_s - ch.score) / (abs(ch.score) + 1e-12)
-                if abs(delta) >= 1e-6:
-                    prob = 1.0 if delta >= 0.0 else math.exp(delta / ch.T)
-                    accepted = rng.random() < prob
-                    if accepted:
-                        ch.cur, ch.score, ch.rej = best_ev, best_s, 0
-                    else:
-                        ch.rej += 1
+                accepted = mh_accept(rng, best_s, ch.score, ch.T)
+                if accepted:
+                    ch.cur, ch.score, ch.rej = best_ev, best_s, 0
+                elif accepted is not None:
+                    ch.rej += 1
                 if p.geometric_cooling:
                     ch.T = max(p.T_min, ch.T * p.T_cool)
                 if p.stag_window > 0 and ch.rej >= p.stag_window:
@@ -582,6 +593,117 @@ def run_chains(rpeg_of_chain, plan_type, alloc_type, space, suite, workload, eva
                     continue
                 _enter(ch, nxt, step, p.T_warm, p)
     return chains
+
+
+def serial_chain(rng, rpeg, base_plan, space, suite, workload, evaluate, tables, params, E_max, E_struct,
+                 R_max=10000):
+    """optimize() (optimizer.py:365-946) for ONE structural setting, as the reference runs it: one chain
+    at a time on one continuous random stream, an evaluation cache (hits cost no budget and are merged
+    before fresh results), the budgets E_max / E_struct counted in cache misses, restarts from the best
+    elite plan.  It shares `propose`, `mh_accept`, `elite_insert` and the bookkeeping with `run_chains`;
+    it exists so that those can be pinned against the reference's own optimize() driven by the same
+    generator (tests/golden/make_golden_optimize.py).  The base plan must be valid and the elite plans
+    stay valid (no random restart is restated).
+
+    Returns (best feasible plan or best plan, evaluation log): the log lists every plan handed to the
+    evaluator (cache misses only), in order."""
+    p = params
+    table, index = tables
+    cache, order = {}, []
+
+    def key(q):
+        return tuple((tuple(q.pi[v]), q.mb[v], tuple(q.sigma[v].origin), tuple(q.sigma[v].extent)) for v in rpeg.vertices)
+
+    def cached(q, gated):
+        """(Evaluated, miss).  The cache stores what the first evaluation stored: evaluate_cached stores the
+        gated score, the merge of fresh candidates the score of _eval_worker (optimizer.py:838, evaluate.py:372-374)."""
+        k = key(q)
+        if k in cache:
+            return cache[k], False
+        ev = evaluate(q)
+        order.append(q)
+        stored = (ev.gated if gated else ev.score, ev.mem_ok and (ev.stale_ok or not gated), ev)
+        cache[k] = stored
+        return stored, True
+
+    ch = Chain(0)
+    (s0, f0, ev0), _ = cached(base_plan, True)
+    ch.best, ch.best_score = ev0, s0
+    if f0:
+        ch.best_feasible, ch.best_feasible_score = ev0, s0
+        elite_insert(s0, ev0, ev0.plan, ch.elite, ch.seen, p.K_elite)
+    E, E_s = 1, 0
+    cur = ev0
+    r, no_progress, exhausted = 0, 0, False
+    while r < R_max and not exhausted:
+        restart_E_s = E_s
+        if r > 0:
+            cur = ch.elite[0][1] if ch.elite else cur          # warm restart (optimizer.py:640-660)
+            no_progress = 0
+        (score_curr, feasible, cur), miss = cached(cur.plan, True)
+        if miss:
+            E += 1; E_s += 1
+        if feasible:
+            elite_insert(score_curr, cur, cur.plan, ch.elite, ch.seen, p.K_elite)
+        if score_curr > ch.best_score * (1.0 + p.score_eps):
+            ch.best, ch.best_score = cur, score_curr
+        if feasible and score_curr > ch.best_feasible_score:
+            ch.best_feasible, ch.best_feasible_score = cur, score_curr
+        T = p.T_warm if r > 0 else p.T_init
+        rej = 0
+        while True:
+            if E >= E_max:
+                return (ch.best_feasible or ch.best).plan, order
+            if E_s >= E_struct:
+                exhausted = True
+                break
+            kind, cands = propose(rng, rpeg, cur, space, suite, workload, table, index, p, T)
+            if cands is None:
+                T = max(p.T_min, T * p.T_cool)
+                continue
+            if not cands:
+                break
+            hits, fresh = [], []
+            for plan in cands:                                  # optimizer.py:781-789
+                k = key(plan)
+                (hits if k in cache else fresh).append(plan)
+            best_ev, best_s = None, -math.inf
+            for plan in hits + fresh:                           # optimizer.py:807-861
+                (s, f, ev), miss = cached(plan, False)
+                if miss:
+                    E += 1; E_s += 1
+                if f:
+                    elite_insert(s, ev, ev.plan, ch.elite, ch.seen, p.K_elite)
+                if s > ch.best_score * (1.0 + p.score_eps):
+                    ch.best, ch.best_score = ev, s
+                if f and s > ch.best_feasible_score:
+                    ch.best_feasible, ch.best_feasible_score = ev, s
+                if s > best_s:
+                    best_ev, best_s = ev, s
+            if E >= E_max:
+                return (ch.best_feasible or ch.best).plan, order
+            if E_s >= E_struct:
+                exhausted = True
+            if not exhausted:
+                accepted = mh_accept(rng, best_s, score_curr, T)
+                if accepted:
+                    cur, score_curr, rej = best_ev, best_s, 0
+                elif accepted is not None:
+                    rej += 1
+            if p.geometric_cooling:
+                T = max(p.T_min, T * p.T_cool)
+            if exhausted:
+                break
+            if p.stag_window > 0 and rej >= p.stag_window:
+                break
+        r += 1
+        if E_s == restart_E_s:
+            no_progress += 1
+            if no_progress >= 2:
+                exhausted = True
+        else:
+            no_progress = 0
+    return (ch.best_feasible or ch.best).plan, order
 
 
 # ----------------------------------------------------------------------------- polish

@@ -1,0 +1,143 @@
+"""Writes tests/golden/ref_optimize.json: the trajectory of the REFERENCE's optimize()
+(RPEG/search/optimizer.py:365-946) for one structural setting of config 1, driven by the counter-based
+generator instead of MT19937.
+
+Run in the development container only (it needs the read-only reference tree):
+
+    python tests/golden/make_golden_optimize.py [--ref /root/reference]
+
+optimize() runs unmodified.  As in make_golden_polish.py, the names its module uses in annotations
+without importing them are made visible, and the functions it imports from the unparsable
+`search/evaluate.py` are written here on the reference's own passes (score arithmetic of evaluate.py:288
+and :396-401, stale-layout rule :115-140, validity rules :143-232, cache key :301-326).  The module
+attribute `random` of optimizer.py and of moves.py is pointed at ONE generator object, and
+`os.cpu_count` reports one core while optimize() runs so that it evaluates candidates in-process, in
+order.  The file records every plan handed to an evaluation function (cache misses only), in order, and
+the plan optimize() returns: the restatement must evaluate the same plans in the same order.
+"""
+
+from __future__ import annotations
+
+import argparse
+import builtins
+import json
+import math
+import os
+import sys
+import typing
+import zlib
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, HERE)
+
+import make_golden as MG      # noqa: E402
+import make_golden_sa as SA   # noqa: E402
+
+CASES = [dict(plan=0, stream=(42, 77, 0, 0), E_max=260, E_struct=200, stag_window=4, T_init=0.05, T_min=0.05, T_warm=0.10),
+         dict(plan=2, stream=(42, 77, 1, 0), E_max=150, E_struct=400, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05)]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--ref", default="/root/reference")
+    args = ap.parse_args()
+    mods, moves, Configuration, ct = SA.load_moves(args.ref)
+    import ir.rpeg
+    import schedule.trace
+    import search.cache as rcache
+    from oracle import rpeg_oracle as O
+    from oracle.sa_oracle import CounterRng
+    stub = sys.modules["search.evaluate"]
+    st = {}
+
+    def rows(config):
+        return SA.plan_rows(config.rpeg, config.plan)
+
+    def _eval(config, gate):
+        p = st["problem"]
+        rpeg, plan, wl = config.rpeg, config.plan, st["wl"]
+        st["log"].append(rows(config))
+        unrolled = mods["passes.unroll"].unroll(rpeg, p.K_eval)
+        lowered = mods["passes.lower"].lower(rpeg, unrolled, plan, st["suite"], p.K_eval, workload=wl)
+        trace = mods["schedule.scheduler"].schedule(lowered, st["cost"], st["space"])
+        raw = trace.throughput(W_step=wl.B * wl.K * (wl.S + wl.T), K=p.K_eval)
+        if gate and not O.stale_publication_layout_valid(rpeg, plan):
+            return 0.0, trace, False
+        violation = mods["model.memory"].mem_worst_violation(lowered, st["mm"])
+        if violation is None:
+            return raw, trace, True
+        _, req, cap = violation
+        return raw * max(math.exp(-40.0 * max(0.0, req / cap - 1.0)), 1e-12), trace, False
+
+    def evaluation_cache_key(config, memory_policy=None):
+        return rcache.config_hash(config.rpeg, config.plan) + ":mem:fusion=0:transfer=destination_only,destination_only:2:1:0:0:activation_cache=0:groups=0"
+
+    def evaluate_cached(config, cache, suite, workload, hw, K_eval, memory_policy=None):
+        h = evaluation_cache_key(config)
+        if h in cache:
+            s, t, f = cache.get(h)
+            return s, t, f, False
+        s, t, f = _eval(config, gate=True)
+        cache.put(h, s, t, f)
+        return s, t, f, True
+
+    def _eval_worker(a):
+        return _eval(a[0], gate=False)
+
+    def is_valid(config, suite, workload, mem_model):
+        rpeg, plan = config.rpeg, config.plan
+        if not O.plan_structurally_valid(rpeg, plan, config.device_space, suite, workload):
+            return False
+        if not O.stale_publication_layout_valid(rpeg, plan):
+            return False
+        unrolled = mods["passes.unroll"].unroll(rpeg, 1)
+        lowered = mods["passes.lower"].lower(rpeg, unrolled, plan, suite, 1, workload=workload)
+        return mods["model.memory"].mem_feasible(lowered, mem_model)
+
+    stub.evaluation_cache_key, stub.evaluate_cached = evaluation_cache_key, evaluate_cached
+    stub._eval_worker, stub.is_valid = _eval_worker, is_valid
+    builtins.TemplateVertex, builtins.List, builtins.Trace = ir.rpeg.TemplateVertex, typing.List, schedule.trace.Trace
+    import search.optimizer as ropt
+
+    from rpeg_amd import configs
+    from rpeg_amd.search import candidates
+    cfg = configs.config(1)
+    p = cfg.problem
+    rpeg0, suite, wl, hw, space, cost, mm = SA.ref_world(mods, p, {"Pi": 0, "V": 0})
+    st.update(problem=p, suite=suite, wl=wl, space=space, cost=cost, mm=mm, log=[])
+    batch = candidates.generate(p, 8, cfg.tau_choices, seed=42, tag=1)
+    Model = ct.Model
+    doc = {"cases": []}
+    real_cpu_count = os.cpu_count
+    for case in CASES:
+        plan = SA.ref_plan(mods, rpeg0, batch, p, case["plan"])
+        base = Configuration(rpeg0, plan, space)
+        assert is_valid(base, suite, wl, mm), "the base plan must be valid"
+        oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
+                                  T_cand={Model.ACTOR: {0}, Model.CRITIC: {0}, Model.AC_SHARE: set()},
+                                  structural_candidates=frozenset({"separate"}), T_init=case["T_init"],
+                                  T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"])
+        rng = CounterRng(*case["stream"])
+        ropt.random = rng
+        moves.random = rng
+        st["log"] = []
+        os.cpu_count = lambda: 1
+        try:
+            out = ropt.optimize(base, suite, wl, hw, p.K_eval, oc, rcache.EvalCache())
+        finally:
+            os.cpu_count = real_cpu_count
+        log = st["log"]
+        doc["cases"].append(dict(case, stream=list(case["stream"]), T_cool=oc.T_cool.hex(), n_eval=len(log),
+                                 n_draws=rng.k, eval_crc=zlib.crc32(json.dumps(log, separators=(",", ":")).encode()),
+                                 first=log[:8], final=rows(out)))
+        print("case", case["plan"], "evaluations", len(log), "draws", rng.k)
+    path = os.path.join(HERE, "ref_optimize.json")
+    with open(path, "w") as f:
+        json.dump(doc, f, separators=(",", ":"))
+    print(path, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()

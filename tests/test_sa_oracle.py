@@ -163,3 +163,34 @@ def test_polish_and_optimizer_config_match_reference():
         assert _rows(rpeg0, out) == case["plan"], case["i"]
         assert score.hex() == case["final_score"], case["i"]
         assert n_eval - 1 == case["evaluations"], case["i"]
+
+
+def test_chain_loop_matches_reference_optimize():
+    """The reference's own optimize() (run unmodified, for one structural setting, on the counter-based
+    generator by tests/golden/make_golden_optimize.py) against `serial_chain`, which is built from the
+    same `propose` / `mh_accept` / elite functions as the population loop `run_chains`: every plan is
+    evaluated in the same order, the same number of draws is consumed, the same plan is returned."""
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        g = json.load(f)
+    cfg, batch, rpeg0, cost, mem = _world(1, 8)
+    p = cfg.problem
+    table, index = S.build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, cost, mem)
+    ev = S.oracle_evaluator(rpeg0, p.device_space, p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+    for case in g["cases"]:
+        _, plan_m, _ = batch.configuration(p, case["plan"])
+        by_id = {v.id: v for v in rpeg0.vertices}
+        plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
+                             pi={by_id[v.id]: x for v, x in plan_m.pi.items()},
+                             mb={by_id[v.id]: x for v, x in plan_m.mb.items()})
+        params = S.SaParams(K_x=6, T_max=50, T_init=case["T_init"], T_warm=case["T_warm"], T_min=case["T_min"],
+                            stag_window=case["stag_window"], E_struct=case["E_struct"])
+        assert params.T_cool.hex() == case["T_cool"]
+        rng = S.CounterRng(*case["stream"])
+        best, order = S.serial_chain(rng, rpeg0, plan, p.device_space, p.suite, p.workload, ev, (table, index),
+                                     params, case["E_max"], case["E_struct"])
+        log = [_rows(rpeg0, q) for q in order]
+        assert log[:8] == case["first"]
+        assert len(log) == case["n_eval"]
+        assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
+        assert rng.k == case["n_draws"]
+        assert _rows(rpeg0, best) == case["final"]
