@@ -250,6 +250,13 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e);
 int rpeg_engine_set_timing(rpeg_engine_t* e, int32_t enabled);
 double rpeg_engine_last_kernel_ms(const rpeg_engine_t* e);
 
+/* Development aid: per-wavefront phase clocks of the evaluation kernel.  enable != 0 makes the following
+   rpeg_eval_batch calls record, per wavefront, seven stamps of the 100 MHz wall clock (start; after the
+   plan load; durations; memory model; ranks; scheduling; outputs) and in the eighth word the node count
+   << 32 | heap pops; with `out` non-NULL the stamps of the last call (8 words per wavefront, at most
+   cap_waves wavefronts) are copied to host memory and their number is returned. */
+int rpeg_engine_profile(rpeg_engine_t* e, int32_t enable, unsigned long long* out, uint64_t cap_waves);
+
 /* exp() as the host C library of an FMA-capable x86-64 computes it, evaluated on the device for n
    inputs; exported for the parity test of the OOM penalty. */
 int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream);

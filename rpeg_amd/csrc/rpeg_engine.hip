@@ -261,7 +261,7 @@ struct rpeg_engine_s {
   size_t cap_n = 0, cap_perm = 0;
   uint64_t* d_sig = nullptr;
   uint64_t* h_sig = nullptr;
-  uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_perm = nullptr, *h_cls = nullptr;
+  uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_cls = nullptr;   // lane -> plan; wavefront -> class blob
   uint8_t* d_ws = nullptr;
   size_t ws_cap = 0;
   // timing / stats
@@ -332,11 +332,10 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
 static int ensure_perm(rpeg_engine_t* e, size_t lanes) {
   if (lanes <= e->cap_perm) return 0;
   size_t cap = std::max<size_t>(lanes + lanes / 4, 8192);
-  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_cls); }
   e->cap_perm = 0;
   HIP_TRY(e, hipMalloc(&e->d_perm, cap * 4));
   HIP_TRY(e, hipMalloc(&e->d_cls, (cap / WAVE + 1) * 4));
-  HIP_TRY(e, hipHostMalloc(&e->h_perm, cap * 4));
   HIP_TRY(e, hipHostMalloc(&e->h_cls, (cap / WAVE + 1) * 4));
   e->cap_perm = cap;
   return 0;
@@ -446,7 +445,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
     hipFree(e->d_ccount); hipFree(e->d_cfirst); hipFree(e->d_clpw);
     hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
   }
-  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_perm); hipHostFree(e->h_cls); }
+  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_cls); }
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
   if (e->ev1) hipEventDestroy(e->ev1);

@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_engine_set_state_lanes")
+           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile")
 
 
 class EngineError(RuntimeError):
@@ -66,6 +66,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_set_state_lanes.argtypes = [vp, i32]
     lib.rpeg_engine_reset_classes.restype = C.c_int
     lib.rpeg_engine_reset_classes.argtypes = [vp]
+    lib.rpeg_engine_profile.restype = C.c_int
+    lib.rpeg_engine_profile.argtypes = [vp, i32, vp, u64]
     lib.rpeg_device_exp.restype = C.c_int
     lib.rpeg_device_exp.argtypes = [vp, u64, vp, vp, vp]
     if path is None:
