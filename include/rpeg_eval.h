@@ -228,6 +228,32 @@ typedef struct rpeg_sa_result_s {   /* per-chain arrays of n_chains elements, an
 int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* params, const int16_t* base_plan,
                 rpeg_sa_result_t* result, void* stream);
 
+/* optimize() as the reference runs it (RPEG/search/optimizer.py:365-946), for the structure of
+   `params`: the staleness variants one after the other, each a sequence of restarts of one chain on the
+   continuous random stream (params->seed, stream_a, stream_b, stream_c); evaluation cache (hits cost no
+   budget and are merged before fresh results, :775-861); budgets E_max / E_struct in cache misses; elites
+   shared by the variants; warm restarts (:640-663).  The K_x candidates of an iteration are one batched
+   evaluation (the reference maps _eval_worker over them, :793-798).  Variant 0 must be the staleness of
+   the base configuration.  n_chains, n_steps, restart_attempts and gate_candidates of `params` are not
+   used.  With the same generator the reference's optimize() evaluates the same plans in the same order
+   and returns the same plan. */
+typedef struct rpeg_sa_serial_result_s {
+  int16_t best_plan[RPEG_MAX_V * RPEG_FIELDS];  /* best feasible plan, else best plan (optimizer.py:946)  */
+  int32_t best_variant, best_feasible;
+  double best_score;
+  int64_t E;                 /* evaluations counted against the budget (cache misses)                   */
+  int64_t n_draws;           /* random words consumed                                                    */
+  int64_t n_uncounted;       /* evaluations made for is_valid only (no budget, no cache)                 */
+  int16_t* eval_log;         /* optional: every plan evaluated as a cache miss, in order, eval_log_cap   */
+  uint8_t* eval_log_variant; /*   rows of RPEG_MAX_V*RPEG_FIELDS values / their staleness variants       */
+  int64_t eval_log_cap, n_eval_log;
+  double wall_s;
+} rpeg_sa_serial_result_t;
+
+int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* params, int32_t E_max, int32_t E_struct,
+                     int32_t R_max, uint64_t stream_a, uint64_t stream_b, uint64_t stream_c,
+                     const int16_t* base_plan, rpeg_sa_serial_result_t* result, void* stream);
+
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,
    [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace). */

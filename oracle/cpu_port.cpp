@@ -241,6 +241,30 @@ int port_sa_run(void* h, const rpeg_sa_params_t* prm, const int16_t* base_plan, 
   return 0;
 }
 
+int port_sa_optimize(void* h, const rpeg_sa_params_t* prm, int32_t E_max, int32_t E_struct, int32_t R_max, uint64_t ka,
+                     uint64_t kb, uint64_t kc, const int16_t* base_plan, rpeg_sa_serial_result_t* res, int threads) {
+  Port* e = (Port*)h;
+  SaContext cx;
+  sa_context(e, prm, cx);
+  SaSettings st;
+  st.K_x = prm->K_x; st.T_max = prm->T_max; st.K_elite = prm->K_elite; st.stag_window = prm->stag_window;
+  st.geometric_cooling = prm->geometric_cooling; st.n_variants = prm->n_variants; st.T_init = prm->T_init;
+  st.T_warm = prm->T_warm; st.T_min = prm->T_min; st.T_cool = prm->T_cool; st.alpha_pair = prm->alpha_pair;
+  st.score_eps = prm->score_eps; st.seed = prm->seed;
+  CpuSaBackend be;
+  be.e = e; be.threads = threads;
+  for (int k = 0; k < prm->n_variants; ++k) {
+    be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
+    be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];
+  }
+  SaSerial run(cx, st, be, E_max, E_struct, R_max, prm->seed, ka, kb, kc);
+  SaPlan base;
+  std::memcpy(&base, base_plan, sizeof base);
+  if (int rc = run.run(base)) return rc;
+  sa_serial_result(run, res);
+  return 0;
+}
+
 // single proposals with the stream (seed, a, b, c): what = 0 move_gen, 1 pair, 2 region sample of vertex `v`
 // in racks [r_lo, r_hi).  Returns the number of plans (or rows) written; *draws = words consumed (in: words
 // to skip).

@@ -31,6 +31,9 @@ def lib():
             [C.c_void_p] * 6 + [C.c_int, C.c_void_p]
         _lib.port_sa_run.restype = C.c_int
         _lib.port_sa_run.argtypes = [C.c_void_p] * 4 + [C.c_int]
+        _lib.port_sa_optimize.restype = C.c_int
+        _lib.port_sa_optimize.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, C.c_uint64,
+                                          C.c_uint64, C.c_void_p, C.c_void_p, C.c_int]
         _lib.port_sa_propose.restype = C.c_int
         _lib.port_sa_propose.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_uint64,
                                          C.c_uint64, C.c_void_p, C.c_void_p, C.c_double, C.c_int, C.c_int, C.c_int,
@@ -125,6 +128,20 @@ class CpuPort:
         out["log"] = out["log"][:, :ns]
         out["wall_s"] = res.wall_s
         return out
+
+    def sa_optimize(self, params, directory, base_plan, E_max, E_struct, R_max=10000, stream_key=(0, 0, 0), log_cap=0,
+                    threads=1):
+        """The reference-style optimize of rpeg_amd/csrc/rpeg_sa.h (SaSerial) over this CPU evaluator."""
+        from rpeg_amd.engine.runtime import serial_dict, serial_result
+        keep = self._set_directory(params, directory)
+        res, log, logv = serial_result(log_cap)
+        base = np.ascontiguousarray(base_plan, dtype=np.int16).reshape(abi.MAX_V * abi.FIELDS)
+        rc = lib().port_sa_optimize(self.h, C.addressof(params), E_max, E_struct, R_max, *[int(x) for x in stream_key],
+                                    base.ctypes.data, C.addressof(res), threads)
+        if rc != 0:
+            raise RuntimeError(f"port_sa_optimize failed ({rc}): {lib().port_error(self.h).decode()}")
+        del keep
+        return serial_dict(res, log, logv)
 
     def sa_propose(self, params, directory, what, stream, plan=None, mass=None, T=0.0, v=0, r_lo=0, r_hi=0, skip=0):
         """One proposal with generator stream (seed, a, b, c): what = 0 move_gen, 1 donor/receiver pair,

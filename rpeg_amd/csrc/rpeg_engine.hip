@@ -900,6 +900,48 @@ int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* ba
   return 0;
 }
 
+int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t E_max, int32_t E_struct, int32_t R_max,
+                     uint64_t stream_a, uint64_t stream_b, uint64_t stream_c, const int16_t* base_plan,
+                     rpeg_sa_serial_result_t* res, void* stream) {
+  if (!e || !prm || !res || !base_plan) return -1;
+  e->err.clear();
+  if (prm->structure < 0 || prm->structure >= e->P.n_struct || prm->split < 0 || prm->split >= e->P.n_split ||
+      prm->n_variants < 1 || prm->n_variants > 8 || prm->K_x < 1 || prm->K_x > 16 || prm->T_max < 0 ||
+      !(prm->T_init > 0.0) || E_max < 1 || E_struct < 1 || R_max < 1) {
+    e->err = "bad annealing parameters";
+    return -1;
+  }
+  SaContext cx;
+  cx.init(e->P, prm->structure);
+  for (int v = 0; v < cx.nv; ++v) {
+    if (prm->dir_n[v] < 0 || (prm->dir_n[v] > 0 && !prm->dir[v])) { e->err = "bad candidate directory"; return -1; }
+    if (const char* msg = cx.set_directory(v, prm->dir[v], prm->dir_n[v])) { e->err = msg; return -1; }
+  }
+  SaSettings st;
+  st.K_x = prm->K_x; st.T_max = prm->T_max; st.K_elite = prm->K_elite; st.stag_window = prm->stag_window;
+  st.geometric_cooling = prm->geometric_cooling; st.n_variants = prm->n_variants; st.T_init = prm->T_init;
+  st.T_warm = prm->T_warm; st.T_min = prm->T_min; st.T_cool = prm->T_cool; st.alpha_pair = prm->alpha_pair;
+  st.score_eps = prm->score_eps; st.seed = prm->seed;
+  GpuSaBackend be(e, (hipStream_t)stream, std::max(prm->K_x, 16));
+  if (be.rc_alloc) return be.rc_alloc;
+  for (int k = 0; k < prm->n_variants; ++k) {
+    be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
+    be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];
+  }
+  SaSerial run(cx, st, be, E_max, E_struct, R_max, prm->seed, stream_a, stream_b, stream_c);
+  SaPlan base;
+  std::memcpy(&base, base_plan, sizeof base);
+  const auto t0 = std::chrono::steady_clock::now();
+  const bool was_timing = e->timing;
+  e->timing = false;
+  const int rc = run.run(base);
+  e->timing = was_timing;
+  if (rc) return rc;
+  sa_serial_result(run, res);
+  res->wall_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  return 0;
+}
+
 int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream) {
   if (!e || !x || !y) return -1;
   if (n == 0) return 0;

@@ -549,5 +549,237 @@ struct SaRun {
   }
 };
 
+// ------------------------------------------------------------------------------------- one chain at a time
+// optimize() as the reference runs it (optimizer.py:365-946): the staleness variants one after the other,
+// each a sequence of restarts of ONE chain on one continuous random stream; an evaluation cache (hits cost
+// no budget and are merged before fresh results); the budgets E_max / E_struct counted in cache misses;
+// elites shared by the variants; warm restarts from the best elite plan, random restarts otherwise.  The
+// K_x candidates of a step are one batched evaluation.
+struct SaSerial {
+  const SaContext& cx;
+  const SaSettings& p;
+  SaBackend& be;
+  int E_max, E_struct, R_max;
+  SaRng rng;
+
+  struct Stored { double score; bool feasible; SaEval ev; };
+  std::unordered_map<std::string, Stored> cache;
+  std::vector<SaPlan> eval_log;          // every plan handed to the evaluator as a cache miss, in order
+  std::vector<uint8_t> eval_log_variant;
+  std::vector<SaEntry> elite;
+  std::set<std::vector<int16_t>> seen;
+  SaEntry best, best_feasible;
+  int best_variant = 0, best_feasible_variant = 0;
+  bool has_feasible = false;
+  double best_score = 0.0, best_feasible_score = -INFINITY;
+  long E = 0, n_uncounted = 0;
+
+  SaSerial(const SaContext& c, const SaSettings& s, SaBackend& b, int e_max, int e_struct, int r_max, uint64_t seed,
+           uint64_t ka, uint64_t kb, uint64_t kc)
+      : cx(c), p(s), be(b), E_max(e_max), E_struct(e_struct), R_max(r_max), rng(seed, ka, kb, kc) {}
+
+  std::string key(const SaPlan& q, int variant) const {
+    std::string k((const char*)&q, sizeof q);
+    k.push_back((char)variant);
+    return k;
+  }
+  std::vector<int16_t> fingerprint(const SaPlan& q) const {
+    std::vector<int16_t> fp;
+    for (int v = 0; v < cx.nv; ++v)
+      for (int x : {SA_DP, SA_PP, SA_TP, SA_OR, SA_ON, SA_OG, SA_MB}) fp.push_back(q.f[v][x]);
+    return fp;
+  }
+  void elite_insert(double raw, const SaPlan& q, const SaEval& ev) {
+    auto fp = fingerprint(q);
+    if (seen.count(fp)) return;
+    if ((int)elite.size() >= p.K_elite && raw <= elite.back().ev.score) return;
+    SaEntry e; e.plan = q; e.ev = ev; e.ev.score = raw;
+    elite.push_back(e);
+    std::stable_sort(elite.begin(), elite.end(), [](const SaEntry& a, const SaEntry& b) { return a.ev.score > b.ev.score; });
+    if ((int)elite.size() > p.K_elite) elite.resize(p.K_elite);
+    seen.insert(fp);
+  }
+  static bool mask_valid(uint8_t m) {
+    return (m & RPEG_MASK_VALID) && (m & RPEG_MASK_STALE_OK) && (m & RPEG_MASK_MEM_OK) && !(m & RPEG_MASK_ERROR);
+  }
+  // is_valid (evaluate.py:143-232) costs no budget and does not touch the cache
+  int is_valid(const SaPlan& q, int variant, bool* ok) {
+    auto it = cache.find(key(q, variant));
+    if (it != cache.end()) { *ok = mask_valid(it->second.ev.mask); return 0; }
+    SaEval ev;
+    const uint8_t var = (uint8_t)variant;
+    if (int rc = be.evaluate(1, &q, &var, &ev)) return rc;
+    ++n_uncounted;
+    *ok = mask_valid(ev.mask);
+    return 0;
+  }
+  // evaluates the cache misses among `plans` in one batch; gated: evaluate_cached's score, else _eval_worker's
+  int evaluate(int n, const SaPlan* plans, int variant, bool gated, std::vector<Stored>& out, std::vector<char>& miss) {
+    out.resize(n);
+    miss.assign(n, 0);
+    std::vector<SaPlan> todo;
+    std::vector<int> idx;
+    for (int i = 0; i < n; ++i) {
+      auto it = cache.find(key(plans[i], variant));
+      if (it != cache.end()) { out[i] = it->second; continue; }
+      bool dup = false;   // the same plan twice among the misses is evaluated once
+      for (size_t j = 0; j < todo.size() && !dup; ++j) dup = std::memcmp(&todo[j], &plans[i], sizeof(SaPlan)) == 0;
+      if (!dup) { todo.push_back(plans[i]); idx.push_back(i); }
+      miss[i] = 1;
+    }
+    if (!todo.empty()) {
+      std::vector<uint8_t> var(todo.size(), (uint8_t)variant);
+      std::vector<SaEval> ev(todo.size());
+      if (int rc = be.evaluate((int)todo.size(), todo.data(), var.data(), ev.data())) return rc;
+      for (size_t j = 0; j < todo.size(); ++j) {
+        const bool stale_ok = (ev[j].mask & RPEG_MASK_STALE_OK) != 0, mem_ok = (ev[j].mask & RPEG_MASK_MEM_OK) != 0;
+        Stored st;
+        st.ev = ev[j];
+        st.score = gated && !stale_ok ? 0.0 : ev[j].score;
+        st.feasible = mem_ok && (stale_ok || !gated);
+        cache[key(todo[j], variant)] = st;
+        eval_log.push_back(todo[j]);
+        eval_log_variant.push_back((uint8_t)variant);
+      }
+      for (int i = 0; i < n; ++i)
+        if (miss[i]) out[i] = cache[key(plans[i], variant)];
+    }
+    return 0;
+  }
+  void note(const SaPlan& q, const Stored& s, int variant) {   // optimizer.py:676-686, 846-861
+    if (s.feasible) elite_insert(s.score, q, s.ev);
+    if (s.score > best_score * (1.0 + p.score_eps)) { best.plan = q; best.ev = s.ev; best_score = s.score; best_variant = variant; }
+    if (s.feasible && s.score > best_feasible_score) {
+      has_feasible = true; best_feasible.plan = q; best_feasible.ev = s.ev; best_feasible_score = s.score;
+      best_feasible_variant = variant;
+    }
+  }
+  // optimizer.py:259-289 on the continuous stream
+  int random_restart(int variant, SaPlan* out, bool* found) {
+    *found = false;
+    for (int a = 0; a < 50; ++a) {
+      SaPlan q;
+      if (!sa_sample_all(rng, cx, &q)) return 0;
+      bool ok = false;
+      if (int rc = is_valid(q, variant, &ok)) return rc;
+      if (ok) { *out = q; *found = true; return 0; }
+    }
+    return 0;
+  }
+
+  int run(const SaPlan& base) {
+    std::vector<Stored> st;
+    std::vector<char> miss;
+    if (int rc = evaluate(1, &base, 0, true, st, miss)) return rc;   // optimizer.py:466-478
+    best.plan = base; best.ev = st[0].ev; best_score = st[0].score; best_variant = 0;
+    if (st[0].feasible) {
+      has_feasible = true; best_feasible = best; best_feasible_score = st[0].score; best_feasible_variant = 0;
+      elite_insert(st[0].score, base, st[0].ev);
+    }
+    E = 1;
+    std::vector<SaPlan> cand(p.K_x);
+    for (int variant = 0; variant < p.n_variants; ++variant) {
+      SaPlan config = base;
+      bool ok = false;
+      if (int rc = is_valid(base, variant, &ok)) return rc;
+      if (!ok) {   // optimizer.py:596-616
+        bool found = false;
+        if (int rc = random_restart(variant, &config, &found)) return rc;
+        if (!found) config = base;
+      }
+      long E_s = 0;
+      int r = 0, no_progress = 0;
+      bool exhausted = false;
+      SaEval cur_ev{};
+      while (r < R_max && !exhausted) {
+        const long restart_E_s = E_s;
+        if (r > 0) {   // optimizer.py:640-663
+          bool restarted = false;
+          if (!elite.empty()) {
+            bool w_ok = false;
+            if (int rc = is_valid(elite[0].plan, variant, &w_ok)) return rc;
+            if (w_ok) { config = elite[0].plan; restarted = true; }
+          }
+          if (!restarted) {
+            bool found = false;
+            if (int rc = random_restart(variant, &config, &found)) return rc;
+            if (!found) {
+              ++r; ++no_progress;
+              if (no_progress >= 2) exhausted = true;
+              continue;
+            }
+          }
+          no_progress = 0;
+        }
+        if (int rc = evaluate(1, &config, variant, true, st, miss)) return rc;
+        double score_curr = st[0].score;
+        cur_ev = st[0].ev;
+        if (miss[0]) { ++E; ++E_s; }
+        note(config, st[0], variant);
+        double T = r > 0 ? p.T_warm : p.T_init;
+        int rej = 0;
+        while (true) {
+          if (E >= E_max) return 0;
+          if (E_s >= E_struct) { exhausted = true; break; }
+          const double frac = std::min(1.0, T / p.T_init);
+          int nc = 0;
+          if (rng.random() < p.alpha_pair * frac) {
+            if (!sa_move_pair(rng, cx, config, &cand[0])) { T = std::max(p.T_min, T * p.T_cool); continue; }
+            nc = 1;
+          } else {
+            nc = sa_move_gen(rng, cx, config, cur_ev.mass, p.K_x, p.T_max, T, p.T_init, cand.data());
+          }
+          if (nc == 0) break;   // "chain stuck"
+          if (int rc = evaluate(nc, cand.data(), variant, false, st, miss)) return rc;
+          int bi = -1;
+          double bs = -INFINITY;
+          for (int pass = 0; pass < 2; ++pass)        // cache hits first, then fresh results (optimizer.py:807-861)
+            for (int i = 0; i < nc; ++i) {
+              if ((miss[i] != 0) != (pass == 1)) continue;
+              if (miss[i]) { ++E; ++E_s; }
+              note(cand[i], st[i], variant);
+              if (st[i].score > bs) { bs = st[i].score; bi = i; }
+            }
+          if (E >= E_max) return 0;
+          if (E_s >= E_struct) exhausted = true;
+          if (bi >= 0 && !exhausted) {
+            const double delta = (bs - score_curr) / (std::fabs(score_curr) + 1e-12);
+            if (std::fabs(delta) >= 1e-6) {
+              const double prob = delta >= 0.0 ? 1.0 : exp_libm(delta / T);
+              if (rng.random() < prob) { config = cand[bi]; cur_ev = st[bi].ev; score_curr = bs; rej = 0; }
+              else ++rej;
+            }
+          }
+          if (p.geometric_cooling) T = std::max(p.T_min, T * p.T_cool);
+          if (exhausted) break;
+          if (p.stag_window > 0 && rej >= p.stag_window) break;
+        }
+        ++r;
+        if (E_s == restart_E_s) { if (++no_progress >= 2) exhausted = true; }
+        else no_progress = 0;
+      }
+    }
+    return 0;
+  }
+};
+
+inline void sa_serial_result(const SaSerial& run, rpeg_sa_serial_result_t* res) {
+  const bool feas = run.has_feasible;
+  const SaEntry& b = feas ? run.best_feasible : run.best;
+  std::memcpy(res->best_plan, &b.plan, sizeof(SaPlan));
+  res->best_variant = feas ? run.best_feasible_variant : run.best_variant;
+  res->best_score = feas ? run.best_feasible_score : run.best_score;
+  res->best_feasible = feas;
+  res->E = run.E;
+  res->n_draws = (int64_t)run.rng.k;
+  res->n_uncounted = run.n_uncounted;
+  res->n_eval_log = (int64_t)run.eval_log.size();
+  const int64_t keep = std::min<int64_t>(res->n_eval_log, res->eval_log_cap);
+  if (res->eval_log)
+    for (int64_t i = 0; i < keep; ++i) std::memcpy(res->eval_log + i * RPEG_MAX_V * RPEG_FIELDS, &run.eval_log[i], sizeof(SaPlan));
+  if (res->eval_log_variant)
+    for (int64_t i = 0; i < keep; ++i) res->eval_log_variant[i] = run.eval_log_variant[i];
+}
+
 }  // namespace rpeg
 #endif

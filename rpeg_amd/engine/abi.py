@@ -99,3 +99,10 @@ class SaResultT(C.Structure):
                 ("cur_score", C.c_void_p), ("restarts", C.c_void_p), ("n_eval", C.c_void_p), ("dead", C.c_void_p),
                 ("log", C.c_void_p), ("wall_s", C.c_double), ("eval_s", C.c_double),
                 ("n_launch", C.c_int64), ("n_plans", C.c_int64)]
+
+
+class SaSerialResultT(C.Structure):
+    _fields_ = [("best_plan", C.c_int16 * (MAX_V * FIELDS)), ("best_variant", C.c_int32), ("best_feasible", C.c_int32),
+                ("best_score", C.c_double), ("E", C.c_int64), ("n_draws", C.c_int64), ("n_uncounted", C.c_int64),
+                ("eval_log", C.c_void_p), ("eval_log_variant", C.c_void_p), ("eval_log_cap", C.c_int64),
+                ("n_eval_log", C.c_int64), ("wall_s", C.c_double)]

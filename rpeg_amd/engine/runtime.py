@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile")
+           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize")
 
 
 class EngineError(RuntimeError):
@@ -52,6 +52,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_eval_batch_mass.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp, vp]
     lib.rpeg_sa_run.restype = C.c_int
     lib.rpeg_sa_run.argtypes = [vp, vp, vp, vp, vp]
+    lib.rpeg_sa_optimize.restype = C.c_int
+    lib.rpeg_sa_optimize.argtypes = [vp, vp, i32, i32, i32, u64, u64, u64, vp, vp, vp]
     lib.rpeg_op_time_batch.restype = C.c_int
     lib.rpeg_op_time_batch.argtypes = [vp, u64, i32, i32, vp, u64, vp, vp, vp]
     lib.rpeg_eval_trace.restype = C.c_int
@@ -73,6 +75,37 @@ def load_library(path: Optional[str] = None):
     if path is None:
         _lib = lib
     return lib
+
+
+def set_directory(params: "abi.SaParamsT", directory):
+    """Points params.dir at per-vertex int16 arrays [n, 6]; returns the arrays (keep them alive)."""
+    keep = []
+    for v in range(abi.MAX_V):
+        if v < len(directory):
+            a = np.ascontiguousarray(directory[v], dtype=np.int16).reshape(-1, 6)
+            keep.append(a)
+            params.dir_n[v] = a.shape[0]
+            params.dir[v] = a.ctypes.data
+        else:
+            params.dir_n[v] = 0
+            params.dir[v] = None
+    return keep
+
+
+def serial_result(log_cap: int):
+    res = abi.SaSerialResultT()
+    log = np.zeros((max(log_cap, 1), abi.MAX_V * abi.FIELDS), np.int16)
+    logv = np.zeros(max(log_cap, 1), np.uint8)
+    res.eval_log, res.eval_log_variant, res.eval_log_cap = log.ctypes.data, logv.ctypes.data, log_cap
+    return res, log, logv
+
+
+def serial_dict(res, log, logv):
+    n = min(res.n_eval_log, res.eval_log_cap)
+    return dict(best_plan=np.array(res.best_plan, dtype=np.int16), best_variant=res.best_variant,
+                best_feasible=bool(res.best_feasible), best_score=res.best_score, E=res.E, n_draws=res.n_draws,
+                n_uncounted=res.n_uncounted, n_eval_log=res.n_eval_log, eval_log=log[:n].copy(),
+                eval_log_variant=logv[:n].copy(), wall_s=res.wall_s)
 
 
 def _torch():
@@ -219,6 +252,21 @@ class Engine:
         out["log"] = out["log"][:, :ns]
         out.update(wall_s=res.wall_s, eval_s=res.eval_s, n_launch=res.n_launch, n_plans=res.n_plans)
         return out
+
+    def sa_optimize(self, params: "abi.SaParamsT", directory, base_plan: np.ndarray, E_max: int, E_struct: int,
+                    R_max: int = 10000, stream_key=(0, 0, 0), log_cap: int = 0) -> Dict[str, object]:
+        """optimize() as the reference runs it (rpeg_sa_optimize): one chain at a time, cache and budgets."""
+        torch = _torch()
+        keep = set_directory(params, directory)
+        res, log, logv = serial_result(log_cap)
+        base = np.ascontiguousarray(base_plan, dtype=np.int16).reshape(abi.MAX_V * abi.FIELDS)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_sa_optimize(self._h, C.addressof(params), E_max, E_struct, R_max,
+                                           *[int(x) for x in stream_key], base.ctypes.data, C.addressof(res), stream)
+        self._check(rc, "rpeg_sa_optimize")
+        del keep
+        return serial_dict(res, log, logv)
 
     def op_time(self, structure: int, vertex: int, strat: np.ndarray):
         """time() and peak_bytes() of mock nodes: strat is int16 [7, n] = dp pp tp mb r_ext n_ext g_ext."""

@@ -182,26 +182,39 @@ def _iter_staleness(tau_models, t_cand) -> List[Tuple[int, ...]]:
 
 
 def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
-             opt_config: OptimizerConfig, cache: Optional[EvalCache] = None, n_chains: int = 64, seed: int = 42) -> Configuration:
+             opt_config: OptimizerConfig, cache: Optional[EvalCache] = None, seed: int = 42,
+             stream_key: Sequence[int] = (0, 0, 0)) -> Configuration:
     """Drop-in for optimize() (RPEG/search/optimizer.py:365-946) on the template of `base_config`.
 
-    The structural outer loop is replaced by running all staleness variants of T_cand side by side
-    (chain c uses variant c mod n); every chain runs the number of iterations the reference's
-    per-structure budget is calibrated for (2 * I_max = E_struct / ((K_x+1)/2), optimizer.py:121-125).
-    AC-share and intra-stage-fusion structures are not entered: the returned configuration keeps the
-    template of `base_config` with the staleness of the winning chain.  `cache` is accepted for
-    signature compatibility; results do not depend on it."""
+    Runs the reference's loop (rpeg_sa_optimize): the staleness variants of T_cand one after the other,
+    the base configuration's own staleness first; per variant a sequence of restarts of one chain, with
+    the evaluation cache, the budgets E_max / E_struct, the elites and the warm restarts of the reference.
+    The K_x candidates of an iteration are one GPU launch.  Given the same random generator the reference
+    evaluates the same plans in the same order and returns the same plan (tests/golden/make_golden_optimize.py);
+    the generator here is the counter-based stream (seed, *stream_key), not MT19937.
+
+    Not entered: the AC-share and intra-stage-fusion structures (`structural_candidates` other than
+    "separate"), deadlines, the utilisation objective.  `cache` is accepted for signature compatibility:
+    the run keeps its own cache (keyed by plan and staleness variant)."""
     _check_supported(base_config)
+    if opt_config.max_throughput_loss > 0.0 or opt_config.deadline is not None:
+        raise NotImplementedError("utilisation objective and deadlines are not part of this engine")
     policy = opt_config.memory_policy()
     eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy)
     t_cand = opt_config.T_cand if opt_config.T_cand is not None else DEFAULT_T_CAND
-    variants = _iter_staleness(st.tau_models, t_cand)
-    res = optimize_chains(eng.problem, opt_config, n_chains, max(1, 2 * opt_config.I_max), variants, seed,
-                          base_config.plan, eng)
-    c = res.argbest()
-    tau = {m: res.variants[c % len(variants)][i] for i, m in enumerate(st.tau_models)}
+    own = tuple(int(base_config.rpeg.tau.get(m, 0)) for m in st.tau_models)
+    variants = [own] + [v for v in _iter_staleness(st.tau_models, t_cand) if v != own]
+    if own not in _iter_staleness(st.tau_models, t_cand):
+        variants = variants[1:] or [own]
+    rpeg0 = eng.problem.template(0, ())
+    table, _ = build_candidate_directory(rpeg0, suite, base_config.device_space, workload, eng)
+    split = 1 if workload.gen_quantiles else 0
+    params = sa_params(opt_config, 1, 1, variants, 0, split, seed)
+    res = eng.sa_optimize(params, directory_arrays(rpeg0, table), plan_row(base_config.rpeg, base_config.plan),
+                          opt_config.E_max, opt_config.E_struct, opt_config.R_max, stream_key)
+    tau = {m: variants[res["best_variant"]][i] for i, m in enumerate(st.tau_models)}
     rpeg = st.build(suite, workload, tau=tau)
-    return Configuration(rpeg, row_plan(rpeg, res.best_plan[c]), base_config.device_space,
+    return Configuration(rpeg, row_plan(rpeg, res["best_plan"]), base_config.device_space,
                          intra_stage_fusion=False, transfer_resource_policy=base_config.transfer_resource_policy)
 
 

@@ -142,3 +142,47 @@ def test_polish_equals_reference():
         score, _, feasible, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
         assert float(score).hex() == case["final_score"] and feasible == case["final_feasible"]
         assert cache.misses - 1 == case["evaluations"]
+
+
+def test_optimize_equals_reference_trajectory():
+    """rpeg_sa_optimize on the GPU evaluator against the trajectory of the reference's own optimize() on the
+    same generator: same plans evaluated in the same order, same draws, same returned plan; and the
+    drop-in optimize() built on it."""
+    from rpeg_amd.ir.plan import ExecutionPlan
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration, evaluate_cached
+    from rpeg_amd.search.optimizer import optimize, plan_row
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        g = json.load(f)
+    cfg, batch = seeded_batch(1, 8)
+    p = cfg.problem
+    eng = engine(1)
+    rpeg0 = p.template(0, ())
+    nv = len(rpeg0.vertices)
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, eng)
+    arrays = directory_arrays(rpeg0, table)
+
+    def rows(r):
+        return [[int(x) for x in r[v * 10:(v + 1) * 10]] for v in range(nv)]
+    for case in g["cases"]:
+        _, plan_m, _ = batch.configuration(p, case["plan"])
+        by_id = {v.id: v for v in rpeg0.vertices}
+        plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
+                             pi={by_id[v.id]: x for v, x in plan_m.pi.items()},
+                             mb={by_id[v.id]: x for v, x in plan_m.mb.items()})
+        opt = OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"], T_init=case["T_init"],
+                              T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"],
+                              T_cand={m: {0} for m in rpeg0.tau})
+        res = eng.sa_optimize(sa_params(opt, 1, 1, [(0, 0)], 0, 1, case["stream"][0]), arrays, plan_row(rpeg0, plan),
+                              case["E_max"], case["E_struct"], stream_key=case["stream"][1:], log_cap=4096)
+        log = [rows(r) for r in res["eval_log"]]
+        assert log[:8] == case["first"] and res["n_eval_log"] == case["n_eval"]
+        assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
+        assert res["n_draws"] == case["n_draws"] and rows(res["best_plan"]) == case["final"]
+        base = Configuration(rpeg0, plan, p.device_space)
+        out = optimize(base, p.suite, p.workload, p.hw, p.K_eval, opt, EvalCache(), seed=case["stream"][0],
+                       stream_key=case["stream"][1:])
+        assert rows(plan_row(out.rpeg, out.plan)) == case["final"]
+        s1, _, f1, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+        s0, _, _, _ = evaluate_cached(base, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+        assert f1 and s1 >= s0

@@ -147,3 +147,36 @@ def test_chain_trajectories_match_restatement(c, n_chains, n_steps, kw):
         assert _rows6(got["best_plan"][cid], nv) == _rows6(plan_row(rpeg, best.plan), nv), cid
         assert got["best_score"][cid].hex() == float(ch.best_feasible_score if feas else ch.best_score).hex(), cid
         assert got["best_step"][cid] == (ch.best_feasible_step if feas else ch.best_step), cid
+
+
+def test_cxx_optimize_matches_reference_optimize():
+    """The shipped reference-style loop (SaSerial in rpeg_amd/csrc/rpeg_sa.h, here over the CPU evaluator)
+    against the trajectory of the reference's own optimize() on the same generator
+    (tests/golden/make_golden_optimize.py): same plans evaluated in the same order, same number of draws,
+    same returned plan."""
+    import zlib
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        g = json.load(f)
+    cfg, batch = seeded_batch(1, 8)
+    p = cfg.problem
+    rpeg0 = p.template(0, ())
+    nv = len(rpeg0.vertices)
+    _, _, arrays = _directory(p, rpeg0)
+    port = CpuPort(p)
+    for case in g["cases"]:
+        _, plan_m, _ = batch.configuration(p, case["plan"])
+        row = plan_row(rpeg0, ExecutionPlan(sigma={v: plan_m.sigma[u] for v, u in zip(rpeg0.vertices, plan_m.sigma)},
+                                            pi={v: plan_m.pi[u] for v, u in zip(rpeg0.vertices, plan_m.pi)},
+                                            mb={v: plan_m.mb[u] for v, u in zip(rpeg0.vertices, plan_m.mb)}))
+        opt = OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"], T_init=case["T_init"],
+                              T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"])
+        assert opt.T_cool.hex() == case["T_cool"]
+        params = sa_params(opt, 1, 1, [(0, 0)], 0, 1, case["stream"][0])
+        res = port.sa_optimize(params, arrays, row, case["E_max"], case["E_struct"], stream_key=case["stream"][1:],
+                               log_cap=4096, threads=4)
+        log = [_rows6(r, nv) for r in res["eval_log"]]
+        assert log[:8] == case["first"]
+        assert res["n_eval_log"] == case["n_eval"] == len(log)
+        assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
+        assert res["n_draws"] == case["n_draws"]
+        assert _rows6(res["best_plan"], nv) == case["final"]
