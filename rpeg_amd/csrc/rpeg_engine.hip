@@ -856,11 +856,7 @@ int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* ba
     if (const char* msg = cx.set_directory(v, prm->dir[v], prm->dir_n[v])) { e->err = msg; return -1; }
   }
   SaSettings st;
-  st.n_chains = prm->n_chains; st.n_steps = prm->n_steps; st.K_x = prm->K_x; st.T_max = prm->T_max;
-  st.K_elite = prm->K_elite; st.stag_window = prm->stag_window; st.restart_attempts = prm->restart_attempts;
-  st.gate_candidates = prm->gate_candidates; st.geometric_cooling = prm->geometric_cooling;
-  st.n_variants = prm->n_variants; st.T_init = prm->T_init; st.T_warm = prm->T_warm; st.T_min = prm->T_min;
-  st.T_cool = prm->T_cool; st.alpha_pair = prm->alpha_pair; st.score_eps = prm->score_eps; st.seed = prm->seed;
+  sa_settings_from(*prm, &st);
   const int cap = prm->n_chains * std::max(prm->K_x, prm->restart_attempts);
   GpuSaBackend be(e, (hipStream_t)stream, cap);
   if (be.rc_alloc) return be.rc_alloc;
@@ -876,24 +872,7 @@ int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* ba
   const int rc = run.run(base_plan ? &base : nullptr);
   e->timing = was_timing;
   if (rc) return rc;
-  const size_t V = RPEG_MAX_V * RPEG_FIELDS;
-  for (int c = 0; c < st.n_chains; ++c) {
-    const SaChain& ch = run.chains[c];
-    const bool feas = ch.has_feasible;
-    const SaEntry& b = feas ? ch.best_feasible : ch.best;
-    if (res->best_plan) std::memcpy(res->best_plan + c * V, &b.plan, V * 2);
-    if (res->best_score) res->best_score[c] = feas ? ch.best_feasible_score : (ch.has_best ? ch.best_score : __builtin_nan(""));
-    if (res->best_step) res->best_step[c] = feas ? ch.best_feasible_step : ch.best_step;
-    if (res->best_time) res->best_time[c] = feas ? ch.best_feasible_time : -1.0;
-    if (res->best_feasible) res->best_feasible[c] = feas;
-    if (res->cur_plan) std::memcpy(res->cur_plan + c * V, &ch.cur.plan, V * 2);
-    if (res->cur_score) res->cur_score[c] = ch.score;
-    if (res->restarts) res->restarts[c] = ch.restarts;
-    if (res->n_eval) res->n_eval[c] = ch.n_eval;
-    if (res->dead) res->dead[c] = ch.dead;
-  }
-  if (res->log) std::memcpy(res->log, run.log.data(), run.log.size());
-  res->wall_s = run.now();
+  sa_run_result(run, res);
   res->eval_s = be.eval_s;
   res->n_launch = be.n_launch;
   res->n_plans = be.n_plans;
@@ -918,10 +897,7 @@ int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t E_ma
     if (const char* msg = cx.set_directory(v, prm->dir[v], prm->dir_n[v])) { e->err = msg; return -1; }
   }
   SaSettings st;
-  st.K_x = prm->K_x; st.T_max = prm->T_max; st.K_elite = prm->K_elite; st.stag_window = prm->stag_window;
-  st.geometric_cooling = prm->geometric_cooling; st.n_variants = prm->n_variants; st.T_init = prm->T_init;
-  st.T_warm = prm->T_warm; st.T_min = prm->T_min; st.T_cool = prm->T_cool; st.alpha_pair = prm->alpha_pair;
-  st.score_eps = prm->score_eps; st.seed = prm->seed;
+  sa_settings_from(*prm, &st);
   GpuSaBackend be(e, (hipStream_t)stream, std::max(prm->K_x, 16));
   if (be.rc_alloc) return be.rc_alloc;
   for (int k = 0; k < prm->n_variants; ++k) {

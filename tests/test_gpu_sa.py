@@ -186,3 +186,24 @@ def test_optimize_equals_reference_trajectory():
         s1, _, f1, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
         s0, _, _, _ = evaluate_cached(base, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
         assert f1 and s1 >= s0
+
+
+def test_annealing_argument_errors_and_edges():
+    from rpeg_amd.engine.runtime import EngineError
+    p = configs.config(1).problem
+    eng = engine(1)
+    rpeg0 = p.template(0, ())
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, eng)
+    arrays = directory_arrays(rpeg0, table)
+    opt = OptimizerConfig(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)
+    res = optimize_chains(p, opt, 4, 0, [(0, 0)], engine=eng, directory=arrays)          # no steps: only the starts
+    assert res.log.shape == (4, 0) and not res.dead.any() and (res.best_step == -1).all()
+    for bad in (dict(K_x=17), dict(K_x=0)):
+        with pytest.raises(EngineError, match="bad annealing parameters"):
+            optimize_chains(p, OptimizerConfig(T_init=0.05, T_min=0.05, **bad), 2, 1, [(0, 0)], engine=eng, directory=arrays)
+    big = [np.full((3, 6), 2000, np.int16)] * 6
+    with pytest.raises(EngineError, match="outside 0..1023"):
+        optimize_chains(p, opt, 2, 1, [(0, 0)], engine=eng, directory=big)
+    empty = [np.zeros((0, 6), np.int16)] * 6                                              # empty directory: placement and pair moves only
+    res = optimize_chains(p, opt, 4, 20, [(0, 0)], engine=eng, directory=empty)
+    assert not res.dead.any() and ((res.log >> 1) & 7).max() <= 1
