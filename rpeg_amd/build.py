@@ -15,7 +15,7 @@ HEADERS = [os.path.join(HERE, "csrc", f) for f in
           [os.path.join(HERE, "..", "include", "rpeg_eval.h")]
 
 # -ffp-contract=off: scores must equal the reference's Python floats, which never fuse a*b+c.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-pthread", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function", "-Wno-unused-value", "-Wno-unused-result"]
 
 

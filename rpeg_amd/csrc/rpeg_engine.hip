@@ -19,6 +19,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -362,17 +363,8 @@ static int ensure_pool(rpeg_engine_t* e, hipStream_t s) {
   return 0;
 }
 
-// returns the pool offset of the class of `sig`, lowering it on first sight; -1 on failure
-static int64_t class_offset(rpeg_engine_t* e, uint64_t sig, bool* is_new) {
-  auto it = e->class_off.find(sig);
-  if (it != e->class_off.end()) return it->second;
-  LoweredClass lc;
-  try {
-    lc = lower_class(e->P, sig);
-  } catch (const std::exception& ex) {
-    e->err = std::string("lowering failed: ") + ex.what();
-    return -1;
-  }
+// appends a lowered class to the engine's tables; returns its pool offset or -1
+static int64_t class_append(rpeg_engine_t* e, uint64_t sig, const LoweredClass& lc) {
   const ClassHdr* h = (const ClassHdr*)lc.blob.data();
   e->max_nodes = std::max(e->max_nodes, h->n_nodes);
   e->max_slots = std::max(e->max_slots, h->n_slots);
@@ -384,8 +376,56 @@ static int64_t class_offset(rpeg_engine_t* e, uint64_t sig, bool* is_new) {
   e->cls_sig.push_back(sig);
   e->cls_off.push_back(off);
   e->cls_nodes.push_back(h->n_nodes);
-  if (is_new) *is_new = true;
   return off;
+}
+
+// returns the pool offset of the class of `sig`, lowering it on first sight; -1 on failure
+static int64_t class_offset(rpeg_engine_t* e, uint64_t sig, bool* is_new) {
+  auto it = e->class_off.find(sig);
+  if (it != e->class_off.end()) return it->second;
+  LoweredClass lc;
+  try {
+    lc = lower_class(e->P, sig);
+  } catch (const std::exception& ex) {
+    e->err = std::string("lowering failed: ") + ex.what();
+    return -1;
+  }
+  if (is_new) *is_new = true;
+  return class_append(e, sig, lc);
+}
+
+// lowers the classes of `sigs` that the engine does not hold yet, on up to eight host threads (lowering a
+// class reads only the problem tables), and appends them in the order of `sigs`
+static int lower_new_classes(rpeg_engine_t* e, const std::vector<uint64_t>& sigs, uint64_t* n_new) {
+  std::vector<uint64_t> todo;
+  {
+    std::unordered_map<uint64_t, char> seen;
+    for (uint64_t sg : sigs)
+      if (!e->class_off.count(sg) && seen.emplace(sg, 1).second) todo.push_back(sg);
+  }
+  if (todo.empty()) return 0;
+  std::vector<LoweredClass> lowered(todo.size());
+  std::vector<std::string> errors(todo.size());
+  const unsigned hw = std::max(1u, std::thread::hardware_concurrency());
+  const size_t n_threads = std::min<size_t>({(size_t)8, (size_t)hw, (todo.size() + 15) / 16});
+  auto work = [&](size_t t) {
+    for (size_t i = t; i < todo.size(); i += n_threads) {
+      try { lowered[i] = lower_class(e->P, todo[i]); } catch (const std::exception& ex) { errors[i] = ex.what(); if (errors[i].empty()) errors[i] = "error"; }
+    }
+  };
+  if (n_threads <= 1) {
+    work(0);
+  } else {
+    std::vector<std::thread> pool;
+    for (size_t t = 0; t < n_threads; ++t) pool.emplace_back(work, t);
+    for (auto& th : pool) th.join();
+  }
+  for (size_t i = 0; i < todo.size(); ++i) {
+    if (!errors[i].empty()) { e->err = "lowering failed: " + errors[i]; return -5; }
+    if (class_append(e, todo[i], lowered[i]) < 0) return -5;
+  }
+  *n_new += todo.size();
+  return 0;
 }
 
 static int ensure_ws(rpeg_engine_t* e, size_t bytes, hipStream_t s) {
@@ -547,15 +587,15 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (round >= 2) { e->err = "class table did not converge"; return -5; }
     HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
+    std::vector<uint64_t> sigs;
     uint64_t last_sig = SIG_INVALID;
     for (uint64_t i = 0; i < n; ++i) {
       const uint64_t sg = e->h_sig[i];
       if (sg == SIG_INVALID || sg == last_sig) continue;
       last_sig = sg;
-      bool is_new = false;
-      if (class_offset(e, sg, &is_new) < 0) return -5;
-      n_new += is_new;
+      sigs.push_back(sg);
     }
+    if (int rc = lower_new_classes(e, sigs, &n_new)) return rc;
   }
   std::vector<uint32_t> offs, counts, cids;   // the classes present in this batch
   for (uint32_t c = 0; c < ncls; ++c)
