@@ -160,7 +160,10 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
 template <int LS>
 __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
   extern __shared__ uint8_t ke_lds[];
-  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) ke_eval_wave<LS>(L, w, ke_lds);
+  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
+    if (LS == 0 && (L.wave_cls[w] & KE_CLS_LDS)) ke_eval_wave<KE_FEW>(L, w, ke_lds);   // uniform branch
+    else ke_eval_wave<LS>(L, w, ke_lds);
+  }
 }
 
 // Generic single-wavefront kernel over the host/device-shared scheduler template; used for the
@@ -369,7 +372,7 @@ static int64_t class_append(rpeg_engine_t* e, uint64_t sig, const LoweredClass& 
   e->max_nodes = std::max(e->max_nodes, h->n_nodes);
   e->max_slots = std::max(e->max_slots, h->n_slots);
   e->max_cls_bytes = std::max(e->max_cls_bytes, h->n_nodes * 8u + h->n_succ * 2u);
-  if (e->pool.size() + lc.blob.size() >= (1ull << 32)) { e->err = "class pool exceeds 4 GiB"; return -1; }
+  if (e->pool.size() + lc.blob.size() >= (1ull << 31)) { e->err = "class pool exceeds 2 GiB"; return -1; }   // bit 31 of an offset is a flag
   uint32_t off = (uint32_t)e->pool.size();
   e->pool.insert(e->pool.end(), lc.blob.begin(), lc.blob.end());
   e->class_off.emplace(sig, off);
@@ -637,7 +640,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     // classes with the largest graphs (at least seven tenths of the largest) get eight plans per wavefront, so
     // that fewer plans wait for the slowest one, unless they are a large share of the batch or the batch
     // is many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest).
-    const uint32_t heavy_lpw = 8u;
+    const uint32_t heavy_lpw = (uint32_t)KE_FEW;
     const uint64_t hfrac = 7ull;   // tenths of the largest node count
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t heavy_plans = 0;
@@ -662,8 +665,14 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     e->h_cfirst[cids[c]] = first[c];
     e->h_clpw[cids[c]] = clpw[c];
   }
-  for (size_t k = 0; k < order.size(); ++k)
-    for (uint32_t w = start[k]; w < start[k + 1]; ++w) e->h_cls[w] = offs[order[k]];
+  // wavefronts of few plans keep their scheduler state in LDS when that needs no more LDS than the ready
+  // lists of a full wavefront do
+  const bool few_in_lds = !ls &&
+      ke_lds_bytes(0, 32, KE_FEW, e->max_nodes, e->max_slots) <= ke_lds_bytes(0, 32, 0, e->max_nodes, e->max_slots);
+  for (size_t k = 0; k < order.size(); ++k) {
+    const uint32_t flag = few_in_lds && clpw[order[k]] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
+    for (uint32_t w = start[k]; w < start[k + 1]; ++w) e->h_cls[w] = offs[order[k]] | flag;
+  }
   if (int rc = ensure_pool(e, s)) return rc;
   HIP_TRY(e, hipMemcpyAsync(e->d_cfirst, e->h_cfirst, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_clpw, e->h_clpw, (size_t)ncls * 4, hipMemcpyHostToDevice, s));

@@ -23,6 +23,8 @@ namespace rpeg {
 
 constexpr int KE_WAVE = 64;
 constexpr uint32_t KE_IDLE = 0xFFFFFFFFu;
+constexpr uint32_t KE_CLS_LDS = 0x80000000u;   // flag in EvalLaunch::wave_cls
+constexpr int KE_FEW = 8;                      // plans of a wavefront so flagged
 
 struct EvalLaunch {              // uniform launch parameters
   const rpeg_problem_t* P;
@@ -30,7 +32,7 @@ struct EvalLaunch {              // uniform launch parameters
   const uint8_t* head;
   uint64_t stride;
   const uint32_t* perm;          // lane -> plan index, KE_IDLE for padding lanes
-  const uint32_t* wave_cls;      // wavefront -> class blob offset
+  const uint32_t* wave_cls;      // wavefront -> class blob offset; KE_CLS_LDS set: few plans, state in LDS
   const uint8_t* pool;
   uint8_t* ws;
   uint64_t n_waves;
@@ -128,7 +130,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   const int lane = threadIdx.x;
   int first_lane = 0;
   const rpeg_problem_t& P = *L.P;
-  const ClassView cv = class_view(L.pool + L.wave_cls[w]);   // uniform
+  const ClassView cv = class_view(L.pool + (L.wave_cls[w] & ~KE_CLS_LDS));   // uniform
   const int n = (int)cv.h->n_nodes, n_slots = (int)cv.h->n_slots, n_succ_all = (int)cv.h->n_succ;
 
   // ---- LDS carve-up
