@@ -256,14 +256,17 @@ int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* params, int32_t E
 
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,
-   [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace). */
+   [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace; 1: one plan per
+   wavefront). */
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
 
 /* Where the evaluation kernel keeps the scheduler state of a plan (ready time, rank and remaining
    in-degree per node, duration per slot).  lanes = 0: in an HBM workspace, 64 plans per wavefront (the
    throughput layout).  lanes = 8, 16, 32 or 64: in LDS, that many plans per wavefront (the latency
    layout: a batch too small to fill the chip finishes sooner); fails at the next call when the state
-   of the problem's largest class does not fit.  lanes = -1 (default): chosen per batch from its size.
+   of the problem's largest class does not fit.  lanes = 1: one plan per wavefront, its nodes spread
+   over the lanes (the layout of lowest latency, for batches of a few thousand plans at most; classes of
+   up to 384 nodes).  lanes = -1 (default): chosen per batch from its size.
    Results do not depend on the setting. */
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
 

@@ -484,67 +484,81 @@ RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) 
 // pairwise-overlap graph.  `order` lists the vertices in order of first appearance among the
 // lowered operator nodes (it fixes the insertion order of the reference's dicts and hence the
 // order of its float sums).  VM provides w_shard(v) (as double), mem_w(v), opt(v), extra(v).
+// Whether some device is covered by exactly the vertex set M and no other set dominates it: M is a maximal
+// clique of the overlap graph.
+RPEG_HD bool maximal_clique(int nv, const PlanMasks& pm, unsigned M) {
+  bool clique = true, maximal = true;
+  for (int v = 0; v < nv; ++v) {
+    const bool in = (M >> v) & 1u;
+    const bool fits = (M & ~mask_row(pm.ovl, v)) == 0;   // every member of M intersects v
+    if (in && !fits) clique = false;
+    if (!in && fits) maximal = false;
+  }
+  return clique && maximal;
+}
+
+// Peak of the devices covered by exactly the vertex set M.
+template <class VM>
+RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
+                                 const StructMasks& sm, const PlanMasks& pm, const VM& vm, unsigned M) {
+  const int nv = st.n_vertex;
+  double persistent = 0.0;
+  int groups = 0;
+  for (int i = 0; i < nv; ++i) {  // distinct (model, allocation) worker keys
+    const int v = order[i];
+    if (!((M >> v) & 1u)) continue;
+    if ((mask_row(pm.eq, v) & M & sm.same_model[v] & sm.before[i]) == 0) ++groups;
+  }
+  for (int i = 0; i < nv; ++i) {  // optimizer shards of the training vertices
+    const int v = order[i];
+    if (((M & sm.train & sm.trainable) >> v) & 1u) persistent += vm.opt(v);
+  }
+  unsigned serving = 0;           // serving shards: one per worker key that is not a training worker
+  for (int i = 0; i < nv; ++i) {
+    const int v = order[i];
+    if (!(((M & sm.trainable & ~(unsigned)sm.train) >> v) & 1u)) continue;
+    const unsigned same_key = mask_row(pm.eq, v) & M & sm.same_model[v];
+    if (same_key & sm.train_same[v]) continue;
+    const bool first = (same_key & serving) == 0;
+    serving |= 1u << v;
+    if (!first) continue;
+    double ws = 0.0;
+    for (int w = 0; w < nv; ++w)
+      if (((same_key & ~(unsigned)sm.train) >> w) & 1u) ws = dmax(ws, vm.w_shard(w));
+    persistent += (double)P.model[st.vertex[v].model].sb * ws;
+  }
+  for (int i = 0; i < nv; ++i) {  // frozen weights: one entry per model, its largest shard
+    const int v = order[i];
+    if (!(((M & ~(unsigned)sm.trainable) >> v) & 1u)) continue;
+    const unsigned same = M & sm.same_model[v];
+    if (same & sm.before[i]) continue;
+    double wb = 0.0;
+    for (int w = 0; w < nv; ++w)
+      if ((same >> w) & 1u) wb = dmax(wb, vm.mem_w(w));
+    persistent += wb;
+  }
+  double top = 0.0;
+  for (int i = 0; i < nv; ++i) {
+    const int v = order[i];
+    if (!((M >> v) & 1u)) continue;
+    const bool resident = !((sm.trainable >> v) & 1u) || (mask_row(pm.eq, v) & serving & sm.same_model[v]) != 0;
+    const double c = resident ? vm.extra(v) : vm.mem_w(v) + vm.extra(v);
+    top = dmax(top, c);
+  }
+  double peak = (double)groups * P.group_overhead + persistent + top;
+  if (P.max_groups > 0 && groups > P.max_groups) peak = __builtin_inf();  // memory.py:699-704
+  return peak;
+}
+
 template <class VM>
 RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
                                const PlanMasks& pm, const VM& vm) {
-  const int nv = st.n_vertex;
   const StructMasks sm = struct_masks(st, order);
-  const unsigned full = (1u << nv) - 1u;
+  const unsigned full = (1u << st.n_vertex) - 1u;
   double best = -1.0;
   for (unsigned M = 1; M <= full; ++M) {
-    bool clique = true, maximal = true;
-    for (int v = 0; v < nv; ++v) {
-      const bool in = (M >> v) & 1u;
-      const bool fits = (M & ~mask_row(pm.ovl, v)) == 0;   // every member of M intersects v
-      if (in && !fits) clique = false;
-      if (!in && fits) maximal = false;
-    }
-    if (!clique || !maximal) continue;
-    double persistent = 0.0;
-    int groups = 0;
-    for (int i = 0; i < nv; ++i) {  // distinct (model, allocation) worker keys
-      const int v = order[i];
-      if (!((M >> v) & 1u)) continue;
-      if ((mask_row(pm.eq, v) & M & sm.same_model[v] & sm.before[i]) == 0) ++groups;
-    }
-    for (int i = 0; i < nv; ++i) {  // optimizer shards of the training vertices
-      const int v = order[i];
-      if (((M & sm.train & sm.trainable) >> v) & 1u) persistent += vm.opt(v);
-    }
-    unsigned serving = 0;           // serving shards: one per worker key that is not a training worker
-    for (int i = 0; i < nv; ++i) {
-      const int v = order[i];
-      if (!(((M & sm.trainable & ~(unsigned)sm.train) >> v) & 1u)) continue;
-      const unsigned same_key = mask_row(pm.eq, v) & M & sm.same_model[v];
-      if (same_key & sm.train_same[v]) continue;
-      const bool first = (same_key & serving) == 0;
-      serving |= 1u << v;
-      if (!first) continue;
-      double ws = 0.0;
-      for (int w = 0; w < nv; ++w)
-        if (((same_key & ~(unsigned)sm.train) >> w) & 1u) ws = dmax(ws, vm.w_shard(w));
-      persistent += (double)P.model[st.vertex[v].model].sb * ws;
-    }
-    for (int i = 0; i < nv; ++i) {  // frozen weights: one entry per model, its largest shard
-      const int v = order[i];
-      if (!(((M & ~(unsigned)sm.trainable) >> v) & 1u)) continue;
-      const unsigned same = M & sm.same_model[v];
-      if (same & sm.before[i]) continue;
-      double wb = 0.0;
-      for (int w = 0; w < nv; ++w)
-        if ((same >> w) & 1u) wb = dmax(wb, vm.mem_w(w));
-      persistent += wb;
-    }
-    double top = 0.0;
-    for (int i = 0; i < nv; ++i) {
-      const int v = order[i];
-      if (!((M >> v) & 1u)) continue;
-      const bool resident = !((sm.trainable >> v) & 1u) || (mask_row(pm.eq, v) & serving & sm.same_model[v]) != 0;
-      const double c = resident ? vm.extra(v) : vm.mem_w(v) + vm.extra(v);
-      top = dmax(top, c);
-    }
-    double peak = (double)groups * P.group_overhead + persistent + top;
-    if (P.max_groups > 0 && groups > P.max_groups) peak = __builtin_inf();  // memory.py:699-704
+    if (!maximal_clique(st.n_vertex, pm, M)) continue;
+    const double peak = device_class_peak(P, st, order, sm, pm, vm, M);
     if (peak > best) best = peak;
   }
   return best;

@@ -24,6 +24,7 @@
 #include <vector>
 
 #include "rpeg_kernel_eval.h"
+#include "rpeg_kernel_plan.h"
 #include "rpeg_lower.h"
 #include "rpeg_plan.h"
 #include "rpeg_sa.h"
@@ -145,16 +146,17 @@ __global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, co
   kidx[i] = k;
 }
 
-// perm[(first wavefront of the class + k / lanes) * 64 + k % lanes] = plan, k = arrival order within the class
+// perm[(first wavefront of the class + k / lanes) * pstride + k % lanes] = plan, k = arrival order within the
+// class; pstride = 64, or 1 when every wavefront takes one plan
 __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const uint32_t* __restrict__ kidx,
                           const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
-                          uint32_t* __restrict__ perm) {
+                          uint32_t* __restrict__ perm, uint32_t pstride) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t c = cid[i];
   if (c >= CID_UNKNOWN) return;
   const uint32_t k = kidx[i], l = clpw[c];
-  perm[(uint64_t)(cfirst[c] + k / l) * WAVE + k % l] = (uint32_t)i;
+  perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
 }
 
 template <int LS>
@@ -163,6 +165,15 @@ __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
   for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
     if (LS == 0 && (L.wave_cls[w] & KE_CLS_LDS)) ke_eval_wave<KE_FEW>(L, w, ke_lds);   // uniform branch
     else ke_eval_wave<LS>(L, w, ke_lds);
+  }
+}
+
+// One plan per wavefront (rpeg_kernel_plan.h); perm[w] is the plan of wavefront task w.
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(4, 8))) void k_plan(const EvalLaunch L) {
+  extern __shared__ uint8_t kp_lds[];
+  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
+    const uint64_t pi = L.perm[w];
+    kp_eval_plan(L, w, pi, class_view(L.pool + L.wave_cls[w]), kp_lds);
   }
 }
 
@@ -257,7 +268,8 @@ struct rpeg_engine_s {
   size_t d_pool_cap = 0, d_pool_used = 0;
   uint32_t max_nodes = 1, max_slots = 1, max_cls_bytes = 16;
   bool lds_attr_set[5] = {false, false, false, false, false};
-  int state_lanes = -1;   // -1: chosen per batch; 0: per-plan state in HBM; 8/16/32/64: in LDS, that many plans per wavefront
+  uint32_t one_plan_waves_per_cu = 32;   // batches of at most this many plans per compute unit take one wavefront per plan
+  int state_lanes = -1;   // -1: chosen per batch; 0: per-plan state in HBM; 8/16/32/64: in LDS, that many plans per wavefront; 1: one plan per wavefront (k_plan)
   bool prof_on = false;
   unsigned long long* d_prof = nullptr;
   uint64_t prof_waves = 0;
@@ -520,7 +532,7 @@ int rpeg_engine_profile(rpeg_engine_t* e, int32_t enable, unsigned long long* ou
 
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
   if (!e) return -1;
-  if (lanes != -1 && lanes != 0 && lanes != 8 && lanes != 16 && lanes != 32 && lanes != 64) {
+  if (lanes != -1 && lanes != 0 && lanes != 1 && lanes != 8 && lanes != 16 && lanes != 32 && lanes != 64) {
     e->err = "state lanes must be -1, 0, 8, 16, 32 or 64";
     return -1;
   }
@@ -607,25 +619,34 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // with the state in the HBM workspace; a batch too small to fill the chip that way is spread over more
   // wavefronts of fewer plans whose state fits in LDS, which shortens every scheduler step.
   int ls = e->state_lanes;
+  bool one = false;   // one plan per wavefront (k_plan)
   {
     auto waves_for = [&](uint32_t per) { uint64_t t = 0; for (uint32_t c : counts) t += (c + per - 1) / per; return t; };
     auto fits = [&](int l) {
       return ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, 32, (uint32_t)l, e->max_nodes, e->max_slots) <= 160 * 1024;
     };
+    const bool one_fits = e->max_nodes <= (uint32_t)(WAVE * KP_MAX_NS) && kp_lds_bytes(e->max_nodes, e->max_slots) <= 64 * 1024;
     if (ls < 0) {
       ls = 0;
-      if (waves_for(WAVE) < (uint64_t)e->n_cu * 2)   // under two wavefronts per compute unit
+      if (one_fits && waves_for(1) <= (uint64_t)e->n_cu * e->one_plan_waves_per_cu) {
+        one = true;   // the batch does not fill the chip with a plan per lane: spread every plan over a wavefront
+      } else if (waves_for(WAVE) < (uint64_t)e->n_cu * 2) {   // under two wavefronts per compute unit
         for (int l : {8, 16, 32, 64}) {              // fewest plans per wavefront that still gives each its own SIMD
           if (!fits(l)) break;
           ls = l;
           if (waves_for((uint32_t)l) <= (uint64_t)e->n_cu * 4) break;
         }
+      }
+    } else if (ls == 1) {
+      if (!one_fits) { e->err = "a class of this problem has too many nodes for one plan per wavefront"; return -8; }
+      one = true;
+      ls = 0;
     } else if (ls > 0 && !fits(ls)) {
       e->err = "per-plan state of this problem does not fit in LDS with that many plans per wavefront";
       return -8;
     }
   }
-  const uint32_t lpw = ls ? (uint32_t)ls : (uint32_t)WAVE;   // plans per wavefront
+  const uint32_t lpw = one ? 1u : ls ? (uint32_t)ls : (uint32_t)WAVE;   // plans per wavefront
   // every class starts on a wavefront boundary; the lanes left over are idle
   // classes with the largest graphs first: their wavefronts run longest and should not start last
   std::vector<uint32_t> order(counts.size());
@@ -635,7 +656,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   });
   // start[k]: first wavefront of the k-th class in launch order
   std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0), clpw(counts.size(), lpw);
-  if (!ls && !order.empty()) {
+  if (!ls && !one && !order.empty()) {
     // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
     // classes with the largest graphs (at least seven tenths of the largest) get eight plans per wavefront, so
     // that fewer plans wait for the slowest one, unless they are a large share of the batch or the batch
@@ -656,6 +677,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     first[order[k]] = start[k];
     start[k + 1] = start[k] + (counts[order[k]] + clpw[order[k]] - 1) / clpw[order[k]];
   }
+  const uint32_t pstride = one ? 1u : (uint32_t)WAVE;
   const uint64_t n_sorted = (uint64_t)start.back() * WAVE;
   e->stats[0] = counts.size();
   e->stats[1] = n_new;
@@ -667,7 +689,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   // wavefronts of few plans keep their scheduler state in LDS when that needs no more LDS than the ready
   // lists of a full wavefront do
-  const bool few_in_lds = !ls &&
+  const bool few_in_lds = !ls && !one &&
       ke_lds_bytes(0, 32, KE_FEW, e->max_nodes, e->max_slots) <= ke_lds_bytes(0, 32, 0, e->max_nodes, e->max_slots);
   for (size_t k = 0; k < order.size(); ++k) {
     const uint32_t flag = few_in_lds && clpw[order[k]] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
@@ -677,14 +699,15 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   HIP_TRY(e, hipMemcpyAsync(e->d_cfirst, e->h_cfirst, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_clpw, e->h_clpw, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted / WAVE * 4, hipMemcpyHostToDevice, s));
-  hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
-  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_perm);
+  if (!one)   // with one plan per wavefront every entry is written by the scatter
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
+  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_perm, pstride);
   HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_sorted / WAVE;
-  const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * 16);
-  const size_t wsb = ls ? 0 : ke_ws_bytes(e->max_nodes, e->max_slots);
-  if (!ls)
+  const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * (one ? 32 : 16));
+  const size_t wsb = ls || one ? 0 : ke_ws_bytes(e->max_nodes, e->max_slots);
+  if (!ls && !one)
     if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
   EvalLaunch L;
   L.P = e->dP; L.vert = plans->vert; L.head = plans->head; L.stride = plans->stride;
@@ -705,21 +728,23 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     e->prof_waves = n_waves;
     L.prof = e->d_prof;
   }
-  const size_t lds = ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots);
+  const size_t lds = one ? kp_lds_bytes(e->max_nodes, e->max_slots)
+                         : ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots);
   if (lds > 160 * 1024) { e->err = "class tables exceed the LDS"; return -8; }
   const void* kfn = ls == 0 ? (const void*)k_eval<0> : ls == 8 ? (const void*)k_eval<8> : ls == 16 ? (const void*)k_eval<16>
                   : ls == 32 ? (const void*)k_eval<32> : (const void*)k_eval<64>;
   const int ki = ls == 0 ? 0 : ls == 8 ? 1 : ls == 16 ? 2 : ls == 32 ? 3 : 4;
-  if (lds > 64 * 1024 && !e->lds_attr_set[ki]) {
+  if (!one && lds > 64 * 1024 && !e->lds_attr_set[ki]) {
     HIP_TRY(e, hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     e->lds_attr_set[ki] = true;
   }
   e->stats[2] = n_waves;
   e->stats[3] = lds;
   e->stats[4] = wsb * grid;
-  e->stats[5] = (uint64_t)ls;
+  e->stats[5] = one ? 1u : (uint64_t)ls;
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
-  switch (ls) {
+  if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
+  else switch (ls) {
     case 0: hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds, s, L); break;
     case 8: hipLaunchKernelGGL(k_eval<8>, dim3(grid), dim3(WAVE), lds, s, L); break;
     case 16: hipLaunchKernelGGL(k_eval<16>, dim3(grid), dim3(WAVE), lds, s, L); break;

@@ -1,0 +1,637 @@
+// rpeg_kernel_plan.h - the evaluation kernel for batches too small to fill the chip with one plan per
+// lane (device only): ONE PLAN PER WAVEFRONT.
+//
+// The lanes share the plan's work instead of each carrying a plan of its own:
+//   cost model      lane = duration slot of the class (NodeCostModel.time of one node variant each)
+//   memory model    lane = template vertex, then lane = vertex subset (candidate device class)
+//   ranks           lane = lowered node; Jacobi rounds of rank = duration + max(rank of successors) until
+//                   nothing changes (the fixed point is the reverse topological pass of scheduler.py:71-100)
+//   list scheduler  lane = lowered node (NS nodes per lane).  Every node keeps its heap key, its tie-break
+//                   word, the latest finish of its predecessors and the availability of the devices it
+//                   reserves in registers.  The heap's pop is a minimum over the wavefront (row shifts and
+//                   broadcasts, no memory); all control flow is uniform, so the loop runs on the scalar unit
+//                   and the successors of the dispatched node are read from the winner lane's registers.
+//
+// The heap key of the reference is (est, comm_prio, topo_idx, -rank, tie).  (comm_prio, topo_idx, -rank) is
+// fixed once the ranks are known, so it is replaced by the node's position in that order (equal triples get
+// equal positions), packed above the tie counter in one 32-bit word: a pop is the minimum of a double and,
+// among equals, of that word.
+//
+// Device availability: a node waits for max(avail[d]) over the devices it reserves, i.e. for the largest
+// finish time of any dispatched node whose reserved vertices intersect its own.  Every lane keeps that
+// maximum for its nodes and raises it at each dispatch (max is exact, so the order does not matter).
+#ifndef RPEG_KERNEL_PLAN_H
+#define RPEG_KERNEL_PLAN_H
+
+#include "rpeg_kernel_eval.h"
+
+namespace rpeg {
+
+constexpr int KP_MAX_NS = 6;                    // nodes per lane: classes of up to 384 nodes
+constexpr uint32_t KP_TIE_BITS = 23u, KP_TIE_MASK = (1u << KP_TIE_BITS) - 1u;
+constexpr int KP_PLAN_I16 = 80;                 // plan fields in LDS (60 used; pair tests may read past them)
+
+// LDS of one wavefront: plan fields, per-vertex memory terms, durations per slot, rank / finish and start
+// per node (plus one neutral element each), tie-break class per node.
+__host__ __device__ inline size_t kp_lds_bytes(uint32_t nodes, uint32_t slots) {
+  return ((size_t)KP_PLAN_I16 * 2 + (size_t)RPEG_MAX_V * 4 * 8 + 8ull * slots + 16ull * (nodes + 1) + nodes + 15) & ~size_t(15);
+}
+
+#if defined(__HIPCC__)
+
+template <int CTRL, int ROWS>
+__device__ inline int kp_dpp(int v) { return __builtin_amdgcn_update_dpp(v, v, CTRL, ROWS, 0xF, false); }
+
+struct KpMin { __device__ double operator()(double a, double b) const { return __builtin_fmin(a, b); } };
+struct KpMax { __device__ double operator()(double a, double b) const { return __builtin_fmax(a, b); } };
+
+template <int CTRL, int ROWS, class OP>
+__device__ inline double kp_step(double v, OP op) {
+  const int lo = kp_dpp<CTRL, ROWS>(__double2loint(v)), hi = kp_dpp<CTRL, ROWS>(__double2hiint(v));
+  return op(v, __hiloint2double(hi, lo));
+}
+// reduction over the 64 lanes (all must be active); the result is uniform
+template <class OP>
+__device__ inline double kp_wave_reduce(double v, OP op) {
+  v = kp_step<0xB1, 0xF>(v, op);    // lanes 1,0,3,2 of each quad
+  v = kp_step<0x4E, 0xF>(v, op);    // lanes 2,3,0,1 of each quad
+  v = kp_step<0x124, 0xF>(v, op);   // row rotated by 4
+  v = kp_step<0x128, 0xF>(v, op);   // row rotated by 8: every lane holds its row's result
+  v = kp_step<0x142, 0xA>(v, op);   // last lane of rows 0 and 2 into rows 1 and 3
+  v = kp_step<0x143, 0xC>(v, op);   // last lane of row 1 into rows 2 and 3: row 3 holds the result
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), 63), __builtin_amdgcn_readlane(__double2loint(v), 63));
+}
+// minimum of an unsigned word over the 64 lanes; the neutral element fills the lanes a step does not
+// write, so that each step is one instruction (the lane move folds into the minimum)
+template <int CTRL, int ROWS>
+__device__ inline uint32_t kp_ustep(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)0xFFFFFFFFu, (int)v, CTRL, ROWS, 0xF, false);
+  return o < v ? o : v;
+}
+__device__ inline uint32_t kp_wave_umin(uint32_t v) {
+  v = kp_ustep<0xB1, 0xF>(v);
+  v = kp_ustep<0x4E, 0xF>(v);
+  v = kp_ustep<0x124, 0xF>(v);
+  v = kp_ustep<0x128, 0xF>(v);
+  v = kp_ustep<0x142, 0xA>(v);
+  v = kp_ustep<0x143, 0xC>(v);
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+__device__ inline double kp_readlane(double v, int l) {
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), l), __builtin_amdgcn_readlane(__double2loint(v), l));
+}
+__device__ inline bool kp_is_inf(double v) {   // on the bits, so that a uniform value stays on the scalar unit
+  return __double2hiint(v) == 0x7FF00000 && __double2loint(v) == 0;
+}
+
+// Ranks, tie-break classes and the list scheduler for a class of at most 64 * NS nodes.  l_rank holds the
+// ranks while they are computed and the finish times afterwards; nd is the index of the neutral element.
+// Returns false on a broken class (cycle).
+template <int NS>
+__device__ inline bool kp_schedule(const ClassView& cv, const int n, const int lane, const uint64_t ovl,
+                                   const uint64_t dpne, const int nd, const double* l_dur, double* l_rank,
+                                   double* l_start, uint8_t* l_pt, const bool keep_trace, double* out_makespan,
+                                   long* out_pops, unsigned long long* stamp) {
+  const double inf = __builtin_inf();
+  double key[NS], tm[NS], dvc[NS], dur[NS], rk[NS];
+  uint32_t ord[NS], info[NS], deg[NS], sxl[NS], sxh[NS], pt[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int v = s * 64 + lane;
+    const bool ok = v < n;
+    const uint64_t bits = ((const uint64_t*)cv.node)[ok ? v : 0];
+    NodeRec nr;
+    __builtin_memcpy(&nr, &bits, 8);
+    info[s] = ok ? (blocked_mask(nr, dpne) | ((uint32_t)nr.n_succ << 8) | ((uint32_t)nr.succ_begin << 16)) : 0u;
+    deg[s] = ok ? (uint32_t)nr.indeg : 0xFFFFu;
+    dur[s] = ok ? l_dur[nr.slot] : 0.0;
+    pt[s] = nr.ptkey;
+    uint32_t q[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q[j] = (ok && j < nr.n_succ) ? (uint32_t)cv.succ[nr.succ_begin + j] : (uint32_t)nd;
+    sxl[s] = q[0] | (q[1] << 16);
+    sxh[s] = q[2] | (q[3] << 16);
+    rk[s] = dur[s];
+    key[s] = inf;
+    tm[s] = 0.0;
+    dvc[s] = 0.0;
+    if (ok) {
+      l_rank[v] = rk[s];
+      l_pt[v] = nr.ptkey;
+    }
+  }
+  if (lane == 0) l_rank[nd] = 0.0;
+  __syncthreads();
+
+  // ---- ranks (scheduler.py:71-100): rounds until no rank changes, at most one per node
+  for (int round = 0; round <= n; ++round) {
+    bool changed = false;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const double r0 = l_rank[sxl[s] & 0xFFFFu], r1 = l_rank[sxl[s] >> 16], r2 = l_rank[sxh[s] & 0xFFFFu],
+                   r3 = l_rank[sxh[s] >> 16];
+      double best = 0.0;
+      best = r0 > best ? r0 : best;
+      best = r1 > best ? r1 : best;
+      best = r2 > best ? r2 : best;
+      best = r3 > best ? r3 : best;
+      const int ns = (int)((info[s] >> 8) & 0xFFu), sb = (int)(info[s] >> 16);
+      for (int j = 4; j < ns; ++j) {
+        const double r = l_rank[cv.succ[sb + j]];
+        best = r > best ? r : best;
+      }
+      const double nr_ = dur[s] + best;
+      changed = changed || nr_ != rk[s];
+      rk[s] = nr_;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (s * 64 + lane < n) l_rank[s * 64 + lane] = rk[s];
+    __syncthreads();
+    if (!__ballot(changed)) break;
+  }
+  // chain inheritance (scheduler.py:367-378): the sub-nodes of one split vertex share the chain's top rank
+  for (unsigned g = lane; g < cv.h->n_groups; g += KE_WAVE) {
+    const GroupRec gr = cv.group[g];
+    double top = l_rank[cv.gmember[gr.begin]];
+    for (int j = 1; j < gr.count; ++j) {
+      const double r = l_rank[cv.gmember[gr.begin + j]];
+      top = r > top ? r : top;
+    }
+    for (int j = 0; j < gr.count; ++j) l_rank[cv.gmember[gr.begin + j]] = top;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < NS; ++s) rk[s] = l_rank[s * 64 + lane < n ? s * 64 + lane : nd];
+
+  if (stamp) stamp[3] = wall_clock64();
+  // ---- position of every node in the order (comm_prio * 8 + topo_idx ascending, rank descending); `shared`
+  // marks the nodes whose position another node has too: only among those does a tie counter ever decide
+  bool shared[NS];
+  {
+    uint32_t eq[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) ord[s] = eq[s] = 0;
+#pragma unroll 4
+    for (int u = 0; u < n; ++u) {
+      const double ru = l_rank[u];
+      const uint32_t pu = l_pt[u];
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        ord[s] += ((pu < pt[s]) | ((pu == pt[s]) & (ru > rk[s]))) ? 1u : 0u;
+        eq[s] += ((pu == pt[s]) & (ru == rk[s])) ? 1u : 0u;
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      ord[s] <<= KP_TIE_BITS;
+      shared[s] = eq[s] > 1u;
+    }
+  }
+  __syncthreads();   // l_rank is reused for the finish times from here on
+  if (stamp) stamp[4] = wall_clock64();
+
+  // ---- list scheduling (scheduler.py:399-546)
+  uint32_t ctr = 0;
+  for (unsigned i = 0; i < cv.h->n_init; ++i) {
+    const int v = __builtin_amdgcn_readfirstlane((int)cv.init[i]);
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (s == (v >> 6) && lane == (v & 63)) {
+        key[s] = 0.0;
+        ord[s] |= ctr;
+      }
+    ++ctr;
+  }
+  double makespan = 0.0;
+  int done = 0;
+  bool ok = true;
+  long pops = 0, slow_decisions = 0;
+  const long guard_max = (long)n * n + 64;
+  long guard = 0;
+  while (done < n && guard < guard_max) {
+    ++guard;
+    ++pops;
+    // ---- One decision of the heap: the pops up to the next dispatch.  The heap pops stale entries (key below
+    // the true start time, because the node's devices are busy) in key order and pushes each back with its
+    // true time and a fresh tie, until the minimum is current.  That entry D is the minimum of (true time,
+    // position, tie); the entries pushed back on the way are exactly the stale ones whose old key is below
+    // D's final key.  When D is alone with its (true time, position) and no other waiting entry has its
+    // position, no tie counter decides which entry D is and the whole decision is taken at once; otherwise
+    // the pops are replayed one by one.
+    int wl, ws;
+    double gk;
+    bool slow;
+    {
+      double e[NS];
+#pragma unroll
+      for (int s = 0; s < NS; ++s) e[s] = dvc[s] > key[s] ? dvc[s] : key[s];
+      double be = e[0];
+      uint32_t bo = ord[0] >> KP_TIE_BITS;
+      int bs = 0;
+#pragma unroll
+      for (int s = 1; s < NS; ++s) {
+        const uint32_t o = ord[s] >> KP_TIE_BITS;
+        const bool lt = (e[s] < be) | ((e[s] == be) & (o < bo));
+        be = lt ? e[s] : be;
+        bo = lt ? o : bo;
+        bs = lt ? s : bs;
+      }
+      const uint32_t ehi = (uint32_t)__double2hiint(be), elo = (uint32_t)__double2loint(be);
+      const uint32_t ghi = kp_wave_umin(ehi);
+      if (ghi >= 0x7FF00000u) { ok = false; break; }   // nothing is ready: cycle (scheduler.py:548-550)
+      bool cand = ehi == ghi;
+      unsigned long long m = __ballot(cand);
+      if (m & (m - 1ull)) {
+        const uint32_t glo = kp_wave_umin(cand ? elo : 0xFFFFFFFFu);
+        cand = cand && elo == glo;
+        m = __ballot(cand);
+        if (m & (m - 1ull)) {
+          const uint32_t go_ = kp_wave_umin(cand ? bo : 0xFFFFFFFFu);
+          m = __ballot(cand && bo == go_);
+        }
+      }
+      wl = __builtin_ctzll(m);
+      ws = __builtin_amdgcn_readlane(bs, wl);
+      gk = __hiloint2double((int)ghi, __builtin_amdgcn_readlane((int)elo, wl));
+      const uint32_t go = (uint32_t)__builtin_amdgcn_readlane((int)bo, wl);
+      bool other = false, in_r[NS];
+      uint32_t n_shared = 0;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const uint32_t o = ord[s] >> KP_TIE_BITS;
+        const bool is_d = (lane == wl) & (s == ws);
+        other = other | ((key[s] < inf) & (o == go) & !is_d);
+        in_r[s] = (dvc[s] > key[s]) & ((key[s] < gk) | ((key[s] == gk) & (o < go)));
+        n_shared += (in_r[s] & shared[s]) ? 1u : 0u;
+      }
+      slow = (m & (m - 1ull)) != 0ull || __ballot(other) != 0ull;
+      if (!slow) {
+        // Fresh ties of the entries pushed back: the heap hands them out in pop order, i.e. in the order of
+        // the old keys.  Entries that share their position with no other node never compare ties and take
+        // any fresh value; two or more entries with shared positions are ranked among themselves first.
+        uint32_t rank[NS], total = 1u;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) rank[s] = 0u;
+        const unsigned long long ms = __ballot(n_shared > 0u);
+        if ((ms & (ms - 1ull)) != 0ull || __ballot(n_shared > 1u) != 0ull) {
+          total = 0u;
+#pragma unroll
+          for (int s = 0; s < NS; ++s) {
+            unsigned long long members = __ballot(in_r[s] & shared[s]);
+            total += (uint32_t)__builtin_popcountll(members);
+            while (members) {
+              const int j = __builtin_ctzll(members);
+              members &= members - 1ull;
+              const double kj = kp_readlane(key[s], j);
+              const uint32_t oj = (uint32_t)__builtin_amdgcn_readlane((int)ord[s], j);
+#pragma unroll
+              for (int t = 0; t < NS; ++t) rank[t] += ((kj < key[t]) | ((kj == key[t]) & (oj < ord[t]))) ? 1u : 0u;
+            }
+          }
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+          if (in_r[s]) {
+            key[s] = dvc[s];
+            ord[s] = (ord[s] & ~KP_TIE_MASK) | (ctr + rank[s]);
+          }
+        ctr += total;
+      }
+    }
+    if (slow) {
+      ++slow_decisions;
+      for (;;) {
+        // the heap's minimum: smallest key, among equals the smallest tie-break word.  Keys are non-negative
+        // doubles or +inf, so they order like their bit patterns: the minimum is taken on the high words,
+        // then (only if lanes still tie) on the low words, then on the tie-break words.
+        double bk = key[0];
+        uint32_t bo = ord[0];
+        int bs = 0;
+#pragma unroll
+        for (int s = 1; s < NS; ++s) {
+          const bool lt = (key[s] < bk) | ((key[s] == bk) & (ord[s] < bo));
+          bk = lt ? key[s] : bk;
+          bo = lt ? ord[s] : bo;
+          bs = lt ? s : bs;
+        }
+        const uint32_t khi = (uint32_t)__double2hiint(bk), klo = (uint32_t)__double2loint(bk);
+        const uint32_t ghi = kp_wave_umin(khi);
+        bool cand = khi == ghi;
+        unsigned long long m = __ballot(cand);
+        if (m & (m - 1ull)) {
+          const uint32_t glo = kp_wave_umin(cand ? klo : 0xFFFFFFFFu);
+          cand = cand && klo == glo;
+          m = __ballot(cand);
+          if (m & (m - 1ull)) {
+            const uint32_t go_ = kp_wave_umin(cand ? bo : 0xFFFFFFFFu);
+            m = __ballot(cand && bo == go_);
+          }
+        }
+        wl = __builtin_ctzll(m);
+        gk = __hiloint2double((int)ghi, __builtin_amdgcn_readlane((int)klo, wl));
+        ws = __builtin_amdgcn_readlane(bs, wl);
+        // stale: push back with the true time and a fresh tie (scheduler.py:437-443)
+        double wdv = dvc[0];
+#pragma unroll
+        for (int s = 1; s < NS; ++s) wdv = s == ws ? dvc[s] : wdv;
+        if (!__ballot(lane == wl && wdv > gk)) break;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+          if (lane == wl && s == ws) {
+            key[s] = dvc[s];
+            ord[s] = (ord[s] & ~KP_TIE_MASK) | ctr;
+          }
+        ++ctr;
+        ++pops;
+        if (++guard >= guard_max) break;
+      }
+      if (guard >= guard_max) break;
+    }
+    const bool mine = lane == wl;
+    // ---- dispatch node ws * 64 + wl at gk
+    double wdur = dur[0];
+    uint32_t winfo = info[0], wsl = sxl[0], wsh = sxh[0];
+#pragma unroll
+    for (int s = 1; s < NS; ++s) {
+      wdur = s == ws ? dur[s] : wdur;
+      winfo = s == ws ? info[s] : winfo;
+      wsl = s == ws ? sxl[s] : wsl;
+      wsh = s == ws ? sxh[s] : wsh;
+    }
+    const double d = kp_readlane(wdur, wl);
+    const uint32_t binfo = (uint32_t)__builtin_amdgcn_readlane((int)winfo, wl);
+    const uint32_t s01 = (uint32_t)__builtin_amdgcn_readlane((int)wsl, wl), s23 = (uint32_t)__builtin_amdgcn_readlane((int)wsh, wl);
+    const double fin = gk + d;
+    makespan = fin > makespan ? fin : makespan;
+    ++done;
+    unsigned touched = 0;
+#pragma unroll
+    for (int x = 0; x < RPEG_MAX_V; ++x)
+      if ((binfo >> x) & 1u) touched |= mask_row(ovl, x);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const bool hit = (info[s] & touched) != 0u;
+      dvc[s] = hit && fin > dvc[s] ? fin : dvc[s];
+      if (mine && s == ws) key[s] = inf;
+    }
+    if (keep_trace && mine) {
+      l_rank[ws * 64 + wl] = fin;
+      l_start[ws * 64 + wl] = gk;
+    }
+    // successors in adjacency order; a node whose last predecessor this was becomes ready
+    const int ns = (int)((binfo >> 8) & 0xFFu), sb = (int)(binfo >> 16);
+    for (int j = 0; j < ns; ++j) {
+      int wn;
+      if (j < 4) wn = (int)(((j < 2 ? s01 : s23) >> ((j & 1) * 16)) & 0xFFFFu);
+      else wn = __builtin_amdgcn_readfirstlane((int)cv.succ[sb + j]);
+      const bool me = lane == (wn & 63);
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        if (me && s == (wn >> 6)) {
+          tm[s] = fin > tm[s] ? fin : tm[s];
+          deg[s] -= 1u;
+          if (deg[s] == 0u) {
+            key[s] = dvc[s] > tm[s] ? dvc[s] : tm[s];
+            ord[s] |= ctr;
+          }
+        }
+      ++ctr;
+    }
+  }
+  if (ctr > KP_TIE_MASK) ok = false;
+  if (done != n) ok = false;
+  *out_makespan = makespan;
+  *out_pops = (slow_decisions << 20) | pops;
+  return ok;
+}
+
+// Pair relations and vertex sets of one plan by POSITION in the order of first appearance (bit 8i+j of a
+// 64-bit word: positions i and j; bit i of a 32-bit word: position i).
+struct KpOrdered {
+  unsigned long long ovl, eq, same_model, train_same;
+  unsigned train, trainable;
+};
+__device__ inline unsigned kp_row(unsigned long long m, int i) { return (unsigned)(m >> (8 * i)) & 0xFFu; }
+
+__device__ inline bool kp_maximal_clique(int nv, unsigned long long ovl, unsigned M) {
+  bool clique = true, maximal = true;
+#pragma unroll
+  for (int i = 0; i < RPEG_MAX_V; ++i) {
+    if (i >= nv) break;
+    const bool in = (M >> i) & 1u;
+    const bool fits = (M & ~kp_row(ovl, i)) == 0;
+    clique = clique && !(in && !fits);
+    maximal = maximal && !(!in && fits);
+  }
+  return clique && maximal;
+}
+
+// device_class_peak of rpeg_core.h on position-indexed masks; vm[i * 4 + f] holds w_shard, mem_w, opt and
+// extra of the vertex at position i.  M is uniform, so is the control flow; every loop runs over the
+// compile-time bound and nothing is indexed dynamically.
+__device__ inline double kp_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order, int nv,
+                                       const KpOrdered& om, const double* vm, unsigned M) {
+  double persistent = 0.0;
+  int groups = 0;
+#pragma unroll
+  for (int i = 0; i < RPEG_MAX_V; ++i) {   // distinct (model, allocation) worker keys
+    if (!((M >> i) & 1u)) continue;
+    if ((kp_row(om.eq, i) & M & kp_row(om.same_model, i) & ((1u << i) - 1u)) == 0) ++groups;
+  }
+#pragma unroll
+  for (int i = 0; i < RPEG_MAX_V; ++i)     // optimizer shards of the training vertices
+    if (((M & om.train & om.trainable) >> i) & 1u) persistent += vm[i * 4 + 2];
+  unsigned serving = 0;                    // serving shards: one per worker key that is not a training worker
+#pragma unroll
+  for (int i = 0; i < RPEG_MAX_V; ++i) {
+    if (!(((M & om.trainable & ~om.train) >> i) & 1u)) continue;
+    const unsigned same_key = kp_row(om.eq, i) & M & kp_row(om.same_model, i);
+    if (same_key & kp_row(om.train_same, i)) continue;
+    const bool first = (same_key & serving) == 0;
+    serving |= 1u << i;
+    if (!first) continue;
+    double ws = 0.0;
+#pragma unroll
+    for (int q = 0; q < RPEG_MAX_V; ++q)
+      if (((same_key & ~om.train) >> q) & 1u) ws = dmax(ws, vm[q * 4 + 0]);
+    persistent += (double)P.model[st.vertex[order[i]].model].sb * ws;
+  }
+#pragma unroll
+  for (int i = 0; i < RPEG_MAX_V; ++i) {   // frozen weights: one entry per model, its largest shard
+    if (!(((M & ~om.trainable) >> i) & 1u)) continue;
+    const unsigned same = M & kp_row(om.same_model, i);
+    if (same & ((1u << i) - 1u)) continue;
+    double wb = 0.0;
+#pragma unroll
+    for (int q = 0; q < RPEG_MAX_V; ++q)
+      if ((same >> q) & 1u) wb = dmax(wb, vm[q * 4 + 1]);
+    persistent += wb;
+  }
+  double top = 0.0;
+#pragma unroll
+  for (int i = 0; i < RPEG_MAX_V; ++i) {
+    if (!((M >> i) & 1u)) continue;
+    const bool resident = !((om.trainable >> i) & 1u) || (kp_row(om.eq, i) & serving & kp_row(om.same_model, i)) != 0;
+    const double c = resident ? vm[i * 4 + 3] : vm[i * 4 + 1] + vm[i * 4 + 3];
+    top = dmax(top, c);
+  }
+  double peak = (double)groups * P.group_overhead + persistent + top;
+  if (P.max_groups > 0 && groups > P.max_groups) peak = __builtin_inf();   // memory.py:699-704
+  (void)nv;
+  return peak;
+}
+
+// One plan, evaluated by the whole wavefront.  pi: plan index (uniform).
+__device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const uint64_t pi, const ClassView cv,
+                                    uint8_t* lds) {
+  const int lane = threadIdx.x;
+  const rpeg_problem_t& P = *L.P;
+  const int n = (int)cv.h->n_nodes, n_slots = (int)cv.h->n_slots;
+  const int nd = (int)L.ws_nodes;
+  int first_lane = 0;
+  (void)first_lane;
+
+  int16_t* l_plan = (int16_t*)lds;
+  double* l_vm = (double*)(lds + KP_PLAN_I16 * 2);
+  double* l_dur = l_vm + RPEG_MAX_V * 4;
+  double* l_rank = l_dur + L.ws_slots;
+  double* l_start = l_rank + (L.ws_nodes + 1);
+  uint8_t* l_pt = (uint8_t*)(l_start + (L.ws_nodes + 1));
+
+  __syncthreads();   // the previous plan of this wavefront is done with LDS
+  KE_STAMP(0);
+  const PlanHead h = load_head(L.head, L.stride, pi);
+  const rpeg_struct_t& st = P.st[cv.h->structure];
+  const int nv = st.n_vertex;
+  if (lane < KP_PLAN_I16) l_plan[lane] = lane < nv * RPEG_FIELDS ? L.vert[(uint64_t)lane * L.stride + pi] : (int16_t)1;
+  __syncthreads();
+
+  // ---- pair relations: lane 8u+v tests vertices u and v, the ballots are the masks
+  PlanMasks pm;
+  {
+    const int u = lane >> 3, v = lane & 7;
+    const bool valid = u < nv && v < nv;
+    const VPlan au = ke_vplan<1>(l_plan, valid ? u : 0), av = ke_vplan<1>(l_plan, valid ? v : 0);
+    pm.ovl = __ballot(valid && !alloc_disjoint(au, av));
+    pm.eq = 0;   // the memory model below works on position-indexed masks of its own
+    pm.dpne = __ballot(valid && au.dp != av.dp);
+  }
+  KE_STAMP(1);
+
+  // ---- durations of the class's slots, one slot per lane
+  bool err = cv.h->error != 0, zero_div = false;
+  const int split = (int)cv.h->split;
+  for (int s = lane; s < n_slots; s += KE_WAVE) l_dur[s] = ke_slot_duration<1>(P, st, split, cv.slot[s], l_plan, &zero_div);
+  err = err || __ballot(zero_div) != 0ull;
+  KE_STAMP(2);
+
+  // ---- memory model (memory.py:608-841), in the order of first appearance of the vertices among the
+  // lowered operator nodes (position i = vertex vorder[i]): that order fixes the order of the float sums.
+  // One vertex per lane, then one vertex subset per lane tests whether it is a device class (a maximal clique
+  // of the overlap graph); the few that are get evaluated one after the other with uniform control flow.
+  const uint8_t* order = cv.h->vorder;
+  if (lane < nv) {
+    const int v = order[lane];
+    const VMem m = vertex_memory(P, st.vertex[v], ke_vplan<1>(l_plan, v));
+    l_vm[lane * 4 + 0] = (double)m.w_shard;
+    l_vm[lane * 4 + 1] = m.mem_w;
+    l_vm[lane * 4 + 2] = m.opt;
+    l_vm[lane * 4 + 3] = m.extra;
+  }
+  KpOrdered om;
+  {
+    const int i = lane >> 3, j = lane & 7;
+    const bool valid = i < nv && j < nv;
+    const int vi = order[valid ? i : 0], vj = order[valid ? j : 0];
+    const VPlan ai = ke_vplan<1>(l_plan, vi), aj = ke_vplan<1>(l_plan, vj);
+    const rpeg_vertex_t &xi = st.vertex[vi], &xj = st.vertex[vj];
+    om.ovl = __ballot(valid && !alloc_disjoint(ai, aj));
+    om.eq = __ballot(valid && alloc_equal(ai, aj));
+    om.same_model = __ballot(valid && xi.model == xj.model);
+    om.train_same = __ballot(valid && xi.model == xj.model && xj.role == RPEG_ROLE_TRAIN);
+    const unsigned long long t = __ballot(valid && j == 0 && xi.role == RPEG_ROLE_TRAIN),
+                             tr = __ballot(valid && j == 0 && st.trainable[xi.model] != 0);   // bit 8i: position i
+    om.train = om.trainable = 0u;
+#pragma unroll
+    for (int q = 0; q < RPEG_MAX_V; ++q) {
+      om.train |= (unsigned)((t >> (8 * q)) & 1ull) << q;
+      om.trainable |= (unsigned)((tr >> (8 * q)) & 1ull) << q;
+    }
+  }
+  __syncthreads();
+  double peak = -1.0;
+  {
+    const unsigned M = (unsigned)lane + 1u;
+    unsigned long long classes = __ballot(M < (1u << nv) && kp_maximal_clique(nv, om.ovl, M));
+    while (classes) {
+      const unsigned Mu = (unsigned)__builtin_ctzll(classes) + 1u;
+      classes &= classes - 1ull;
+      const double p = kp_class_peak(P, st, order, nv, om, l_vm, Mu);
+      peak = p > peak ? p : peak;
+    }
+  }
+  const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
+  const bool mem_ok = !(peak > P.cap);
+  KE_STAMP(3);
+  unsigned long long* stamp = L.prof && lane == 0 ? L.prof + w * 8 : nullptr;
+
+  // ---- ranks and list scheduling
+  double makespan = 0.0;
+  long pops = 0;
+  if (!err) {
+    bool ok;
+    if (n <= 64) ok = kp_schedule<1>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    else if (n <= 128) ok = kp_schedule<2>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    else if (n <= 192) ok = kp_schedule<3>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    else if (n <= 256) ok = kp_schedule<4>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    else if (n <= 320) ok = kp_schedule<5>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    else ok = kp_schedule<6>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    err = !ok;
+  }
+  KE_STAMP(5);
+  if (L.prof && lane == 0) L.prof[w * 8 + 7] = ((unsigned long long)n << 32) | (unsigned long long)pops;
+
+  // ---- outputs
+  uint8_t mask = RPEG_MASK_VALID;
+  if (stale_ok) mask |= RPEG_MASK_STALE_OK;
+  if (mem_ok) mask |= RPEG_MASK_MEM_OK;
+  double out_makespan, out_score;
+  if (err || makespan == 0.0) {
+    out_makespan = out_score = __builtin_nan("");
+    mask |= RPEG_MASK_ERROR;
+  } else {
+    double score = P.score_num / makespan;
+    if (!mem_ok) score = score * oom_penalty(peak, P.cap);
+    if ((L.flags & RPEG_GATE_STALE) && !stale_ok) score = 0.0;
+    out_makespan = makespan;
+    out_score = score;
+  }
+  double m[RPEG_MAX_V];
+  if (L.mass) {
+    __syncthreads();
+    if (err) {
+#pragma unroll
+      for (int x = 0; x < RPEG_MAX_V; ++x) m[x] = __builtin_nan("");
+    } else {
+      critical_mass(cv, [&](int i) { return l_rank[i]; }, [&](int i) { return l_start[i]; }, m);
+    }
+  }
+  if (lane == 0) {
+    if (L.makespan) L.makespan[pi] = out_makespan;
+    if (L.peak) L.peak[pi] = peak;
+    if (L.score) L.score[pi] = out_score;
+    if (L.mask) L.mask[pi] = mask;
+    if (L.mass) {
+#pragma unroll
+      for (int x = 0; x < RPEG_MAX_V; ++x) L.mass[pi * RPEG_MAX_V + x] = m[x];
+    }
+  }
+  KE_STAMP(6);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace rpeg
+#endif

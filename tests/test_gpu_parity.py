@@ -223,24 +223,24 @@ def test_drop_in_calls():
 @pytest.mark.parametrize("c,n", [(1, 2048), (2, 8192), (5, 1024)])
 def test_every_state_layout_gives_the_same_bits(c, n):
     """Scheduler state in the HBM workspace (64 plans per wavefront) or in LDS (8/16/32/64 plans per
-    wavefront), and the per-batch automatic choice: identical outputs."""
+    wavefront), one plan per wavefront, and the per-batch automatic choice: identical outputs."""
     from rpeg_amd.engine.runtime import Engine, EngineError
     cfg, batch = seeded_batch(c, n)
     eng = Engine(cfg.problem)
     ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
     seen = set()
-    for lanes in (0, 8, 16, 32, 64, -1):
+    for lanes in (0, 1, 8, 16, 32, 64, -1):
         eng.set_state_lanes(lanes)
         try:
             out = eng.eval(batch, gate_stale=True)
         except EngineError as ex:
-            assert lanes > 0 and "does not fit in LDS" in str(ex)   # the largest class is too big for that many plans
+            assert lanes > 1 and "does not fit in LDS" in str(ex)   # the largest class is too big for that many plans
             continue
         seen.add(eng.stats()["state_lanes"])
         assert np.array_equal(out["mask"], ref["mask"]), lanes
         assert same_bits(out["makespan"], ref["makespan"]) and same_bits(out["score"], ref["score"]), lanes
         assert same_bits(out["peak"], ref["peak"]), lanes
-    assert 0 in seen and 8 in seen
+    assert 0 in seen and 1 in seen and 8 in seen
     with pytest.raises(EngineError):
         eng.set_state_lanes(12)
 
