@@ -165,6 +165,17 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
 int rpeg_eval_batch_mass(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
                          double* makespan, double* peak, double* score, uint8_t* mask, double* mass, void* stream);
 
+/* rpeg_eval_batch_mass for plans and results in HOST memory (any of the result pointers may be null).  This
+   is what one step of the reference's search hands to its evaluation pool: a handful of candidate
+   configurations held by the host (RPEG/search/optimizer.py:793-798, the `map` over `_eval_worker`; and
+   every single call of evaluate / evaluate_cached, RPEG/search/evaluate.py:235-403).  For a batch of at most
+   32 plans per compute unit the host computes the lowering class of each plan itself and the call is one
+   copy to the device, one launch (one plan per wavefront) whose results land in pinned host memory, and one
+   wait; larger batches are staged through device memory and take the path of rpeg_eval_batch.  Returns when
+   the results are in place. */
+int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                   double* peak, double* score, uint8_t* mask, double* mass, void* stream);
+
 /* Single-node durations and isolated peaks: the batched form of the candidate-directory loop
    (RPEG/search/moves.py:532-549): for strategy i, time = NodeCostModel.time(mock node) and
    peak = NodeMemoryModel.peak_bytes(mock node) of vertex `vertex` of structure `structure` placed at

@@ -172,7 +172,7 @@ __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(4, 8))) void k_plan(const EvalLaunch L) {
   extern __shared__ uint8_t kp_lds[];
   for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
-    const uint64_t pi = L.perm[w];
+    const uint64_t pi = L.perm ? L.perm[w] : w;
     kp_eval_plan(L, w, pi, class_view(L.pool + L.wave_cls[w]), kp_lds);
   }
 }
@@ -268,7 +268,13 @@ struct rpeg_engine_s {
   size_t d_pool_cap = 0, d_pool_used = 0;
   uint32_t max_nodes = 1, max_slots = 1, max_cls_bytes = 16;
   bool lds_attr_set[5] = {false, false, false, false, false};
-  uint32_t one_plan_waves_per_cu = 32;   // batches of at most this many plans per compute unit take one wavefront per plan
+  // staging of the host-pointer path: plans and class offsets in (pinned, then device), results out (pinned,
+  // written by the kernel itself)
+  uint8_t *hs_in = nullptr, *ds_in = nullptr, *hs_out = nullptr;
+  size_t hs_cap = 0;
+  std::vector<uint32_t> hs_idx;
+  uint32_t one_plan_waves_per_cu = 128;   // batches of at most this many plans per compute unit take one wavefront per plan
+  uint32_t host_small_max = 1024;          // rpeg_eval_host: largest batch whose classes the host looks up itself
   int state_lanes = -1;   // -1: chosen per batch; 0: per-plan state in HBM; 8/16/32/64: in LDS, that many plans per wavefront; 1: one plan per wavefront (k_plan)
   bool prof_on = false;
   unsigned long long* d_prof = nullptr;
@@ -456,6 +462,8 @@ static int ensure_ws(rpeg_engine_t* e, size_t bytes, hipStream_t s) {
 
 static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                            double* peak, double* score, uint8_t* mask, double* mass, void* stream);
+static int eval_host_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                          double* peak, double* score, uint8_t* mask, double* mass, void* stream);
 
 extern "C" {
 
@@ -501,6 +509,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
     hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
   }
   if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_cls); }
+  if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
   if (e->ev1) hipEventDestroy(e->ev1);
@@ -533,7 +542,7 @@ int rpeg_engine_profile(rpeg_engine_t* e, int32_t enable, unsigned long long* ou
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
   if (!e) return -1;
   if (lanes != -1 && lanes != 0 && lanes != 1 && lanes != 8 && lanes != 16 && lanes != 32 && lanes != 64) {
-    e->err = "state lanes must be -1, 0, 8, 16, 32 or 64";
+    e->err = "state lanes must be -1, 0, 1, 8, 16, 32 or 64";
     return -1;
   }
   e->state_lanes = lanes;
@@ -567,6 +576,11 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
 int rpeg_eval_batch_mass(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                          double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
   return eval_batch_impl(e, n, plans, flags, makespan, peak, score, mask, mass, stream);
+}
+
+int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                   double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
+  return eval_host_impl(e, n, plans, flags, makespan, peak, score, mask, mass, stream);
 }
 
 }  // extern "C"
@@ -843,6 +857,179 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
 // host memory into structure-of-arrays device tensors, scored by the batch kernel (with critical-chain
 // masses) and read back in one synchronisation.
 namespace {
+
+constexpr size_t HS_IN_BYTES = (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 + 4 + 4;   // per plan: fields, header, class offset
+constexpr size_t HS_OUT_BYTES = 3 * 8 + (size_t)RPEG_MAX_V * 8 + 8;            // makespan, peak, score, mass, mask (padded)
+
+int ensure_host_stage(rpeg_engine_t* e, size_t n, hipStream_t s) {
+  if (n <= e->hs_cap) return 0;
+  HIP_TRY(e, hipStreamSynchronize(s));
+  if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
+  e->hs_in = e->ds_in = e->hs_out = nullptr;
+  e->hs_cap = 0;
+  const size_t cap = (std::max<size_t>(n + n / 2, 1024) + 63) & ~size_t(63);
+  HIP_TRY(e, hipHostMalloc(&e->hs_in, HS_IN_BYTES * cap));
+  HIP_TRY(e, hipMalloc(&e->ds_in, HS_IN_BYTES * cap));
+  HIP_TRY(e, hipHostMalloc(&e->hs_out, HS_OUT_BYTES * cap));
+  e->hs_cap = cap;
+  return 0;
+}
+
+// Plans in host memory, results to host memory, for a batch small enough for one plan per wavefront: the
+// host computes the class of every plan itself (validity gate, signature, table lookup: ~100 ns per plan),
+// so the call is one copy to the device, one launch of k_plan, whose first lanes write the results straight
+// into pinned host memory, and one wait.  get(i, head, a) yields plan i.  Returns 1 when the batch is not
+// eligible (a class too large for k_plan); the caller then takes the device path.  Output arrays may be null.
+template <class GET>
+int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, double* makespan, double* peak, double* score,
+                    uint8_t* mask, double* mass, hipStream_t s) {
+  e->last_ms = -1.0;
+  if (n == 0) return 0;
+  const size_t stride = ((size_t)n + 63) & ~size_t(63);
+  if (int rc = ensure_host_stage(e, stride, s)) return rc;
+  int16_t* in_vert = (int16_t*)e->hs_in;
+  uint8_t* in_head = e->hs_in + (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 * stride;
+  uint32_t* in_cls = (uint32_t*)(in_head + 4 * stride);
+  e->hs_idx.clear();
+  const double nan = __builtin_nan("");
+  uint64_t n_new = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    PlanHead h;
+    VPlan a[RPEG_MAX_V];
+    get(i, h, a);
+    const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;
+    if (nv == 0 || !plan_valid(e->P, h, a)) {
+      if (makespan) makespan[i] = nan;
+      if (peak) peak[i] = nan;
+      if (score) score[i] = nan;
+      if (mask) mask[i] = 0;
+      if (mass)
+        for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
+      continue;
+    }
+    bool is_new = false;
+    const int64_t off = class_offset(e, plan_signature(e->P, h.structure, h.split, h.tau0, h.tau1, a), &is_new);
+    if (off < 0) return -5;
+    n_new += is_new ? 1 : 0;
+    const size_t j = e->hs_idx.size();
+    e->hs_idx.push_back((uint32_t)i);
+    for (int v = 0; v < nv; ++v) {
+      int16_t* p = in_vert + (size_t)v * RPEG_FIELDS * stride + j;
+      p[0 * stride] = (int16_t)a[v].dp; p[1 * stride] = (int16_t)a[v].pp; p[2 * stride] = (int16_t)a[v].tp; p[3 * stride] = (int16_t)a[v].mb;
+      p[4 * stride] = (int16_t)a[v].o[0]; p[5 * stride] = (int16_t)a[v].o[1]; p[6 * stride] = (int16_t)a[v].o[2];
+      p[7 * stride] = (int16_t)a[v].e[0]; p[8 * stride] = (int16_t)a[v].e[1]; p[9 * stride] = (int16_t)a[v].e[2];
+    }
+    in_head[0 * stride + j] = (uint8_t)h.structure; in_head[1 * stride + j] = (uint8_t)h.split;
+    in_head[2 * stride + j] = (uint8_t)h.tau0; in_head[3 * stride + j] = (uint8_t)h.tau1;
+    in_cls[j] = (uint32_t)off;
+  }
+  const size_t m = e->hs_idx.size();
+  e->stats[0] = 0; e->stats[1] = n_new; e->stats[2] = m; e->stats[3] = 0; e->stats[4] = 0; e->stats[5] = 1;
+  if (m == 0) return 0;
+  if (e->max_nodes > (uint32_t)(WAVE * KP_MAX_NS) || kp_lds_bytes(e->max_nodes, e->max_slots) > 64 * 1024) return 1;
+  if (int rc = ensure_pool(e, s)) return rc;
+  HIP_TRY(e, hipMemcpyAsync(e->ds_in, e->hs_in, HS_IN_BYTES * stride, hipMemcpyHostToDevice, s));
+  double* o_makespan = (double*)e->hs_out;
+  double* o_peak = o_makespan + stride;
+  double* o_score = o_peak + stride;
+  double* o_mass = o_score + stride;
+  uint8_t* o_mask = (uint8_t*)(o_mass + (size_t)RPEG_MAX_V * stride);
+  EvalLaunch L;
+  L.P = e->dP;
+  L.vert = (const int16_t*)e->ds_in;
+  L.head = e->ds_in + (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 * stride;
+  L.stride = stride;
+  L.perm = nullptr;
+  L.wave_cls = (const uint32_t*)(L.head + 4 * stride);
+  L.pool = e->d_pool; L.ws = nullptr;
+  L.n_waves = m; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
+  L.cls_bytes = 0; L.rcap = 0;
+  L.flags = flags; L.makespan = o_makespan; L.peak = o_peak; L.score = o_score; L.mask = o_mask;
+  L.mass = mass ? o_mass : nullptr;
+  L.prof = nullptr;
+  const size_t lds = kp_lds_bytes(e->max_nodes, e->max_slots);
+  const unsigned grid = (unsigned)std::min<uint64_t>(m, (uint64_t)e->n_cu * 32);
+  e->stats[3] = lds;
+  if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
+  hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
+  HIP_TRY(e, hipGetLastError());
+  if (e->timing) HIP_TRY(e, hipEventRecord(e->ev1, s));
+  HIP_TRY(e, hipStreamSynchronize(s));
+  if (e->timing) {
+    float ms = 0.f;
+    HIP_TRY(e, hipEventElapsedTime(&ms, e->ev0, e->ev1));
+    e->last_ms = ms;
+  }
+  for (size_t j = 0; j < m; ++j) {
+    const uint32_t i = e->hs_idx[j];
+    if (makespan) makespan[i] = o_makespan[j];
+    if (peak) peak[i] = o_peak[j];
+    if (score) score[i] = o_score[j];
+    if (mask) mask[i] = o_mask[j];
+    if (mass)
+      for (int x = 0; x < RPEG_MAX_V; ++x) mass[(size_t)i * RPEG_MAX_V + x] = o_mass[j * RPEG_MAX_V + x];
+  }
+  return 0;
+}
+
+}  // namespace
+
+// rpeg_eval_host: plans and results in host memory.  Small batches go through eval_host_small; larger ones
+// (or problems whose classes are too large for it) are copied to the device and take the batch path.
+static int eval_host_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                          double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
+  if (!e || !plans) return -1;
+  e->err.clear();
+  e->last_ms = -1.0;
+  if (n == 0) return 0;
+  if (n >= (1ull << 32)) { e->err = "at most 2^32-1 plans per call"; return -1; }
+  if (!plans->vert || !plans->head || plans->stride < n) { e->err = "bad plan tensors"; return -1; }
+  hipStream_t s = (hipStream_t)stream;
+  const int16_t* vert = plans->vert;
+  const uint8_t* head = plans->head;
+  const uint64_t stride = plans->stride;
+  if (e->state_lanes != 0 && e->state_lanes < 8 && n <= (uint64_t)e->host_small_max) {
+    auto get = [&](uint64_t i, PlanHead& h, VPlan (&a)[RPEG_MAX_V]) {
+      h = load_head(head, stride, i);
+      const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;
+      for (int v = 0; v < nv; ++v) load_vertex(vert, stride, i, v, &a[v]);
+    };
+    const int rc = eval_host_small(e, n, get, flags, makespan, peak, score, mask, mass, s);
+    if (rc <= 0) return rc;
+  }
+  // device path: stage the tensors and the results in device memory for this call
+  const size_t V = (size_t)RPEG_MAX_V * RPEG_FIELDS;
+  uint8_t* d = nullptr;
+  const size_t b_vert = V * 2 * n, b_head = 4 * n, b_f64 = 8 * n;
+  const size_t o_head = (b_vert + 255) & ~size_t(255), o_mk = (o_head + b_head + 255) & ~size_t(255), o_pk = o_mk + b_f64,
+               o_sc = o_pk + b_f64, o_ms = o_sc + b_f64, o_mask = o_ms + (mass ? b_f64 * RPEG_MAX_V : 0), total = o_mask + n;
+  HIP_TRY(e, hipMalloc(&d, total));
+  int rc = 0;
+  auto fail = [&](hipError_t st, const char* what) { e->err = std::string(what) + ": " + hipGetErrorString(st); rc = -2; };
+  hipError_t st = hipMemcpy2DAsync(d, n * 2, vert, stride * 2, n * 2, V, hipMemcpyHostToDevice, s);
+  if (st != hipSuccess) fail(st, "hipMemcpy2DAsync");
+  if (!rc && (st = hipMemcpy2DAsync(d + o_head, n, head, stride, n, 4, hipMemcpyHostToDevice, s)) != hipSuccess) fail(st, "hipMemcpy2DAsync");
+  if (!rc) {
+    rpeg_plan_soa_t soa{(const int16_t*)d, d + o_head, n};
+    rc = eval_batch_impl(e, n, &soa, flags, (double*)(d + o_mk), (double*)(d + o_pk), (double*)(d + o_sc), d + o_mask,
+                         mass ? (double*)(d + o_ms) : nullptr, stream);
+  }
+  const double last_ms = e->last_ms;
+  auto back = [&](void* dst, size_t off, size_t bytes) {
+    if (rc || !dst) return;
+    const hipError_t c = hipMemcpyAsync(dst, d + off, bytes, hipMemcpyDeviceToHost, s);
+    if (c != hipSuccess) fail(c, "hipMemcpyAsync");
+  };
+  back(makespan, o_mk, b_f64); back(peak, o_pk, b_f64); back(score, o_sc, b_f64); back(mask, o_mask, n);
+  back(mass, o_ms, b_f64 * RPEG_MAX_V);
+  const hipError_t sy = hipStreamSynchronize(s);
+  if (!rc && sy != hipSuccess) fail(sy, "hipStreamSynchronize");
+  hipFree(d);
+  e->last_ms = last_ms;
+  return rc;
+}
+
+namespace {
 struct GpuSaBackend : SaBackend {
   rpeg_engine_t* e;
   hipStream_t s;
@@ -882,6 +1069,33 @@ struct GpuSaBackend : SaBackend {
 
   int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override {
     if (n > cap) { e->err = "annealing batch exceeds its buffers"; return -1; }
+    {  // a step's proposals are a small batch: one copy, one launch (eval_host_small)
+      const auto t0 = std::chrono::steady_clock::now();
+      auto get = [&](uint64_t i, PlanHead& h, VPlan (&a)[RPEG_MAX_V]) {
+        const uint8_t* hd = head_of[variant[i]];
+        h.structure = hd[0]; h.split = hd[1]; h.tau0 = hd[2]; h.tau1 = hd[3];
+        const int nv = e->P.st[hd[0]].n_vertex;
+        for (int v = 0; v < nv; ++v) {
+          const int16_t* f = plans[i].f[v];
+          a[v].dp = f[0]; a[v].pp = f[1]; a[v].tp = f[2]; a[v].mb = f[3];
+          a[v].o[0] = f[4]; a[v].o[1] = f[5]; a[v].o[2] = f[6];
+          a[v].e[0] = f[7]; a[v].e[1] = f[8]; a[v].e[2] = f[9];
+        }
+      };
+      const int rc = eval_host_small(e, (uint64_t)n, get, 0u, nullptr, nullptr, h_score, h_mask, h_mass, s);
+      if (rc < 0) return rc;
+      if (rc == 0) {
+        for (int i = 0; i < n; ++i) {
+          out[i].score = h_score[i];
+          out[i].mask = h_mask[i];
+          for (int x = 0; x < RPEG_MAX_V; ++x) out[i].mass[x] = h_mass[(size_t)i * RPEG_MAX_V + x];
+        }
+        eval_s += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        ++n_launch;
+        n_plans += n;
+        return 0;
+      }
+    }
     const auto t0 = std::chrono::steady_clock::now();
     const size_t V = RPEG_MAX_V * RPEG_FIELDS;
     for (int i = 0; i < n; ++i) {

@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize")
+           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host")
 
 
 class EngineError(RuntimeError):
@@ -50,6 +50,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_eval_batch.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp]
     lib.rpeg_eval_batch_mass.restype = C.c_int
     lib.rpeg_eval_batch_mass.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp, vp]
+    lib.rpeg_eval_host.restype = C.c_int
+    lib.rpeg_eval_host.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp, vp]
     lib.rpeg_sa_run.restype = C.c_int
     lib.rpeg_sa_run.argtypes = [vp, vp, vp, vp, vp]
     lib.rpeg_sa_optimize.restype = C.c_int
@@ -196,14 +198,32 @@ class Engine:
         self._check(rc, "rpeg_eval_batch")
         return out
 
-    def eval(self, batch: PlanBatch, gate_stale: bool = True) -> Dict[str, np.ndarray]:
-        """Host convenience: upload, evaluate, download."""
-        out = self.eval_device(DeviceBatch(batch, self.device), gate_stale=gate_stale)
-        _torch().cuda.synchronize(self.device)
-        return {k: v.cpu().numpy() for k, v in out.items()}
+    def eval(self, batch: PlanBatch, gate_stale: bool = True, mass: bool = False) -> Dict[str, np.ndarray]:
+        """Plans and results in host memory (rpeg_eval_host): a batch of up to a few thousand plans is one
+        copy, one launch and one wait; larger ones are staged through device memory by the library."""
+        torch = _torch()
+        n = batch.n
+        vert = np.ascontiguousarray(batch.vert, dtype=np.int16)
+        head = np.ascontiguousarray(batch.head, dtype=np.uint8)
+        soa = abi.PlanSoaT(vert.ctypes.data, head.ctypes.data, vert.shape[1])
+        out = dict(makespan=np.empty(n, np.float64), peak=np.empty(n, np.float64), score=np.empty(n, np.float64),
+                   mask=np.empty(n, np.uint8))
+        if mass:
+            out["mass"] = np.empty((n, abi.MAX_V), np.float64)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_eval_host(self._h, n, C.addressof(soa), abi.GATE_STALE if gate_stale else 0,
+                                         out["makespan"].ctypes.data, out["peak"].ctypes.data, out["score"].ctypes.data,
+                                         out["mask"].ctypes.data, out["mass"].ctypes.data if mass else None, stream)
+        self._check(rc, "rpeg_eval_host")
+        return out
 
     def eval_mass(self, batch: PlanBatch, gate_stale: bool = False) -> Dict[str, np.ndarray]:
         """`eval` plus the critical-chain mass per template vertex, float64 [n, MAX_V]."""
+        return self.eval(batch, gate_stale=gate_stale, mass=True)
+
+    def eval_mass_device(self, batch: PlanBatch, gate_stale: bool = False) -> Dict[str, np.ndarray]:
+        """The same through device tensors (rpeg_eval_batch_mass)."""
         torch = _torch()
         db = DeviceBatch(batch, self.device)
         out = self.alloc_outputs(db.n)
@@ -216,6 +236,12 @@ class Engine:
                                                out["mass"].data_ptr(), stream)
         self._check(rc, "rpeg_eval_batch_mass")
         torch.cuda.synchronize(self.device)
+        return {k: v.cpu().numpy() for k, v in out.items()}
+
+    def eval_resident(self, batch: PlanBatch, gate_stale: bool = True) -> Dict[str, np.ndarray]:
+        """Upload with torch, evaluate device tensors (rpeg_eval_batch), download."""
+        out = self.eval_device(DeviceBatch(batch, self.device), gate_stale=gate_stale)
+        _torch().cuda.synchronize(self.device)
         return {k: v.cpu().numpy() for k, v in out.items()}
 
     def sa_run(self, params: "abi.SaParamsT", directory, base_plan: Optional[np.ndarray] = None) -> Dict[str, object]:

@@ -245,6 +245,23 @@ def test_every_state_layout_gives_the_same_bits(c, n):
         eng.set_state_lanes(12)
 
 
+@pytest.mark.parametrize("c,n", [(1, 1500), (2, 3000), (2, 20000), (3, 600), (4, 5000)])
+def test_host_and_device_entry_points_agree(c, n):
+    """rpeg_eval_host (plans and results in host memory; one plan per wavefront for small batches, staged
+    through device memory for larger ones and for classes too large for that kernel), rpeg_eval_batch and
+    rpeg_eval_batch_mass on device tensors: identical outputs, equal to the host build."""
+    cfg, batch = seeded_batch(c, n)
+    eng = engine(c)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16, want_mass=True)
+    for out in (eng.eval(batch, gate_stale=True, mass=True), eng.eval_mass_device(batch, gate_stale=True),
+                eng.eval_resident(batch, gate_stale=True)):
+        assert np.array_equal(out["mask"], ref["mask"])
+        for k in ("makespan", "peak", "score"):
+            assert same_bits(out[k], ref[k]), k
+        if "mass" in out:
+            assert same_bits(out["mass"], ref["mass"])
+
+
 def test_small_batches_pick_the_latency_layout():
     cfg, batch = seeded_batch(2, 512)
     eng = engine(2)
