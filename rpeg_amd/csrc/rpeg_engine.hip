@@ -155,8 +155,9 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
   if (i >= n) return;
   const uint32_t c = cid[i];
   if (c >= CID_UNKNOWN) return;
-  const uint32_t k = kidx[i], l = clpw[c];
-  perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
+  const uint32_t k = kidx[i], l = clpw[c] & 0xFFFFu;
+  if (clpw[c] >> 16) perm[(uint64_t)cfirst[c] + k] = (uint32_t)i;   // a class of single-plan wavefronts: cfirst is its first entry
+  else perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
 }
 
 template <int LS>
@@ -280,7 +281,10 @@ struct rpeg_engine_s {
   unsigned long long* d_prof = nullptr;
   uint64_t prof_waves = 0;
   // per-batch buffers
-  size_t cap_n = 0, cap_perm = 0;
+  size_t cap_n = 0, cap_perm = 0, cap_cls = 0;
+  hipStream_t s2 = nullptr;                     // second stream: single-plan wavefronts of a large batch run beside the others
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  int split_heavy = 1;                          // 0: the classes with the largest graphs stay in the main kernel
   uint64_t* d_sig = nullptr;
   uint64_t* h_sig = nullptr;
   uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_cls = nullptr;   // lane -> plan; wavefront -> class blob
@@ -351,15 +355,24 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
 }
 
 // permutation (one entry per lane, classes padded to wavefronts) and class offset per wavefront
-static int ensure_perm(rpeg_engine_t* e, size_t lanes) {
-  if (lanes <= e->cap_perm) return 0;
-  size_t cap = std::max<size_t>(lanes + lanes / 4, 8192);
-  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_cls); }
-  e->cap_perm = 0;
-  HIP_TRY(e, hipMalloc(&e->d_perm, cap * 4));
-  HIP_TRY(e, hipMalloc(&e->d_cls, (cap / WAVE + 1) * 4));
-  HIP_TRY(e, hipHostMalloc(&e->h_cls, (cap / WAVE + 1) * 4));
-  e->cap_perm = cap;
+static int ensure_perm(rpeg_engine_t* e, size_t lanes, size_t tasks) {
+  if (lanes > e->cap_perm) {
+    size_t cap = std::max<size_t>(lanes + lanes / 4, 8192);
+    if (e->d_perm) hipFree(e->d_perm);
+    e->d_perm = nullptr;
+    e->cap_perm = 0;
+    HIP_TRY(e, hipMalloc(&e->d_perm, cap * 4));
+    e->cap_perm = cap;
+  }
+  if (tasks > e->cap_cls) {
+    size_t cap = std::max<size_t>(tasks + tasks / 4, 1024);
+    if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
+    e->d_cls = e->h_cls = nullptr;
+    e->cap_cls = 0;
+    HIP_TRY(e, hipMalloc(&e->d_cls, cap * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_cls, cap * 4));
+    e->cap_cls = cap;
+  }
   return 0;
 }
 
@@ -487,6 +500,7 @@ int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
   hipGetDevice(&e->device);
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, e->device) == hipSuccess) e->n_cu = prop.multiProcessorCount;
+
   if (hipMalloc(&e->dP, sizeof(rpeg_problem_t)) != hipSuccess ||
       hipMemcpy(e->dP, problem, sizeof(rpeg_problem_t), hipMemcpyHostToDevice) != hipSuccess ||
       hipEventCreate(&e->ev0) != hipSuccess || hipEventCreate(&e->ev1) != hipSuccess) {
@@ -508,7 +522,9 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
     hipFree(e->d_ccount); hipFree(e->d_cfirst); hipFree(e->d_clpw);
     hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
   }
-  if (e->d_perm) { hipFree(e->d_perm); hipFree(e->d_cls); hipHostFree(e->h_cls); }
+  if (e->d_perm) hipFree(e->d_perm);
+  if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
+  if (e->s2) { hipStreamDestroy(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
   if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
@@ -668,35 +684,66 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
     return ((const ClassHdr*)(e->pool.data() + offs[a]))->n_nodes > ((const ClassHdr*)(e->pool.data() + offs[b]))->n_nodes;
   });
-  // start[k]: first wavefront of the k-th class in launch order
-  std::vector<uint32_t> start(counts.size() + 1, 0), first(counts.size(), 0), clpw(counts.size(), lpw);
+  // first[c]: first wavefront of class c in launch order (first permutation entry for a class of
+  // single-plan wavefronts, which follow the others in the permutation and in the task list)
+  std::vector<uint32_t> first(counts.size(), 0), clpw(counts.size(), lpw);
+  std::vector<uint8_t> solo(counts.size(), 0);
   if (!ls && !one && !order.empty()) {
     // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
-    // classes with the largest graphs (at least seven tenths of the largest) get eight plans per wavefront, so
-    // that fewer plans wait for the slowest one, unless they are a large share of the batch or the batch
-    // is many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest).
+    // classes with the largest graphs (up to a quarter of the batch) are taken out of it, unless the batch is
+    // many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest): their plans
+    // get a wavefront each (k_plan, on a second stream, filling the registers and LDS the main kernel leaves
+    // free; graphs of at least six tenths of the largest node count) or, where that kernel does not fit,
+    // eight plans per wavefront (at least seven tenths).
     const uint32_t heavy_lpw = (uint32_t)KE_FEW;
-    const uint64_t hfrac = 7ull;   // tenths of the largest node count
+    const bool one_fits = e->max_nodes <= (uint32_t)(WAVE * KP_MAX_NS) && kp_lds_bytes(e->max_nodes, e->max_slots) <= 64 * 1024;
+    const bool split = e->split_heavy && one_fits;
+    // node count from which a class counts as large: the smallest one, not under `floor` percent of the
+    // largest, such that the large classes hold at most `share` percent of the batch
+    const uint64_t floor_pct = split ? 60ull : 70ull, share_pct = 25ull;
     const uint32_t top = e->cls_nodes[cids[order[0]]];
-    uint64_t heavy_plans = 0;
-    for (size_t c = 0; c < counts.size(); ++c)
-      if (10ull * e->cls_nodes[cids[c]] >= hfrac * top) heavy_plans += counts[c];
     uint64_t waves64 = 0;
     for (uint32_t c : counts) waves64 += (c + WAVE - 1) / WAVE;
-    if (heavy_plans * 4 <= n && waves64 <= (uint64_t)e->n_cu * 16 && heavy_lpw >= 1 && heavy_lpw <= WAVE)
+    uint32_t cut = 0xFFFFFFFFu;   // classes of at least `cut` nodes are large
+    uint64_t heavy_plans = 0;
+    for (size_t k = 0; k < order.size();) {
+      const uint32_t nodes = e->cls_nodes[cids[order[k]]];
+      if (100ull * nodes < floor_pct * top) break;
+      uint64_t group = 0;
+      size_t k2 = k;
+      for (; k2 < order.size() && e->cls_nodes[cids[order[k2]]] == nodes; ++k2) group += counts[order[k2]];
+      if ((heavy_plans + group) * 100 > (uint64_t)n * share_pct) break;
+      heavy_plans += group;
+      cut = nodes;
+      k = k2;
+    }
+    if (waves64 <= (uint64_t)e->n_cu * 16 && heavy_lpw >= 1 && heavy_lpw <= WAVE)
       for (size_t c = 0; c < counts.size(); ++c)
-        if (10ull * e->cls_nodes[cids[c]] >= hfrac * top) clpw[c] = heavy_lpw;
+        if (e->cls_nodes[cids[c]] >= cut) {
+          if (split) solo[c] = 1;
+          else clpw[c] = heavy_lpw;
+        }
   }
+  uint32_t n_eval_waves = 0, n_solo = 0;
   for (size_t k = 0; k < order.size(); ++k) {
-    first[order[k]] = start[k];
-    start[k + 1] = start[k] + (counts[order[k]] + clpw[order[k]] - 1) / clpw[order[k]];
+    const uint32_t c = order[k];
+    if (solo[c]) continue;
+    first[c] = n_eval_waves;
+    n_eval_waves += (counts[c] + clpw[c] - 1) / clpw[c];
   }
   const uint32_t pstride = one ? 1u : (uint32_t)WAVE;
-  const uint64_t n_sorted = (uint64_t)start.back() * WAVE;
+  const uint64_t n_sorted = (uint64_t)n_eval_waves * pstride;   // permutation entries of the main kernel
+  for (size_t k = 0; k < order.size(); ++k) {
+    const uint32_t c = order[k];
+    if (!solo[c]) continue;
+    first[c] = (uint32_t)n_sorted + n_solo;
+    clpw[c] = 1u | (1u << 16);
+    n_solo += counts[c];
+  }
   e->stats[0] = counts.size();
   e->stats[1] = n_new;
-  if (n_sorted == 0) return 0;
-  if (int rc = ensure_perm(e, n_sorted)) return rc;
+  if (n_sorted + n_solo == 0) return 0;
+  if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_eval_waves + n_solo)) return rc;
   for (size_t c = 0; c < counts.size(); ++c) {
     e->h_cfirst[cids[c]] = first[c];
     e->h_clpw[cids[c]] = clpw[c];
@@ -706,20 +753,27 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   const bool few_in_lds = !ls && !one &&
       ke_lds_bytes(0, 32, KE_FEW, e->max_nodes, e->max_slots) <= ke_lds_bytes(0, 32, 0, e->max_nodes, e->max_slots);
   for (size_t k = 0; k < order.size(); ++k) {
-    const uint32_t flag = few_in_lds && clpw[order[k]] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
-    for (uint32_t w = start[k]; w < start[k + 1]; ++w) e->h_cls[w] = offs[order[k]] | flag;
+    const uint32_t c = order[k];
+    if (solo[c]) {
+      const uint32_t t0 = n_eval_waves + (first[c] - (uint32_t)n_sorted);
+      for (uint32_t t = 0; t < counts[c]; ++t) e->h_cls[t0 + t] = offs[c];
+    } else {
+      const uint32_t flag = few_in_lds && clpw[c] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
+      const uint32_t nw = (counts[c] + clpw[c] - 1) / clpw[c];
+      for (uint32_t t = 0; t < nw; ++t) e->h_cls[first[c] + t] = offs[c] | flag;
+    }
   }
   if (int rc = ensure_pool(e, s)) return rc;
   HIP_TRY(e, hipMemcpyAsync(e->d_cfirst, e->h_cfirst, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_clpw, e->h_clpw, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
-  HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, n_sorted / WAVE * 4, hipMemcpyHostToDevice, s));
-  if (!one)   // with one plan per wavefront every entry is written by the scatter
+  HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, ((size_t)n_eval_waves + n_solo) * 4, hipMemcpyHostToDevice, s));
+  if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
   hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_perm, pstride);
   HIP_TRY(e, hipGetLastError());
 
-  const uint64_t n_waves = n_sorted / WAVE;
-  const unsigned grid = (unsigned)std::min<uint64_t>(n_waves, (uint64_t)e->n_cu * (one ? 32 : 16));
+  const uint64_t n_waves = n_eval_waves;
+  const unsigned grid = (unsigned)std::min<uint64_t>(std::max<uint64_t>(n_waves, 1), (uint64_t)e->n_cu * (one ? 32 : 16));
   const size_t wsb = ls || one ? 0 : ke_ws_bytes(e->max_nodes, e->max_slots);
   if (!ls && !one)
     if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
@@ -737,13 +791,13 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.prof = nullptr;
   if (e->prof_on) {
     if (e->d_prof) hipFree(e->d_prof);
-    HIP_TRY(e, hipMalloc(&e->d_prof, n_waves * 64));
-    HIP_TRY(e, hipMemsetAsync(e->d_prof, 0, n_waves * 64, s));
-    e->prof_waves = n_waves;
+    HIP_TRY(e, hipMalloc(&e->d_prof, (n_waves + n_solo) * 64));
+    HIP_TRY(e, hipMemsetAsync(e->d_prof, 0, (n_waves + n_solo) * 64, s));
+    e->prof_waves = n_waves + n_solo;
     L.prof = e->d_prof;
   }
   const size_t lds = one ? kp_lds_bytes(e->max_nodes, e->max_slots)
-                         : ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots);
+                   : ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots);
   if (lds > 160 * 1024) { e->err = "class tables exceed the LDS"; return -8; }
   const void* kfn = ls == 0 ? (const void*)k_eval<0> : ls == 8 ? (const void*)k_eval<8> : ls == 16 ? (const void*)k_eval<16>
                   : ls == 32 ? (const void*)k_eval<32> : (const void*)k_eval<64>;
@@ -752,12 +806,23 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     HIP_TRY(e, hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     e->lds_attr_set[ki] = true;
   }
-  e->stats[2] = n_waves;
+  e->stats[2] = n_waves + n_solo;
   e->stats[3] = lds;
   e->stats[4] = wsb * grid;
   e->stats[5] = one ? 1u : (uint64_t)ls;
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
-  if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
+  // The main kernel is submitted first: it needs 26 KB of LDS per wavefront, and once single-plan wavefronts
+  // fill a compute unit its wavefronts only fit in as those retire.
+  if (n_solo) {
+    if (!e->s2) {
+      HIP_TRY(e, hipStreamCreateWithFlags(&e->s2, hipStreamNonBlocking));
+      HIP_TRY(e, hipEventCreateWithFlags(&e->ev_fork, hipEventDisableTiming));
+      HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join, hipEventDisableTiming));
+    }
+    HIP_TRY(e, hipEventRecord(e->ev_fork, s));
+  }
+  if (n_waves == 0) {
+  } else if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
   else switch (ls) {
     case 0: hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds, s, L); break;
     case 8: hipLaunchKernelGGL(k_eval<8>, dim3(grid), dim3(WAVE), lds, s, L); break;
@@ -766,6 +831,19 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     default: hipLaunchKernelGGL(k_eval<64>, dim3(grid), dim3(WAVE), lds, s, L); break;
   }
   HIP_TRY(e, hipGetLastError());
+  if (n_solo) {   // the single-plan wavefronts, beside the main kernel
+    EvalLaunch S = L;
+    S.perm = e->d_perm + n_sorted;
+    S.wave_cls = e->d_cls + n_eval_waves;
+    S.n_waves = n_solo;
+    if (L.prof) S.prof = L.prof + n_waves * 8;
+    HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
+    hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n_solo, (uint64_t)e->n_cu * 32)), dim3(WAVE),
+                       kp_lds_bytes(e->max_nodes, e->max_slots), e->s2, S);
+    HIP_TRY(e, hipGetLastError());
+    HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
+  }
+  if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
   if (e->timing) {
     HIP_TRY(e, hipEventRecord(e->ev1, s));
     HIP_TRY(e, hipEventSynchronize(e->ev1));
@@ -814,7 +892,7 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   if (off < 0) return -5;
   hipStream_t s = nullptr;
   if (int rc = ensure_pool(e, s)) return rc;
-  if (int rc = ensure_perm(e, WAVE)) return rc;
+  if (int rc = ensure_perm(e, WAVE, 1)) return rc;
   if (int rc = ensure_ws(e, wave_ws_bytes(e->max_nodes, e->max_slots), s)) return rc;
   int16_t* d_vert = nullptr;
   uint8_t* d_head = nullptr;
