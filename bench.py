@@ -22,9 +22,10 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 FP64_PEAK_TFLOPS = 78.6     # MI355X vector FP64, published
 # algorithmic bytes per plan: int16 plan fields (10 per vertex) + 4 header bytes in, 3 doubles + 1 mask byte out
 ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
-# HBM bytes per launch of k_eval measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB
-# copy (profiles/k_eval_cfg2_grpo_65536.md); None where no counter run exists
-MEASURED_TRAFFIC = {2: 718.6e6}
+# HBM bytes per step of the evaluation kernels measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# a 256 MiB copy (the counter summary of this workload is committed under profiles/); None where no counter
+# run exists
+MEASURED_TRAFFIC = {2: 830.2e6}
 # algorithmic fp64 operations per plan (cost model + scheduler + memory model of the fully split DAG)
 ALG_FLOPS = {1: 3.7e3, 2: 2.5e3, 3: 6.0e3, 4: 0.83e3, 5: 3.7e3}
 
@@ -185,7 +186,8 @@ def main():
     torch.cuda.synchronize()
     cold_ms = (time.perf_counter() - t0) / cold_steps * 1e3
 
-    # dominant kernel (k_eval) duration: HIP events on the launch stream, recorded by the library
+    # duration of the evaluation launch (k_eval, k_plan, or both side by side from fork to join): HIP events on
+    # the launch stream, recorded by the library
     eng.set_timing(True)
     k_ms = []
     for _ in range(args.steps):
@@ -232,6 +234,14 @@ def main():
     score = out["score"].cpu().numpy()
     valid = (mask & abi.MASK_VALID) != 0
     alg_bytes = ALG_BYTES[c] * n
+    # what the timed launch consists of: one plan per wavefront for a batch that would not fill the chip
+    # otherwise; else the throughput kernel, for mid-size batches with the largest graphs on a second stream
+    if stats["state_lanes"] == 1:
+        kernel_name = "k_plan"
+    elif stats["single_plan_tasks"]:
+        kernel_name = f"k_eval<0> beside k_plan ({stats['single_plan_tasks']} plans), one launch each, timed from fork to join"
+    else:
+        kernel_name = f"k_eval<{stats['state_lanes']}>"
     achieved_gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
     achieved_tflops = ALG_FLOPS[c] * n / (kernel_ms * 1e-3) / 1e12
     line = {
@@ -244,7 +254,7 @@ def main():
                    "classes": stats["classes"], "inputs": "resident in HBM", "outputs": "left in HBM"},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(c),
-                     "kernel": "k_eval", "kernel_ms": kernel_ms, "algorithmic_bytes_per_plan": ALG_BYTES[c]},
+                     "kernel": kernel_name, "kernel_ms": kernel_ms, "algorithmic_bytes_per_plan": ALG_BYTES[c]},
         "fp64_valu": {"achieved": achieved_tflops, "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
                       "frac": achieved_tflops / FP64_PEAK_TFLOPS, "algorithmic_flops_per_plan": ALG_FLOPS[c]},
         "kernel_only_evals_per_s": n / (kernel_ms * 1e-3),

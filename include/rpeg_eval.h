@@ -268,7 +268,8 @@ int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* params, int32_t E
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,
    [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace; 1: one plan per
-   wavefront). */
+   wavefront), [6] plans of a large batch that ran one per wavefront beside the main kernel (included
+   in [2]). */
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
 
 /* Where the evaluation kernel keeps the scheduler state of a plan (ready time, rank and remaining

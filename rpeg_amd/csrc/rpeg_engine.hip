@@ -272,6 +272,10 @@ struct rpeg_engine_s {
   // staging of the host-pointer path: plans and class offsets in (pinned, then device), results out (pinned,
   // written by the kernel itself)
   uint8_t *hs_in = nullptr, *ds_in = nullptr, *hs_out = nullptr;
+  uint8_t* d_stage = nullptr;   // device copy of host tensors and results for larger host-pointer batches
+  size_t d_stage_cap = 0;
+  uint8_t* h_stage = nullptr;   // pinned mirror of the result region of d_stage
+  size_t h_stage_cap = 0;
   size_t hs_cap = 0;
   std::vector<uint32_t> hs_idx;
   uint32_t one_plan_waves_per_cu = 128;   // batches of at most this many plans per compute unit take one wavefront per plan
@@ -294,7 +298,7 @@ struct rpeg_engine_s {
   bool timing = false;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   double last_ms = -1.0;
-  uint64_t stats[6] = {0, 0, 0, 0, 0, 0};
+  uint64_t stats[7] = {0, 0, 0, 0, 0, 0, 0};
   int n_cu = 256;
 };
 
@@ -526,6 +530,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
   if (e->s2) { hipStreamDestroy(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
   if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
+  if (e->d_stage) hipFree(e->d_stage);
+  if (e->h_stage) hipHostFree(e->h_stage);
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
   if (e->ev1) hipEventDestroy(e->ev1);
@@ -580,7 +586,7 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
 
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n) {
   if (!e || !out) return -1;
-  for (int i = 0; i < n && i < 6; ++i) out[i] = e->stats[i];
+  for (int i = 0; i < n && i < 7; ++i) out[i] = e->stats[i];
   return 0;
 }
 
@@ -742,6 +748,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   e->stats[0] = counts.size();
   e->stats[1] = n_new;
+  e->stats[6] = 0;
   if (n_sorted + n_solo == 0) return 0;
   if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_eval_waves + n_solo)) return rc;
   for (size_t c = 0; c < counts.size(); ++c) {
@@ -810,6 +817,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   e->stats[3] = lds;
   e->stats[4] = wsb * grid;
   e->stats[5] = one ? 1u : (uint64_t)ls;
+  e->stats[6] = n_solo;
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
   // The main kernel is submitted first: it needs 26 KB of LDS per wavefront, and once single-plan wavefronts
   // fill a compute unit its wavefronts only fit in as those retire.
@@ -1002,7 +1010,7 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
     in_cls[j] = (uint32_t)off;
   }
   const size_t m = e->hs_idx.size();
-  e->stats[0] = 0; e->stats[1] = n_new; e->stats[2] = m; e->stats[3] = 0; e->stats[4] = 0; e->stats[5] = 1;
+  e->stats[0] = 0; e->stats[1] = n_new; e->stats[2] = m; e->stats[3] = 0; e->stats[4] = 0; e->stats[5] = 1; e->stats[6] = 0;
   if (m == 0) return 0;
   if (e->max_nodes > (uint32_t)(WAVE * KP_MAX_NS) || kp_lds_bytes(e->max_nodes, e->max_slots) > 64 * 1024) return 1;
   if (int rc = ensure_pool(e, s)) return rc;
@@ -1077,32 +1085,55 @@ static int eval_host_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* p
   }
   // device path: stage the tensors and the results in device memory for this call
   const size_t V = (size_t)RPEG_MAX_V * RPEG_FIELDS;
-  uint8_t* d = nullptr;
   const size_t b_vert = V * 2 * n, b_head = 4 * n, b_f64 = 8 * n;
   const size_t o_head = (b_vert + 255) & ~size_t(255), o_mk = (o_head + b_head + 255) & ~size_t(255), o_pk = o_mk + b_f64,
                o_sc = o_pk + b_f64, o_ms = o_sc + b_f64, o_mask = o_ms + (mass ? b_f64 * RPEG_MAX_V : 0), total = o_mask + n;
-  HIP_TRY(e, hipMalloc(&d, total));
+  if (total > e->d_stage_cap) {   // grow-only staging block, kept by the engine
+    HIP_TRY(e, hipStreamSynchronize(s));
+    if (e->d_stage) hipFree(e->d_stage);
+    e->d_stage = nullptr;
+    e->d_stage_cap = 0;
+    HIP_TRY(e, hipMalloc(&e->d_stage, total + total / 4));
+    e->d_stage_cap = total + total / 4;
+  }
+  uint8_t* d = e->d_stage;
   int rc = 0;
   auto fail = [&](hipError_t st, const char* what) { e->err = std::string(what) + ": " + hipGetErrorString(st); rc = -2; };
-  hipError_t st = hipMemcpy2DAsync(d, n * 2, vert, stride * 2, n * 2, V, hipMemcpyHostToDevice, s);
-  if (st != hipSuccess) fail(st, "hipMemcpy2DAsync");
-  if (!rc && (st = hipMemcpy2DAsync(d + o_head, n, head, stride, n, 4, hipMemcpyHostToDevice, s)) != hipSuccess) fail(st, "hipMemcpy2DAsync");
+  // results come back in one copy into a pinned mirror of the output region
+  const size_t b_out = total - o_mk;
+  if (b_out > e->h_stage_cap) {
+    HIP_TRY(e, hipStreamSynchronize(s));
+    if (e->h_stage) hipHostFree(e->h_stage);
+    e->h_stage = nullptr;
+    e->h_stage_cap = 0;
+    HIP_TRY(e, hipHostMalloc(&e->h_stage, b_out + b_out / 4));
+    e->h_stage_cap = b_out + b_out / 4;
+  }
+  hipError_t st = stride == n ? hipMemcpyAsync(d, vert, b_vert, hipMemcpyHostToDevice, s)
+                              : hipMemcpy2DAsync(d, n * 2, vert, stride * 2, n * 2, V, hipMemcpyHostToDevice, s);
+  if (st != hipSuccess) fail(st, "hipMemcpyAsync");
+  if (!rc) {
+    st = stride == n ? hipMemcpyAsync(d + o_head, head, b_head, hipMemcpyHostToDevice, s)
+                     : hipMemcpy2DAsync(d + o_head, n, head, stride, n, 4, hipMemcpyHostToDevice, s);
+    if (st != hipSuccess) fail(st, "hipMemcpyAsync");
+  }
   if (!rc) {
     rpeg_plan_soa_t soa{(const int16_t*)d, d + o_head, n};
     rc = eval_batch_impl(e, n, &soa, flags, (double*)(d + o_mk), (double*)(d + o_pk), (double*)(d + o_sc), d + o_mask,
                          mass ? (double*)(d + o_ms) : nullptr, stream);
   }
   const double last_ms = e->last_ms;
-  auto back = [&](void* dst, size_t off, size_t bytes) {
-    if (rc || !dst) return;
-    const hipError_t c = hipMemcpyAsync(dst, d + off, bytes, hipMemcpyDeviceToHost, s);
-    if (c != hipSuccess) fail(c, "hipMemcpyAsync");
-  };
-  back(makespan, o_mk, b_f64); back(peak, o_pk, b_f64); back(score, o_sc, b_f64); back(mask, o_mask, n);
-  back(mass, o_ms, b_f64 * RPEG_MAX_V);
+  if (!rc && (st = hipMemcpyAsync(e->h_stage, d + o_mk, b_out, hipMemcpyDeviceToHost, s)) != hipSuccess) fail(st, "hipMemcpyAsync");
   const hipError_t sy = hipStreamSynchronize(s);
   if (!rc && sy != hipSuccess) fail(sy, "hipStreamSynchronize");
-  hipFree(d);
+  if (!rc) {
+    const uint8_t* h = e->h_stage - o_mk;   // same offsets as in the device block
+    if (makespan) std::memcpy(makespan, h + o_mk, b_f64);
+    if (peak) std::memcpy(peak, h + o_pk, b_f64);
+    if (score) std::memcpy(score, h + o_sc, b_f64);
+    if (mass) std::memcpy(mass, h + o_ms, b_f64 * RPEG_MAX_V);
+    if (mask) std::memcpy(mask, h + o_mask, n);
+  }
   e->last_ms = last_ms;
   return rc;
 }

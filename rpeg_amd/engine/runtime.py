@@ -172,10 +172,10 @@ class Engine:
         return float(self.lib.rpeg_engine_last_kernel_ms(self._h))
 
     def stats(self) -> Dict[str, int]:
-        buf = (C.c_uint64 * 6)()
-        self.lib.rpeg_engine_stats(self._h, buf, 6)
+        buf = (C.c_uint64 * 7)()
+        self.lib.rpeg_engine_stats(self._h, buf, 7)
         return dict(classes=buf[0], classes_lowered=buf[1], wave_tasks=buf[2], lds_bytes=buf[3], workspace_bytes=buf[4],
-                    state_lanes=buf[5])
+                    state_lanes=buf[5], single_plan_tasks=buf[6])
 
     def alloc_outputs(self, n: int):
         torch = _torch()
