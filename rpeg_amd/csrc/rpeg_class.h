@@ -24,7 +24,9 @@ namespace rpeg {
 constexpr int SIG_REL_SHIFT = 9;
 constexpr uint64_t SIG_INVALID = ~0ull;
 
-RPEG_HD uint64_t plan_signature(const rpeg_problem_t& P, int s, int split, int tau0, int tau1, const VPlan* a) {
+// `a[v]` yields the plan fields of vertex v (an array of VPlan, or an accessor returning VPlan by value).
+template <class PLANS>
+RPEG_HD uint64_t plan_signature(const rpeg_problem_t& P, int s, int split, int tau0, int tau1, const PLANS& a) {
   const rpeg_struct_t& st = P.st[s];
   uint64_t sig = (uint64_t)s | ((uint64_t)split << 2) | ((uint64_t)tau0 << 5) | ((uint64_t)tau1 << 7);
   for (int r = 0; r < st.n_rel; ++r) {

@@ -73,6 +73,9 @@ __host__ __device__ inline size_t wave_ws_bytes(uint32_t nodes, uint32_t slots) 
 }
 
 constexpr uint32_t CID_INVALID = 0xFFFFFFFFu, CID_UNKNOWN = 0xFFFFFFFEu;
+// Every class counts its plans in `shards` counters (the blocks of k_signature spread over them): thousands of
+// wavefronts adding to the same few addresses serialise in the L2.  classes * shards stays near COUNT_SLOTS.
+constexpr uint32_t COUNT_SLOTS = 16384, MAX_SHARDS = 64;
 
 __host__ __device__ inline uint64_t sig_hash(uint64_t x) {
   x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -86,76 +89,114 @@ __global__ void k_fill_u32(uint32_t* p, uint64_t n, uint32_t v) {
 }
 
 // Integer validity gate, class signature, class id (open-addressing table of the classes lowered so far)
-// and the per-class plan count.  count[n_classes] counts the plans of classes not lowered yet.
-__global__ void k_signature(const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
-                            const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig,
-                            double* makespan, double* peak, double* score, uint8_t* mask, double* mass,
-                            const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval, uint32_t hmask,
-                            uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
-                            uint32_t n_classes) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  PlanHead h = load_head(head, stride, i);
-  VPlan a[RPEG_MAX_V];
-  const int nv = (h.structure < P->n_struct) ? P->st[h.structure].n_vertex : 0;
-  for (int v = 0; v < RPEG_MAX_V; ++v)
-    if (v < nv) load_vertex(vert, stride, i, v, &a[v]);
-  if (nv == 0 || !plan_valid(*P, h, a)) {
-    sig[i] = SIG_INVALID;
-    const double nan = __builtin_nan("");
-    if (makespan) makespan[i] = nan;
-    if (peak) peak[i] = nan;
-    if (score) score[i] = nan;
-    if (mask) mask[i] = 0;
-    if (mass)
-      for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
-    cid[i] = CID_INVALID;
-    return;
-  }
-  const uint64_t sg = plan_signature(*P, h.structure, h.split, h.tau0, h.tau1, a);
-  sig[i] = sg;
-  uint32_t c = CID_UNKNOWN;
-  for (uint32_t slot = (uint32_t)sig_hash(sg) & hmask, probes = 0; probes <= hmask; slot = (slot + 1) & hmask, ++probes) {
-    const uint64_t key = hkey[slot];
-    if (key == sg) { c = hval[slot]; break; }
-    if (key == SIG_INVALID) break;
-  }
-  cid[i] = c;
-  // arrival index within the class.  The plans of the (up to four) first classes met in a wavefront share
-  // one atomic per class: batches of few classes would otherwise serialise on a handful of counters.  The
-  // rest (many classes, few plans each) add themselves one by one.
-  const uint32_t key = c == CID_UNKNOWN ? n_classes : c;
-  const int lane = (int)(threadIdx.x & (WAVE - 1));
-  bool pending = true;
-  uint32_t k = 0;
-  for (int round = 0; round < 4; ++round) {
-    const unsigned long long am = __ballot(pending);
-    if (!am) break;
-    const int leader = __ffsll(am) - 1;
-    const uint32_t k0 = (uint32_t)__shfl((int)key, leader);
-    const unsigned long long same = __ballot(pending && key == k0);
-    uint32_t base = 0;
-    if (lane == leader) base = atomicAdd(&count[k0], (uint32_t)__popcll(same));
-    base = (uint32_t)__shfl((int)base, leader);
-    if (pending && key == k0) {
-      k = base + (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
-      pending = false;
+// and the per-class plan counts.  Blocks of SIG_BLOCK plans; shard = block mod shards.
+constexpr int SIG_BLOCK = 256, SIG_TABLE = 512;
+struct SigPlans {   // the plan fields of one thread's plan, a column of an LDS array [field][thread]
+  const int16_t* col;
+  __device__ VPlan operator[](int v) const { return ke_vplan<SIG_BLOCK>(col, v); }
+};
+__global__ __launch_bounds__(SIG_BLOCK) void k_signature(
+    const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
+    const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig, double* makespan, double* peak,
+    double* score, uint8_t* mask, double* mass, const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval,
+    uint32_t hmask, uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
+    uint32_t n_classes, uint32_t shards) {
+  // counters met in this block: key, plans of the block, and the block's first arrival index
+  __shared__ uint32_t t_key[SIG_TABLE], t_cnt[SIG_TABLE], t_base[SIG_TABLE];
+  // plan fields: the gate and the signature index the vertices with run-time values, which would put a
+  // per-thread array into scratch memory
+  __shared__ int16_t s_plan[RPEG_MAX_V * RPEG_FIELDS * SIG_BLOCK];
+  constexpr uint32_t NONE = 0xFFFFFFFFu;
+  for (int j = threadIdx.x; j < SIG_TABLE; j += SIG_BLOCK) { t_key[j] = NONE; t_cnt[j] = 0u; }
+  __syncthreads();
+  const uint64_t i = (uint64_t)blockIdx.x * SIG_BLOCK + threadIdx.x;
+  const bool active = i < n;
+  PlanHead h;
+  h.structure = h.split = h.tau0 = h.tau1 = 0;
+  if (active) h = load_head(head, stride, i);
+  // The structure decides which tables the gate and the signature read.  It is made uniform (one pass per
+  // distinct structure among the plans of the wavefront) so that those reads are scalar loads.
+  uint64_t sg = SIG_INVALID;
+  const bool known = active && h.structure >= 0 && h.structure < P->n_struct;
+  unsigned long long todo = __ballot(known);
+  while (todo) {
+    const int su = __builtin_amdgcn_readlane(h.structure, __builtin_ctzll(todo));
+    const bool mine = known && h.structure == su;
+    todo &= ~__ballot(mine);
+    if (mine) {
+      const int nv = P->st[su].n_vertex;
+      {  // every load of a vertex is issued before the first is waited for
+        const int16_t* src = vert + i;
+        int16_t* dst = s_plan + threadIdx.x;
+#pragma unroll
+        for (int v = 0; v < RPEG_MAX_V; ++v) {
+          if (v >= nv) break;
+          int16_t t[RPEG_FIELDS];
+#pragma unroll
+          for (int f = 0; f < RPEG_FIELDS; ++f) t[f] = src[(uint64_t)(v * RPEG_FIELDS + f) * stride];
+#pragma unroll
+          for (int f = 0; f < RPEG_FIELDS; ++f) dst[(v * RPEG_FIELDS + f) * SIG_BLOCK] = t[f];
+        }
+      }
+      const SigPlans a{s_plan + threadIdx.x};
+      PlanHead hu = h;
+      hu.structure = su;
+      if (nv != 0 && plan_valid(*P, hu, a)) sg = plan_signature(*P, su, h.split, h.tau0, h.tau1, a);
     }
   }
-  if (pending) k = atomicAdd(&count[key], 1u);
-  kidx[i] = k;
+  uint32_t key = NONE;
+  if (active) {
+    sig[i] = sg;
+    if (sg == SIG_INVALID) {
+      const double nan = __builtin_nan("");
+      if (makespan) makespan[i] = nan;
+      if (peak) peak[i] = nan;
+      if (score) score[i] = nan;
+      if (mask) mask[i] = 0;
+      if (mass)
+        for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
+      cid[i] = CID_INVALID;
+    } else {
+      uint32_t c = CID_UNKNOWN;
+      for (uint32_t slot = (uint32_t)sig_hash(sg) & hmask, probes = 0; probes <= hmask; slot = (slot + 1) & hmask, ++probes) {
+        const uint64_t k = hkey[slot];
+        if (k == sg) { c = hval[slot]; break; }
+        if (k == SIG_INVALID) break;
+      }
+      cid[i] = c;
+      // count[class * shards + shard]; the plans of classes not lowered yet share count[n_classes * shards]
+      key = c == CID_UNKNOWN ? n_classes * shards : c * shards + (blockIdx.x & (shards - 1u));
+    }
+  }
+  // Arrival index within (class, shard): the plans of the block are counted in LDS first, then every counter
+  // the block met takes one atomic: thousands of wavefronts adding to the same address serialise in the L2.
+  uint32_t slot = 0, local = 0;
+  if (key != NONE) {
+    slot = (key * 2654435761u >> 16) & (SIG_TABLE - 1);
+    for (;;) {   // at most SIG_BLOCK distinct keys in SIG_TABLE slots: a free slot is always found
+      const uint32_t prev = atomicCAS(&t_key[slot], NONE, key);
+      if (prev == NONE || prev == key) break;
+      slot = (slot + 1) & (SIG_TABLE - 1);
+    }
+    local = atomicAdd(&t_cnt[slot], 1u);
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < SIG_TABLE; j += SIG_BLOCK)
+    if (t_cnt[j]) t_base[j] = atomicAdd(&count[t_key[j]], t_cnt[j]);
+  __syncthreads();
+  if (key != NONE) kidx[i] = t_base[slot] + local;
 }
 
-// perm[(first wavefront of the class + k / lanes) * pstride + k % lanes] = plan, k = arrival order within the
-// class; pstride = 64, or 1 when every wavefront takes one plan
+// cbase[class * shards + shard]: plans of the class in lower shards; shard as in k_signature.
 __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const uint32_t* __restrict__ kidx,
                           const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
-                          uint32_t* __restrict__ perm, uint32_t pstride) {
+                          const uint32_t* __restrict__ cbase, uint32_t shards, uint32_t* __restrict__ perm,
+                          uint32_t pstride) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t c = cid[i];
   if (c >= CID_UNKNOWN) return;
-  const uint32_t k = kidx[i], l = clpw[c] & 0xFFFFu;
+  const uint32_t k = cbase[c * shards + ((uint32_t)(i / SIG_BLOCK) & (shards - 1u))] + kidx[i], l = clpw[c] & 0xFFFFu;
   if (clpw[c] >> 16) perm[(uint64_t)cfirst[c] + k] = (uint32_t)i;   // a class of single-plan wavefronts: cfirst is its first entry
   else perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
 }
@@ -346,10 +387,10 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
       hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
     }
     e->d_ccount = nullptr; e->ccap = 0;
-    HIP_TRY(e, hipMalloc(&e->d_ccount, (size_t)cap * 4));
+    HIP_TRY(e, hipMalloc(&e->d_ccount, ((size_t)cap + COUNT_SLOTS + 64) * 4));
     HIP_TRY(e, hipMalloc(&e->d_cfirst, (size_t)cap * 4));
     HIP_TRY(e, hipMalloc(&e->d_clpw, (size_t)cap * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (size_t)cap * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_ccount, ((size_t)cap + COUNT_SLOTS + 64) * 4));
     HIP_TRY(e, hipHostMalloc(&e->h_cfirst, (size_t)cap * 4));
     HIP_TRY(e, hipHostMalloc(&e->h_clpw, (size_t)cap * 4));
     e->ccap = cap;
@@ -623,18 +664,21 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // per-class counts come back.  Plans of classes not lowered yet make the call take the slow round:
   // their signatures are read back, the classes are lowered on the host, the tables are rebuilt.
   uint64_t n_new = 0;
-  uint32_t ncls = 0;
+  uint32_t ncls = 0, shards = 1;
   for (int round = 0;; ++round) {
     if (int rc = ensure_class_tables(e, s)) return rc;
     ncls = (uint32_t)e->cls_sig.size();
-    hipLaunchKernelGGL(k_fill_u32, dim3((ncls + 1 + blk - 1) / blk), dim3(blk), 0, s, e->d_ccount, (uint64_t)ncls + 1, 0u);
-    hipLaunchKernelGGL(k_signature, dim3(nblk), dim3(blk), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
+    shards = MAX_SHARDS;
+    while (shards > 1 && (uint64_t)ncls * shards > COUNT_SLOTS) shards >>= 1;
+    const uint64_t n_count = (uint64_t)ncls * shards + 1;
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_count + blk - 1) / blk)), dim3(blk), 0, s, e->d_ccount, n_count, 0u);
+    hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
                        e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
-                       e->d_kidx, e->d_ccount, ncls);
+                       e->d_kidx, e->d_ccount, ncls, shards);
     HIP_TRY(e, hipGetLastError());
-    HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, ((size_t)ncls + 1) * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, n_count * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
-    if (e->h_ccount[ncls] == 0) break;
+    if (e->h_ccount[n_count - 1] == 0) break;
     if (round >= 2) { e->err = "class table did not converge"; return -5; }
     HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
@@ -649,8 +693,15 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (int rc = lower_new_classes(e, sigs, &n_new)) return rc;
   }
   std::vector<uint32_t> offs, counts, cids;   // the classes present in this batch
-  for (uint32_t c = 0; c < ncls; ++c)
-    if (e->h_ccount[c]) { cids.push_back(c); offs.push_back(e->cls_off[c]); counts.push_back(e->h_ccount[c]); }
+  for (uint32_t c = 0; c < ncls; ++c) {   // per-shard counts become the shards' offsets within the class
+    uint32_t total = 0;
+    for (uint32_t sh = 0; sh < shards; ++sh) {
+      const uint32_t cnt = e->h_ccount[(size_t)c * shards + sh];
+      e->h_ccount[(size_t)c * shards + sh] = total;
+      total += cnt;
+    }
+    if (total) { cids.push_back(c); offs.push_back(e->cls_off[c]); counts.push_back(total); }
+  }
   // Plans per wavefront and where their scheduler state lives.  A full batch keeps 64 plans per wavefront
   // with the state in the HBM workspace; a batch too small to fill the chip that way is spread over more
   // wavefronts of fewer plans whose state fits in LDS, which shortens every scheduler step.
@@ -773,10 +824,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (int rc = ensure_pool(e, s)) return rc;
   HIP_TRY(e, hipMemcpyAsync(e->d_cfirst, e->h_cfirst, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_clpw, e->h_clpw, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, (size_t)ncls * shards * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, ((size_t)n_eval_waves + n_solo) * 4, hipMemcpyHostToDevice, s));
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
-  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_perm, pstride);
+  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_ccount, shards, e->d_perm, pstride);
   HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_eval_waves;

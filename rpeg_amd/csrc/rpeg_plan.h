@@ -30,7 +30,8 @@ RPEG_HD void load_vertex(const int16_t* vert, uint64_t stride, uint64_t i, int s
 }
 
 // Integer gate: header ranges plus evaluate.py:172-196 per vertex.
-RPEG_HD bool plan_valid(const rpeg_problem_t& P, const PlanHead& h, const VPlan* a) {
+template <class PLANS>
+RPEG_HD bool plan_valid(const rpeg_problem_t& P, const PlanHead& h, const PLANS& a) {
   if (h.structure < 0 || h.structure >= P.n_struct) return false;
   if (h.split < 0 || h.split >= P.n_split) return false;
   if (h.tau0 > 3 || h.tau1 > 3) return false;
