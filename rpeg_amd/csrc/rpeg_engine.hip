@@ -302,8 +302,9 @@ struct rpeg_engine_s {
   uint32_t* d_hval = nullptr;
   uint32_t hcap = 0, tables_for = 0;                 // table capacity; class count the device tables reflect
   uint32_t ccap = 0;                                 // capacity of the per-class device arrays
-  uint32_t *d_ccount = nullptr, *d_cfirst = nullptr, *d_clpw = nullptr;
-  uint32_t *h_ccount = nullptr, *h_cfirst = nullptr, *h_clpw = nullptr;
+  // per-class tables of a call, one block on each side: counters per (class, shard), which become the shards'
+  // offsets, then first wavefront and plans per wavefront of every class
+  uint32_t *d_ccount = nullptr, *h_ccount = nullptr;
   uint32_t *d_cid = nullptr, *d_kidx = nullptr;   // per plan: class id, arrival index within the class
   std::vector<uint8_t> pool;
   uint8_t* d_pool = nullptr;
@@ -383,16 +384,12 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
   if (ncls + 1 > e->ccap) {
     const uint32_t cap = std::max<uint32_t>(2 * (ncls + 1), 4096);
     if (e->d_ccount) {
-      hipFree(e->d_ccount); hipFree(e->d_cfirst); hipFree(e->d_clpw);
-      hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
+      hipFree(e->d_ccount);
+      hipHostFree(e->h_ccount);
     }
     e->d_ccount = nullptr; e->ccap = 0;
-    HIP_TRY(e, hipMalloc(&e->d_ccount, ((size_t)cap + COUNT_SLOTS + 64) * 4));
-    HIP_TRY(e, hipMalloc(&e->d_cfirst, (size_t)cap * 4));
-    HIP_TRY(e, hipMalloc(&e->d_clpw, (size_t)cap * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_ccount, ((size_t)cap + COUNT_SLOTS + 64) * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_cfirst, (size_t)cap * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_clpw, (size_t)cap * 4));
+    HIP_TRY(e, hipMalloc(&e->d_ccount, (3 * (size_t)cap + COUNT_SLOTS + 64) * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (3 * (size_t)cap + COUNT_SLOTS + 64) * 4));
     e->ccap = cap;
   }
   e->tables_for = ncls;
@@ -564,8 +561,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); }
   if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
   if (e->d_ccount) {
-    hipFree(e->d_ccount); hipFree(e->d_cfirst); hipFree(e->d_clpw);
-    hipHostFree(e->h_ccount); hipHostFree(e->h_cfirst); hipHostFree(e->h_clpw);
+    hipFree(e->d_ccount);
+    hipHostFree(e->h_ccount);
   }
   if (e->d_perm) hipFree(e->d_perm);
   if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
@@ -738,9 +735,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // classes with the largest graphs first: their wavefronts run longest and should not start last
   std::vector<uint32_t> order(counts.size());
   for (size_t c = 0; c < counts.size(); ++c) order[c] = (uint32_t)c;
-  std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
-    return ((const ClassHdr*)(e->pool.data() + offs[a]))->n_nodes > ((const ClassHdr*)(e->pool.data() + offs[b]))->n_nodes;
-  });
+  std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) { return e->cls_nodes[cids[a]] > e->cls_nodes[cids[b]]; });
   // first[c]: first wavefront of class c in launch order (first permutation entry for a class of
   // single-plan wavefronts, which follow the others in the permutation and in the task list)
   std::vector<uint32_t> first(counts.size(), 0), clpw(counts.size(), lpw);
@@ -802,9 +797,13 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   e->stats[6] = 0;
   if (n_sorted + n_solo == 0) return 0;
   if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_eval_waves + n_solo)) return rc;
+  uint32_t* const h_cfirst = e->h_ccount + (size_t)ncls * shards;   // behind the shard offsets
+  uint32_t* const h_clpw = h_cfirst + ncls;
+  const uint32_t* const d_cfirst = e->d_ccount + (size_t)ncls * shards;
+  const uint32_t* const d_clpw = d_cfirst + ncls;
   for (size_t c = 0; c < counts.size(); ++c) {
-    e->h_cfirst[cids[c]] = first[c];
-    e->h_clpw[cids[c]] = clpw[c];
+    h_cfirst[cids[c]] = first[c];
+    h_clpw[cids[c]] = clpw[c];
   }
   // wavefronts of few plans keep their scheduler state in LDS when that needs no more LDS than the ready
   // lists of a full wavefront do
@@ -822,13 +821,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     }
   }
   if (int rc = ensure_pool(e, s)) return rc;
-  HIP_TRY(e, hipMemcpyAsync(e->d_cfirst, e->h_cfirst, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
-  HIP_TRY(e, hipMemcpyAsync(e->d_clpw, e->h_clpw, (size_t)ncls * 4, hipMemcpyHostToDevice, s));
-  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, (size_t)ncls * shards * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, ((size_t)ncls * shards + 2 * (size_t)ncls) * 4, hipMemcpyHostToDevice, s));
   HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, ((size_t)n_eval_waves + n_solo) * 4, hipMemcpyHostToDevice, s));
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
-  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, e->d_cfirst, e->d_clpw, e->d_ccount, shards, e->d_perm, pstride);
+  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride);
   HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_eval_waves;
