@@ -126,6 +126,39 @@ def test_empty_single_and_invalid():
     assert list(eng.eval(allbad)["mask"]) == [0, 0, 0]
 
 
+def test_empty_single_and_invalid_device_tensors_and_argument_errors():
+    """The same edge cases through rpeg_eval_batch on device tensors (a batch of 8 plans and one of 3,000:
+    one plan per wavefront and the main kernel), and the argument checks of rpeg_eval_host."""
+    import ctypes as C
+    from rpeg_amd.engine.runtime import EngineError
+    eng = engine(2)
+    for n in (8, 3000, 40000):
+        cfg, batch = seeded_batch(2, n)
+        batch.vert[0, 1] = 3
+        batch.vert[3, 2] = 5
+        batch.head[1, 3] = 7
+        batch.vert[7, 4] = 99
+        out = eng.eval_resident(batch)
+        host = eng.eval(batch)
+        assert list(out["mask"][1:5]) == [0, 0, 0, 0] and np.all(np.isnan(out["score"][1:5]))
+        assert np.array_equal(out["mask"], host["mask"]) and same_bits(out["score"], host["score"])
+        assert same_bits(out["makespan"], host["makespan"]) and same_bits(out["peak"], host["peak"])
+    assert list(eng.eval_resident(PlanBatch.empty(3))["mask"]) == [0, 0, 0]
+    cfg, batch = seeded_batch(2, 16)
+    vert = np.ascontiguousarray(batch.vert)
+    head = np.ascontiguousarray(batch.head)
+    score = np.empty(16)
+    bad_stride = abi.PlanSoaT(vert.ctypes.data, head.ctypes.data, 8)        # stride below n
+    assert eng.lib.rpeg_eval_host(eng._h, 16, C.addressof(bad_stride), 0, None, None, score.ctypes.data, None, None, None) < 0
+    assert b"bad plan tensors" in eng.lib.rpeg_last_error(eng._h)
+    no_vert = abi.PlanSoaT(None, head.ctypes.data, 16)
+    assert eng.lib.rpeg_eval_host(eng._h, 16, C.addressof(no_vert), 0, None, None, score.ctypes.data, None, None, None) < 0
+    assert eng.lib.rpeg_eval_host(eng._h, 16, None, 0, None, None, score.ctypes.data, None, None, None) < 0
+    ok = abi.PlanSoaT(vert.ctypes.data, head.ctypes.data, 16)               # only the score is asked for
+    assert eng.lib.rpeg_eval_host(eng._h, 16, C.addressof(ok), 0, None, None, score.ctypes.data, None, None, None) == 0
+    assert same_bits(score, eng.eval(batch, gate_stale=False)["score"])
+
+
 def test_mixed_structures_config3():
     cfg, batch = seeded_batch(3, 2000, start=500_000)
     out = engine(3).eval(batch)
