@@ -328,6 +328,13 @@ struct rpeg_engine_s {
   uint64_t prof_waves = 0;
   // per-batch buffers
   size_t cap_n = 0, cap_perm = 0, cap_cls = 0;
+  // Ready-list capacity of k_eval: learned from the longest list seen so far (running maxima kept by the
+  // kernel, read back with the class counts of the next call); plans that outgrow it are flagged and redone
+  // with the full capacity by a second launch.
+  uint8_t* d_ovf = nullptr;
+  uint32_t *d_need = nullptr, *h_need = nullptr;
+  uint32_t need = 0;
+  uint32_t max_v = RPEG_MAX_V;   // largest vertex count of the problem's structures
   hipStream_t s2 = nullptr;                     // second stream: single-plan wavefronts of a large batch run beside the others
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   int split_heavy = 1;                          // 0: the classes with the largest graphs stay in the main kernel
@@ -347,8 +354,16 @@ struct rpeg_engine_s {
 static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (n <= e->cap_n) return 0;
   size_t cap = std::max<size_t>(n, 4096);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
   e->cap_n = 0;
+  HIP_TRY(e, hipMalloc(&e->d_ovf, cap));
+  HIP_TRY(e, hipMemset(e->d_ovf, 0, cap));   // flags are cleared again by the launch that consumes them
+  if (!e->d_need) {
+    HIP_TRY(e, hipMalloc(&e->d_need, KE_NEED_SHARDS * 4));
+    HIP_TRY(e, hipMemset(e->d_need, 0, KE_NEED_SHARDS * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_need, KE_NEED_SHARDS * 4));
+    std::memset(e->h_need, 0, KE_NEED_SHARDS * 4);
+  }
   HIP_TRY(e, hipMalloc(&e->d_sig, cap * 8));
   HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
   HIP_TRY(e, hipMalloc(&e->d_cid, cap * 4));
@@ -542,6 +557,8 @@ int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
   hipGetDevice(&e->device);
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, e->device) == hipSuccess) e->n_cu = prop.multiProcessorCount;
+  e->max_v = 1;
+  for (int q = 0; q < e->P.n_struct; ++q) e->max_v = std::max<uint32_t>(e->max_v, (uint32_t)e->P.st[q].n_vertex);
 
   if (hipMalloc(&e->dP, sizeof(rpeg_problem_t)) != hipSuccess ||
       hipMemcpy(e->dP, problem, sizeof(rpeg_problem_t), hipMemcpyHostToDevice) != hipSuccess ||
@@ -558,7 +575,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   hipDeviceSynchronize();
   if (e->dP) hipFree(e->dP);
   if (e->d_pool) hipFree(e->d_pool);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
+  if (e->d_need) { hipFree(e->d_need); hipHostFree(e->h_need); }
   if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
   if (e->d_ccount) {
     hipFree(e->d_ccount);
@@ -674,7 +692,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
                        e->d_kidx, e->d_ccount, ncls, shards);
     HIP_TRY(e, hipGetLastError());
     HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, n_count * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipMemcpyAsync(e->h_need, e->d_need, KE_NEED_SHARDS * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
+    for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_need[q]);
     if (e->h_ccount[n_count - 1] == 0) break;
     if (round >= 2) { e->err = "class table did not converge"; return -5; }
     HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
@@ -707,7 +727,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   {
     auto waves_for = [&](uint32_t per) { uint64_t t = 0; for (uint32_t c : counts) t += (c + per - 1) / per; return t; };
     auto fits = [&](int l) {
-      return ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, 32, (uint32_t)l, e->max_nodes, e->max_slots) <= 160 * 1024;
+      return ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, 32, (uint32_t)l, e->max_nodes, e->max_slots, e->max_v) <= 160 * 1024;
     };
     const bool one_fits = e->max_nodes <= (uint32_t)(WAVE * KP_MAX_NS) && kp_lds_bytes(e->max_nodes, e->max_slots) <= 64 * 1024;
     if (ls < 0) {
@@ -807,8 +827,13 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   // wavefronts of few plans keep their scheduler state in LDS when that needs no more LDS than the ready
   // lists of a full wavefront do
+  // Ready-list capacity: the full 32 entries until the longest list of earlier launches is known, then a
+  // short list (less LDS, more wavefronts per compute unit); plans that outgrow it are redone below.
+  const uint32_t rcap_full = 32;
+  const bool short_list = !ls && !one && e->need > 0 && ((e->need + 2 + 7) & ~7u) < rcap_full;
+  const uint32_t rcap = short_list ? std::max(8u, (e->need + 2 + 7) & ~7u) : rcap_full;
   const bool few_in_lds = !ls && !one &&
-      ke_lds_bytes(0, 32, KE_FEW, e->max_nodes, e->max_slots) <= ke_lds_bytes(0, 32, 0, e->max_nodes, e->max_slots);
+      ke_lds_bytes(0, rcap, KE_FEW, e->max_nodes, e->max_slots, e->max_v) <= ke_lds_bytes(0, rcap, 0, e->max_nodes, e->max_slots, e->max_v);
   for (size_t k = 0; k < order.size(); ++k) {
     const uint32_t c = order[k];
     if (solo[c]) {
@@ -841,7 +866,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // ready-list capacity (a multiple of the scan's batch of 8); classes with more than 4095 nodes or
   // tie-break keys above 15 cannot be packed into a ready entry
   if (e->max_nodes > 4095) { e->err = "class with more than 4095 nodes"; return -8; }
-  L.rcap = 32;
+  L.rcap = rcap;
+  L.max_v = e->max_v;
+  L.ovf = !ls && !one ? e->d_ovf : nullptr;
+  L.need = !ls && !one ? e->d_need : nullptr;
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
   L.prof = nullptr;
@@ -853,7 +881,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     L.prof = e->d_prof;
   }
   const size_t lds = one ? kp_lds_bytes(e->max_nodes, e->max_slots)
-                   : ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots);
+                   : ke_lds_bytes(L.cls_bytes, L.rcap, (uint32_t)ls, e->max_nodes, e->max_slots, e->max_v);
   if (lds > 160 * 1024) { e->err = "class tables exceed the LDS"; return -8; }
   const void* kfn = ls == 0 ? (const void*)k_eval<0> : ls == 8 ? (const void*)k_eval<8> : ls == 16 ? (const void*)k_eval<16>
                   : ls == 32 ? (const void*)k_eval<32> : (const void*)k_eval<64>;
@@ -888,6 +916,19 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     default: hipLaunchKernelGGL(k_eval<64>, dim3(grid), dim3(WAVE), lds, s, L); break;
   }
   HIP_TRY(e, hipGetLastError());
+  if (short_list && n_waves) {   // the plans whose ready list outgrew the short one, with the full one
+    EvalLaunch F = L;
+    F.rcap = rcap_full;
+    F.flags = flags | KE_FIXUP;
+    const size_t lds_full = ke_lds_bytes(F.cls_bytes, F.rcap, 0, e->max_nodes, e->max_slots, e->max_v);
+    if (lds_full > 160 * 1024) { e->err = "class tables exceed the LDS"; return -8; }
+    if (lds_full > 64 * 1024 && !e->lds_attr_set[0]) {
+      HIP_TRY(e, hipFuncSetAttribute((const void*)k_eval<0>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      e->lds_attr_set[0] = true;
+    }
+    hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds_full, s, F);
+    HIP_TRY(e, hipGetLastError());
+  }
   if (n_solo) {   // the single-plan wavefronts, beside the main kernel
     EvalLaunch S = L;
     S.perm = e->d_perm + n_sorted;
@@ -1078,7 +1119,7 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
   L.wave_cls = (const uint32_t*)(L.head + 4 * stride);
   L.pool = e->d_pool; L.ws = nullptr;
   L.n_waves = m; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
-  L.cls_bytes = 0; L.rcap = 0;
+  L.cls_bytes = 0; L.rcap = 0; L.max_v = e->max_v; L.ovf = nullptr; L.need = nullptr;
   L.flags = flags; L.makespan = o_makespan; L.peak = o_peak; L.score = o_score; L.mask = o_mask;
   L.mass = mass ? o_mass : nullptr;
   L.prof = nullptr;

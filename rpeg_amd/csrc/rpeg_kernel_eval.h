@@ -39,6 +39,7 @@ struct EvalLaunch {              // uniform launch parameters
   uint32_t ws_nodes, ws_slots;   // workspace row counts (maxima over the engine's classes)
   uint32_t cls_bytes;            // LDS bytes reserved for class tables
   uint32_t rcap;                 // ready-list capacity per plan
+  uint32_t max_v;                // largest vertex count of the problem's structures
   uint32_t flags;
   double* makespan;
   double* peak;
@@ -46,7 +47,12 @@ struct EvalLaunch {              // uniform launch parameters
   uint8_t* mask;
   double* mass;                  // optional critical-chain mass, [plan][RPEG_MAX_V], or null
   unsigned long long* prof;      // optional per-wavefront phase clocks (8 per wavefront), or null
+  uint8_t* ovf;                  // per plan: its ready list outgrew rcap (set by a launch with a short list,
+                                 // consumed by the KE_FIXUP launch with the full one), or null
+  uint32_t* need;                // KE_NEED_SHARDS running maxima of the ready-list length, or null
 };
+constexpr uint32_t KE_FIXUP = 0x80000000u;   // EvalLaunch::flags: only the plans flagged in `ovf` are evaluated
+constexpr int KE_NEED_SHARDS = 64;
 
 __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
   size_t lane = (16ull * nodes + 8ull * slots + nodes + 63) & ~size_t(63);
@@ -54,17 +60,19 @@ __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
 }
 // Dynamic LDS of one wavefront.  ls = 0: the per-plan state lives in the HBM workspace and all 64 lanes
 // carry plans.  ls > 0: only the first `ls` lanes carry plans and their state (ready time, rank,
-// in-degree per node, duration per slot) lives in LDS too, interleaved by lane.
-__host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls) {
+// in-degree per node, duration per slot) lives in LDS too, interleaved by lane.  One area serves, one after
+// the other, the plan fields (read by the cost model), the per-vertex memory terms and the ready list; nv is
+// the largest vertex count of the problem's structures.
+__host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls, uint32_t nv) {
   const size_t rw = ls ? ls : KE_WAVE;
-  // ready list: key (8 bytes) and meta (4 bytes) per entry
-  size_t ready = (size_t)rcap * rw * 12;
-  size_t plan = (size_t)RPEG_MAX_V * RPEG_FIELDS * rw * 2 + (size_t)RPEG_MAX_V * 4 * rw * 8;
-  return ((ready > plan ? ready : plan) + 15) & ~size_t(15);
+  const size_t ready = (size_t)rcap * rw * 12;                 // key (8 bytes) and meta (4 bytes) per entry
+  const size_t plan = (size_t)nv * RPEG_FIELDS * rw * 2, vmem = (size_t)nv * 4 * rw * 8;
+  const size_t top = ready > plan ? (ready > vmem ? ready : vmem) : (plan > vmem ? plan : vmem);
+  return (top + 15) & ~size_t(15);
 }
-__host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap, uint32_t ls = 0, uint32_t nodes = 0,
-                                               uint32_t slots = 0) {
-  return cls_bytes + ke_dyn_bytes(rcap, ls) + (size_t)ls * ((16ull * nodes + 8ull * slots + nodes + 15) & ~15ull);
+__host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap, uint32_t ls, uint32_t nodes,
+                                               uint32_t slots, uint32_t nv) {
+  return cls_bytes + ke_dyn_bytes(rcap, ls, nv) + (size_t)ls * ((16ull * nodes + 8ull * slots + nodes + 15) & ~15ull);
 }
 
 #if defined(__HIPCC__)
@@ -138,17 +146,21 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   uint16_t* l_succ = (uint16_t*)(lds + (size_t)n * 8);                // uint16[n_succ]
   uint8_t* dyn = lds + L.cls_bytes;
   int16_t* l_plan = (int16_t*)dyn + lane;                             // [60][64], aliased with the ready list
-  double* l_vm = (double*)(dyn + (size_t)RPEG_MAX_V * RPEG_FIELDS * RW * 2) + lane;  // [24][RW], aliased too
+  double* l_vm = (double*)dyn + lane;   // [4 * vertices][RW]: written once the cost model is done with the plan fields
   double* r_key = (double*)dyn + lane;                                       // [rcap][RW]
   uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * RW * 8) + lane;        // [rcap][RW] meta, see below
 
+  // which plan this lane carries; a fix-up launch only takes the plans whose list outgrew the short one
+  uint64_t pi = (LS && lane >= LS) ? (uint64_t)KE_IDLE : (uint64_t)L.perm[w * KE_WAVE + lane];
+  if (L.flags & KE_FIXUP) {
+    if (pi != KE_IDLE && !L.ovf[pi]) pi = KE_IDLE;
+    if (!__ballot(pi != KE_IDLE)) return;   // uniform: nothing to redo in this wavefront
+  }
   __syncthreads();  // the previous task of this wavefront is done with LDS
   for (int i = lane; i < n; i += KE_WAVE) l_node[i] = ((const uint64_t*)cv.node)[i];
   for (int i = lane; i < n_succ_all; i += KE_WAVE) l_succ[i] = cv.succ[i];
   __syncthreads();
 
-  if (LS && lane >= LS) return;
-  const uint64_t pi = L.perm[w * KE_WAVE + lane];
   if (pi == KE_IDLE) return;
   first_lane = __builtin_ctzll(__ballot(1));
   KE_STAMP(0);
@@ -157,7 +169,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   double *g_time, *g_rank, *g_dur;
   uint8_t* g_deg;
   if (LS) {  // LDS, [row][lane]: time[nodes] rank[nodes] dur[slots] deg[nodes]
-    uint8_t* sbase = dyn + ke_dyn_bytes(L.rcap, LS);
+    uint8_t* sbase = dyn + ke_dyn_bytes(L.rcap, LS, L.max_v);
     g_time = (double*)sbase + lane;
     g_rank = g_time + (size_t)L.ws_nodes * LS;
     g_dur = g_rank + (size_t)L.ws_nodes * LS;
@@ -257,7 +269,8 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   double lf[RPEG_MAX_V];
 #pragma unroll
   for (int x = 0; x < RPEG_MAX_V; ++x) lf[x] = 0.0;
-  int n_ready = 0, done = 0;
+  int n_ready = 0, done = 0, max_ready = 0;
+  bool ovf = false;
   const int rcap = (int)L.rcap;   // a multiple of eight
   const double inf = __builtin_inf();
   constexpr uint32_t SAME = 1u << 22;
@@ -331,10 +344,11 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
       r_nt[idx * RW] = nm[q] | (same ? SAME : 0u);
     }
     n_ready += cnt;
+    max_ready = n_ready > max_ready ? n_ready : max_ready;
   };
   for (unsigned i = 0; i < cv.h->n_init && !err; ++i) {
     const int v = cv.init[i];
-    if (n_ready >= rcap - 1) { err = true; break; }
+    if (n_ready >= rcap - 1) { err = ovf = true; break; }
     const uint32_t nm[4] = {make_meta(v, cv.node[v]), 0u, 0u, 0u};
     const double nk[4] = {0.0, 0.0, 0.0, 0.0}, nrk[4] = {g_rank[(v) * SS], 0.0, 0.0, 0.0};
     push_many(std::integral_constant<int, 1>{}, 1, nm, nk, nrk);
@@ -483,7 +497,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
           g_deg[(wn) * SS] = left;
         }
       }
-      if (n_ready + cnt >= rcap) { err = true; break; }
+      if (n_ready + cnt >= rcap) { err = ovf = true; break; }
       // the widest push of the wavefront selects the code: most dispatches release one or two successors
       if (__ballot(cnt > 2)) {
         if (cnt) push_many(std::integral_constant<int, 4>{}, cnt, nm, nk, nrk);
@@ -495,6 +509,20 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     }
   }
   if (done != n) err = true;
+  if (L.ovf) {
+    if (L.flags & KE_FIXUP) L.ovf[pi] = 0;
+    else if (ovf) L.ovf[pi] = 1;
+  }
+  if (L.need) {   // longest ready list of the wavefront, folded into one of the running maxima
+    int m = max_ready;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const int o = __shfl_xor(m, off);
+      m = o > m ? o : m;
+    }
+    uint32_t* slot = L.need + (blockIdx.x & (KE_NEED_SHARDS - 1));
+    if (lane == first_lane && (uint32_t)m > *slot) atomicMax(slot, (uint32_t)m);
+  }
   KE_STAMP(5);
   if (L.prof) atomicMax(&L.prof[w * 8 + 7], ((unsigned long long)n << 32) | (unsigned long long)guard_total);
 

@@ -159,6 +159,31 @@ def test_empty_single_and_invalid_device_tensors_and_argument_errors():
     assert same_bits(score, eng.eval(batch, gate_stale=False)["score"])
 
 
+def test_plans_that_outgrow_the_learned_ready_list_are_redone():
+    """The main kernel sizes its ready lists by the longest list it has seen.  An engine that has only seen
+    chain-like graphs (every vertex on vertex 0's allocation and strategy) then meets the seeded set: the plans
+    whose lists outgrow the short capacity are flagged and redone with the full one."""
+    from rpeg_amd.engine.runtime import Engine
+    n = 40000                                       # above the one-plan-per-wavefront range
+    cfg, batch = seeded_batch(2, n)
+    chains = PlanBatch(batch.vert.copy(), batch.head.copy())
+    for v in range(1, 4):
+        chains.vert[v * 10:(v + 1) * 10, :] = chains.vert[0:10, :]
+    port = CpuPort(cfg.problem)
+    eng = Engine(cfg.problem)
+    lds = []
+    for b in (chains, batch, chains, batch):
+        out = eng.eval_resident(b)
+        ref = port.eval(b, flags=abi.GATE_STALE, threads=16)
+        assert np.array_equal(out["mask"], ref["mask"])
+        assert same_bits(out["makespan"], ref["makespan"]) and same_bits(out["score"], ref["score"])
+        assert eng.stats()["state_lanes"] == 0
+        lds.append(eng.stats()["lds_bytes"])
+    assert lds[1] < lds[0] and lds[1] < lds[3]      # the second call ran with the capacity learned from the chains
+    assert (ref["mask"] & abi.MASK_VALID).sum() > n // 2
+    eng.close()
+
+
 def test_mixed_structures_config3():
     cfg, batch = seeded_batch(3, 2000, start=500_000)
     out = engine(3).eval(batch)
