@@ -4,14 +4,16 @@
 //
 // Memory placement, chosen for the latency of the list scheduler's dependent accesses:
 //   LDS   class tables (node records, successor lists): read with per-lane node indices
-//         plan fields [field][lane] int16, aliased with ...
-//         ... the ready list [entry][lane]: key (est), rank, node|tie.  The arg-min scan, the
-//         stale-key update and the removal never leave LDS.
-//   HBM   per-plan arrays in a per-wavefront workspace laid out [row][lane] (a row is 512
-//         contiguous bytes, so accesses coalesce whenever lanes agree on the row): durations per
-//         slot, rank / ready-time / remaining in-degree per node.  A scheduling step issues all of
-//         its loads (duration of the dispatched node; ready-time, in-degree and rank of up to four
-//         successors) before it waits, i.e. one memory round trip per dispatched node.
+//         one area [row][lane] that holds, one after the other, the plan fields (int16, read by the cost
+//         model), the per-vertex memory terms and the ready list: key (est) and a meta word (node, tie-break
+//         class, reserved vertices) per entry.  The arg-min scan, the stale-key update and the removal never
+//         leave LDS.
+//   HBM   (LS = 0) per-plan arrays in a workspace, one contiguous block per lane: ready time and rank per
+//         node, duration per slot, remaining in-degree per node.  The lanes of a wavefront dispatch different
+//         nodes at any moment, so a row-per-node layout would not coalesce either, and a lane's block keeps
+//         its neighbouring nodes in one cache line.  A scheduling step issues all of its loads (duration of
+//         the dispatched node; ready time, in-degree and rank of up to four successors) before it waits.
+//         With LS > 0 the same arrays sit in LDS, interleaved by lane.
 #ifndef RPEG_KERNEL_EVAL_H
 #define RPEG_KERNEL_EVAL_H
 
