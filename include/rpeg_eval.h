@@ -190,12 +190,14 @@ int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t 
    0 operator, 1 COMM, 2 RESHARD; node_vertex: the operator's vertex, or a transfer's destination
    vertex; node_src: a transfer's source vertex; node_sub: quantile phase or -1; edges: (src,dst)
    node index pairs; dispatch_index (may be NULL): position of the node in the scheduler's dispatch order,
-   the insertion order of the reference's Trace.start (scheduler.py:517-518).  Returns the node count, or
-   a negative status. */
+   the insertion order of the reference's Trace.start (scheduler.py:517-518); node_reserved (may be NULL):
+   bit v set when the scheduler reserves the allocation of vertex v for the node
+   (RPEG/passes/transfer_resources.py:18-148, Trace.reserved_allocations).  Returns the node count, or a
+   negative status. */
 int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4,
                     double* start, double* finish, int32_t* dispatch_index, int32_t* node_kind, int32_t* node_vertex,
                     int32_t* node_step, int32_t* node_sub, int32_t* node_src, int32_t* edges,
-                    int32_t* n_edges, int32_t cap);
+                    int32_t* n_edges, int32_t cap, uint8_t* node_reserved);
 
 /* Batched simulated annealing: n_chains independent Metropolis-Hastings chains of n_steps steps.  One
    step of a chain is one iteration of the inner loop of optimize() (RPEG/search/optimizer.py:702-930):

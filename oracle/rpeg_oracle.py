@@ -1175,6 +1175,58 @@ def schedule(nodes, edges, cost, space, policy=("destination_only", "destination
     return start, finish, order
 
 
+def reserved_by_node(nodes, edges, policy=("destination_only", "destination_only")):
+    """node id -> tuple of the allocations the scheduler reserves for it (scheduler.py:334-343)."""
+    preds = {n.id: set() for n in nodes}
+    succs = {n.id: set() for n in nodes}
+    for a, b in edges:
+        preds[b.id].add(a.id)
+        succs[a.id].add(b.id)
+    by_id = {n.id: n for n in nodes}
+    return {n.id: reserved_allocations(n, preds, succs, by_id, policy) for n in nodes}
+
+
+def utilization(start, finish, order, reserved):
+    """Trace.utilization (RPEG/schedule/trace.py:53-101): per device the merged busy intervals of the nodes
+    that reserve it, divided by the makespan, averaged over the devices any node reserves.  `order` is the
+    dispatch order (the insertion order of Trace.start), which fixes the order of the devices in the
+    reference's dict and hence of its float sum."""
+    ms = max(finish.values())
+    if ms <= 0:
+        return 0.0
+    intervals = {}
+    for nid in order:
+        for a in reserved[nid]:
+            for dv in alloc_devices(a):
+                intervals.setdefault(dv, []).append((start[nid], finish[nid]))
+    if not intervals:
+        return 0.0
+    total = 0.0
+    for spans in intervals.values():
+        merged = 0.0
+        cs = ce = None
+        for s, e in sorted(spans):
+            if ce is None or s > ce:
+                if ce is not None:
+                    merged += ce - cs
+                cs, ce = s, e
+            else:
+                ce = max(ce, e)
+        if ce is not None:
+            merged += ce - cs
+        total += merged / ms    # the builtin sum of this interpreter (3.10) is a plain left fold
+    return total / len(intervals)
+
+
+def n_active(nodes):
+    """Trace.n_active (trace.py:103-118): devices inside any allocation of any node."""
+    devices = set()
+    for n in nodes:
+        for a in n.allocs:
+            devices.update(alloc_devices(a))
+    return len(devices)
+
+
 # --------------------------------------------------------------------------- evaluate
 def make_mem_model(rpeg, suite, workload, hw, policy):
     return MemModel(

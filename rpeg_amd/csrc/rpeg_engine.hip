@@ -972,7 +972,7 @@ int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t 
 
 int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* start, double* finish,
                     int32_t* dispatch_index, int32_t* node_kind, int32_t* node_vertex, int32_t* node_step, int32_t* node_sub, int32_t* node_src,
-                    int32_t* edges, int32_t* n_edges, int32_t cap) {
+                    int32_t* edges, int32_t* n_edges, int32_t cap, uint8_t* node_reserved) {
   if (!e || !vert_fields || !head4 || !start || !finish) return -1;
   e->err.clear();
   PlanHead h = load_head(head4, 1, 0);
@@ -1020,6 +1020,11 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
     if (node_step) node_step[i] = lc.nodes[i].step;
     if (node_sub) node_sub[i] = lc.nodes[i].sub;
     if (node_src) node_src[i] = lc.nodes[i].kind == 0 ? lc.nodes[i].vertex : lc.nodes[i].a0;
+  }
+  if (node_reserved) {   // the vertices whose allocations the scheduler reserves for the node
+    const ClassView cv = class_view(e->pool.data() + off);
+    const uint64_t dpne = plan_masks(a, e->P.st[h.structure].n_vertex).dpne;
+    for (int i = 0; i < n; ++i) node_reserved[i] = (uint8_t)blocked_mask(cv.node[i], dpne);
   }
   if (edges)
     for (size_t j = 0; j < lc.edges.size(); ++j) { edges[2 * j] = lc.edges[j].first; edges[2 * j + 1] = lc.edges[j].second; }

@@ -59,7 +59,7 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_op_time_batch.restype = C.c_int
     lib.rpeg_op_time_batch.argtypes = [vp, u64, i32, i32, vp, u64, vp, vp, vp]
     lib.rpeg_eval_trace.restype = C.c_int
-    lib.rpeg_eval_trace.argtypes = [vp] * 13 + [i32]
+    lib.rpeg_eval_trace.argtypes = [vp] * 13 + [i32, vp]
     lib.rpeg_engine_stats.restype = C.c_int
     lib.rpeg_engine_stats.argtypes = [vp, vp, i32]
     lib.rpeg_engine_set_timing.restype = C.c_int
@@ -317,14 +317,16 @@ class Engine:
         start, finish = np.zeros(cap), np.zeros(cap)
         kind, vertex, step, sub, src, order = (np.zeros(cap, np.int32) for _ in range(6))
         edges = np.zeros(2 * cap, np.int32)
+        reserved = np.zeros(cap, np.uint8)
         ne = C.c_int32(0)
         with torch.cuda.device(self.device):
             n = self.lib.rpeg_eval_trace(self._h, vert.ctypes.data, head.ctypes.data, start.ctypes.data,
                                          finish.ctypes.data, order.ctypes.data, kind.ctypes.data, vertex.ctypes.data, step.ctypes.data,
-                                         sub.ctypes.data, src.ctypes.data, edges.ctypes.data, C.addressof(ne), cap)
+                                         sub.ctypes.data, src.ctypes.data, edges.ctypes.data, C.addressof(ne), cap,
+                                         reserved.ctypes.data)
         self._check(n, "rpeg_eval_trace")
         return dict(start=start[:n], finish=finish[:n], order=order[:n], kind=kind[:n], vertex=vertex[:n], step=step[:n],
-                    sub=sub[:n], src=src[:n], edges=edges[:2 * ne.value].reshape(-1, 2))
+                    sub=sub[:n], src=src[:n], edges=edges[:2 * ne.value].reshape(-1, 2), reserved=reserved[:n])
 
     def device_exp(self, x: np.ndarray) -> np.ndarray:
         torch = _torch()

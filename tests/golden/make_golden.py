@@ -110,7 +110,8 @@ def reference_eval(mods, problem, batch, i):
     return dict(makespan=makespan.hex(), raw=raw.hex(), peak=float(max_peak).hex(), score=score.hex(),
                 feasible=feasible, n_nodes=len(lowered.nodes), n_edges=len(lowered.edges),
                 order_crc=zlib.crc32(order.encode()),
-                finish_sum=math.fsum(trace.finish.values()).hex()), lowered, cost, mm
+                finish_sum=math.fsum(trace.finish.values()).hex(),
+                utilization=float(trace.utilization()).hex(), n_active=trace.n_active()), lowered, cost, mm
 
 
 def node_vectors(lowered, cost, mm, limit):

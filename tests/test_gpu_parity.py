@@ -244,6 +244,25 @@ def test_device_exp_equals_host_libm():
     assert same_bits(y, want)
 
 
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_trace_utilization_and_active_devices_equal_reference(c):
+    """Trace.utilization() and Trace.n_active() of the drop-in evaluate(): the engine's start/finish times and
+    reserved allocations, folded on the host as the reference folds them, against the values the reference
+    computed from its own traces (tests/golden/ref_cfg*.json)."""
+    from rpeg_amd.search.evaluate import Configuration, evaluate
+    gold = load_golden(c)
+    cfg, batch = seeded_batch(c, gold["n"])
+    p = cfg.problem
+    for i in range(0, gold["n"], 16):
+        rpeg, plan, wl = batch.configuration(p, i)
+        score, trace, lowered = evaluate(Configuration(rpeg, plan, p.device_space), p.suite, wl, p.hw, p.K_eval,
+                                         p.memory_policy)
+        want = gold["plans"][i]
+        assert float(trace.utilization()).hex() == want["utilization"], i
+        assert trace.n_active() == want["n_active"], i
+        assert trace.makespan().hex() == want["makespan"], i
+
+
 def test_drop_in_calls():
     from rpeg_amd.search.evaluate import Configuration, _eval_worker, evaluate, evaluate_batch, evaluate_cached
     from rpeg_amd.search.cache import EvalCache

@@ -1,6 +1,7 @@
 """The Python oracle against vectors written by the reference implementation itself
 (tests/golden/make_golden.py): bit-exact makespan, raw score, worst device peak, penalised
-score, feasibility, lowered graph size and dispatch order."""
+score, feasibility, lowered graph size, dispatch order, mean device utilisation and number of active
+devices."""
 
 import math
 
@@ -30,6 +31,11 @@ def test_plans_match_reference(c):
         assert got["feasible"] == want["feasible"], i
         assert got["score"].hex() == want["score"], i
         assert math.fsum(got["finish"].values()).hex() == want["finish_sum"], i
+        if i % 4 == 0:   # Trace.utilization / Trace.n_active of the reference's own trace
+            reserved = oracle.reserved_by_node(got["nodes"], got["edges"])
+            util = oracle.utilization(got["start"], got["finish"], got["order"], reserved)
+            assert float(util).hex() == want["utilization"], i
+            assert oracle.n_active(got["nodes"]) == want["n_active"], i
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
