@@ -207,3 +207,29 @@ def test_annealing_argument_errors_and_edges():
     empty = [np.zeros((0, 6), np.int16)] * 6                                              # empty directory: placement and pair moves only
     res = optimize_chains(p, opt, 4, 20, [(0, 0)], engine=eng, directory=empty)
     assert not res.dead.any() and ((res.log >> 1) & 7).max() <= 1
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_start_plans_equal_the_reference_pipelines(c):
+    """The greedy, fully colocated and hand-partitioned start plans (RPEG/pipeline.py:389-435, 1051-1201)
+    from the engine's directory: same rows as the reference built on the same template, and where the
+    reference finds no plan, the same error with the same text."""
+    from rpeg_amd.search import baselines
+    with open(os.path.join(GOLDEN, "ref_baselines.json")) as f:
+        g = json.load(f)["configs"][str(c)]
+    p = configs.config(c).problem
+    rpeg0 = p.template(0, ())
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, engine(c))
+    for name, want in g.items():
+        build = getattr(baselines, name)
+        if "error" in want:
+            with pytest.raises(RuntimeError) as ex:
+                build(rpeg0, p.device_space, p.suite, p.workload, engine(c), table=table)
+            assert str(ex.value) == want["message"]
+            continue
+        plan = build(rpeg0, p.device_space, p.suite, p.workload, engine(c), table=table)
+        rows = [[*plan.pi[v], plan.mb[v], *plan.sigma[v].origin, *plan.sigma[v].extent] for v in rpeg0.vertices]
+        assert rows == want["rows"], name
+    # without a directory handed in the constructor builds its own
+    plan = baselines.build_valid_baseline_plan(rpeg0, p.device_space, p.suite, p.workload, engine(c))
+    assert [[*plan.pi[v], plan.mb[v]] for v in rpeg0.vertices] == [r[:4] for r in g["build_valid_baseline_plan"]["rows"]]
