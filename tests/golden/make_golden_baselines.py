@@ -1,6 +1,6 @@
 """Writes tests/golden/ref_baselines.json: the start plans the REFERENCE's pipeline builds before it calls
-optimize() (pipeline.py:389-435 greedy per-vertex plan, :1051-1108 fully colocated plan, :1111-1201 the
-hand-partitioned concurrent plan), for the templates of the benchmark configurations.
+optimize() (pipeline.py:389-435 greedy per-vertex plan, :437-1048 topology-aware concurrent plan, :1051-1108
+fully colocated plan, :1111-1201 the hand-partitioned concurrent plan), for the templates of the benchmark configurations.
 
 Run in the development container only (it needs the read-only reference tree):
 
@@ -9,15 +9,18 @@ Run in the development container only (it needs the read-only reference tree):
 pipeline.py is imported unmodified.  Its import chain reaches `search/evaluate.py` (does not parse; served by
 the record and function names make_golden_sa.py / make_golden_optimize.py register, none of which the three
 constructors call), `search/optimizer.py` (three names it uses in annotations are made visible) and
-`scripts/visualize.py` (plotting helpers, served by an empty module).  The constructors only use the
-reference's candidate directory, `packing_geometry` and the plan records.
+`scripts/visualize.py` (plotting helpers, served by an empty module).  The constructors use the reference's
+candidate directory, `packing_geometry`, the plan records and, for the concurrent plan, its lowering and
+memory check.
 """
 
 from __future__ import annotations
 
 import argparse
 import builtins
+import contextlib
 import importlib.util
+import io
 import json
 import os
 import sys
@@ -68,8 +71,30 @@ def main():
                 rec[name] = dict(rows=SA.plan_rows(rpeg, plan))
             except (RuntimeError, KeyError) as ex:
                 rec[name] = dict(error=type(ex).__name__, message=str(ex))
+        # the topology-aware plan (pipeline.py:908-1048): every plan it lowers for its memory check, with the
+        # verdict of that check, and what it returns.  The two names it calls are wrapped to listen in.
+        tried = []
+        real_lower, real_check = pipe.lower, pipe.mem_worst_violation
+
+        def lower(rpeg_, unrolled, plan, *a, **k):
+            tried.append(dict(rows=SA.plan_rows(rpeg_, plan)))
+            return real_lower(rpeg_, unrolled, plan, *a, **k)
+
+        def check(executable, mem_model):
+            v = real_check(executable, mem_model)
+            tried[-1]["peak_over_cap"] = None if v is None else float(v[1]).hex()
+            return v
+
+        pipe.lower, pipe.mem_worst_violation = lower, check
+        try:
+            with contextlib.redirect_stdout(io.StringIO()):
+                plan, found = pipe.build_concurrent_baseline_plan(rpeg, space, suite, wl, cost, mm)
+        finally:
+            pipe.lower, pipe.mem_worst_violation = real_lower, real_check
+        rec["build_concurrent_baseline_plan"] = dict(rows=SA.plan_rows(rpeg, plan), found=bool(found), tried=tried)
         doc["configs"][str(c)] = rec
-        print(c, {k: ("error " + v["error"]) if "error" in v else "ok" for k, v in rec.items()})
+        print(c, {k: ("error " + v["error"]) if "error" in v else "ok" for k, v in rec.items()},
+              "concurrent: found", found, "after", len(tried), "plans")
     path = os.path.join(HERE, "ref_baselines.json")
     with open(path, "w") as f:
         json.dump(doc, f, separators=(",", ":"))

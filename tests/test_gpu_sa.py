@@ -220,8 +220,8 @@ def test_start_plans_equal_the_reference_pipelines(c):
     p = configs.config(c).problem
     rpeg0 = p.template(0, ())
     table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, engine(c))
-    for name, want in g.items():
-        build = getattr(baselines, name)
+    for name in ("build_valid_baseline_plan", "build_fullycolocated_baseline_plan", "build_naive_concurrent_plan"):
+        want, build = g[name], getattr(baselines, name)
         if "error" in want:
             with pytest.raises(RuntimeError) as ex:
                 build(rpeg0, p.device_space, p.suite, p.workload, engine(c), table=table)
@@ -233,3 +233,43 @@ def test_start_plans_equal_the_reference_pipelines(c):
     # without a directory handed in the constructor builds its own
     plan = baselines.build_valid_baseline_plan(rpeg0, p.device_space, p.suite, p.workload, engine(c))
     assert [[*plan.pi[v], plan.mb[v]] for v in rpeg0.vertices] == [r[:4] for r in g["build_valid_baseline_plan"]["rows"]]
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_concurrent_start_plan_takes_the_reference_cascade(c):
+    """build_concurrent_baseline_plan (RPEG/pipeline.py:908-1048): the plans it would try are the plans the
+    reference lowered for its memory check, in the same order (1 to 473 of them; on config 3 all 345 fail and
+    the greedy plan is returned); the engine's peak of each failing one equals the peak the reference's K = 1
+    check reported, bit for bit; the returned plan and flag are the reference's."""
+    from rpeg_amd.engine.problem import PlanBatch
+    from rpeg_amd.search import baselines
+    with open(os.path.join(GOLDEN, "ref_baselines.json")) as f:
+        g = json.load(f)["configs"][str(c)]["build_concurrent_baseline_plan"]
+    p = configs.config(c).problem
+    rpeg0 = p.template(0, ())
+    eng = engine(c)
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, eng)
+
+    def rows(plan):
+        return [[*plan.pi[v], plan.mb[v], *plan.sigma[v].origin, *plan.sigma[v].extent] for v in rpeg0.vertices]
+
+    cascade = baselines.concurrent_plan_cascade(rpeg0, p.device_space, table)
+    tried = g["tried"]
+    assert len(cascade) >= len(tried)
+    assert [rows(pl) for pl, _, _ in cascade[:len(tried)]] == [t["rows"] for t in tried]
+    if not g["found"]:
+        assert len(cascade) == len(tried)
+
+    batch = PlanBatch.empty(len(tried))
+    taus = [int(rpeg0.tau[m]) for m in p.structures[0].tau_models]
+    for i, (pl, _, _) in enumerate(cascade[:len(tried)]):
+        batch.set_plan(i, 0, 1 if p.workload.gen_quantiles else 0, taus, rpeg0, pl)
+    out = eng.eval(batch, gate_stale=False)
+    for i, t in enumerate(tried):
+        fits = bool(out["mask"][i] & abi.MASK_MEM_OK)
+        assert fits == (t["peak_over_cap"] is None), i
+        if not fits:
+            assert float(out["peak"][i]).hex() == t["peak_over_cap"], i
+
+    plan, found = baselines.build_concurrent_baseline_plan(rpeg0, p.device_space, p.suite, p.workload, eng, table=table)
+    assert found == g["found"] and rows(plan) == g["rows"]

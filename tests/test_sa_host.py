@@ -180,3 +180,39 @@ def test_cxx_optimize_matches_reference_optimize():
         assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
         assert res["n_draws"] == case["n_draws"]
         assert _rows6(res["best_plan"], nv) == case["final"]
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_start_plan_host_logic_against_reference_vectors(c):
+    """The start-plan constructors are host logic over a candidate directory.  Fed the directory of the
+    Python restatement, the greedy plan and the cascade of the concurrent constructor (groups by depth,
+    partition enumeration, ranking, demotion order) equal what the reference built and lowered; every
+    partition with several allocations is pairwise disjoint and inside the device space."""
+    from rpeg_amd.search import baselines as B
+    with open(os.path.join(GOLDEN, "ref_baselines.json")) as f:
+        g = json.load(f)["configs"][str(c)]
+    p = configs.config(c).problem
+    rpeg0 = p.template(0, ())
+    table, _, _ = _directory(p, rpeg0)
+
+    def rows(plan):
+        return [[*plan.pi[v], plan.mb[v], *plan.sigma[v].origin, *plan.sigma[v].extent] for v in rpeg0.vertices]
+
+    assert rows(B.build_valid_baseline_plan(rpeg0, p.device_space, p.suite, p.workload, None, table=table)) \
+        == g["build_valid_baseline_plan"]["rows"]
+    tried = g["build_concurrent_baseline_plan"]["tried"]
+    cascade = B.concurrent_plan_cascade(rpeg0, p.device_space, table)
+    assert [rows(pl) for pl, _, _ in cascade[:len(tried)]] == [t["rows"] for t in tried]
+
+    sp = p.device_space
+    for group in B._find_concurrent_groups(rpeg0):
+        for part in B._enumerate_group_partitions(group, sp):
+            assert len(part) == len(group)
+            seen = set()
+            for a in set(part):
+                devs = {(r, n, d) for r in range(a.origin[0], a.origin[0] + a.extent[0])
+                        for n in range(a.origin[1], a.origin[1] + a.extent[1])
+                        for d in range(a.origin[2], a.origin[2] + a.extent[2])}
+                assert all(r < sp.R and n < sp.N and d < sp.G for r, n, d in devs)
+                assert not (devs & seen)
+                seen |= devs
