@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define RPEG_ABI_VERSION 1
+#define RPEG_ABI_VERSION 2
 
 #define RPEG_MAX_V 6       /* template vertices per structure                */
 #define RPEG_MAX_E 9       /* within-step data edges                          */
@@ -29,7 +29,7 @@ extern "C" {
 #define RPEG_MAX_PH 6      /* generation phases (quantiles)                   */
 #define RPEG_MAX_SPLIT 7   /* split variants: 0 = unsplit, j = quantiles[j-1:] */
 #define RPEG_MAX_MODEL 5
-#define RPEG_MAX_STRUCT 2
+#define RPEG_MAX_STRUCT 3
 #define RPEG_FIELDS 10     /* per-vertex plan fields: dp pp tp mb o_r o_n o_g e_r e_n e_g */
 
 enum { RPEG_ROLE_GEN = 0, RPEG_ROLE_INF = 1, RPEG_ROLE_TRAIN = 2 };
@@ -107,7 +107,13 @@ typedef struct rpeg_struct_s {
   rpeg_pair_t pair[RPEG_MAX_PAIR];     /* within_step_priors over the LIFO topological order (lower.py:135-220) */
   rpeg_rel_t rel[RPEG_MAX_REL];
   uint8_t reach[RPEG_MAX_V][RPEG_MAX_V];  /* transitive closure of data edges (lower.py:170-193) */
-  uint8_t trainable[RPEG_MAX_MODEL + 3];
+  uint8_t trainable[RPEG_MAX_MODEL + 3];      /* RPEG.trainable: what lowering sees (lower.py:626-793)          */
+  uint8_t mem_trainable[RPEG_MAX_MODEL + 3];  /* NodeMemoryModel.trainable: what the memory model sees
+                                                 (memory.py:647-790).  evaluate_cached builds it from the template
+                                                 (evaluate.py:378-385) and then the two agree; optimize() hands
+                                                 is_valid the memory model of its BASE configuration
+                                                 (optimizer.py:449-458), which for the AC-share template is another
+                                                 set: that view of a template is a structure of its own           */
 } rpeg_struct_t;
 
 typedef struct rpeg_phase_s { int32_t n_active, n_seqs, steps, t_start, prefill, pad; } rpeg_phase_t;
@@ -261,11 +267,40 @@ typedef struct rpeg_sa_serial_result_s {
   uint8_t* eval_log_variant; /*   rows of RPEG_MAX_V*RPEG_FIELDS values / their staleness variants       */
   int64_t eval_log_cap, n_eval_log;
   double wall_s;
+  int32_t best_family, pad;  /* family of best_plan (0 from rpeg_sa_optimize)                            */
 } rpeg_sa_serial_result_t;
 
 int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* params, int32_t E_max, int32_t E_struct,
                      int32_t R_max, uint64_t stream_a, uint64_t stream_b, uint64_t stream_c,
                      const int16_t* base_plan, rpeg_sa_serial_result_t* result, void* stream);
+
+/* The same loop over several structural families, one after the other, as optimize() walks
+   Iter_inter_model_candidates (RPEG/search/inter_model.py:68-121, optimizer.py:541-628): the separate
+   template with its staleness variants, then the AC-share template with its own.  (The intra-stage-fusion
+   settings in between are not entered: that pass does not run upstream.)  A family is a template
+   (params->structure), its staleness variants in the order they are walked (params->tau) and its candidate
+   directory (params->dir); the annealing settings are those of family 0.  `base_plan` is a plan of family
+   0's template with staleness `base_tau`; a family of another template starts from a random valid plan
+   and is skipped when 50 draws find none (optimizer.py:596-626).
+     score_scale      multiplies every score of the family before it is compared (1 - lambda_ac for
+                      AC-share, optimizer.py:132-145); elites keep raw scores
+     elite_family     families with the same number share their elites (optimizer.py:500-515)
+     valid_structure  structure whose memory verdict is_valid() uses for this family's plans: the
+                      reference checks restarts against the memory model of the base configuration
+                      (optimizer.py:449-458, 596-616, 640-663), see rpeg_struct_t.mem_trainable; equal to
+                      params->structure when the two models agree
+   result->best_variant counts within result->best_family; eval_log_variant holds family * 8 + variant,
+   and 255 for the base configuration when its staleness is not among family 0's variants. */
+typedef struct rpeg_sa_family_s {
+  const rpeg_sa_params_t* params;
+  double score_scale;
+  int32_t elite_family, valid_structure;
+} rpeg_sa_family_t;
+
+int rpeg_sa_optimize_families(rpeg_engine_t* e, int32_t n_families, const rpeg_sa_family_t* families,
+                              const uint8_t base_tau[2], int32_t E_max, int32_t E_struct, int32_t R_max,
+                              uint64_t stream_a, uint64_t stream_b, uint64_t stream_c, const int16_t* base_plan,
+                              rpeg_sa_serial_result_t* result, void* stream);
 
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,

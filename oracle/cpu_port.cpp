@@ -171,7 +171,7 @@ int port_op_time(void* h, uint64_t n, int structure, int vertex, const int16_t* 
 namespace {
 struct CpuSaBackend : SaBackend {
   Port* e;
-  uint8_t head_of[8][4];
+  uint8_t head_of[256][4] = {};
   int threads = 1;
   int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override {
     const size_t V = RPEG_MAX_V * RPEG_FIELDS;
@@ -220,25 +220,29 @@ int port_sa_run(void* h, const rpeg_sa_params_t* prm, const int16_t* base_plan, 
   return 0;
 }
 
-int port_sa_optimize(void* h, const rpeg_sa_params_t* prm, int32_t E_max, int32_t E_struct, int32_t R_max, uint64_t ka,
-                     uint64_t kb, uint64_t kc, const int16_t* base_plan, rpeg_sa_serial_result_t* res, int threads) {
+int port_sa_optimize_families(void* h, int32_t n_families, const rpeg_sa_family_t* families, const uint8_t* base_tau,
+                              int32_t E_max, int32_t E_struct, int32_t R_max, uint64_t ka, uint64_t kb, uint64_t kc,
+                              const int16_t* base_plan, rpeg_sa_serial_result_t* res, int threads) {
   Port* e = (Port*)h;
-  SaContext cx;
-  sa_context(e, prm, cx);
-  SaSettings st;
-  sa_settings_from(*prm, &st);
   CpuSaBackend be;
   be.e = e; be.threads = threads;
-  for (int k = 0; k < prm->n_variants; ++k) {
-    be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
-    be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];
-  }
-  SaSerial run(cx, st, be, E_max, E_struct, R_max, prm->seed, ka, kb, kc);
+  SaFamilySetup setup;
+  if (setup.init(e->P, n_families, families, base_tau, be.head_of)) return -1;
+  const rpeg_sa_params_t* prm = families[0].params;
+  SaSettings st;
+  sa_settings_from(*prm, &st);
+  SaSerial run(setup.fam, st, be, E_max, E_struct, R_max, prm->seed, ka, kb, kc);
   SaPlan base;
   std::memcpy(&base, base_plan, sizeof base);
-  if (int rc = run.run(base)) return rc;
+  if (int rc = run.run(base, setup.base_variant)) return rc;
   sa_serial_result(run, res);
   return 0;
+}
+
+int port_sa_optimize(void* h, const rpeg_sa_params_t* prm, int32_t E_max, int32_t E_struct, int32_t R_max, uint64_t ka,
+                     uint64_t kb, uint64_t kc, const int16_t* base_plan, rpeg_sa_serial_result_t* res, int threads) {
+  const rpeg_sa_family_t one{prm, 1.0, 0, prm->structure};
+  return port_sa_optimize_families(h, 1, &one, prm->tau[0], E_max, E_struct, R_max, ka, kb, kc, base_plan, res, threads);
 }
 
 // single proposals with the stream (seed, a, b, c): what = 0 move_gen, 1 pair, 2 region sample of vertex `v`

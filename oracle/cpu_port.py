@@ -34,6 +34,10 @@ def lib():
         _lib.port_sa_optimize.restype = C.c_int
         _lib.port_sa_optimize.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, C.c_uint64,
                                           C.c_uint64, C.c_void_p, C.c_void_p, C.c_int]
+        _lib.port_sa_optimize_families.restype = C.c_int
+        _lib.port_sa_optimize_families.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                                   C.c_int32, C.c_uint64, C.c_uint64, C.c_uint64, C.c_void_p, C.c_void_p,
+                                                   C.c_int]
         _lib.port_sa_propose.restype = C.c_int
         _lib.port_sa_propose.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_uint64,
                                          C.c_uint64, C.c_void_p, C.c_void_p, C.c_double, C.c_int, C.c_int, C.c_int,
@@ -140,6 +144,21 @@ class CpuPort:
                                     base.ctypes.data, C.addressof(res), threads)
         if rc != 0:
             raise RuntimeError(f"port_sa_optimize failed ({rc}): {lib().port_error(self.h).decode()}")
+        del keep
+        return serial_dict(res, log, logv)
+
+    def sa_optimize_families(self, families, base_tau, base_plan, E_max, E_struct, R_max=10000, stream_key=(0, 0, 0),
+                             log_cap=0, threads=1):
+        """SaSerial over several structural families (the CPU twin of rpeg_sa_optimize_families)."""
+        from rpeg_amd.engine.runtime import family_array, serial_dict, serial_result
+        arr, keep = family_array(families)
+        res, log, logv = serial_result(log_cap)
+        base = np.ascontiguousarray(base_plan, dtype=np.int16).reshape(abi.MAX_V * abi.FIELDS)
+        tau = (C.c_uint8 * 2)(*([int(t) for t in base_tau] + [0, 0])[:2])
+        rc = lib().port_sa_optimize_families(self.h, len(families), arr, tau, E_max, E_struct, R_max,
+                                             *[int(x) for x in stream_key], base.ctypes.data, C.addressof(res), threads)
+        if rc != 0:
+            raise RuntimeError(f"port_sa_optimize_families failed ({rc})")
         del keep
         return serial_dict(res, log, logv)
 

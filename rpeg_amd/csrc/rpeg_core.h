@@ -467,7 +467,7 @@ RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) 
   for (int i = 0; i < RPEG_MAX_V; ++i) { m.same_model[i] = m.train_same[i] = m.before[i] = 0; }
   for (int v = 0; v < st.n_vertex; ++v) {
     if (st.vertex[v].role == RPEG_ROLE_TRAIN) m.train |= (uint8_t)(1u << v);
-    if (st.trainable[st.vertex[v].model]) m.trainable |= (uint8_t)(1u << v);
+    if (st.mem_trainable[st.vertex[v].model]) m.trainable |= (uint8_t)(1u << v);
     for (int w = 0; w < st.n_vertex; ++w)
       if (st.vertex[w].model == st.vertex[v].model) {
         m.same_model[v] |= (uint8_t)(1u << w);

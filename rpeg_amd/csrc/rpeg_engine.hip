@@ -1238,7 +1238,7 @@ struct GpuSaBackend : SaBackend {
   rpeg_engine_t* e;
   hipStream_t s;
   int cap = 0;
-  uint8_t head_of[8][4];
+  uint8_t head_of[256][4] = {};
   int16_t *h_vert = nullptr, *d_vert = nullptr;
   uint8_t *h_head = nullptr, *d_head = nullptr, *h_mask = nullptr, *d_mask = nullptr;
   double *h_score = nullptr, *d_score = nullptr, *h_mass = nullptr, *d_mass = nullptr;
@@ -1371,43 +1371,44 @@ int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* ba
   return 0;
 }
 
-int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t E_max, int32_t E_struct, int32_t R_max,
-                     uint64_t stream_a, uint64_t stream_b, uint64_t stream_c, const int16_t* base_plan,
-                     rpeg_sa_serial_result_t* res, void* stream) {
-  if (!e || !prm || !res || !base_plan) return -1;
+int rpeg_sa_optimize_families(rpeg_engine_t* e, int32_t n_families, const rpeg_sa_family_t* families,
+                              const uint8_t base_tau[2], int32_t E_max, int32_t E_struct, int32_t R_max,
+                              uint64_t stream_a, uint64_t stream_b, uint64_t stream_c, const int16_t* base_plan,
+                              rpeg_sa_serial_result_t* res, void* stream) {
+  if (!e || !families || !base_tau || !res || !base_plan || n_families < 1 || !families[0].params) return -1;
   e->err.clear();
-  if (prm->structure < 0 || prm->structure >= e->P.n_struct || prm->split < 0 || prm->split >= e->P.n_split ||
-      prm->n_variants < 1 || prm->n_variants > 8 || prm->K_x < 1 || prm->K_x > 16 || prm->T_max < 0 ||
-      !(prm->T_init > 0.0) || E_max < 1 || E_struct < 1 || R_max < 1) {
+  const rpeg_sa_params_t* prm = families[0].params;
+  if (prm->K_x < 1 || prm->K_x > 16 || prm->T_max < 0 || !(prm->T_init > 0.0) || E_max < 1 || E_struct < 1 || R_max < 1) {
     e->err = "bad annealing parameters";
     return -1;
   }
-  SaContext cx;
-  cx.init(e->P, prm->structure);
-  for (int v = 0; v < cx.nv; ++v) {
-    if (prm->dir_n[v] < 0 || (prm->dir_n[v] > 0 && !prm->dir[v])) { e->err = "bad candidate directory"; return -1; }
-    if (const char* msg = cx.set_directory(v, prm->dir[v], prm->dir_n[v])) { e->err = msg; return -1; }
-  }
-  SaSettings st;
-  sa_settings_from(*prm, &st);
   GpuSaBackend be(e, (hipStream_t)stream, std::max(prm->K_x, 16));
   if (be.rc_alloc) return be.rc_alloc;
-  for (int k = 0; k < prm->n_variants; ++k) {
-    be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
-    be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];
-  }
-  SaSerial run(cx, st, be, E_max, E_struct, R_max, prm->seed, stream_a, stream_b, stream_c);
+  SaFamilySetup setup;
+  if (const char* msg = setup.init(e->P, n_families, families, base_tau, be.head_of)) { e->err = msg; return -1; }
+  SaSettings st;
+  sa_settings_from(*prm, &st);
+  SaSerial run(setup.fam, st, be, E_max, E_struct, R_max, prm->seed, stream_a, stream_b, stream_c);
   SaPlan base;
   std::memcpy(&base, base_plan, sizeof base);
   const auto t0 = std::chrono::steady_clock::now();
   const bool was_timing = e->timing;
   e->timing = false;
-  const int rc = run.run(base);
+  const int rc = run.run(base, setup.base_variant);
   e->timing = was_timing;
   if (rc) return rc;
   sa_serial_result(run, res);
   res->wall_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
   return 0;
+}
+
+int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t E_max, int32_t E_struct, int32_t R_max,
+                     uint64_t stream_a, uint64_t stream_b, uint64_t stream_c, const int16_t* base_plan,
+                     rpeg_sa_serial_result_t* res, void* stream) {
+  if (!e || !prm) return -1;
+  const rpeg_sa_family_t one{prm, 1.0, 0, prm->structure};
+  return rpeg_sa_optimize_families(e, 1, &one, prm->tau[0], E_max, E_struct, R_max, stream_a, stream_b, stream_c,
+                                   base_plan, res, stream);
 }
 
 int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream) {

@@ -552,7 +552,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     om.same_model = __ballot(valid && xi.model == xj.model);
     om.train_same = __ballot(valid && xi.model == xj.model && xj.role == RPEG_ROLE_TRAIN);
     const unsigned long long t = __ballot(valid && j == 0 && xi.role == RPEG_ROLE_TRAIN),
-                             tr = __ballot(valid && j == 0 && st.trainable[xi.model] != 0);   // bit 8i: position i
+                             tr = __ballot(valid && j == 0 && st.mem_trainable[xi.model] != 0);   // bit 8i: position i
     om.train = om.trainable = 0u;
 #pragma unroll
     for (int q = 0; q < RPEG_MAX_V; ++q) {

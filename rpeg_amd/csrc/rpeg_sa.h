@@ -18,6 +18,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <map>
 #include <set>
 #include <string>
 #include <unordered_map>
@@ -550,13 +551,26 @@ struct SaRun {
 };
 
 // ------------------------------------------------------------------------------------- one chain at a time
-// optimize() as the reference runs it (optimizer.py:365-946): the staleness variants one after the other,
-// each a sequence of restarts of ONE chain on one continuous random stream; an evaluation cache (hits cost
-// no budget and are merged before fresh results); the budgets E_max / E_struct counted in cache misses;
-// elites shared by the variants; warm restarts from the best elite plan, random restarts otherwise.  The
-// K_x candidates of a step are one batched evaluation.
+// optimize() as the reference runs it (optimizer.py:365-946): the structural families one after the other
+// (the separate template, then AC-share: inter_model.py:68-121 without the fused settings), within a family
+// its staleness variants one after the other, each a sequence of restarts of ONE chain on one continuous
+// random stream; an evaluation cache (hits cost no budget and are merged before fresh results); the
+// budgets E_max / E_struct counted in cache misses; elites shared by the variants of a family; warm
+// restarts from the best elite plan, random restarts otherwise.  The K_x candidates of a step are one
+// batched evaluation.
+struct SaFamily {
+  const SaContext* cx = nullptr;  // template and candidate directory
+  int first_variant = 0;          // backend variants first_variant .. first_variant + n_variants - 1, walked in order
+  int n_variants = 1;
+  int first_valid = 0;            // backend variants whose masks stand for is_valid(): the reference checks restarts
+                                  // with the memory model of the base configuration (optimizer.py:449-458), which can
+                                  // differ from the one evaluate_cached builds; == first_variant when they agree
+  double scale = 1.0;             // 1 - lambda_ac for the AC-share template (optimizer.py:132-145)
+  int elite_family = 0;           // families with one number share elites (optimizer.py:500-515)
+};
+
 struct SaSerial {
-  const SaContext& cx;
+  std::vector<SaFamily> fam;
   const SaSettings& p;
   SaBackend& be;
   int E_max, E_struct, R_max;
@@ -566,31 +580,33 @@ struct SaSerial {
   std::unordered_map<std::string, Stored> cache;
   std::vector<SaPlan> eval_log;          // every plan handed to the evaluator as a cache miss, in order
   std::vector<uint8_t> eval_log_variant;
-  std::vector<SaEntry> elite;
-  std::set<std::vector<int16_t>> seen;
+  std::map<int, std::vector<SaEntry>> elites;
+  std::map<int, std::set<std::vector<int16_t>>> seens;
   SaEntry best, best_feasible;
   int best_variant = 0, best_feasible_variant = 0;
   bool has_feasible = false;
   double best_score = 0.0, best_feasible_score = -INFINITY;
   long E = 0, n_uncounted = 0;
 
-  SaSerial(const SaContext& c, const SaSettings& s, SaBackend& b, int e_max, int e_struct, int r_max, uint64_t seed,
-           uint64_t ka, uint64_t kb, uint64_t kc)
-      : cx(c), p(s), be(b), E_max(e_max), E_struct(e_struct), R_max(r_max), rng(seed, ka, kb, kc) {}
+  SaSerial(const std::vector<SaFamily>& f, const SaSettings& s, SaBackend& b, int e_max, int e_struct, int r_max,
+           uint64_t seed, uint64_t ka, uint64_t kb, uint64_t kc)
+      : fam(f), p(s), be(b), E_max(e_max), E_struct(e_struct), R_max(r_max), rng(seed, ka, kb, kc) {}
 
   std::string key(const SaPlan& q, int variant) const {
     std::string k((const char*)&q, sizeof q);
     k.push_back((char)variant);
     return k;
   }
-  std::vector<int16_t> fingerprint(const SaPlan& q) const {
+  static std::vector<int16_t> fingerprint(const SaPlan& q, int nv) {
     std::vector<int16_t> fp;
-    for (int v = 0; v < cx.nv; ++v)
+    for (int v = 0; v < nv; ++v)
       for (int x : {SA_DP, SA_PP, SA_TP, SA_OR, SA_ON, SA_OG, SA_MB}) fp.push_back(q.f[v][x]);
     return fp;
   }
-  void elite_insert(double raw, const SaPlan& q, const SaEval& ev) {
-    auto fp = fingerprint(q);
+  void elite_insert(const SaFamily& f, double raw, const SaPlan& q, const SaEval& ev) {
+    std::vector<SaEntry>& elite = elites[f.elite_family];
+    std::set<std::vector<int16_t>>& seen = seens[f.elite_family];
+    auto fp = fingerprint(q, f.cx->nv);
     if (seen.count(fp)) return;
     if ((int)elite.size() >= p.K_elite && raw <= elite.back().ev.score) return;
     SaEntry e; e.plan = q; e.ev = ev; e.ev.score = raw;
@@ -603,11 +619,13 @@ struct SaSerial {
     return (m & RPEG_MASK_VALID) && (m & RPEG_MASK_STALE_OK) && (m & RPEG_MASK_MEM_OK) && !(m & RPEG_MASK_ERROR);
   }
   // is_valid (evaluate.py:143-232) costs no budget and does not touch the cache
-  int is_valid(const SaPlan& q, int variant, bool* ok) {
-    auto it = cache.find(key(q, variant));
-    if (it != cache.end()) { *ok = mask_valid(it->second.ev.mask); return 0; }
+  int is_valid(const SaPlan& q, int variant, int valid_variant, bool* ok) {
+    if (variant == valid_variant) {
+      auto it = cache.find(key(q, variant));
+      if (it != cache.end()) { *ok = mask_valid(it->second.ev.mask); return 0; }
+    }
     SaEval ev;
-    const uint8_t var = (uint8_t)variant;
+    const uint8_t var = (uint8_t)valid_variant;
     if (int rc = be.evaluate(1, &q, &var, &ev)) return rc;
     ++n_uncounted;
     *ok = mask_valid(ev.mask);
@@ -646,46 +664,58 @@ struct SaSerial {
     }
     return 0;
   }
-  void note(const SaPlan& q, const Stored& s, int variant) {   // optimizer.py:676-686, 846-861
-    if (s.feasible) elite_insert(s.score, q, s.ev);
-    if (s.score > best_score * (1.0 + p.score_eps)) { best.plan = q; best.ev = s.ev; best_score = s.score; best_variant = variant; }
-    if (s.feasible && s.score > best_feasible_score) {
-      has_feasible = true; best_feasible.plan = q; best_feasible.ev = s.ev; best_feasible_score = s.score;
+  // optimizer.py:676-686, 846-861; returns the score as the family compares it
+  double note(const SaFamily& f, const SaPlan& q, const Stored& s, int variant) {
+    const double score = s.score * f.scale;
+    if (s.feasible) elite_insert(f, s.score, q, s.ev);
+    if (score > best_score * (1.0 + p.score_eps)) { best.plan = q; best.ev = s.ev; best_score = score; best_variant = variant; }
+    if (s.feasible && score > best_feasible_score) {
+      has_feasible = true; best_feasible.plan = q; best_feasible.ev = s.ev; best_feasible_score = score;
       best_feasible_variant = variant;
     }
+    return score;
   }
   // optimizer.py:259-289 on the continuous stream
-  int random_restart(int variant, SaPlan* out, bool* found) {
+  int random_restart(const SaFamily& f, int variant, int valid_variant, SaPlan* out, bool* found) {
     *found = false;
     for (int a = 0; a < 50; ++a) {
       SaPlan q;
-      if (!sa_sample_all(rng, cx, &q)) return 0;
+      if (!sa_sample_all(rng, *f.cx, &q)) return 0;
       bool ok = false;
-      if (int rc = is_valid(q, variant, &ok)) return rc;
+      if (int rc = is_valid(q, variant, valid_variant, &ok)) return rc;
       if (ok) { *out = q; *found = true; return 0; }
     }
     return 0;
   }
 
-  int run(const SaPlan& base) {
+  // `base` is a plan of family 0's template; base_variant the backend variant of the base configuration
+  int run(const SaPlan& base, int base_variant) {
     std::vector<Stored> st;
     std::vector<char> miss;
-    if (int rc = evaluate(1, &base, 0, true, st, miss)) return rc;   // optimizer.py:466-478
-    best.plan = base; best.ev = st[0].ev; best_score = st[0].score; best_variant = 0;
+    if (int rc = evaluate(1, &base, base_variant, true, st, miss)) return rc;   // optimizer.py:466-478
+    best.plan = base; best.ev = st[0].ev; best_score = st[0].score; best_variant = base_variant;
     if (st[0].feasible) {
-      has_feasible = true; best_feasible = best; best_feasible_score = st[0].score; best_feasible_variant = 0;
-      elite_insert(st[0].score, base, st[0].ev);
+      has_feasible = true; best_feasible = best; best_feasible_score = st[0].score; best_feasible_variant = base_variant;
+      elite_insert(fam[0], st[0].score, base, st[0].ev);
     }
     E = 1;
     std::vector<SaPlan> cand(p.K_x);
-    for (int variant = 0; variant < p.n_variants; ++variant) {
+    for (const SaFamily& f : fam)
+     for (int k = 0; k < f.n_variants; ++k) {
+      const SaContext& cx = *f.cx;
+      const int variant = f.first_variant + k, valid_variant = f.first_valid + k;
+      const bool own_template = f.cx == fam[0].cx;
       SaPlan config = base;
       bool ok = false;
-      if (int rc = is_valid(base, variant, &ok)) return rc;
-      if (!ok) {   // optimizer.py:596-616
+      if (own_template)
+        if (int rc = is_valid(base, variant, valid_variant, &ok)) return rc;
+      if (!ok) {   // optimizer.py:596-626
         bool found = false;
-        if (int rc = random_restart(variant, &config, &found)) return rc;
-        if (!found) config = base;
+        if (int rc = random_restart(f, variant, valid_variant, &config, &found)) return rc;
+        if (!found) {
+          if (!own_template) continue;   // the base plan has no meaning on another template: setting skipped
+          config = base;
+        }
       }
       long E_s = 0;
       int r = 0, no_progress = 0;
@@ -695,14 +725,15 @@ struct SaSerial {
         const long restart_E_s = E_s;
         if (r > 0) {   // optimizer.py:640-663
           bool restarted = false;
+          const std::vector<SaEntry>& elite = elites[f.elite_family];
           if (!elite.empty()) {
             bool w_ok = false;
-            if (int rc = is_valid(elite[0].plan, variant, &w_ok)) return rc;
+            if (int rc = is_valid(elite[0].plan, variant, valid_variant, &w_ok)) return rc;
             if (w_ok) { config = elite[0].plan; restarted = true; }
           }
           if (!restarted) {
             bool found = false;
-            if (int rc = random_restart(variant, &config, &found)) return rc;
+            if (int rc = random_restart(f, variant, valid_variant, &config, &found)) return rc;
             if (!found) {
               ++r; ++no_progress;
               if (no_progress >= 2) exhausted = true;
@@ -712,10 +743,9 @@ struct SaSerial {
           no_progress = 0;
         }
         if (int rc = evaluate(1, &config, variant, true, st, miss)) return rc;
-        double score_curr = st[0].score;
         cur_ev = st[0].ev;
         if (miss[0]) { ++E; ++E_s; }
-        note(config, st[0], variant);
+        double score_curr = note(f, config, st[0], variant);
         double T = r > 0 ? p.T_warm : p.T_init;
         int rej = 0;
         while (true) {
@@ -737,8 +767,8 @@ struct SaSerial {
             for (int i = 0; i < nc; ++i) {
               if ((miss[i] != 0) != (pass == 1)) continue;
               if (miss[i]) { ++E; ++E_s; }
-              note(cand[i], st[i], variant);
-              if (st[i].score > bs) { bs = st[i].score; bi = i; }
+              const double sc = note(f, cand[i], st[i], variant);
+              if (sc > bs) { bs = sc; bi = i; }
             }
           if (E >= E_max) return 0;
           if (E_s >= E_struct) exhausted = true;
@@ -760,6 +790,55 @@ struct SaSerial {
       }
     }
     return 0;
+  }
+};
+
+// What rpeg_sa_optimize_families and its CPU twin share: contexts, families and the backend's variant table
+// (family f, variant k -> backend variant f * 8 + k for evaluation, 128 + f * 8 + k for is_valid; the base
+// configuration is the variant of family 0 with its staleness, else 255).  Returns an error text or null.
+struct SaFamilySetup {
+  std::vector<SaContext> cx;
+  std::vector<SaFamily> fam;
+  int base_variant = 0;
+  const char* init(const rpeg_problem_t& P, int n_families, const rpeg_sa_family_t* families, const uint8_t* base_tau,
+                   uint8_t (*head_of)[4]) {
+    if (n_families < 1 || n_families > 8 || !families) return "bad number of families";
+    cx.resize(n_families);
+    fam.resize(n_families);
+    for (int f = 0; f < n_families; ++f) {
+      const rpeg_sa_params_t* prm = families[f].params;
+      if (!prm) return "family without parameters";
+      const int vs = families[f].valid_structure;
+      if (prm->structure < 0 || prm->structure >= P.n_struct || vs < 0 || vs >= P.n_struct ||
+          P.st[vs].n_vertex != P.st[prm->structure].n_vertex || prm->split < 0 || prm->split >= P.n_split ||
+          prm->n_variants < 1 || prm->n_variants > 8)
+        return "bad family parameters";
+      cx[f].init(P, prm->structure);
+      for (int v = 0; v < cx[f].nv; ++v) {
+        if (prm->dir_n[v] < 0 || (prm->dir_n[v] > 0 && !prm->dir[v])) return "bad candidate directory";
+        if (const char* msg = cx[f].set_directory(v, prm->dir[v], prm->dir_n[v])) return msg;
+      }
+      fam[f].n_variants = prm->n_variants;
+      fam[f].first_variant = f * 8;
+      fam[f].first_valid = vs == prm->structure ? f * 8 : 128 + f * 8;
+      fam[f].scale = families[f].score_scale;
+      fam[f].elite_family = families[f].elite_family;
+      for (int k = 0; k < prm->n_variants; ++k) {
+        uint8_t* h = head_of[f * 8 + k];
+        h[0] = (uint8_t)prm->structure; h[1] = (uint8_t)prm->split; h[2] = prm->tau[k][0]; h[3] = prm->tau[k][1];
+        uint8_t* hv = head_of[128 + f * 8 + k];
+        hv[0] = (uint8_t)vs; hv[1] = h[1]; hv[2] = h[2]; hv[3] = h[3];
+      }
+    }
+    for (int f = 0; f < n_families; ++f) fam[f].cx = &cx[f];   // cx no longer moves
+    const rpeg_sa_params_t* p0 = families[0].params;
+    base_variant = 255;
+    uint8_t* hb = head_of[255];
+    hb[0] = (uint8_t)p0->structure; hb[1] = (uint8_t)p0->split; hb[2] = base_tau[0]; hb[3] = base_tau[1];
+    const int n_tau = P.st[p0->structure].n_tau;
+    for (int k = p0->n_variants - 1; k >= 0; --k)
+      if (p0->tau[k][0] == base_tau[0] && (n_tau < 2 || p0->tau[k][1] == base_tau[1])) base_variant = k;
+    return nullptr;
   }
 };
 
@@ -796,7 +875,14 @@ inline void sa_serial_result(const SaSerial& run, rpeg_sa_serial_result_t* res) 
   const bool feas = run.has_feasible;
   const SaEntry& b = feas ? run.best_feasible : run.best;
   std::memcpy(res->best_plan, &b.plan, sizeof(SaPlan));
-  res->best_variant = feas ? run.best_feasible_variant : run.best_variant;
+  const int bv = feas ? run.best_feasible_variant : run.best_variant;
+  res->best_family = 0;
+  res->best_variant = bv;   // the base configuration's own variant when no family holds it
+  for (size_t f = 0; f < run.fam.size(); ++f)
+    if (bv >= run.fam[f].first_variant && bv < run.fam[f].first_variant + run.fam[f].n_variants) {
+      res->best_family = (int32_t)f;
+      res->best_variant = bv - run.fam[f].first_variant;
+    }
   res->best_score = feas ? run.best_feasible_score : run.best_score;
   res->best_feasible = feas;
   res->E = run.E;

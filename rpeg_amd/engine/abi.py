@@ -2,8 +2,8 @@
 
 import ctypes as C
 
-ABI_VERSION = 1
-MAX_V, MAX_E, MAX_PUB, MAX_PAIR, MAX_REL, MAX_PH, MAX_SPLIT, MAX_MODEL, MAX_STRUCT = 6, 9, 2, 4, 13, 6, 7, 5, 2
+ABI_VERSION = 2
+MAX_V, MAX_E, MAX_PUB, MAX_PAIR, MAX_REL, MAX_PH, MAX_SPLIT, MAX_MODEL, MAX_STRUCT = 6, 9, 2, 4, 13, 6, 7, 5, 3
 FIELDS = 10
 ROLE = {"GEN": 0, "INF": 1, "TRAIN": 2}
 MODEL = {"Pi": 0, "V": 1, "Ref": 2, "R": 3, "AC": 4}
@@ -57,7 +57,8 @@ class StructT(C.Structure):
                 ("n_rel", C.c_int32), ("n_tau", C.c_int32),
                 ("vertex", VertexT * MAX_V), ("edge", EdgeT * MAX_E), ("pub", PubT * MAX_PUB),
                 ("pair", PairT * MAX_PAIR), ("rel", RelT * MAX_REL),
-                ("reach", (C.c_uint8 * MAX_V) * MAX_V), ("trainable", C.c_uint8 * (MAX_MODEL + 3))]
+                ("reach", (C.c_uint8 * MAX_V) * MAX_V), ("trainable", C.c_uint8 * (MAX_MODEL + 3)),
+                ("mem_trainable", C.c_uint8 * (MAX_MODEL + 3))]
 
 
 class PhaseT(C.Structure):
@@ -105,4 +106,9 @@ class SaSerialResultT(C.Structure):
     _fields_ = [("best_plan", C.c_int16 * (MAX_V * FIELDS)), ("best_variant", C.c_int32), ("best_feasible", C.c_int32),
                 ("best_score", C.c_double), ("E", C.c_int64), ("n_draws", C.c_int64), ("n_uncounted", C.c_int64),
                 ("eval_log", C.c_void_p), ("eval_log_variant", C.c_void_p), ("eval_log_cap", C.c_int64),
-                ("n_eval_log", C.c_int64), ("wall_s", C.c_double)]
+                ("n_eval_log", C.c_int64), ("wall_s", C.c_double), ("best_family", C.c_int32), ("pad", C.c_int32)]
+
+
+class SaFamilyT(C.Structure):
+    _fields_ = [("params", C.c_void_p), ("score_scale", C.c_double), ("elite_family", C.c_int32),
+                ("valid_structure", C.c_int32)]

@@ -188,6 +188,8 @@ def compile_problem(problem: EvalProblem) -> abi.ProblemT:
             raise ValueError("structure tau_models must list exactly the trainable models")
         for m in rpeg.trainable:
             S_.trainable[abi.MODEL[m.value]] = 1
+        for m in (rpeg.trainable if structure.memory_trainable is None else structure.memory_trainable):
+            S_.mem_trainable[abi.MODEL[m.value]] = 1
         sorted_ids = sorted(v.id for v in rpeg.vertices)
         for i, v in enumerate(rpeg.vertices):
             rec = S_.vertex[i]

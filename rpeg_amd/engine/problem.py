@@ -16,7 +16,7 @@ per-call argument of `evaluate` (RPEG/search/evaluate.py:235-241).
 from __future__ import annotations
 
 from dataclasses import dataclass, field, replace
-from typing import Callable, Dict, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, FrozenSet, List, Optional, Sequence, Tuple
 
 import numpy as np
 
@@ -43,6 +43,11 @@ class Structure:
     name: str
     build: Callable[..., RPEG]
     tau_models: Tuple[Model, ...]
+    # The models the MEMORY model treats as trainable when that is not the template's own set.  The
+    # reference's evaluate_cached builds its memory model from the template (evaluate.py:378-385), but
+    # optimize() checks restarts (is_valid) with the memory model of its base configuration
+    # (optimizer.py:449-458): under that model the AC-share template's shared model counts as frozen.
+    memory_trainable: Optional[FrozenSet[Model]] = None
 
 
 PPO = Structure("ppo", build_PPO_RPEG, (Model.ACTOR, Model.CRITIC))
@@ -50,6 +55,12 @@ GRPO = Structure("grpo", build_GRPO_RPEG, (Model.ACTOR,))
 DPO = Structure("dpo", build_DPO_RPEG, (Model.ACTOR,))
 AC_SHARE = Structure("ac_share", build_AC_share_RPEG, (Model.AC_SHARE,))
 STRUCTURES = {s.name: s for s in (PPO, GRPO, DPO, AC_SHARE)}
+
+
+def as_seen_from(structure: Structure, base: Structure) -> Structure:
+    """`structure` under the memory model of a configuration of `base` (what is_valid sees inside
+    optimize(), RPEG/search/optimizer.py:449-458, 596-663)."""
+    return replace(structure, memory_trainable=frozenset(base.tau_models))
 
 
 @dataclass(frozen=True)

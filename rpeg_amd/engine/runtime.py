@@ -23,7 +23,8 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host")
+           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_optimize_families")
 
 
 class EngineError(RuntimeError):
@@ -56,6 +57,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_sa_run.argtypes = [vp, vp, vp, vp, vp]
     lib.rpeg_sa_optimize.restype = C.c_int
     lib.rpeg_sa_optimize.argtypes = [vp, vp, i32, i32, i32, u64, u64, u64, vp, vp, vp]
+    lib.rpeg_sa_optimize_families.restype = C.c_int
+    lib.rpeg_sa_optimize_families.argtypes = [vp, i32, vp, vp, i32, i32, i32, u64, u64, u64, vp, vp, vp]
     lib.rpeg_op_time_batch.restype = C.c_int
     lib.rpeg_op_time_batch.argtypes = [vp, u64, i32, i32, vp, u64, vp, vp, vp]
     lib.rpeg_eval_trace.restype = C.c_int
@@ -94,6 +97,20 @@ def set_directory(params: "abi.SaParamsT", directory):
     return keep
 
 
+def family_array(families):
+    """rpeg_sa_family_t[] from [(params, directory, score_scale, elite_family, valid_structure)]; returns
+    (array, objects to keep alive)."""
+    arr = (abi.SaFamilyT * len(families))()
+    keep = []
+    for f, (params, directory, scale, elite_family, valid_structure) in enumerate(families):
+        keep.append((params, set_directory(params, directory)))
+        arr[f].params = C.addressof(params)
+        arr[f].score_scale = float(scale)
+        arr[f].elite_family = int(elite_family)
+        arr[f].valid_structure = int(params.structure if valid_structure is None else valid_structure)
+    return arr, keep
+
+
 def serial_result(log_cap: int):
     res = abi.SaSerialResultT()
     log = np.zeros((max(log_cap, 1), abi.MAX_V * abi.FIELDS), np.int16)
@@ -106,7 +123,7 @@ def serial_dict(res, log, logv):
     n = min(res.n_eval_log, res.eval_log_cap)
     return dict(best_plan=np.array(res.best_plan, dtype=np.int16), best_variant=res.best_variant,
                 best_feasible=bool(res.best_feasible), best_score=res.best_score, E=res.E, n_draws=res.n_draws,
-                n_uncounted=res.n_uncounted, n_eval_log=res.n_eval_log, eval_log=log[:n].copy(),
+                best_family=res.best_family, n_uncounted=res.n_uncounted, n_eval_log=res.n_eval_log, eval_log=log[:n].copy(),
                 eval_log_variant=logv[:n].copy(), wall_s=res.wall_s)
 
 
@@ -291,6 +308,25 @@ class Engine:
             rc = self.lib.rpeg_sa_optimize(self._h, C.addressof(params), E_max, E_struct, R_max,
                                            *[int(x) for x in stream_key], base.ctypes.data, C.addressof(res), stream)
         self._check(rc, "rpeg_sa_optimize")
+        del keep
+        return serial_dict(res, log, logv)
+
+    def sa_optimize_families(self, families, base_tau, base_plan: np.ndarray, E_max: int, E_struct: int,
+                             R_max: int = 10000, stream_key=(0, 0, 0), log_cap: int = 0) -> Dict[str, object]:
+        """optimize() over several structural families (rpeg_sa_optimize_families).  `families` is a list of
+        (params, directory, score_scale, elite_family, valid_structure or None); `base_plan` belongs to
+        family 0's template and has staleness `base_tau`."""
+        torch = _torch()
+        arr, keep = family_array(families)
+        res, log, logv = serial_result(log_cap)
+        base = np.ascontiguousarray(base_plan, dtype=np.int16).reshape(abi.MAX_V * abi.FIELDS)
+        tau = (C.c_uint8 * 2)(*([int(t) for t in base_tau] + [0, 0])[:2])
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_sa_optimize_families(self._h, len(families), arr, tau, E_max, E_struct, R_max,
+                                                    *[int(x) for x in stream_key], base.ctypes.data,
+                                                    C.addressof(res), stream)
+        self._check(rc, "rpeg_sa_optimize_families")
         del keep
         return serial_dict(res, log, logv)
 
