@@ -89,13 +89,17 @@ _TEMPLATE_IDS = {"ppo": ("g_pi", "i_ref", "i_R", "i_V", "t_pi", "t_V"), "grpo": 
 
 
 def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware, space: DeviceSpace, K_eval: int,
-                policy: MemoryPolicy):
+                policy: MemoryPolicy, more_structures=()):
+    """(engine, structure of `rpeg`): one engine per problem, kept for the life of the process.  The
+    structure of `rpeg` is structure 0 of the engine, `more_structures` follow."""
     from ..engine.runtime import Engine
     st = _structure_of(rpeg)
-    key = (st.name, tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
+    structures = (st,) + tuple(more_structures)
+    key = (tuple((s.name, s.memory_trainable) for s in structures),
+           tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
     eng = _engines.get(key)
     if eng is None:
-        problem = EvalProblem(structures=(st,), suite=suite, workload=workload, hw=hw, device_space=space,
+        problem = EvalProblem(structures=structures, suite=suite, workload=workload, hw=hw, device_space=space,
                               K_eval=K_eval, memory_policy=policy)
         eng = _engines[key] = Engine(problem)
     return eng, st

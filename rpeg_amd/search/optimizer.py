@@ -181,39 +181,86 @@ def _iter_staleness(tau_models, t_cand) -> List[Tuple[int, ...]]:
     return [tuple(c) for c in itertools.product(*[sorted(t_cand[m]) for m in tau_models])]
 
 
+def optimize_families(problem: EvalProblem, opt_config: OptimizerConfig, engine_directory) -> List[tuple]:
+    """The structural families optimize() walks for structure 0 of `problem`, in the reference's order
+    (RPEG/search/inter_model.py:68-121 filtered by `structural_candidates`, optimizer.py:541-553): the
+    separate template with the staleness variants of T_cand, then -- for a template that trains an actor
+    and a critic, when `problem` holds the AC-share template as structure 1 and its view under the base
+    configuration's memory model as structure 2 -- AC-share with its own, scored times (1 - lambda_ac).
+    The fused settings are not entered (that lowering pass does not run upstream).  Returns the list
+    Engine.sa_optimize_families takes; `engine_directory(structure)` supplies the candidate directory."""
+    t_cand = opt_config.T_cand if opt_config.T_cand is not None else DEFAULT_T_CAND
+    names = opt_config.structural_candidates
+    split = 1 if problem.workload.gen_quantiles else 0
+    st = problem.structures[0]
+    families = []
+    if names is None or "separate" in names:
+        variants = _iter_staleness(st.tau_models, t_cand)
+        if variants:
+            families.append((sa_params(opt_config, 1, 1, variants, 0, split, 0), engine_directory(0), 1.0, 0, None))
+    shares = set(st.tau_models) >= {Model.ACTOR, Model.CRITIC}      # is_AC_share_applicable (ir/ac_share.py:17-26)
+    if shares and len(problem.structures) >= 3 and (names is None or "ac_share" in names):
+        ac = problem.structures[1]
+        variants = _iter_staleness(ac.tau_models, t_cand)
+        if variants:
+            scale = 1.0 - opt_config.lambda_ac if opt_config.lambda_ac != 0.0 else 1.0
+            families.append((sa_params(opt_config, 1, 1, variants, 1, split, 0), engine_directory(1), scale, 1, 2))
+    if not families:
+        raise ValueError("structural_candidates exclude every inter-model candidate for "
+                         f"algorithm={opt_config.algorithm}")
+    return families
+
+
 def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
              opt_config: OptimizerConfig, cache: Optional[EvalCache] = None, seed: int = 42,
              stream_key: Sequence[int] = (0, 0, 0)) -> Configuration:
     """Drop-in for optimize() (RPEG/search/optimizer.py:365-946) on the template of `base_config`.
 
-    Runs the reference's loop (rpeg_sa_optimize): the staleness variants of T_cand one after the other,
-    the base configuration's own staleness first; per variant a sequence of restarts of one chain, with
-    the evaluation cache, the budgets E_max / E_struct, the elites and the warm restarts of the reference.
-    The K_x candidates of an iteration are one GPU launch.  Given the same random generator the reference
-    evaluates the same plans in the same order and returns the same plan (tests/golden/make_golden_optimize.py);
-    the generator here is the counter-based stream (seed, *stream_key), not MT19937.
+    Runs the reference's loop (rpeg_sa_optimize_families): the structural families one after the other --
+    the template of `base_config` with the staleness variants of T_cand, then, for a PPO template, the
+    AC-share template with its own, scored times (1 - lambda_ac) -- and per variant a sequence of restarts
+    of one chain, with the evaluation cache, the budgets E_max / E_struct, the per-family elites and the
+    warm restarts of the reference.  The K_x candidates of an iteration are one GPU launch.  Given the same
+    random generator the reference evaluates the same plans in the same order and returns the same
+    configuration (tests/golden/make_golden_optimize.py); the generator here is the counter-based stream
+    (seed, *stream_key), not MT19937.
 
-    Not entered: the AC-share and intra-stage-fusion structures (`structural_candidates` other than
-    "separate"), deadlines, the utilisation objective.  `cache` is accepted for signature compatibility:
-    the run keeps its own cache (keyed by plan and staleness variant)."""
+    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused"), deadlines, the
+    utilisation objective.  `cache` is accepted for signature compatibility: the run keeps its own cache
+    (keyed by plan, template and staleness)."""
+    from ..engine.problem import STRUCTURES, as_seen_from
     _check_supported(base_config)
     if opt_config.max_throughput_loss > 0.0 or opt_config.deadline is not None:
         raise NotImplementedError("utilisation objective and deadlines are not part of this engine")
     policy = opt_config.memory_policy()
-    eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy)
-    t_cand = opt_config.T_cand if opt_config.T_cand is not None else DEFAULT_T_CAND
-    own = tuple(int(base_config.rpeg.tau.get(m, 0)) for m in st.tau_models)
-    variants = [own] + [v for v in _iter_staleness(st.tau_models, t_cand) if v != own]
-    if own not in _iter_staleness(st.tau_models, t_cand):
-        variants = variants[1:] or [own]
-    rpeg0 = eng.problem.template(0, ())
-    table, _ = build_candidate_directory(rpeg0, suite, base_config.device_space, workload, eng)
-    split = 1 if workload.gen_quantiles else 0
-    params = sa_params(opt_config, 1, 1, variants, 0, split, seed)
-    res = eng.sa_optimize(params, directory_arrays(rpeg0, table), plan_row(base_config.rpeg, base_config.plan),
-                          opt_config.E_max, opt_config.E_struct, opt_config.R_max, stream_key)
-    tau = {m: variants[res["best_variant"]][i] for i, m in enumerate(st.tau_models)}
-    rpeg = st.build(suite, workload, tau=tau)
+    st = _structure_of(base_config.rpeg)
+    names = opt_config.structural_candidates
+    more = ()
+    if set(st.tau_models) >= {Model.ACTOR, Model.CRITIC} and (names is None or "ac_share" in names):
+        more = (STRUCTURES["ac_share"], as_seen_from(STRUCTURES["ac_share"], st))
+    eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy, more)
+
+    def directory(structure: int):
+        rpeg = eng.problem.template(structure, ())
+        table, _ = build_candidate_directory(rpeg, suite, base_config.device_space, workload, eng, structure)
+        return directory_arrays(rpeg, table)
+
+    families = optimize_families(eng.problem, opt_config, directory)
+    families[0][0].seed = seed
+    own = [int(base_config.rpeg.tau.get(m, 0)) for m in st.tau_models]
+    res = eng.sa_optimize_families(families, own, plan_row(base_config.rpeg, base_config.plan), opt_config.E_max,
+                                   opt_config.E_struct, opt_config.R_max, stream_key)
+    return configuration_of(eng.problem, families, res, own, suite, workload, base_config)
+
+
+def configuration_of(problem: EvalProblem, families, res, base_tau, suite, workload, base_config) -> Configuration:
+    """The configuration a result of sa_optimize_families names: template of the best family, staleness of
+    its best variant (the base configuration's own when that is what was best), best plan."""
+    params = families[res["best_family"]][0]
+    st = problem.structures[params.structure]
+    k = res["best_variant"]
+    taus = list(base_tau) if k >= params.n_variants else [int(params.tau[k][i]) for i in range(len(st.tau_models))]
+    rpeg = st.build(suite, workload, tau={m: taus[i] for i, m in enumerate(st.tau_models)})
     return Configuration(rpeg, row_plan(rpeg, res["best_plan"]), base_config.device_space,
                          intra_stage_fusion=False, transfer_resource_policy=base_config.transfer_resource_policy)
 

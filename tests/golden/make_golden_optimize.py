@@ -1,6 +1,7 @@
-"""Writes tests/golden/ref_optimize.json: the trajectory of the REFERENCE's optimize()
-(RPEG/search/optimizer.py:365-946) for one structural setting of config 1, driven by the counter-based
-generator instead of MT19937.
+"""Writes tests/golden/ref_optimize.json: trajectories of the REFERENCE's optimize()
+(RPEG/search/optimizer.py:365-946) on config 1, driven by the counter-based generator instead of MT19937:
+two cases with one structural setting, and cases that walk the separate template's staleness variants and
+then the AC-share template's (structural_candidates "separate" and "ac_share", lambda_ac > 0).
 
 Run in the development container only (it needs the read-only reference tree):
 
@@ -13,7 +14,10 @@ and :396-401, stale-layout rule :115-140, validity rules :143-232, cache key :30
 attribute `random` of optimizer.py and of moves.py is pointed at ONE generator object, and
 `os.cpu_count` reports one core while optimize() runs so that it evaluates candidates in-process, in
 order.  The file records every plan handed to an evaluation function (cache misses only), in order, and
-the plan optimize() returns: the restatement must evaluate the same plans in the same order.
+the plan optimize() returns: the restatement must evaluate the same plans in the same order.  Like the
+reference's evaluate_cached (evaluate.py:378-385) the evaluation functions here build the memory model from
+the evaluated configuration's own template, while `is_valid` receives the one optimize() built from its base
+configuration (optimizer.py:449-458) -- for AC-share plans these differ, and the trajectory depends on it.
 """
 
 from __future__ import annotations
@@ -36,7 +40,16 @@ import make_golden as MG      # noqa: E402
 import make_golden_sa as SA   # noqa: E402
 
 CASES = [dict(plan=0, stream=(42, 77, 0, 0), E_max=260, E_struct=200, stag_window=4, T_init=0.05, T_min=0.05, T_warm=0.10),
-         dict(plan=2, stream=(42, 77, 1, 0), E_max=150, E_struct=400, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05)]
+         dict(plan=2, stream=(42, 77, 1, 0), E_max=150, E_struct=400, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05),
+         # structural families: T_cand as (actor, critic, shared), base staleness, AC-share penalty
+         dict(plan=0, stream=(42, 77, 2, 0), E_max=420, E_struct=70, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
+              families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05),
+         dict(plan=2, stream=(42, 77, 3, 0), E_max=300, E_struct=60, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
+              families=True, T_cand=[[0, 1], [0], [1, 0]], base_tau=[1, 0], lambda_ac=0.0),
+         # tight memory: is_valid's verdict on AC-share restarts (base configuration's memory model) and the
+         # evaluation's (the template's own) disagree, and the trajectory shows which one the reference asks
+         dict(plan=0, stream=(42, 77, 4, 0), E_max=420, E_struct=70, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
+              families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05, memory_per_gpu=1.25e10)]
 
 
 def main():
@@ -55,17 +68,36 @@ def main():
     def rows(config):
         return SA.plan_rows(config.rpeg, config.plan)
 
+    def memory_model(rpeg):
+        key = tuple(sorted(m.value for m in rpeg.trainable))
+        if key not in st["mms"]:
+            pol, mem_mod = st["problem"].memory_policy, mods["model.memory"]
+            st["mms"][key] = mem_mod.NodeMemoryModel.from_policy(
+                st["hw"], st["suite"], st["wl"], mem_mod.MemoryPolicy(
+                    optimizer_stage=pol.optimizer_stage, activation_checkpointing=pol.activation_checkpointing,
+                    runtime_overhead_fraction=pol.runtime_overhead_fraction,
+                    worker_overhead_bytes=pol.worker_overhead_bytes,
+                    semantic_activation_cache_bytes=pol.semantic_activation_cache_bytes,
+                    max_worker_groups_per_gpu=pol.max_worker_groups_per_gpu),
+                trainable=frozenset(rpeg.trainable),
+                shadow_models=frozenset(m for m in rpeg.trainable if rpeg.tau.get(m, 0) > 0))
+        return st["mms"][key]
+
     def _eval(config, gate):
         p = st["problem"]
         rpeg, plan, wl = config.rpeg, config.plan, st["wl"]
-        st["log"].append(rows(config))
+        if st["families"]:
+            st["log"].append([[v.id for v in rpeg.vertices][0], [rpeg.tau[m] for m in sorted(rpeg.tau, key=lambda m: m.value)],
+                              rows(config)])
+        else:
+            st["log"].append(rows(config))
         unrolled = mods["passes.unroll"].unroll(rpeg, p.K_eval)
         lowered = mods["passes.lower"].lower(rpeg, unrolled, plan, st["suite"], p.K_eval, workload=wl)
         trace = mods["schedule.scheduler"].schedule(lowered, st["cost"], st["space"])
         raw = trace.throughput(W_step=wl.B * wl.K * (wl.S + wl.T), K=p.K_eval)
         if gate and not O.stale_publication_layout_valid(rpeg, plan):
             return 0.0, trace, False
-        violation = mods["model.memory"].mem_worst_violation(lowered, st["mm"])
+        violation = mods["model.memory"].mem_worst_violation(lowered, memory_model(rpeg))
         if violation is None:
             return raw, trace, True
         _, req, cap = violation
@@ -88,6 +120,8 @@ def main():
 
     def is_valid(config, suite, workload, mem_model):
         rpeg, plan = config.rpeg, config.plan
+        if any(v not in plan.sigma or v not in plan.pi or v not in plan.mb for v in rpeg.vertices):
+            return False                      # evaluate.py:165-170: coverage first
         if not O.plan_structurally_valid(rpeg, plan, config.device_space, suite, workload):
             return False
         if not O.stale_publication_layout_valid(rpeg, plan):
@@ -106,19 +140,36 @@ def main():
     cfg = configs.config(1)
     p = cfg.problem
     rpeg0, suite, wl, hw, space, cost, mm = SA.ref_world(mods, p, {"Pi": 0, "V": 0})
-    st.update(problem=p, suite=suite, wl=wl, space=space, cost=cost, mm=mm, log=[])
+    st.update(problem=p, suite=suite, wl=wl, hw=hw, space=space, cost=cost, mm=mm, mms={}, log=[], families=False)
     batch = candidates.generate(p, 8, cfg.tau_choices, seed=42, tag=1)
     Model = ct.Model
     doc = {"cases": []}
     real_cpu_count = os.cpu_count
+    import dataclasses
+    p_config = p
     for case in CASES:
+        if "memory_per_gpu" in case:
+            p = dataclasses.replace(p_config, hw=dataclasses.replace(p_config.hw, memory_per_gpu=case["memory_per_gpu"]))
+            rpeg0, suite, wl, hw, space, cost, mm = SA.ref_world(mods, p, {"Pi": 0, "V": 0})
+            st.update(problem=p, suite=suite, wl=wl, hw=hw, space=space, cost=cost, mm=mm, mms={})
         plan = SA.ref_plan(mods, rpeg0, batch, p, case["plan"])
-        base = Configuration(rpeg0, plan, space)
-        assert is_valid(base, suite, wl, mm), "the base plan must be valid"
-        oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
-                                  T_cand={Model.ACTOR: {0}, Model.CRITIC: {0}, Model.AC_SHARE: set()},
-                                  structural_candidates=frozenset({"separate"}), T_init=case["T_init"],
-                                  T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"])
+        st["families"] = bool(case.get("families"))
+        if st["families"]:
+            base_rpeg = dataclasses.replace(rpeg0, tau={Model.ACTOR: case["base_tau"][0], Model.CRITIC: case["base_tau"][1]})
+            base = Configuration(base_rpeg, plan, space)
+            a, c, s_ = case["T_cand"]
+            oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
+                                      T_cand={Model.ACTOR: set(a), Model.CRITIC: set(c), Model.AC_SHARE: set(s_)},
+                                      structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"],
+                                      T_init=case["T_init"], T_warm=case["T_warm"], T_min=case["T_min"],
+                                      stag_window=case["stag_window"])
+        else:
+            base = Configuration(rpeg0, plan, space)
+            assert is_valid(base, suite, wl, mm), "the base plan must be valid"
+            oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
+                                      T_cand={Model.ACTOR: {0}, Model.CRITIC: {0}, Model.AC_SHARE: set()},
+                                      structural_candidates=frozenset({"separate"}), T_init=case["T_init"],
+                                      T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"])
         rng = CounterRng(*case["stream"])
         ropt.random = rng
         moves.random = rng
@@ -131,8 +182,14 @@ def main():
         log = st["log"]
         doc["cases"].append(dict(case, stream=list(case["stream"]), T_cool=oc.T_cool.hex(), n_eval=len(log),
                                  n_draws=rng.k, eval_crc=zlib.crc32(json.dumps(log, separators=(",", ":")).encode()),
-                                 first=log[:8], final=rows(out)))
-        print("case", case["plan"], "evaluations", len(log), "draws", rng.k)
+                                 first=log[:8], final=rows(out), final_first_vertex=out.rpeg.vertices[0].id,
+                                 final_tau=[out.rpeg.tau[m] for m in sorted(out.rpeg.tau, key=lambda m: m.value)]))
+        if st["families"]:
+            import collections
+            doc["cases"][-1]["per_setting"] = [[k[0], list(k[1]), n] for k, n in collections.Counter(
+                (e[0], tuple(e[1])) for e in log).items()]
+        print("case", case["plan"], "evaluations", len(log), "draws", rng.k, doc["cases"][-1].get("per_setting", ""),
+              "->", doc["cases"][-1]["final_first_vertex"], doc["cases"][-1]["final_tau"])
     path = os.path.join(HERE, "ref_optimize.json")
     with open(path, "w") as f:
         json.dump(doc, f, separators=(",", ":"))

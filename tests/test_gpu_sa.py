@@ -14,7 +14,7 @@ from rpeg_amd import configs
 from rpeg_amd.engine import abi
 from rpeg_amd.search.moves import build_candidate_directory, directory_arrays
 from rpeg_amd.search.optimizer import OptimizerConfig, optimize_chains, sa_params
-from tests.helpers import GOLDEN, seeded_batch
+from tests.helpers import GOLDEN, check_family_case, family_case_setup, family_problem, seeded_batch
 
 pytestmark = pytest.mark.gpu
 
@@ -164,7 +164,7 @@ def test_optimize_equals_reference_trajectory():
 
     def rows(r):
         return [[int(x) for x in r[v * 10:(v + 1) * 10]] for v in range(nv)]
-    for case in g["cases"]:
+    for case in [c for c in g["cases"] if not c.get("families")]:
         _, plan_m, _ = batch.configuration(p, case["plan"])
         by_id = {v.id: v for v in rpeg0.vertices}
         plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
@@ -172,7 +172,7 @@ def test_optimize_equals_reference_trajectory():
                              mb={by_id[v.id]: x for v, x in plan_m.mb.items()})
         opt = OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"], T_init=case["T_init"],
                               T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"],
-                              T_cand={m: {0} for m in rpeg0.tau})
+                              T_cand={m: {0} for m in rpeg0.tau}, structural_candidates=frozenset({"separate"}))
         res = eng.sa_optimize(sa_params(opt, 1, 1, [(0, 0)], 0, 1, case["stream"][0]), arrays, plan_row(rpeg0, plan),
                               case["E_max"], case["E_struct"], stream_key=case["stream"][1:], log_cap=4096)
         log = [rows(r) for r in res["eval_log"]]
@@ -273,3 +273,46 @@ def test_concurrent_start_plan_takes_the_reference_cascade(c):
 
     plan, found = baselines.build_concurrent_baseline_plan(rpeg0, p.device_space, p.suite, p.workload, eng, table=table)
     assert found == g["found"] and rows(plan) == g["rows"]
+
+
+def test_optimize_over_structural_families_equals_reference():
+    """rpeg_sa_optimize_families on the GPU evaluator against the reference's optimize() with
+    structural_candidates {"separate", "ac_share"} (RPEG/search/optimizer.py:541-946): the separate
+    template's staleness variants, then the AC-share template's, started from random plans that is_valid
+    checks with the base configuration's memory model (structure 2 of the problem).  Every evaluated
+    (template, staleness, plan) in order, the number of draws, the returned configuration -- an AC-share one
+    in two of the three cases; the third runs with 12.5 GB per device, where the two memory models disagree.
+    The drop-in optimize() returns the same configurations."""
+    from rpeg_amd.core.types import Model
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration
+    from rpeg_amd.search.optimizer import optimize, plan_row, row_plan
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        g = json.load(f)
+    cases = [c for c in g["cases"] if c.get("families")]
+    assert len(cases) == 3
+    for case in cases:
+        p = family_problem(case)
+        eng = Engine(p)
+
+        def directory_of(structure):
+            rpeg = p.template(structure, ())
+            return directory_arrays(rpeg, build_candidate_directory(rpeg, p.suite, p.device_space, p.workload, eng,
+                                                                    structure)[0])
+
+        families, row, opt = family_case_setup(p, case, directory_of)
+        res = eng.sa_optimize_families(families, case["base_tau"], row, case["E_max"], case["E_struct"],
+                                       stream_key=case["stream"][1:], log_cap=4096)
+        check_family_case(p, case, families, res)
+
+        base_rpeg = p.template(0, case["base_tau"])
+        base = Configuration(base_rpeg, row_plan(base_rpeg, row), p.device_space)
+        out = optimize(base, p.suite, p.workload, p.hw, p.K_eval, opt, EvalCache(), seed=case["stream"][0],
+                       stream_key=case["stream"][1:])
+        assert out.rpeg.vertices[0].id == case["final_first_vertex"]
+        assert [out.rpeg.tau[m] for m in sorted(out.rpeg.tau, key=lambda m: m.value)] == case["final_tau"]
+        nv = len(out.rpeg.vertices)
+        got = plan_row(out.rpeg, out.plan)
+        assert [[int(x) for x in got[v * 10:(v + 1) * 10]] for v in range(nv)] == case["final"]
+        eng.close()

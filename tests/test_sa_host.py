@@ -23,7 +23,7 @@ from rpeg_amd.engine import abi
 from rpeg_amd.engine.problem import PlanBatch
 from rpeg_amd.ir.plan import ExecutionPlan
 from rpeg_amd.search.optimizer import OptimizerConfig, plan_row, row_plan, sa_params
-from tests.helpers import GOLDEN, seeded_batch
+from tests.helpers import GOLDEN, check_family_case, family_case_setup, family_problem, seeded_batch
 
 
 def _directory(p, rpeg0):
@@ -163,7 +163,7 @@ def test_cxx_optimize_matches_reference_optimize():
     nv = len(rpeg0.vertices)
     _, _, arrays = _directory(p, rpeg0)
     port = CpuPort(p)
-    for case in g["cases"]:
+    for case in [c for c in g["cases"] if not c.get("families")]:
         _, plan_m, _ = batch.configuration(p, case["plan"])
         row = plan_row(rpeg0, ExecutionPlan(sigma={v: plan_m.sigma[u] for v, u in zip(rpeg0.vertices, plan_m.sigma)},
                                             pi={v: plan_m.pi[u] for v, u in zip(rpeg0.vertices, plan_m.pi)},
@@ -216,3 +216,32 @@ def test_start_plan_host_logic_against_reference_vectors(c):
                 assert all(r < sp.R and n < sp.N and d < sp.G for r, n, d in devs)
                 assert not (devs & seen)
                 seen |= devs
+
+
+def test_cxx_optimize_over_structural_families_matches_reference_optimize():
+    """SaSerial over the separate template's staleness variants and then the AC-share template's, on the CPU
+    evaluator, against the reference's optimize() with structural_candidates {"separate", "ac_share"}: every
+    evaluated (template, staleness, plan) in order -- including the random restarts that start the AC-share
+    settings, which the reference validates with the memory model of its base configuration --, the number of
+    draws, and the returned configuration (an AC-share one in the second and third case).  In the third case
+    memory is tight and the two memory models disagree on the restarts: the run equals the reference's only
+    with the base configuration's view, which the last lines check."""
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        g = json.load(f)
+    cases = [c for c in g["cases"] if c.get("families")]
+    assert len(cases) == 3
+    for case in cases:
+        p = family_problem(case)
+        port = CpuPort(p)
+
+        def directory_of(structure):
+            return _directory(p, p.template(structure, ()))[2]
+
+        families, row, opt = family_case_setup(p, case, directory_of)
+        res = port.sa_optimize_families(families, case["base_tau"], row, case["E_max"], case["E_struct"],
+                                        stream_key=case["stream"][1:], log_cap=4096, threads=4)
+        check_family_case(p, case, families, res)
+    families[1] = families[1][:4] + (None,)      # the template's own memory model for is_valid: another run
+    res = port.sa_optimize_families(families, case["base_tau"], row, case["E_max"], case["E_struct"],
+                                    stream_key=case["stream"][1:], log_cap=4096, threads=4)
+    assert res["n_draws"] != case["n_draws"]
