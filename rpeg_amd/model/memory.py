@@ -1,7 +1,8 @@
-"""Memory policy (mirror of RPEG/model/memory.py:138-185).  The per-device peak
-arithmetic itself runs on the GPU; only the policy record lives on the host."""
+"""Memory policy and memory-model record (mirror of RPEG/model/memory.py:138-250).  The per-device peak
+arithmetic itself runs on the GPU; only the records live on the host."""
 
 from dataclasses import dataclass
+from typing import FrozenSet
 
 
 @dataclass(frozen=True)
@@ -35,3 +36,20 @@ def optimizer_stage(name: str) -> int:
     if key not in table:
         raise ValueError(f"unsupported distributed optimizer mode {name!r}")
     return table[key]
+
+
+@dataclass(frozen=True)
+class NodeMemoryModel:
+    """What the reference's NodeMemoryModel is constructed from (RPEG/model/memory.py:188-250): hardware,
+    models, workload, the policy's fields and the set of models it treats as trainable.  It is the
+    argument `is_valid` takes; the arithmetic behind it is the engine's."""
+    hw: object
+    suite: object
+    workload: object
+    policy: MemoryPolicy = MemoryPolicy()
+    trainable: FrozenSet = frozenset()
+    shadow_models: FrozenSet = frozenset()   # kept as the reference keeps it; no formula reads it
+
+    @classmethod
+    def from_policy(cls, hw, suite, workload, policy: MemoryPolicy, trainable=frozenset(), shadow_models=frozenset()):
+        return cls(hw, suite, workload, policy, frozenset(trainable), frozenset(shadow_models))

@@ -4,6 +4,7 @@ RPEG/search/evaluate.py, computed by the GPU engine.
   evaluate(config, suite, workload, hw, K_eval, memory_policy)          -> (score, trace, lowered)
   evaluate_cached(config, cache, suite, workload, hw, K_eval, policy)   -> (score, trace, feasible, miss)
   _eval_worker((config, suite, workload, hw, K_eval[, policy]))         -> (score, trace, feasible)
+  is_valid(config, suite, workload, mem_model)                          -> bool
   evaluate_batch(configs, suite, workload, hw, K_eval, policy)          -> BatchResult   (new: the
       batched form of Pool.map(_eval_worker, ...), RPEG/search/optimizer.py:793-798)
 
@@ -25,7 +26,7 @@ from ..engine.problem import STRUCTURES, EvalProblem, PlanBatch
 from ..ir.plan import ExecutionPlan
 from ..ir.rpeg import RPEG
 from ..model.hardware import Hardware
-from ..model.memory import MemoryPolicy
+from ..model.memory import MemoryPolicy, NodeMemoryModel
 from ..model.models import ModelSuite
 from ..model.workload import Workload
 from .cache import EvalCache, config_hash
@@ -89,11 +90,15 @@ _TEMPLATE_IDS = {"ppo": ("g_pi", "i_ref", "i_R", "i_V", "t_pi", "t_V"), "grpo": 
 
 
 def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware, space: DeviceSpace, K_eval: int,
-                policy: MemoryPolicy, more_structures=()):
+                policy: MemoryPolicy, more_structures=(), memory_trainable=None):
     """(engine, structure of `rpeg`): one engine per problem, kept for the life of the process.  The
-    structure of `rpeg` is structure 0 of the engine, `more_structures` follow."""
+    structure of `rpeg` is structure 0 of the engine (with `memory_trainable` as the memory model's set of
+    trainable models when that is given and differs from the template's), `more_structures` follow."""
+    from dataclasses import replace
     from ..engine.runtime import Engine
     st = _structure_of(rpeg)
+    if memory_trainable is not None and frozenset(memory_trainable) != frozenset(st.tau_models):
+        st = replace(st, memory_trainable=frozenset(memory_trainable))
     structures = (st,) + tuple(more_structures)
     key = (tuple((s.name, s.memory_trainable) for s in structures),
            tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
@@ -303,6 +308,24 @@ def evaluate(config: Configuration, suite: ModelSuite, workload: Workload, hw: H
     trace, lowered = _trace_of(eng, st, config, batch)
     score = trace.throughput(W_step=workload.B * workload.K * (workload.S + workload.T), K=K_eval)
     return score, trace, lowered
+
+
+def is_valid(config: Configuration, suite: ModelSuite, workload: Workload, mem_model: NodeMemoryModel) -> bool:
+    """Drop-in for is_valid (RPEG/search/evaluate.py:143-232): plan coverage, divisibility, micro-batch and
+    packing rules, the stale-publication layout rule, and memory fit of the K_eval = 1 lowering under
+    `mem_model` -- whose set of trainable models need not be the template's (optimize() passes the model of
+    its base configuration).  Coverage is checked here; everything else is the mask of one engine call."""
+    _check_supported(config)
+    plan = config.plan
+    for v in config.rpeg.vertices:
+        if v not in plan.sigma or v not in plan.pi or v not in plan.mb:
+            return False
+    if not mem_model.trainable:
+        raise NotImplementedError("the co-resident memory model (no trainable model) is not part of this engine")
+    eng, st = _engine_for(config.rpeg, suite, workload, mem_model.hw, config.device_space, 1, mem_model.policy,
+                          memory_trainable=mem_model.trainable)
+    mask = int(eng.eval(_pack([config], st, workload), gate_stale=False)["mask"][0])
+    return bool(mask & abi.MASK_VALID) and bool(mask & abi.MASK_STALE_OK) and bool(mask & abi.MASK_MEM_OK)
 
 
 def evaluation_cache_key(config: Configuration, memory_policy: MemoryPolicy = MemoryPolicy()) -> str:

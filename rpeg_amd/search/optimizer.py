@@ -28,9 +28,9 @@ from ..model.workload import Workload
 from .cache import EvalCache
 from .evaluate import (Configuration, _check_supported, _engine_for, _structure_of, evaluate_batch, evaluate_cached,
                        evaluation_cache_key)
+from .inter_model import DEFAULT_T_CAND, _iter_staleness as _staleness_assignments
 from .moves import build_candidate_directory, directory_arrays
 
-DEFAULT_T_CAND: Dict[Model, Set[int]] = {Model.ACTOR: {0, 1}, Model.CRITIC: {0, 1}, Model.AC_SHARE: {0, 1}}
 
 
 @dataclass
@@ -176,9 +176,19 @@ def optimize_chains(problem: EvalProblem, opt: OptimizerConfig, n_chains: int, n
 
 
 def _iter_staleness(tau_models, t_cand) -> List[Tuple[int, ...]]:
-    """RPEG/search/inter_model.py:43-62 in the order of the structure's trainable models."""
-    import itertools
-    return [tuple(c) for c in itertools.product(*[sorted(t_cand[m]) for m in tau_models])]
+    """The staleness variants in the reference's order (RPEG/search/inter_model.py:43-65), each as one
+    value per entry of `tau_models`."""
+    return [tuple(tau[m] for m in tau_models) for tau in _staleness_assignments(tau_models, t_cand)]
+
+
+def _ac_penalty(score: float, lambda_ac: float) -> float:
+    """RPEG/search/optimizer.py:132-145."""
+    return score if lambda_ac == 0.0 else score * (1.0 - lambda_ac)
+
+
+def penalized_score(raw_score: float, rpeg, opt_config: "OptimizerConfig", ac_share: bool) -> float:
+    """The score optimize() ranks by (RPEG/search/optimizer.py:148-170): only the AC-share penalty."""
+    return _ac_penalty(raw_score, opt_config.lambda_ac) if ac_share else raw_score
 
 
 def optimize_families(problem: EvalProblem, opt_config: OptimizerConfig, engine_directory) -> List[tuple]:

@@ -373,3 +373,69 @@ def test_execution_schedule_artifact_equals_reference(c):
         assert zlib.crc32(",".join(n["node_id"] for n in got["nodes"]).encode()) == want["order_crc"]
         assert [[n["node_id"], n["dispatch_index"], n["predicted_start_s"].hex(), n["predicted_finish_s"].hex()]
                 for n in got["nodes"][:6]] == want["head"]
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_is_valid_drop_in_equals_restatement(c):
+    """is_valid (RPEG/search/evaluate.py:143-232) through the engine against its restatement on the oracle's
+    passes (integer rules, stale-layout rule, memory fit of the K_eval = 1 lowering): seeded plans of every
+    structure and staleness of the configuration as they are, then broken one rule at a time; under the
+    template's own memory model and under one whose trainable set is another template's (what optimize()
+    passes for AC-share plans)."""
+    import dataclasses
+    from oracle import rpeg_oracle as O
+    from rpeg_amd.core.types import Allocation, Model
+    from rpeg_amd.ir.plan import ExecutionPlan
+    from rpeg_amd.model.memory import NodeMemoryModel
+    from rpeg_amd.search.evaluate import Configuration, is_valid
+    cfg, batch = seeded_batch(c, 40)
+    p = cfg.problem
+    pol = p.memory_policy
+
+    def restated(rpeg, plan, wl, trainable):
+        if not O.plan_structurally_valid(rpeg, plan, p.device_space, p.suite, wl):
+            return False
+        if not O.stale_publication_layout_valid(rpeg, plan):
+            return False
+        nodes, _ = O.lower(rpeg, plan, p.suite, 1, wl)
+        mm = O.MemModel(p.hw, p.suite, wl, trainable, eps_rt=pol.runtime_overhead_fraction,
+                        optimizer_stage=pol.optimizer_stage, worker_overhead_bytes=pol.worker_overhead_bytes,
+                        semantic_activation_cache_bytes=pol.semantic_activation_cache_bytes,
+                        max_worker_groups_per_gpu=pol.max_worker_groups_per_gpu,
+                        activation_checkpointing=pol.activation_checkpointing)
+        return not (max(O.device_peaks(nodes, mm).values()) > mm.capacity())
+
+    def broken(plan, v, k):
+        sigma, pi, mb = dict(plan.sigma), dict(plan.pi), dict(plan.mb)
+        dp, pp, tp = pi[v]
+        a = sigma[v]
+        if k == 0:
+            mb[v] = mb[v] + 1                                      # micro-batch rule
+        elif k == 1:
+            pi[v] = (dp, pp, 3)                                    # tp does not divide G
+        elif k == 2:
+            sigma[v] = Allocation(origin=(a.origin[0], a.origin[1] + p.device_space.N, a.origin[2]), extent=a.extent)
+        elif k == 3:
+            sigma[v] = Allocation(origin=a.origin, extent=(a.extent[0], a.extent[1], a.extent[2] + 1))
+        elif k == 4:
+            del mb[v]                                              # coverage
+        return ExecutionPlan(sigma, pi, mb)
+
+    n_true = n_false = n_view = 0
+    for i in range(batch.n):
+        rpeg, plan, wl = batch.configuration(p, i)
+        views = [frozenset(rpeg.trainable)]
+        if Model.AC_SHARE in rpeg.trainable:
+            views.append(frozenset({Model.ACTOR, Model.CRITIC}))
+        for trainable in views:
+            mm = NodeMemoryModel.from_policy(p.hw, p.suite, wl, pol, trainable=trainable)
+            variants = [plan] + ([broken(plan, rpeg.vertices[i % len(rpeg.vertices)], i % 5)] if trainable == views[0] else [])
+            for q in variants:
+                got = is_valid(Configuration(rpeg, q, p.device_space), p.suite, wl, mm)
+                assert got == restated(rpeg, q, wl, trainable), (i, sorted(m.value for m in trainable))
+                n_true += got
+                n_false += not got
+        if len(views) == 2:
+            n_view += restated(rpeg, plan, wl, views[0]) != restated(rpeg, plan, wl, views[1])
+    assert n_true > 0 and n_false > 0
+    print("valid", n_true, "invalid", n_false, "plans on which the two memory views disagree", n_view)

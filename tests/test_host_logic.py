@@ -152,3 +152,37 @@ def test_engine_refuses_without_gpu():
     from rpeg_amd.engine.runtime import Engine, EngineError
     with pytest.raises(EngineError):
         Engine(configs.config(4).problem)
+
+
+def test_structural_settings_in_reference_order():
+    """Iter_inter_model_candidates against what the reference's yields (tests/golden/make_golden_inter_model.py):
+    templates, staleness assignments (models ordered by value string, last fastest), the fused settings
+    interleaved, AC-share last; and the families optimize() derives from the same rules."""
+    import json
+    import os
+    from rpeg_amd import configs
+    from rpeg_amd.core.types import Model
+    from rpeg_amd.search.inter_model import Iter_inter_model_candidates
+    from rpeg_amd.search.optimizer import OptimizerConfig, _ac_penalty, optimize_families, penalized_score
+    from tests.helpers import GOLDEN, family_problem
+    with open(os.path.join(GOLDEN, "ref_inter_model.json")) as f:
+        g = json.load(f)
+    p = configs.config(1).problem
+    for name, cand in g["t_cands"].items():
+        t_cand = None if cand is None else {Model(m): set(v) for m, v in cand.items()}
+        for algorithm in ("ppo", "grpo", "dpo"):
+            got = [dict(vertices=[v.id for v in rpeg.vertices], tau=[[m.value, t] for m, t in cfg.tau.items()],
+                        ac_share=cfg.ac_share, fused=cfg.intra_stage_fusion, algorithm=cfg.algorithm)
+                   for rpeg, cfg in Iter_inter_model_candidates(p.suite, p.workload, t_cand, algorithm=algorithm)]
+            assert got == g[f"{name}/{algorithm}"], (name, algorithm)
+        # the families of optimize(): the same settings without the fused ones, grouped by template
+        fp = family_problem()
+        fams = optimize_families(fp, OptimizerConfig(T_cand=t_cand, lambda_ac=0.15), lambda s: [])
+        walked = [(prm.structure, tuple(int(prm.tau[k][i]) for i in range(len(fp.structures[prm.structure].tau_models))))
+                  for prm, *_ in fams for k in range(prm.n_variants)]
+        want = [(int(s["ac_share"]), tuple(t for _, t in s["tau"])) for s in g[f"{name}/ppo"] if not s["fused"]]
+        assert walked == want
+        assert [f[2] for f in fams] == [1.0, 0.85][:len(fams)] and [f[4] for f in fams] == [None, 2][:len(fams)]
+    assert _ac_penalty(3.0, 0.0) == 3.0 and _ac_penalty(3.0, 0.15) == 3.0 * (1.0 - 0.15)
+    assert penalized_score(2.0, None, OptimizerConfig(lambda_ac=0.5), False) == 2.0
+    assert penalized_score(2.0, None, OptimizerConfig(lambda_ac=0.5), True) == 1.0
