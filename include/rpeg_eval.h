@@ -205,6 +205,14 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
                     int32_t* node_step, int32_t* node_sub, int32_t* node_src, int32_t* edges,
                     int32_t* n_edges, int32_t cap, uint8_t* node_reserved);
 
+/* Trace.utilization() and Trace.n_active() of ONE plan (RPEG/schedule/trace.py:53-118): the plan is traced on
+   the GPU as by rpeg_eval_trace, then the busy intervals are merged device by device on the host in the
+   insertion order of the reference's dictionaries (nodes in dispatch order, a node's reserved allocations
+   source first, devices rack-major), so the sum has the reference's rounding.  Either output may be NULL.
+   The metric steers optimize() when max_throughput_loss > 0 (optimizer.py:461-486). */
+int rpeg_eval_trace_metrics(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4,
+                            double* utilization, int32_t* n_active);
+
 /* Batched simulated annealing: n_chains independent Metropolis-Hastings chains of n_steps steps.  One
    step of a chain is one iteration of the inner loop of optimize() (RPEG/search/optimizer.py:702-930):
    with probability alpha_pair*min(1,T/T_init) a donor/receiver proposal (multi_move_pair,
@@ -225,6 +233,10 @@ typedef struct rpeg_sa_params_s {
   uint64_t seed;
   int32_t dir_n[RPEG_MAX_V];  /* candidate directory (moves.py:464-551): entries per vertex ...      */
   const int16_t* dir[RPEG_MAX_V]; /* ... rows of dp pp tp r_ext n_ext mb, ascending by time          */
+  double max_throughput_loss; /* rpeg_sa_optimize*: > 0 ranks by throughput x Trace.utilization() above the
+                                 floor (1 - loss) x best throughput so far, and by throughput x 1e-12 below
+                                 it (optimizer.py:461-486); every evaluated plan is then traced once more
+                                 for its utilisation (rpeg_eval_trace_metrics).  rpeg_sa_run ignores it  */
 } rpeg_sa_params_t;
 
 typedef struct rpeg_sa_result_s {   /* per-chain arrays of n_chains elements, any may be NULL */

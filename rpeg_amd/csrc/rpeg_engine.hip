@@ -1032,6 +1032,81 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   return n;
 }
 
+int rpeg_eval_trace_metrics(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* utilization,
+                            int32_t* n_active) {
+  if (!e || !vert_fields || !head4) return -1;
+  const int cap = 4096;
+  std::vector<double> start(cap), finish(cap);
+  std::vector<int32_t> order(cap), kind(cap), vertex(cap), src(cap);
+  std::vector<uint8_t> reserved(cap);
+  const int n = rpeg_eval_trace(e, vert_fields, head4, start.data(), finish.data(), order.data(), kind.data(),
+                                vertex.data(), nullptr, nullptr, src.data(), nullptr, nullptr, cap, reserved.data());
+  if (n < 0) return n;
+  const int N = e->P.N, G = e->P.G;
+  const int nv = e->P.st[head4[0]].n_vertex;
+  auto field = [&](int v, int f) { return (int)vert_fields[v * RPEG_FIELDS + f]; };
+  auto same_box = [&](int u, int v) {
+    for (int f = 4; f < 10; ++f) if (field(u, f) != field(v, f)) return false;
+    return true;
+  };
+  auto for_devices = [&](int v, auto&& fn) {   // rack-major, as the reference enumerates an allocation
+    for (int r = field(v, 4); r < field(v, 4) + field(v, 7); ++r)
+      for (int q = field(v, 5); q < field(v, 5) + field(v, 8); ++q)
+        for (int g = field(v, 6); g < field(v, 6) + field(v, 9); ++g) fn((r * N + q) * G + g);
+  };
+  if (n_active) {   // devices inside any allocation of any node: every vertex has operator nodes
+    std::vector<char> seen((size_t)e->P.R * N * G, 0);
+    int cnt = 0;
+    for (int v = 0; v < nv; ++v) for_devices(v, [&](int d) { if (!seen[d]) { seen[d] = 1; ++cnt; } });
+    *n_active = cnt;
+  }
+  if (!utilization) return 0;
+  double ms = 0.0;
+  for (int i = 0; i < n; ++i) ms = i == 0 ? finish[0] : std::max(ms, finish[i]);
+  *utilization = 0.0;
+  if (n == 0 || ms <= 0) return 0;
+  std::vector<int> by_dispatch(n);
+  for (int i = 0; i < n; ++i) by_dispatch[i] = i;
+  std::stable_sort(by_dispatch.begin(), by_dispatch.end(), [&](int x, int y) { return order[x] < order[y]; });
+  std::vector<int> slot((size_t)e->P.R * N * G, -1);           // device -> position in first-touch order
+  std::vector<std::vector<std::pair<double, double>>> spans;
+  for (int i : by_dispatch) {
+    int owners[2], no = 0;
+    if (kind[i] == 0) owners[no++] = vertex[i];
+    else { owners[no++] = src[i]; owners[no++] = vertex[i]; }
+    int used[2], nu = 0;
+    for (int k = 0; k < no; ++k) {
+      if (!((reserved[i] >> owners[k]) & 1)) continue;
+      if (nu == 1 && same_box(used[0], owners[k])) continue;   // identical allocations once
+      used[nu++] = owners[k];
+    }
+    for (int k = 0; k < nu; ++k)
+      for_devices(used[k], [&](int d) {
+        if (slot[d] < 0) { slot[d] = (int)spans.size(); spans.emplace_back(); }
+        spans[slot[d]].emplace_back(start[i], finish[i]);
+      });
+  }
+  if (spans.empty()) return 0;
+  double total = 0.0;
+  for (auto& sp : spans) {
+    std::sort(sp.begin(), sp.end());
+    double merged = 0.0, cs = 0.0, ce = 0.0;
+    bool open = false;
+    for (const auto& se : sp) {
+      if (!open || se.first > ce) {
+        if (open) merged += ce - cs;
+        cs = se.first; ce = se.second; open = true;
+      } else {
+        ce = std::max(ce, se.second);
+      }
+    }
+    if (open) merged += ce - cs;
+    total += merged / ms;
+  }
+  *utilization = total / (double)spans.size();
+  return 0;
+}
+
 }  // extern "C"
 
 // Evaluates the candidates of a simulated-annealing step on the GPU: plans are staged through pinned
@@ -1269,6 +1344,10 @@ struct GpuSaBackend : SaBackend {
     if (d_score) hipFree(d_score);
     if (h_mass) hipHostFree(h_mass);
     if (d_mass) hipFree(d_mass);
+  }
+
+  int utilization(const SaPlan& plan, uint8_t variant, double* out) override {
+    return rpeg_eval_trace_metrics(e, &plan.f[0][0], head_of[variant], out, nullptr);
   }
 
   int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override {

@@ -69,6 +69,7 @@ struct SaPlan { int16_t f[RPEG_MAX_V][RPEG_FIELDS]; };
 struct SaEval {          // what one evaluation returns
   double score;          // throughput times the soft memory penalty, without the stale-layout gate
   double mass[RPEG_MAX_V];
+  double util = 0.0;     // Trace.utilization(), filled only where the utilisation objective asks for it
   uint8_t mask;          // RPEG_MASK_*
 };
 
@@ -78,12 +79,15 @@ struct SaBackend {
   virtual ~SaBackend() {}
   // evaluates n plans; variant[i] selects the staleness variant of plan i
   virtual int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) = 0;
+  // Trace.utilization() of one plan (trace.py:53-101); backends without traces refuse
+  virtual int utilization(const SaPlan& plan, uint8_t variant, double* out) { (void)plan; (void)variant; (void)out; return -1; }
 };
 
 struct SaSettings {
   int n_chains = 64, n_steps = 2000, K_x = 6, T_max = 50, K_elite = 3, stag_window = 20, restart_attempts = 50;
   int gate_candidates = 0, geometric_cooling = 0, n_variants = 1;
   double T_init = 0.30, T_warm = 0.05, T_min = 0.01, T_cool = 1.0, alpha_pair = 0.28, score_eps = 1e-4;
+  double max_throughput_loss = 0.0;
   uint64_t seed = 42;
 };
 
@@ -649,6 +653,9 @@ struct SaSerial {
       std::vector<uint8_t> var(todo.size(), (uint8_t)variant);
       std::vector<SaEval> ev(todo.size());
       if (int rc = be.evaluate((int)todo.size(), todo.data(), var.data(), ev.data())) return rc;
+      if (p.max_throughput_loss > 0.0)
+        for (size_t j = 0; j < todo.size(); ++j)
+          if (int rc = be.utilization(todo[j], (uint8_t)variant, &ev[j].util)) return rc;
       for (size_t j = 0; j < todo.size(); ++j) {
         const bool stale_ok = (ev[j].mask & RPEG_MASK_STALE_OK) != 0, mem_ok = (ev[j].mask & RPEG_MASK_MEM_OK) != 0;
         Stored st;
@@ -664,9 +671,17 @@ struct SaSerial {
     }
     return 0;
   }
+  // optimizer.py:461-486: throughput x utilisation above the floor (1 - loss) x best throughput so far
+  double best_raw = 0.0;
+  double eff(double raw, double util) {
+    if (!(p.max_throughput_loss > 0.0)) return raw;
+    if (raw > best_raw) best_raw = raw;
+    if (raw < (1.0 - p.max_throughput_loss) * best_raw) return raw * 1e-12;
+    return raw * std::max(util, 1e-6);
+  }
   // optimizer.py:676-686, 846-861; returns the score as the family compares it
   double note(const SaFamily& f, const SaPlan& q, const Stored& s, int variant) {
-    const double score = s.score * f.scale;
+    const double score = eff(s.score, s.ev.util) * f.scale;
     if (s.feasible) elite_insert(f, s.score, q, s.ev);
     if (score > best_score * (1.0 + p.score_eps)) { best.plan = q; best.ev = s.ev; best_score = score; best_variant = variant; }
     if (s.feasible && score > best_feasible_score) {
@@ -693,9 +708,9 @@ struct SaSerial {
     std::vector<Stored> st;
     std::vector<char> miss;
     if (int rc = evaluate(1, &base, base_variant, true, st, miss)) return rc;   // optimizer.py:466-478
-    best.plan = base; best.ev = st[0].ev; best_score = st[0].score; best_variant = base_variant;
+    best.plan = base; best.ev = st[0].ev; best_score = eff(st[0].score, st[0].ev.util); best_variant = base_variant;
     if (st[0].feasible) {
-      has_feasible = true; best_feasible = best; best_feasible_score = st[0].score; best_feasible_variant = base_variant;
+      has_feasible = true; best_feasible = best; best_feasible_score = best_score; best_feasible_variant = base_variant;
       elite_insert(fam[0], st[0].score, base, st[0].ev);
     }
     E = 1;
@@ -848,6 +863,7 @@ inline void sa_settings_from(const rpeg_sa_params_t& prm, SaSettings* st) {
   st->gate_candidates = prm.gate_candidates; st->geometric_cooling = prm.geometric_cooling;
   st->n_variants = prm.n_variants; st->T_init = prm.T_init; st->T_warm = prm.T_warm; st->T_min = prm.T_min;
   st->T_cool = prm.T_cool; st->alpha_pair = prm.alpha_pair; st->score_eps = prm.score_eps; st->seed = prm.seed;
+  st->max_throughput_loss = prm.max_throughput_loss;
 }
 
 inline void sa_run_result(const SaRun& run, rpeg_sa_result_t* res) {

@@ -91,7 +91,7 @@ class SaParamsT(C.Structure):
                 ("T_init", C.c_double), ("T_warm", C.c_double), ("T_min", C.c_double), ("T_cool", C.c_double),
                 ("alpha_pair", C.c_double), ("score_eps", C.c_double),
                 ("seed", C.c_uint64),
-                ("dir_n", C.c_int32 * MAX_V), ("dir", C.c_void_p * MAX_V)]
+                ("dir_n", C.c_int32 * MAX_V), ("dir", C.c_void_p * MAX_V), ("max_throughput_loss", C.c_double)]
 
 
 class SaResultT(C.Structure):

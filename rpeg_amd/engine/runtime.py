@@ -24,7 +24,7 @@ EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
            "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
-           "rpeg_sa_optimize_families")
+           "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics")
 
 
 class EngineError(RuntimeError):
@@ -63,6 +63,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_op_time_batch.argtypes = [vp, u64, i32, i32, vp, u64, vp, vp, vp]
     lib.rpeg_eval_trace.restype = C.c_int
     lib.rpeg_eval_trace.argtypes = [vp] * 13 + [i32, vp]
+    lib.rpeg_eval_trace_metrics.restype = C.c_int
+    lib.rpeg_eval_trace_metrics.argtypes = [vp] * 5
     lib.rpeg_engine_stats.restype = C.c_int
     lib.rpeg_engine_stats.argtypes = [vp, vp, i32]
     lib.rpeg_engine_set_timing.restype = C.c_int
@@ -363,6 +365,18 @@ class Engine:
         self._check(n, "rpeg_eval_trace")
         return dict(start=start[:n], finish=finish[:n], order=order[:n], kind=kind[:n], vertex=vertex[:n], step=step[:n],
                     sub=sub[:n], src=src[:n], edges=edges[:2 * ne.value].reshape(-1, 2), reserved=reserved[:n])
+
+    def trace_metrics(self, batch: PlanBatch, i: int):
+        """(Trace.utilization(), Trace.n_active()) of plan i, folded by the library (rpeg_eval_trace_metrics)."""
+        torch = _torch()
+        vert = np.ascontiguousarray(batch.vert[:, i], dtype=np.int16)
+        head = np.ascontiguousarray(batch.head[:, i], dtype=np.uint8)
+        util, act = C.c_double(0.0), C.c_int32(0)
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_eval_trace_metrics(self._h, vert.ctypes.data, head.ctypes.data, C.addressof(util),
+                                                  C.addressof(act))
+        self._check(rc, "rpeg_eval_trace_metrics")
+        return util.value, act.value
 
     def device_exp(self, x: np.ndarray) -> np.ndarray:
         torch = _torch()

@@ -137,6 +137,7 @@ def sa_params(opt: OptimizerConfig, n_chains: int, n_steps: int, variants: Seque
             p.tau[k][t] = int(taus[t]) if t < len(taus) else 0
     p.T_init, p.T_warm, p.T_min, p.T_cool = opt.T_init, opt.T_warm, opt.T_min, opt.T_cool
     p.alpha_pair, p.score_eps, p.seed = opt.alpha_pair, opt.score_eps, seed
+    p.max_throughput_loss = float(opt.max_throughput_loss)
     return p
 
 
@@ -235,13 +236,15 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
     configuration (tests/golden/make_golden_optimize.py); the generator here is the counter-based stream
     (seed, *stream_key), not MT19937.
 
-    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused"), deadlines, the
-    utilisation objective.  `cache` is accepted for signature compatibility: the run keeps its own cache
+    With `max_throughput_loss` > 0 plans are ranked by throughput x utilisation above the throughput floor
+    (optimizer.py:461-486); every evaluated plan is then traced once more for its utilisation.
+
+    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused") and deadlines.  `cache` is accepted for signature compatibility: the run keeps its own cache
     (keyed by plan, template and staleness)."""
     from ..engine.problem import STRUCTURES, as_seen_from
     _check_supported(base_config)
-    if opt_config.max_throughput_loss > 0.0 or opt_config.deadline is not None:
-        raise NotImplementedError("utilisation objective and deadlines are not part of this engine")
+    if opt_config.deadline is not None:
+        raise NotImplementedError("deadlines are not part of this engine")
     policy = opt_config.memory_policy()
     st = _structure_of(base_config.rpeg)
     names = opt_config.structural_candidates
@@ -275,6 +278,23 @@ def configuration_of(problem: EvalProblem, families, res, base_tau, suite, workl
                          intra_stage_fusion=False, transfer_resource_policy=base_config.transfer_resource_policy)
 
 
+class _Utilization:
+    """Stands in a cache entry for the trace of a polish candidate: its one number the objective reads."""
+
+    def __init__(self, value: float):
+        self.value = value
+
+    def utilization(self) -> float:
+        return self.value
+
+
+def _trace_utilization(config: Configuration, suite, workload, hw, K_eval, policy) -> float:
+    """Trace.utilization() of one configuration, folded by the library (rpeg_eval_trace_metrics)."""
+    from .evaluate import _pack
+    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, policy)
+    return eng.trace_metrics(_pack([config], st, workload), 0)[0]
+
+
 def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
            opt_config: OptimizerConfig, cache: EvalCache, table, index, ac_share: bool = False,
            max_rounds: int = 50) -> Configuration:
@@ -285,19 +305,22 @@ def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw
     ones is applied; passes repeat until one brings no improvement.  Cache hits are merged before fresh
     results, as in the reference, so equal scores resolve the same way."""
     _check_supported(best_config)
-    if opt_config.max_throughput_loss > 0.0:
-        raise NotImplementedError("the utilisation-weighted objective needs per-candidate traces")
     policy = opt_config.memory_policy()
     config, rpeg = best_config, best_config.rpeg
     G = config.device_space.G
+    delta, best_raw = opt_config.max_throughput_loss, [0.0]
 
-    def _score(raw: float) -> float:
-        return raw * (1.0 - opt_config.lambda_ac) if ac_share and opt_config.lambda_ac != 0.0 else raw
+    def _score(raw: float, trace=None) -> float:   # optimizer.py:1021-1044
+        s = raw
+        if delta > 0.0 and trace is not None:
+            best_raw[0] = max(best_raw[0], raw)
+            s = raw * 1e-12 if raw < (1.0 - delta) * best_raw[0] else raw * max(trace.utilization(), 1e-6)
+        return _ac_penalty(s, opt_config.lambda_ac) if ac_share else s
 
     vertices = sorted(rpeg.vertices, key=lambda v: v.id)
     w_frac = opt_config.T_min / opt_config.T_init
     raw, _trace, _feasible, _miss = evaluate_cached(config, cache, suite, workload, hw, K_eval, policy)
-    score = _score(raw)
+    score = _score(raw, _trace)
     for _round in range(max_rounds):
         improved = False
         for v in vertices:
@@ -325,7 +348,7 @@ def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw
                 h = evaluation_cache_key(nb, policy)
                 if h in cache:
                     s, t, f = cache.get(h)
-                    hits.append((nb, s, f))
+                    hits.append((nb, s, t, f))
                 else:
                     misses.append((nb, h))
             fresh = []
@@ -333,11 +356,16 @@ def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw
                 res = evaluate_batch([nb for nb, _ in misses], suite, workload, hw, K_eval, policy, gate_stale=False)
                 for (nb, h), s, m in zip(misses, res.score, res.mask):
                     f = bool(m & abi.MASK_MEM_OK)
-                    cache.put(h, float(s), None, f)
-                    fresh.append((nb, float(s), f))
-            for nb, s, f in hits + fresh:
-                if f and _score(s) > best_score:
-                    best_score, best = _score(s), nb
+                    # the utilisation objective reads one number of a candidate's trace: keep that
+                    t = _Utilization(_trace_utilization(nb, suite, workload, hw, K_eval, policy)) if delta > 0.0 else None
+                    cache.put(h, float(s), t, f)
+                    fresh.append((nb, float(s), t, f))
+            for nb, s, t, f in hits + fresh:
+                if not f:
+                    continue
+                score_n = _score(s, t)
+                if score_n > best_score:
+                    best_score, best = score_n, nb
             if best is not None:
                 config, score, improved = best, best_score, True
         if not improved:

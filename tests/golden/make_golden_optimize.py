@@ -49,7 +49,10 @@ CASES = [dict(plan=0, stream=(42, 77, 0, 0), E_max=260, E_struct=200, stag_windo
          # tight memory: is_valid's verdict on AC-share restarts (base configuration's memory model) and the
          # evaluation's (the template's own) disagree, and the trajectory shows which one the reference asks
          dict(plan=0, stream=(42, 77, 4, 0), E_max=420, E_struct=70, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
-              families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05, memory_per_gpu=1.25e10)]
+              families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05, memory_per_gpu=1.25e10),
+         # utilisation objective (optimizer.py:461-486): throughput x Trace.utilization() above the floor
+         dict(plan=0, stream=(42, 77, 5, 0), E_max=330, E_struct=120, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
+              families=True, T_cand=[[0, 1], [0], [0]], base_tau=[0, 0], lambda_ac=0.15, max_throughput_loss=0.10)]
 
 
 def main():
@@ -148,8 +151,9 @@ def main():
     import dataclasses
     p_config = p
     for case in CASES:
-        if "memory_per_gpu" in case:
-            p = dataclasses.replace(p_config, hw=dataclasses.replace(p_config.hw, memory_per_gpu=case["memory_per_gpu"]))
+        if p is not p_config or "memory_per_gpu" in case:
+            p = dataclasses.replace(p_config, hw=dataclasses.replace(
+                p_config.hw, memory_per_gpu=case.get("memory_per_gpu", p_config.hw.memory_per_gpu)))
             rpeg0, suite, wl, hw, space, cost, mm = SA.ref_world(mods, p, {"Pi": 0, "V": 0})
             st.update(problem=p, suite=suite, wl=wl, hw=hw, space=space, cost=cost, mm=mm, mms={})
         plan = SA.ref_plan(mods, rpeg0, batch, p, case["plan"])
@@ -161,6 +165,7 @@ def main():
             oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
                                       T_cand={Model.ACTOR: set(a), Model.CRITIC: set(c), Model.AC_SHARE: set(s_)},
                                       structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"],
+                                      max_throughput_loss=case.get("max_throughput_loss", 0.0),
                                       T_init=case["T_init"], T_warm=case["T_warm"], T_min=case["T_min"],
                                       stag_window=case["stag_window"])
         else:

@@ -99,7 +99,7 @@ def main():
                                 "cfg5": [ropt.OptimizerConfig(K_x=6, T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10).I_max,
                                          ropt.OptimizerConfig(K_x=6, T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10).T_cool.hex()],
                                 "e800": [ropt.OptimizerConfig(E_struct=800, K_x=4).I_max, ropt.OptimizerConfig(E_struct=800, K_x=4).T_cool.hex()]},
-           "T_init": 0.30, "T_min": 0.03, "cases": []}
+           "T_init": 0.30, "T_min": 0.03, "cases": [], "utilisation_cases": []}
     done = 0
     for i in range(64):
         if done >= 4:
@@ -114,6 +114,14 @@ def main():
         s1, _, f1 = _eval(out, gate=True)
         doc["cases"].append(dict(i=i, start_score=s0.hex(), final_score=s1.hex(), final_feasible=f1,
                                  evaluations=state["n_worker"], plan=SA.plan_rows(rpeg0, out.plan)))
+        # the same start under the utilisation objective (optimizer.py:1021-1044)
+        oc_u = ropt.OptimizerConfig(K_x=1, T_init=0.30, T_min=0.03, max_throughput_loss=0.10)
+        state["n_worker"] = 0
+        out = ropt.polish(start, suite, wl, hw, p.K_eval, oc_u, rcache.EvalCache(), table, index)
+        s1, tr1, f1 = _eval(out, gate=True)
+        doc["utilisation_cases"].append(dict(i=i, max_throughput_loss=0.10, final_score=s1.hex(), final_feasible=f1,
+                                             final_utilization=float(tr1.utilization()).hex(),
+                                             evaluations=state["n_worker"], plan=SA.plan_rows(rpeg0, out.plan)))
         done += 1
     path = os.path.join(HERE, "ref_polish.json")
     with open(path, "w") as f:

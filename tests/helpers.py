@@ -63,7 +63,8 @@ def family_case_setup(p, case, directory_of):
     opt = OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"], T_init=case["T_init"],
                           T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"],
                           T_cand={Model.ACTOR: set(a), Model.CRITIC: set(c_), Model.AC_SHARE: set(s_)},
-                          structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"])
+                          structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"],
+                          max_throughput_loss=case.get("max_throughput_loss", 0.0))
     assert opt.T_cool.hex() == case["T_cool"]
     families = optimize_families(p, opt, directory_of)
     families[0][0].seed = case["stream"][0]

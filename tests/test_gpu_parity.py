@@ -261,6 +261,11 @@ def test_trace_utilization_and_active_devices_equal_reference(c):
         assert float(trace.utilization()).hex() == want["utilization"], i
         assert trace.n_active() == want["n_active"], i
         assert trace.makespan().hex() == want["makespan"], i
+    # the same two metrics folded by the library (rpeg_eval_trace_metrics), every plan of the vectors
+    eng = engine(c)
+    for i in range(gold["n"]):
+        util, act = eng.trace_metrics(batch, i)
+        assert float(util).hex() == gold["plans"][i]["utilization"] and act == gold["plans"][i]["n_active"], i
 
 
 def test_drop_in_calls():

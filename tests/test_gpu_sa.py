@@ -142,6 +142,23 @@ def test_polish_equals_reference():
         score, _, feasible, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
         assert float(score).hex() == case["final_score"] and feasible == case["final_feasible"]
         assert cache.misses - 1 == case["evaluations"]
+    # the same starts under the utilisation objective (max_throughput_loss > 0, optimizer.py:1021-1044): other
+    # final plans, again the reference's
+    for case in g["utilisation_cases"]:
+        _, plan_m, _ = batch.configuration(p, case["i"])
+        by_id = {v.id: v for v in rpeg0.vertices}
+        plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
+                             pi={by_id[v.id]: x for v, x in plan_m.pi.items()},
+                             mb={by_id[v.id]: x for v, x in plan_m.mb.items()})
+        opt_u = OptimizerConfig(K_x=1, T_init=g["T_init"], T_min=g["T_min"], max_throughput_loss=case["max_throughput_loss"])
+        cache = EvalCache()
+        out = polish(Configuration(rpeg0, plan, p.device_space), p.suite, p.workload, p.hw, p.K_eval, opt_u, cache, table, index)
+        rows = plan_row(rpeg0, out.plan)
+        assert [[int(x) for x in rows[v * 10:(v + 1) * 10]] for v in range(nv)] == case["plan"], case["i"]
+        score, trace, feasible, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+        assert float(score).hex() == case["final_score"] and feasible == case["final_feasible"]
+        assert float(trace.utilization()).hex() == case["final_utilization"]
+        assert cache.misses - 1 == case["evaluations"]
 
 
 def test_optimize_equals_reference_trajectory():
@@ -281,8 +298,9 @@ def test_optimize_over_structural_families_equals_reference():
     template's staleness variants, then the AC-share template's, started from random plans that is_valid
     checks with the base configuration's memory model (structure 2 of the problem).  Every evaluated
     (template, staleness, plan) in order, the number of draws, the returned configuration -- an AC-share one
-    in two of the three cases; the third runs with 12.5 GB per device, where the two memory models disagree.
-    The drop-in optimize() returns the same configurations."""
+    in two of the four cases; the third runs with 12.5 GB per device, where the two memory models disagree; the
+    fourth ranks by throughput x utilisation (max_throughput_loss = 0.1, optimizer.py:461-486), every evaluated
+    plan traced for Trace.utilization().  The drop-in optimize() returns the same configurations."""
     from rpeg_amd.core.types import Model
     from rpeg_amd.engine.runtime import Engine
     from rpeg_amd.search.cache import EvalCache
@@ -291,7 +309,7 @@ def test_optimize_over_structural_families_equals_reference():
     with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
         g = json.load(f)
     cases = [c for c in g["cases"] if c.get("families")]
-    assert len(cases) == 3
+    assert len(cases) == 4 and cases[3]["max_throughput_loss"] > 0
     for case in cases:
         p = family_problem(case)
         eng = Engine(p)
