@@ -186,9 +186,7 @@ RPEG_HD double list_schedule(const ClassView& c, MEM& mem, const uint8_t* ovl, u
   double makespan = 0.0;
   int done = 0;
   // every iteration either schedules a node or raises one node's key; the bound guards a broken class
-  long guard_iters = 0;
   for (long guard = 0; done < n && guard < (long)n * n + 64; ++guard) {
-    ++guard_iters;
     if (n_ready == 0) { *error = true; return 0.0; }  // cycle (scheduler.py:548-550)
     int bj = 0;
     int bv = mem.rd_node(0);
@@ -243,9 +241,6 @@ RPEG_HD double list_schedule(const ClassView& c, MEM& mem, const uint8_t* ovl, u
       mem.time(w) = t;
     }
   }
-#ifdef RPEG_COUNT_ITERS
-  RPEG_COUNT_ITERS(n, guard_iters);
-#endif
   if (done != n) *error = true;
   return makespan;
 }

@@ -318,6 +318,8 @@ struct rpeg_engine_s {
   size_t d_stage_cap = 0;
   uint8_t* h_stage = nullptr;   // pinned mirror of the result region of d_stage
   size_t h_stage_cap = 0;
+  uint8_t* d_trace = nullptr;   // rpeg_eval_trace: one plan's fields and header, then start / finish / dispatch index
+  size_t d_trace_nodes = 0;
   size_t hs_cap = 0;
   std::vector<uint32_t> hs_idx;
   uint32_t one_plan_waves_per_cu = 128;   // batches of at most this many plans per compute unit take one wavefront per plan
@@ -588,6 +590,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
   if (e->d_stage) hipFree(e->d_stage);
   if (e->h_stage) hipHostFree(e->h_stage);
+  if (e->d_trace) hipFree(e->d_trace);
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
   if (e->ev1) hipEventDestroy(e->ev1);
@@ -992,12 +995,16 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   if (int rc = ensure_pool(e, s)) return rc;
   if (int rc = ensure_perm(e, WAVE, 1)) return rc;
   if (int rc = ensure_ws(e, wave_ws_bytes(e->max_nodes, e->max_slots), s)) return rc;
-  int16_t* d_vert = nullptr;
-  uint8_t* d_head = nullptr;
-  double* d_tr = nullptr;
-  HIP_TRY(e, hipMalloc(&d_vert, RPEG_MAX_V * RPEG_FIELDS * 2));
-  HIP_TRY(e, hipMalloc(&d_head, 4));
-  HIP_TRY(e, hipMalloc(&d_tr, (size_t)n * 20));
+  constexpr size_t IN_BYTES = 256;   // fields (120 B) and header (4 B) of the plan, padded
+  if (!e->d_trace || (size_t)n > e->d_trace_nodes) {
+    if (e->d_trace) hipFree(e->d_trace);
+    e->d_trace = nullptr;
+    e->d_trace_nodes = std::max<size_t>(512, (size_t)n * 2);
+    HIP_TRY(e, hipMalloc(&e->d_trace, IN_BYTES + e->d_trace_nodes * 20));
+  }
+  int16_t* d_vert = (int16_t*)e->d_trace;
+  uint8_t* d_head = e->d_trace + RPEG_MAX_V * RPEG_FIELDS * 2;
+  double* d_tr = (double*)(e->d_trace + IN_BYTES);
   HIP_TRY(e, hipMemcpy(d_vert, vert_fields, RPEG_MAX_V * RPEG_FIELDS * 2, hipMemcpyHostToDevice));
   HIP_TRY(e, hipMemcpy(d_head, head4, 4, hipMemcpyHostToDevice));
   uint32_t lanes[WAVE];
@@ -1013,7 +1020,6 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   HIP_TRY(e, hipMemcpy(start, d_tr, (size_t)n * 8, hipMemcpyDeviceToHost));
   HIP_TRY(e, hipMemcpy(finish, d_tr + n, (size_t)n * 8, hipMemcpyDeviceToHost));
   if (dispatch_index) HIP_TRY(e, hipMemcpy(dispatch_index, d_tr + 2 * (size_t)n, (size_t)n * 4, hipMemcpyDeviceToHost));
-  hipFree(d_vert); hipFree(d_head); hipFree(d_tr);
   for (int i = 0; i < n; ++i) {
     if (node_kind) node_kind[i] = lc.nodes[i].kind;
     if (node_vertex) node_vertex[i] = lc.nodes[i].kind == 0 ? lc.nodes[i].vertex : lc.nodes[i].a1;
