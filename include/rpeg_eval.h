@@ -280,6 +280,12 @@ typedef struct rpeg_sa_serial_result_s {
   int64_t eval_log_cap, n_eval_log;
   double wall_s;
   int32_t best_family, pad;  /* family of best_plan (0 from rpeg_sa_optimize)                            */
+  double* eval_log_score;    /* optional, eval_log_cap entries each: what the run's cache holds for the   */
+  uint8_t* eval_log_feasible;/*   logged plan -- score and feasibility as evaluate_cached stores them for a */
+  double* eval_log_util;     /*   current plan (stale-layout gate applied) or as the merge of fresh         */
+                             /*   candidates stores them (optimizer.py:838), and Trace.utilization() when   */
+                             /*   the utilisation objective is on; a caller can carry them into its own     */
+                             /*   EvalCache, which polish() reads next (RPEG/pipeline.py:1549-1560)         */
 } rpeg_sa_serial_result_t;
 
 int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* params, int32_t E_max, int32_t E_struct,

@@ -584,6 +584,7 @@ struct SaSerial {
   std::unordered_map<std::string, Stored> cache;
   std::vector<SaPlan> eval_log;          // every plan handed to the evaluator as a cache miss, in order
   std::vector<uint8_t> eval_log_variant;
+  std::vector<Stored> eval_log_stored;   // what the cache holds for each of them
   std::map<int, std::vector<SaEntry>> elites;
   std::map<int, std::set<std::vector<int16_t>>> seens;
   SaEntry best, best_feasible;
@@ -665,6 +666,7 @@ struct SaSerial {
         cache[key(todo[j], variant)] = st;
         eval_log.push_back(todo[j]);
         eval_log_variant.push_back((uint8_t)variant);
+        eval_log_stored.push_back(st);
       }
       for (int i = 0; i < n; ++i)
         if (miss[i]) out[i] = cache[key(plans[i], variant)];
@@ -910,6 +912,11 @@ inline void sa_serial_result(const SaSerial& run, rpeg_sa_serial_result_t* res) 
     for (int64_t i = 0; i < keep; ++i) std::memcpy(res->eval_log + i * RPEG_MAX_V * RPEG_FIELDS, &run.eval_log[i], sizeof(SaPlan));
   if (res->eval_log_variant)
     for (int64_t i = 0; i < keep; ++i) res->eval_log_variant[i] = run.eval_log_variant[i];
+  for (int64_t i = 0; i < keep; ++i) {
+    if (res->eval_log_score) res->eval_log_score[i] = run.eval_log_stored[i].score;
+    if (res->eval_log_feasible) res->eval_log_feasible[i] = run.eval_log_stored[i].feasible;
+    if (res->eval_log_util) res->eval_log_util[i] = run.eval_log_stored[i].ev.util;
+  }
 }
 
 }  // namespace rpeg

@@ -106,7 +106,8 @@ class SaSerialResultT(C.Structure):
     _fields_ = [("best_plan", C.c_int16 * (MAX_V * FIELDS)), ("best_variant", C.c_int32), ("best_feasible", C.c_int32),
                 ("best_score", C.c_double), ("E", C.c_int64), ("n_draws", C.c_int64), ("n_uncounted", C.c_int64),
                 ("eval_log", C.c_void_p), ("eval_log_variant", C.c_void_p), ("eval_log_cap", C.c_int64),
-                ("n_eval_log", C.c_int64), ("wall_s", C.c_double), ("best_family", C.c_int32), ("pad", C.c_int32)]
+                ("n_eval_log", C.c_int64), ("wall_s", C.c_double), ("best_family", C.c_int32), ("pad", C.c_int32),
+                ("eval_log_score", C.c_void_p), ("eval_log_feasible", C.c_void_p), ("eval_log_util", C.c_void_p)]
 
 
 class SaFamilyT(C.Structure):

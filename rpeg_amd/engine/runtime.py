@@ -118,6 +118,9 @@ def serial_result(log_cap: int):
     log = np.zeros((max(log_cap, 1), abi.MAX_V * abi.FIELDS), np.int16)
     logv = np.zeros(max(log_cap, 1), np.uint8)
     res.eval_log, res.eval_log_variant, res.eval_log_cap = log.ctypes.data, logv.ctypes.data, log_cap
+    stored = (np.zeros(max(log_cap, 1)), np.zeros(max(log_cap, 1), np.uint8), np.zeros(max(log_cap, 1)))
+    res.eval_log_score, res.eval_log_feasible, res.eval_log_util = (a.ctypes.data for a in stored)
+    res._stored = stored     # kept alive with the record
     return res, log, logv
 
 
@@ -126,7 +129,9 @@ def serial_dict(res, log, logv):
     return dict(best_plan=np.array(res.best_plan, dtype=np.int16), best_variant=res.best_variant,
                 best_feasible=bool(res.best_feasible), best_score=res.best_score, E=res.E, n_draws=res.n_draws,
                 best_family=res.best_family, n_uncounted=res.n_uncounted, n_eval_log=res.n_eval_log, eval_log=log[:n].copy(),
-                eval_log_variant=logv[:n].copy(), wall_s=res.wall_s)
+                eval_log_variant=logv[:n].copy(), eval_log_score=res._stored[0][:n].copy(),
+                eval_log_feasible=res._stored[1][:n].astype(bool), eval_log_util=res._stored[2][:n].copy(),
+                wall_s=res.wall_s)
 
 
 def _torch():

@@ -100,13 +100,17 @@ def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware,
     if memory_trainable is not None and frozenset(memory_trainable) != frozenset(st.tau_models):
         st = replace(st, memory_trainable=frozenset(memory_trainable))
     structures = (st,) + tuple(more_structures)
-    key = (tuple((s.name, s.memory_trainable) for s in structures),
-           tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
+    rest = (tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
+    key = (tuple((s.name, s.memory_trainable) for s in structures),) + rest
     eng = _engines.get(key)
+    if eng is None and not more_structures:
+        # an engine that holds this template as structure 0 beside others serves as well (and keeps its classes)
+        eng = _engines.get(((st.name, st.memory_trainable), "first") + rest)
     if eng is None:
         problem = EvalProblem(structures=structures, suite=suite, workload=workload, hw=hw, device_space=space,
                               K_eval=K_eval, memory_policy=policy)
         eng = _engines[key] = Engine(problem)
+        _engines.setdefault(((st.name, st.memory_trainable), "first") + rest, eng)
     return eng, st
 
 

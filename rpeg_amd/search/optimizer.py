@@ -222,6 +222,18 @@ def optimize_families(problem: EvalProblem, opt_config: OptimizerConfig, engine_
     return families
 
 
+def family_structures(rpeg, opt_config: OptimizerConfig) -> tuple:
+    """The structures an engine for optimize() on the template of `rpeg` holds besides that template: for a
+    template that trains an actor and a critic, unless `structural_candidates` leaves AC-share out, the AC-share
+    template and its view under the base configuration's memory model."""
+    from ..engine.problem import STRUCTURES, as_seen_from
+    st = _structure_of(rpeg)
+    names = opt_config.structural_candidates
+    if set(st.tau_models) >= {Model.ACTOR, Model.CRITIC} and (names is None or "ac_share" in names):
+        return (STRUCTURES["ac_share"], as_seen_from(STRUCTURES["ac_share"], st))
+    return ()
+
+
 def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
              opt_config: OptimizerConfig, cache: Optional[EvalCache] = None, seed: int = 42,
              stream_key: Sequence[int] = (0, 0, 0)) -> Configuration:
@@ -239,18 +251,14 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
     With `max_throughput_loss` > 0 plans are ranked by throughput x utilisation above the throughput floor
     (optimizer.py:461-486); every evaluated plan is then traced once more for its utilisation.
 
-    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused") and deadlines.  `cache` is accepted for signature compatibility: the run keeps its own cache
-    (keyed by plan, template and staleness)."""
-    from ..engine.problem import STRUCTURES, as_seen_from
+    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused") and deadlines.  The run
+    keeps its own cache (keyed by plan, template and staleness); what it evaluated is put into `cache`
+    afterwards under the reference's keys, entries `cache` held before are not consulted."""
     _check_supported(base_config)
     if opt_config.deadline is not None:
         raise NotImplementedError("deadlines are not part of this engine")
     policy = opt_config.memory_policy()
-    st = _structure_of(base_config.rpeg)
-    names = opt_config.structural_candidates
-    more = ()
-    if set(st.tau_models) >= {Model.ACTOR, Model.CRITIC} and (names is None or "ac_share" in names):
-        more = (STRUCTURES["ac_share"], as_seen_from(STRUCTURES["ac_share"], st))
+    more = family_structures(base_config.rpeg, opt_config)
     eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy, more)
 
     def directory(structure: int):
@@ -262,8 +270,34 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
     families[0][0].seed = seed
     own = [int(base_config.rpeg.tau.get(m, 0)) for m in st.tau_models]
     res = eng.sa_optimize_families(families, own, plan_row(base_config.rpeg, base_config.plan), opt_config.E_max,
-                                   opt_config.E_struct, opt_config.R_max, stream_key)
+                                   opt_config.E_struct, opt_config.R_max, stream_key,
+                                   log_cap=opt_config.E_max + 64 if cache is not None else 0)
+    if cache is not None:
+        _carry_into(cache, eng.problem, families, res, own, suite, workload, base_config, policy,
+                    opt_config.max_throughput_loss > 0.0)
     return configuration_of(eng.problem, families, res, own, suite, workload, base_config)
+
+
+def _carry_into(cache: EvalCache, problem, families, res, base_tau, suite, workload, base_config, policy, with_util):
+    """Puts what the run evaluated into the caller's cache under the reference's keys, so that what runs next on
+    the same cache -- polish() in the reference's pipeline (RPEG/pipeline.py:1549-1560) -- finds the entries
+    optimize() would have left there: score and feasibility as stored, and in the trace's place the
+    utilisation (the one number of a trace that polish reads) when the utilisation objective is on."""
+    templates = {}
+    for row, var, score, feasible, util in zip(res["eval_log"], res["eval_log_variant"], res["eval_log_score"],
+                                               res["eval_log_feasible"], res["eval_log_util"]):
+        var = int(var)
+        if var not in templates:
+            f, k = (0, None) if var == 255 else (var // 8, var % 8)
+            st = problem.structures[families[f][0].structure]
+            taus = list(base_tau) if k is None else [int(families[f][0].tau[k][i]) for i in range(len(st.tau_models))]
+            templates[var] = st.build(suite, workload, tau={m: taus[i] for i, m in enumerate(st.tau_models)})
+        rpeg = templates[var]
+        config = Configuration(rpeg, row_plan(rpeg, row), base_config.device_space, intra_stage_fusion=False,
+                               transfer_resource_policy=base_config.transfer_resource_policy)
+        h = evaluation_cache_key(config, policy)
+        if h not in cache:
+            cache.put(h, float(score), _Utilization(float(util)) if with_util else None, bool(feasible))
 
 
 def configuration_of(problem: EvalProblem, families, res, base_tau, suite, workload, base_config) -> Configuration:

@@ -1,0 +1,78 @@
+"""The search part of the reference's pipeline as one call (RPEG/pipeline.py:1405-1560, without the command
+line, plots and reports): start plans from the candidate directory, the three evaluations that open the cache,
+optimize() over the structural families, polish() on the same cache.  Every step runs on the GPU engine."""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Optional, Sequence
+
+from ..core.types import DeviceSpace, Model
+from ..ir.plan import ExecutionPlan
+from ..model.hardware import Hardware
+from ..model.models import ModelSuite
+from ..model.workload import Workload
+from .baselines import build_concurrent_baseline_plan, build_valid_baseline_plan
+from .cache import EvalCache
+from .evaluate import Configuration, _engine_for, evaluate_cached
+from .moves import build_candidate_directory
+from .optimizer import OptimizerConfig, family_structures, optimize, polish
+
+def _template(algorithm: str, suite: ModelSuite, workload: Workload, tau: Optional[Dict[Model, int]]):
+    """The synchronous template of an algorithm (RPEG/pipeline.py:1405-1410)."""
+    from ..ir.dpo import build_DPO_RPEG
+    from ..ir.grpo import build_GRPO_RPEG
+    from ..ir.ppo import build_PPO_RPEG
+    build = {"dpo": build_DPO_RPEG, "grpo": build_GRPO_RPEG}.get(algorithm, build_PPO_RPEG)
+    return build(suite, workload, tau) if tau is not None else build(suite, workload)
+
+
+@dataclass
+class SearchResult:
+    start: Configuration                 # what optimize() was seeded with: the concurrent start plan or `seed_plan`
+    greedy: Configuration
+    concurrent_found: bool               # False: no concurrent plan fits, the start is the greedy plan
+    optimized: Configuration
+    polished: Configuration              # == optimized when polish was skipped (infeasible result, no_polish)
+    scores: Dict[str, float] = field(default_factory=dict)     # greedy, start, optimized, polished
+    seconds: Dict[str, float] = field(default_factory=dict)    # directory + start plans, optimize, polish
+    cache: Optional[EvalCache] = None
+
+
+def search_plan(suite: ModelSuite, workload: Workload, hw: Hardware, device_space: DeviceSpace, K_eval: int,
+                opt_config: OptimizerConfig, algorithm: Optional[str] = None, tau_sync: Optional[Dict[Model, int]] = None,
+                seed_plan: Optional[ExecutionPlan] = None, cache: Optional[EvalCache] = None, seed: int = 42,
+                stream_key: Sequence[int] = (0, 0, 0), no_polish: bool = False) -> SearchResult:
+    """Start plans -> optimize -> polish, in the order and on the shared cache of RPEG/pipeline.py:1412-1560."""
+    algorithm = algorithm or opt_config.algorithm
+    policy = opt_config.memory_policy()
+    cache = cache if cache is not None else EvalCache()
+    rpeg = _template(algorithm, suite, workload, tau_sync)
+    t0 = time.perf_counter()
+    eng, _ = _engine_for(rpeg, suite, workload, hw, device_space, K_eval, policy, family_structures(rpeg, opt_config))
+    table, _ = build_candidate_directory(rpeg, suite, device_space, workload, eng)
+    conc_plan, found = build_concurrent_baseline_plan(rpeg, device_space, suite, workload, eng, table=table)
+    greedy_plan = build_valid_baseline_plan(rpeg, device_space, suite, workload, eng, table=table)
+    t1 = time.perf_counter()
+    greedy = Configuration(rpeg, greedy_plan, device_space)
+    conc = Configuration(rpeg, conc_plan, device_space)
+    start = Configuration(rpeg, seed_plan if seed_plan is not None else conc_plan, device_space)
+    scores = {}
+    scores["greedy"] = evaluate_cached(greedy, cache, suite, workload, hw, K_eval, policy)[0]
+    scores["concurrent"] = evaluate_cached(conc, cache, suite, workload, hw, K_eval, policy)[0]
+    scores["start"] = evaluate_cached(start, cache, suite, workload, hw, K_eval, policy)[0]
+    t2 = time.perf_counter()
+    optimized = optimize(start, suite, workload, hw, K_eval, opt_config, cache, seed=seed, stream_key=stream_key)
+    t3 = time.perf_counter()
+    scores["optimized"], _, feasible, _ = evaluate_cached(optimized, cache, suite, workload, hw, K_eval, policy)
+    polished = optimized
+    if feasible and not no_polish:      # pipeline.py:1553-1560
+        ac_share = Model.AC_SHARE in optimized.rpeg.trainable
+        structure = 1 if ac_share else 0
+        p_table, p_index = build_candidate_directory(optimized.rpeg, suite, device_space, workload, eng, structure)
+        polished = polish(optimized, suite, workload, hw, K_eval, opt_config, cache, p_table, p_index, ac_share=ac_share)
+    t4 = time.perf_counter()
+    scores["polished"] = evaluate_cached(polished, cache, suite, workload, hw, K_eval, policy)[0]
+    return SearchResult(start=start, greedy=greedy, concurrent_found=found, optimized=optimized, polished=polished,
+                        scores=scores, seconds=dict(start_plans=t1 - t0, optimize=t3 - t2, polish=t4 - t3), cache=cache)

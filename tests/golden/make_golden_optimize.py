@@ -55,6 +55,73 @@ CASES = [dict(plan=0, stream=(42, 77, 0, 0), E_max=260, E_struct=200, stag_windo
               families=True, T_cand=[[0, 1], [0], [0]], base_tau=[0, 0], lambda_ac=0.15, max_throughput_loss=0.10)]
 
 
+PIPELINE = dict(stream=(42, 77, 6, 0), E_max=300, E_struct=60, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
+                lambda_ac=0.05)
+
+
+def pipeline_case(ref, mods, moves, ropt, rcache, Configuration, st, ct, problem, rows):
+    """The search part of the reference's pipeline on config 1 (pipeline.py:1412-1560): concurrent start plan,
+    the three evaluations that fill the cache, optimize() over both families, polish() on the same cache."""
+    import contextlib
+    import importlib.util
+    import io
+    import types
+    from oracle.sa_oracle import CounterRng
+    vis = types.ModuleType("scripts.visualize")
+    for name in ("dot_to_img", "exec_to_dot", "rpeg_to_dot", "unrolled_to_dot", "safe_unlink", "trace_to_gantt"):
+        setattr(vis, name, None)
+    pkg = types.ModuleType("scripts")
+    pkg.__path__ = []
+    sys.modules["scripts"], sys.modules["scripts.visualize"] = pkg, vis
+    spec = importlib.util.spec_from_file_location("ref_pipeline", os.path.join(ref, "pipeline.py"))
+    pipe = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(pipe)
+    stub = sys.modules["search.evaluate"]
+
+    rpeg0, suite, wl, hw, space, cost, mm = SA.ref_world(mods, problem, {"Pi": 0, "V": 0})
+    st.update(problem=problem, suite=suite, wl=wl, hw=hw, space=space, cost=cost, mm=mm, mms={}, log=[], families=True)
+    with contextlib.redirect_stdout(io.StringIO()):
+        conc_plan, found = pipe.build_concurrent_baseline_plan(rpeg0, space, suite, wl, cost, mm)
+        greedy_plan = pipe.build_valid_baseline_plan(rpeg0, space, suite, wl, cost, mm)
+    cache = rcache.EvalCache()
+    base = Configuration(rpeg0, conc_plan, space)
+    for config in (Configuration(rpeg0, greedy_plan, space), Configuration(rpeg0, conc_plan, space), base):
+        stub.evaluate_cached(config, cache, suite, wl, hw, problem.K_eval)
+    case = PIPELINE
+    oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
+                              structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"],
+                              T_init=case["T_init"], T_warm=case["T_warm"], T_min=case["T_min"],
+                              stag_window=case["stag_window"])
+    rng = CounterRng(*case["stream"])
+    ropt.random = rng
+    moves.random = rng
+    st["log"] = []
+    real_cpu_count = os.cpu_count
+    os.cpu_count = lambda: 1
+    try:
+        out = ropt.optimize(base, suite, wl, hw, problem.K_eval, oc, cache)
+        n_opt = len(st["log"])
+        _, _, feasible, _ = stub.evaluate_cached(out, cache, suite, wl, hw, problem.K_eval)
+        assert feasible
+        ac = ct.Model.AC_SHARE in out.rpeg.trainable
+        table, index = moves.build_candidate_directory(out.rpeg, suite, space, wl, cost, mm)
+        pol = ropt.polish(out, suite, wl, hw, problem.K_eval, oc, cache, table, index, ac_share=ac)
+    finally:
+        os.cpu_count = real_cpu_count
+    s_opt = stub.evaluate_cached(out, cache, suite, wl, hw, problem.K_eval)[0]
+    s_pol = stub.evaluate_cached(pol, cache, suite, wl, hw, problem.K_eval)[0]
+
+    def setting(config):
+        return dict(first_vertex=config.rpeg.vertices[0].id, rows=rows(config),
+                    tau=[config.rpeg.tau[m] for m in sorted(config.rpeg.tau, key=lambda m: m.value)])
+    print("pipeline: optimize evaluations", n_opt, "polish evaluations", len(st["log"]) - n_opt, "draws", rng.k,
+          "scores", s_opt, "->", s_pol, setting(pol)["first_vertex"], setting(pol)["tau"])
+    return dict(case, stream=list(case["stream"]), concurrent_found=bool(found), start=rows(base),
+                greedy=rows(Configuration(rpeg0, greedy_plan, space)), n_optimize=n_opt,
+                n_polish=len(st["log"]) - n_opt, n_draws=rng.k, optimized=setting(out), optimized_score=float(s_opt).hex(),
+                polished=setting(pol), polished_score=float(s_pol).hex())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--ref", default="/root/reference")
@@ -195,6 +262,7 @@ def main():
                 (e[0], tuple(e[1])) for e in log).items()]
         print("case", case["plan"], "evaluations", len(log), "draws", rng.k, doc["cases"][-1].get("per_setting", ""),
               "->", doc["cases"][-1]["final_first_vertex"], doc["cases"][-1]["final_tau"])
+    doc["pipeline"] = pipeline_case(args.ref, mods, moves, ropt, rcache, Configuration, st, ct, p_config, rows)
     path = os.path.join(HERE, "ref_optimize.json")
     with open(path, "w") as f:
         json.dump(doc, f, separators=(",", ":"))

@@ -334,3 +334,35 @@ def test_optimize_over_structural_families_equals_reference():
         got = plan_row(out.rpeg, out.plan)
         assert [[int(x) for x in got[v * 10:(v + 1) * 10]] for v in range(nv)] == case["final"]
         eng.close()
+
+
+def test_search_pipeline_equals_reference_pipeline():
+    """search_plan on config 1 against the same steps of the reference's pipeline (RPEG/pipeline.py:1412-1560,
+    tests/golden/make_golden_optimize.py): the concurrent and the greedy start plan, the configuration optimize()
+    returns over both structural families when seeded with the concurrent plan, what polish() makes of it on
+    the shared cache, their scores, and the number of evaluations that end up in the cache."""
+    from rpeg_amd.search.optimizer import plan_row
+    from rpeg_amd.search.pipeline import search_plan
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        g = json.load(f)["pipeline"]
+    p = configs.config(1).problem
+    opt = OptimizerConfig(K_x=6, T_max=50, E_max=g["E_max"], E_struct=g["E_struct"], T_init=g["T_init"],
+                          T_warm=g["T_warm"], T_min=g["T_min"], stag_window=g["stag_window"], lambda_ac=g["lambda_ac"],
+                          structural_candidates=frozenset({"separate", "ac_share"}))
+    res = search_plan(p.suite, p.workload, p.hw, p.device_space, p.K_eval, opt, algorithm="ppo", seed=g["stream"][0],
+                      stream_key=g["stream"][1:])
+
+    def rows(config):
+        r = plan_row(config.rpeg, config.plan)
+        return [[int(x) for x in r[v * 10:(v + 1) * 10]] for v in range(len(config.rpeg.vertices))]
+
+    def setting(config):
+        return dict(first_vertex=config.rpeg.vertices[0].id, rows=rows(config),
+                    tau=[config.rpeg.tau[m] for m in sorted(config.rpeg.tau, key=lambda m: m.value)])
+
+    assert res.concurrent_found == g["concurrent_found"]
+    assert rows(res.start) == g["start"] and rows(res.greedy) == g["greedy"]
+    assert setting(res.optimized) == g["optimized"] and float(res.scores["optimized"]).hex() == g["optimized_score"]
+    assert setting(res.polished) == g["polished"] and float(res.scores["polished"]).hex() == g["polished_score"]
+    n_before = len({json.dumps(g["start"]), json.dumps(g["greedy"])})
+    assert res.cache.misses == n_before + g["n_optimize"] + g["n_polish"]
