@@ -73,7 +73,8 @@ def stale_publication_layout_valid(config: Configuration) -> bool:
 
 
 # ----------------------------------------------------------------------------- engine plumbing
-_engines: Dict[tuple, object] = {}
+_engines: Dict[tuple, object] = {}   # insertion-ordered: least recently used first
+_MAX_ENGINES = 16
 
 
 def _structure_of(rpeg: RPEG):
@@ -102,15 +103,19 @@ def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware,
     structures = (st,) + tuple(more_structures)
     rest = (tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
     key = (tuple((s.name, s.memory_trainable) for s in structures),) + rest
-    eng = _engines.get(key)
-    if eng is None and not more_structures:
-        # an engine that holds this template as structure 0 beside others serves as well (and keeps its classes)
-        eng = _engines.get(((st.name, st.memory_trainable), "first") + rest)
-    if eng is None:
-        problem = EvalProblem(structures=structures, suite=suite, workload=workload, hw=hw, device_space=space,
-                              K_eval=K_eval, memory_policy=policy)
-        eng = _engines[key] = Engine(problem)
-        _engines.setdefault(((st.name, st.memory_trainable), "first") + rest, eng)
+    alias = ((st.name, st.memory_trainable), "first") + rest
+    hit = key if key in _engines else alias if not more_structures and alias in _engines else None
+    if hit is not None:
+        # (an engine that holds this template as structure 0 beside others serves as well, and keeps its classes)
+        eng = _engines.pop(hit)
+        _engines[hit] = eng          # most recently used last
+        return eng, st
+    problem = EvalProblem(structures=structures, suite=suite, workload=workload, hw=hw, device_space=space,
+                          K_eval=K_eval, memory_policy=policy)
+    eng = _engines[key] = Engine(problem)
+    _engines.setdefault(alias, eng)
+    while len(_engines) > _MAX_ENGINES:      # a long-lived process that sees many problems keeps the recent ones;
+        _engines.pop(next(iter(_engines)))   # an engine frees its device memory when its last holder lets go
     return eng, st
 
 
