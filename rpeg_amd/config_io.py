@@ -44,6 +44,24 @@ def load_config(path: str) -> Dict:
         return yaml.load(f, Loader=_Loader)
 
 
+def merge_hardware_overlay(cfg: Dict, path: str) -> Dict:
+    """Overlays the `key: value` lines of a calibrated-hardware file on cfg["hardware"] as the reference's
+    `--hw` option does (pipeline.py:1288-1302): comment and blank lines skipped, text after `#` dropped, values
+    that do not read as floats ignored.  Returns cfg."""
+    overlay = {}
+    with open(path) as f:
+        for line in f:
+            if not line.strip() or line.strip().startswith("#") or ":" not in line:
+                continue
+            key, val = line.split(":", 1)
+            try:
+                overlay[key.strip()] = float(val.split("#")[0].strip())
+            except ValueError:
+                pass
+    cfg.setdefault("hardware", {}).update(overlay)
+    return cfg
+
+
 def _require(d: Dict, *keys: str, section: str = "") -> None:
     prefix = f"[{section}] " if section else ""
     for k in keys:

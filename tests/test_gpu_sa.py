@@ -366,3 +366,33 @@ def test_search_pipeline_equals_reference_pipeline():
     assert setting(res.polished) == g["polished"] and float(res.scores["polished"]).hex() == g["polished_score"]
     n_before = len({json.dumps(g["start"]), json.dumps(g["greedy"])})
     assert res.cache.misses == n_before + g["n_optimize"] + g["n_polish"]
+
+
+def test_search_from_config_file_writes_loadable_plans(tmp_path):
+    """search_from_config on the YAML of config 1 (the reference's schema) with small budgets: the plan files named
+    in its output section are written in the reference's plan schema and load back to the plans returned; the
+    polished plan is feasible and no worse than the start."""
+    import yaml
+    from rpeg_amd import config_io
+    from rpeg_amd.ir.serialize import load_plan
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import evaluate_cached
+    from rpeg_amd.search.optimizer import plan_row
+    from rpeg_amd.search.pipeline import search_from_config
+    here = os.path.dirname(os.path.abspath(config_io.__file__))
+    cfg = config_io.load_config(os.path.join(here, "config_files", "cfg1.yaml"))
+    cfg["optimizer"].update(e_max=200, e_struct=60, stag_window=4)
+    cfg["output"] = {"base_plan": str(tmp_path / "base.yaml"), "opt_plan": str(tmp_path / "opt.yaml"), "seed": 7}
+    hw = tmp_path / "hw.yaml"
+    hw.write_text(f"memory_per_gpu: {cfg['hardware']['memory_per_gpu']}  # unchanged\n")
+    res = search_from_config(cfg, hw_overlay=str(hw))
+    assert res.scores["polished"] >= res.scores["optimized"] >= res.scores["start"] > 0
+    for config, name in ((res.start, "base.yaml"), (res.polished, "opt.yaml")):
+        back = load_plan(str(tmp_path / name), config.rpeg)
+        assert list(plan_row(config.rpeg, back)) == list(plan_row(config.rpeg, config.plan))
+    p = config_io.problem_from_config(cfg)
+    _, _, feasible, _ = evaluate_cached(res.polished, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+    assert feasible
+    # the run is a function of the seed
+    again = search_from_config(cfg, hw_overlay=str(hw))
+    assert list(plan_row(again.polished.rpeg, again.polished.plan)) == list(plan_row(res.polished.rpeg, res.polished.plan))

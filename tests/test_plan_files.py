@@ -93,3 +93,17 @@ def test_config_loader_and_validation(tmp_path):
         config_io.validate_config(bad)
     grpo = config_io.build_optimizer_config(config_io.load_config(os.path.join(CONFIG_DIR, "cfg2.yaml")), False, "grpo")
     assert grpo.T_cand == {Model.ACTOR: {0, 1}}
+
+
+def test_hardware_overlay_merges_like_the_reference(tmp_path):
+    """The `--hw` overlay of RPEG/pipeline.py:1288-1302: key: value lines, comments and trailing comments dropped,
+    non-numeric values ignored, later keys win over the configuration's."""
+    from rpeg_amd import config_io
+    path = tmp_path / "hw.yaml"
+    path.write_text("# calibrated\n\nflops_per_gpu: 9.5e14   # measured\nmemory_bandwidth: 3.1e12\nname: mi355x\n"
+                    "  gemm_m_half : 512\nnot a pair\n")
+    cfg = {"hardware": {"flops_per_gpu": 1.0, "racks": 2}}
+    out = config_io.merge_hardware_overlay(cfg, str(path))
+    assert out is cfg
+    assert cfg["hardware"] == {"flops_per_gpu": 9.5e14, "racks": 2, "memory_bandwidth": 3.1e12, "gemm_m_half": 512.0}
+    assert config_io.merge_hardware_overlay({}, str(path))["hardware"]["memory_bandwidth"] == 3.1e12
