@@ -5,7 +5,6 @@ The library is built in-tree; it has no CPU fallback and refuses to create an en
 
 import os
 import subprocess
-import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "librpeg_eval.so")

@@ -16,11 +16,11 @@ per-call argument of `evaluate` (RPEG/search/evaluate.py:235-241).
 from __future__ import annotations
 
 from dataclasses import dataclass, field, replace
-from typing import Callable, Dict, FrozenSet, List, Optional, Sequence, Tuple
+from typing import Callable, FrozenSet, Optional, Sequence, Tuple
 
 import numpy as np
 
-from ..core.types import Allocation, DeviceSpace, Model, TemplateVertex
+from ..core.types import Allocation, DeviceSpace, Model
 from ..ir.plan import ExecutionPlan
 from ..ir.rpeg import RPEG
 from ..ir.ppo import build_PPO_RPEG

@@ -16,7 +16,7 @@ set, and the generation-split index uniform over 0..Q.
 
 from __future__ import annotations
 
-from typing import Dict, List, Sequence, Tuple
+from typing import Dict, Sequence
 
 import numpy as np
 

@@ -8,7 +8,7 @@ import pytest
 from oracle import rpeg_oracle as oracle
 from oracle.cpu_port import CpuPort, exp_libm
 from rpeg_amd.engine import abi
-from tests.helpers import load_golden, oracle_eval, seeded_batch
+from tests.helpers import load_golden, seeded_batch
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])

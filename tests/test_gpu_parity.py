@@ -387,7 +387,6 @@ def test_is_valid_drop_in_equals_restatement(c):
     structure and staleness of the configuration as they are, then broken one rule at a time; under the
     template's own memory model and under one whose trainable set is another template's (what optimize()
     passes for AC-share plans)."""
-    import dataclasses
     from oracle import rpeg_oracle as O
     from rpeg_amd.core.types import Allocation, Model
     from rpeg_amd.ir.plan import ExecutionPlan

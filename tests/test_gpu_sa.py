@@ -301,7 +301,6 @@ def test_optimize_over_structural_families_equals_reference():
     in two of the four cases; the third runs with 12.5 GB per device, where the two memory models disagree; the
     fourth ranks by throughput x utilisation (max_throughput_loss = 0.1, optimizer.py:461-486), every evaluated
     plan traced for Trace.utilization().  The drop-in optimize() returns the same configurations."""
-    from rpeg_amd.core.types import Model
     from rpeg_amd.engine.runtime import Engine
     from rpeg_amd.search.cache import EvalCache
     from rpeg_amd.search.evaluate import Configuration

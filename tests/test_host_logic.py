@@ -11,7 +11,7 @@ import pytest
 
 from oracle import rpeg_oracle as oracle
 from rpeg_amd import configs
-from rpeg_amd.core.types import Allocation, DeviceSpace, Model, packing_geometry, rectangular_node_layouts
+from rpeg_amd.core.types import Allocation, Model, packing_geometry, rectangular_node_layouts
 from rpeg_amd.engine import abi
 from rpeg_amd.engine.compile import compile_problem, gen_phases
 from rpeg_amd.engine.problem import PlanBatch

@@ -10,11 +10,8 @@ import pytest
 
 from oracle import rpeg_oracle as oracle
 from rpeg_amd import configs
-from rpeg_amd.core.types import Allocation, DeviceSpace, Model, Role
-from rpeg_amd.engine.problem import EvalProblem
+from rpeg_amd.core.types import Allocation, Model
 from rpeg_amd.ir.plan import ExecutionPlan
-from rpeg_amd.model.models import ModelSpec, ModelSuite
-from rpeg_amd.model.workload import Workload
 from tests.helpers import oracle_eval, seeded_batch
 
 

@@ -20,9 +20,8 @@ from oracle.cpu_port import CpuPort
 from rpeg_amd import configs
 from rpeg_amd.core.types import Allocation
 from rpeg_amd.engine import abi
-from rpeg_amd.engine.problem import PlanBatch
 from rpeg_amd.ir.plan import ExecutionPlan
-from rpeg_amd.search.optimizer import OptimizerConfig, plan_row, row_plan, sa_params
+from rpeg_amd.search.optimizer import OptimizerConfig, plan_row, sa_params
 from tests.helpers import GOLDEN, check_family_case, family_case_setup, family_problem, seeded_batch
 
 

@@ -11,7 +11,6 @@ import pytest
 
 from oracle import rpeg_oracle as O
 from oracle import sa_oracle as S
-from rpeg_amd.core.types import Allocation
 from rpeg_amd.ir.plan import ExecutionPlan
 from tests.helpers import GOLDEN, seeded_batch
 
