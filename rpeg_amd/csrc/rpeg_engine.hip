@@ -204,6 +204,7 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
 template <int LS>
 __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
   extern __shared__ uint8_t ke_lds[];
+  if ((L.flags & KE_FIXUP) && L.need && L.need[KE_NEED_SHARDS] == 0u) return;   // no plan outgrew its list
   for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
     if (LS == 0 && (L.wave_cls[w] & KE_CLS_LDS)) ke_eval_wave<KE_FEW>(L, w, ke_lds);   // uniform branch
     else ke_eval_wave<LS>(L, w, ke_lds);
@@ -361,8 +362,8 @@ static int ensure_batch(rpeg_engine_t* e, size_t n) {
   HIP_TRY(e, hipMalloc(&e->d_ovf, cap));
   HIP_TRY(e, hipMemset(e->d_ovf, 0, cap));   // flags are cleared again by the launch that consumes them
   if (!e->d_need) {
-    HIP_TRY(e, hipMalloc(&e->d_need, KE_NEED_SHARDS * 4));
-    HIP_TRY(e, hipMemset(e->d_need, 0, KE_NEED_SHARDS * 4));
+    HIP_TRY(e, hipMalloc(&e->d_need, (KE_NEED_SHARDS + 1) * 4));
+    HIP_TRY(e, hipMemset(e->d_need, 0, (KE_NEED_SHARDS + 1) * 4));
     HIP_TRY(e, hipHostMalloc(&e->h_need, KE_NEED_SHARDS * 4));
     std::memset(e->h_need, 0, KE_NEED_SHARDS * 4);
   }
@@ -929,7 +930,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       HIP_TRY(e, hipFuncSetAttribute((const void*)k_eval<0>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       e->lds_attr_set[0] = true;
     }
-    hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds_full, s, F);
+    // a small grid: the launch almost always finds the count of flagged plans at zero and ends at once
+    hipLaunchKernelGGL(k_eval<0>, dim3(std::min<unsigned>(grid, (unsigned)e->n_cu * 2u)), dim3(WAVE), lds_full, s, F);
     HIP_TRY(e, hipGetLastError());
   }
   if (n_solo) {   // the single-plan wavefronts, beside the main kernel

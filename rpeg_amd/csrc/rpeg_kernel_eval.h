@@ -51,7 +51,8 @@ struct EvalLaunch {              // uniform launch parameters
   unsigned long long* prof;      // optional per-wavefront phase clocks (8 per wavefront), or null
   uint8_t* ovf;                  // per plan: its ready list outgrew rcap (set by a launch with a short list,
                                  // consumed by the KE_FIXUP launch with the full one), or null
-  uint32_t* need;                // KE_NEED_SHARDS running maxima of the ready-list length, or null
+  uint32_t* need;                // KE_NEED_SHARDS running maxima of the ready-list length, then one word that
+                                 // counts the plans flagged in `ovf` and not yet redone; or null
 };
 constexpr uint32_t KE_FIXUP = 0x80000000u;   // EvalLaunch::flags: only the plans flagged in `ovf` are evaluated
 constexpr int KE_NEED_SHARDS = 64;
@@ -512,8 +513,15 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   }
   if (done != n) err = true;
   if (L.ovf) {
-    if (L.flags & KE_FIXUP) L.ovf[pi] = 0;
+    const bool fix = (L.flags & KE_FIXUP) != 0;
+    if (fix) L.ovf[pi] = 0;
     else if (ovf) L.ovf[pi] = 1;
+    // the count of flagged plans lets a fix-up launch that has nothing to redo end at once
+    const int k = __builtin_popcountll(__ballot(fix || ovf));
+    if (k && L.need && lane == first_lane) {
+      if (fix) atomicSub(L.need + KE_NEED_SHARDS, (uint32_t)k);
+      else atomicAdd(L.need + KE_NEED_SHARDS, (uint32_t)k);
+    }
   }
   if (L.need) {   // longest ready list of the wavefront, folded into one of the running maxima
     int m = max_ready;
