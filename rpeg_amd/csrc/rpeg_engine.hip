@@ -920,6 +920,19 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     default: hipLaunchKernelGGL(k_eval<64>, dim3(grid), dim3(WAVE), lds, s, L); break;
   }
   HIP_TRY(e, hipGetLastError());
+  if (n_solo) {   // the single-plan wavefronts, beside the main kernel
+    EvalLaunch S = L;
+    S.perm = e->d_perm + n_sorted;
+    S.wave_cls = e->d_cls + n_eval_waves;
+    S.n_waves = n_solo;
+    if (L.prof) S.prof = L.prof + n_waves * 8;
+    HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
+    hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n_solo, (uint64_t)e->n_cu * 32)), dim3(WAVE),
+                       kp_lds_bytes(e->max_nodes, e->max_slots), e->s2, S);
+    HIP_TRY(e, hipGetLastError());
+    HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
+  }
+  // (after the submission of k_plan, which is the longer of the two kernels and should not wait for this one)
   if (short_list && n_waves) {   // the plans whose ready list outgrew the short one, with the full one
     EvalLaunch F = L;
     F.rcap = rcap_full;
@@ -933,18 +946,6 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     // a small grid: the launch almost always finds the count of flagged plans at zero and ends at once
     hipLaunchKernelGGL(k_eval<0>, dim3(std::min<unsigned>(grid, (unsigned)e->n_cu * 2u)), dim3(WAVE), lds_full, s, F);
     HIP_TRY(e, hipGetLastError());
-  }
-  if (n_solo) {   // the single-plan wavefronts, beside the main kernel
-    EvalLaunch S = L;
-    S.perm = e->d_perm + n_sorted;
-    S.wave_cls = e->d_cls + n_eval_waves;
-    S.n_waves = n_solo;
-    if (L.prof) S.prof = L.prof + n_waves * 8;
-    HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
-    hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n_solo, (uint64_t)e->n_cu * 32)), dim3(WAVE),
-                       kp_lds_bytes(e->max_nodes, e->max_slots), e->s2, S);
-    HIP_TRY(e, hipGetLastError());
-    HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
   }
   if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
   if (e->timing) {
