@@ -191,14 +191,17 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
 __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const uint32_t* __restrict__ kidx,
                           const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
                           const uint32_t* __restrict__ cbase, uint32_t shards, uint32_t* __restrict__ perm,
-                          uint32_t pstride) {
+                          uint32_t pstride, const uint32_t* __restrict__ coff, uint32_t* __restrict__ task_cls,
+                          uint32_t first_entry) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t c = cid[i];
   if (c >= CID_UNKNOWN) return;
   const uint32_t k = cbase[c * shards + ((uint32_t)(i / SIG_BLOCK) & (shards - 1u))] + kidx[i], l = clpw[c] & 0xFFFFu;
-  if (clpw[c] >> 16) perm[(uint64_t)cfirst[c] + k] = (uint32_t)i;   // a class of single-plan wavefronts: cfirst is its first entry
-  else perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
+  if (clpw[c] >> 16) {   // a class of single-plan wavefronts: cfirst is its first entry; the task learns its class here
+    perm[(uint64_t)cfirst[c] + k] = (uint32_t)i;
+    task_cls[cfirst[c] + k - first_entry] = coff[c];
+  } else perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
 }
 
 template <int LS>
@@ -406,8 +409,8 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
       hipHostFree(e->h_ccount);
     }
     e->d_ccount = nullptr; e->ccap = 0;
-    HIP_TRY(e, hipMalloc(&e->d_ccount, (3 * (size_t)cap + COUNT_SLOTS + 64) * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (3 * (size_t)cap + COUNT_SLOTS + 64) * 4));
+    HIP_TRY(e, hipMalloc(&e->d_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4));
+    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4));
     e->ccap = cap;
   }
   e->tables_for = ncls;
@@ -823,11 +826,17 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_eval_waves + n_solo)) return rc;
   uint32_t* const h_cfirst = e->h_ccount + (size_t)ncls * shards;   // behind the shard offsets
   uint32_t* const h_clpw = h_cfirst + ncls;
+  uint32_t* const h_coff = h_clpw + ncls;
   const uint32_t* const d_cfirst = e->d_ccount + (size_t)ncls * shards;
   const uint32_t* const d_clpw = d_cfirst + ncls;
+  const uint32_t* const d_coff = d_clpw + ncls;
+  // tasks of one plan get their class from the scatter kernel, not from the host: with one plan per wavefront
+  // throughout that is every task of the launch, otherwise the tasks of the classes taken out of the main kernel
+  const uint32_t n_host_tasks = one ? 0u : n_eval_waves;
   for (size_t c = 0; c < counts.size(); ++c) {
     h_cfirst[cids[c]] = first[c];
-    h_clpw[cids[c]] = clpw[c];
+    h_clpw[cids[c]] = one ? (1u | (1u << 16)) : clpw[c];
+    h_coff[cids[c]] = offs[c];
   }
   // wavefronts of few plans keep their scheduler state in LDS when that needs no more LDS than the ready
   // lists of a full wavefront do
@@ -840,9 +849,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       ke_lds_bytes(0, rcap, KE_FEW, e->max_nodes, e->max_slots, e->max_v) <= ke_lds_bytes(0, rcap, 0, e->max_nodes, e->max_slots, e->max_v);
   for (size_t k = 0; k < order.size(); ++k) {
     const uint32_t c = order[k];
-    if (solo[c]) {
-      const uint32_t t0 = n_eval_waves + (first[c] - (uint32_t)n_sorted);
-      for (uint32_t t = 0; t < counts[c]; ++t) e->h_cls[t0 + t] = offs[c];
+    if (solo[c] || one) {
+      continue;
     } else {
       const uint32_t flag = few_in_lds && clpw[c] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
       const uint32_t nw = (counts[c] + clpw[c] - 1) / clpw[c];
@@ -850,11 +858,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     }
   }
   if (int rc = ensure_pool(e, s)) return rc;
-  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, ((size_t)ncls * shards + 2 * (size_t)ncls) * 4, hipMemcpyHostToDevice, s));
-  HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, ((size_t)n_eval_waves + n_solo) * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, ((size_t)ncls * shards + 3 * (size_t)ncls) * 4, hipMemcpyHostToDevice, s));
+  if (n_host_tasks) HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, (size_t)n_host_tasks * 4, hipMemcpyHostToDevice, s));
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
-  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride);
+  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
+                     d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted);
   HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_eval_waves;
