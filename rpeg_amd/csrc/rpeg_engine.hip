@@ -100,7 +100,7 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
     const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig, double* makespan, double* peak,
     double* score, uint8_t* mask, double* mass, const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval,
     uint32_t hmask, uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
-    uint32_t n_classes, uint32_t shards) {
+    uint32_t n_classes, uint32_t shards, const uint32_t* __restrict__ need) {
   // counters met in this block: key, plans of the block, and the block's first arrival index
   __shared__ uint32_t t_key[SIG_TABLE], t_cnt[SIG_TABLE], t_base[SIG_TABLE];
   // plan fields: the gate and the signature index the vertices with run-time values, which would put a
@@ -185,6 +185,8 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
     if (t_cnt[j]) t_base[j] = atomicAdd(&count[t_key[j]], t_cnt[j]);
   __syncthreads();
   if (key != NONE) kidx[i] = t_base[slot] + local;
+  // the running maxima of the ready-list length ride behind the counters, so that one copy brings both to the host
+  if (blockIdx.x == 0 && threadIdx.x < KE_NEED_SHARDS) count[(size_t)n_classes * shards + 1 + threadIdx.x] = need[threadIdx.x];
 }
 
 // cbase[class * shards + shard]: plans of the class in lower shards; shard as in k_signature.
@@ -338,7 +340,7 @@ struct rpeg_engine_s {
   // kernel, read back with the class counts of the next call); plans that outgrow it are flagged and redone
   // with the full capacity by a second launch.
   uint8_t* d_ovf = nullptr;
-  uint32_t *d_need = nullptr, *h_need = nullptr;
+  uint32_t* d_need = nullptr;
   uint32_t need = 0;
   uint32_t max_v = RPEG_MAX_V;   // largest vertex count of the problem's structures
   hipStream_t s2 = nullptr;                     // second stream: single-plan wavefronts of a large batch run beside the others
@@ -367,8 +369,6 @@ static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (!e->d_need) {
     HIP_TRY(e, hipMalloc(&e->d_need, (KE_NEED_SHARDS + 1) * 4));
     HIP_TRY(e, hipMemset(e->d_need, 0, (KE_NEED_SHARDS + 1) * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_need, KE_NEED_SHARDS * 4));
-    std::memset(e->h_need, 0, KE_NEED_SHARDS * 4);
   }
   HIP_TRY(e, hipMalloc(&e->d_sig, cap * 8));
   HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
@@ -582,7 +582,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->dP) hipFree(e->dP);
   if (e->d_pool) hipFree(e->d_pool);
   if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
-  if (e->d_need) { hipFree(e->d_need); hipHostFree(e->h_need); }
+  if (e->d_need) hipFree(e->d_need);
   if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
   if (e->d_ccount) {
     hipFree(e->d_ccount);
@@ -696,12 +696,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_count + blk - 1) / blk)), dim3(blk), 0, s, e->d_ccount, n_count, 0u);
     hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
                        e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
-                       e->d_kidx, e->d_ccount, ncls, shards);
+                       e->d_kidx, e->d_ccount, ncls, shards, e->d_need);
     HIP_TRY(e, hipGetLastError());
-    HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, n_count * 4, hipMemcpyDeviceToHost, s));
-    HIP_TRY(e, hipMemcpyAsync(e->h_need, e->d_need, KE_NEED_SHARDS * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, (n_count + KE_NEED_SHARDS) * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
-    for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_need[q]);
+    for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_ccount[n_count + q]);
     if (e->h_ccount[n_count - 1] == 0) break;
     if (round >= 2) { e->err = "class table did not converge"; return -5; }
     HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
@@ -833,6 +832,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // tasks of one plan get their class from the scatter kernel, not from the host: with one plan per wavefront
   // throughout that is every task of the launch, otherwise the tasks of the classes taken out of the main kernel
   const uint32_t n_host_tasks = one ? 0u : n_eval_waves;
+  // their class offsets ride behind the per-class tables when the block has room, else in a copy of their own
+  const size_t block_words = (size_t)ncls * shards + 3 * (size_t)ncls;
+  const bool tasks_in_block = block_words + n_host_tasks <= 4 * (size_t)e->ccap + COUNT_SLOTS;
+  uint32_t* const h_tasks = tasks_in_block ? e->h_ccount + block_words : e->h_cls;
   for (size_t c = 0; c < counts.size(); ++c) {
     h_cfirst[cids[c]] = first[c];
     h_clpw[cids[c]] = one ? (1u | (1u << 16)) : clpw[c];
@@ -854,12 +857,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     } else {
       const uint32_t flag = few_in_lds && clpw[c] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
       const uint32_t nw = (counts[c] + clpw[c] - 1) / clpw[c];
-      for (uint32_t t = 0; t < nw; ++t) e->h_cls[first[c] + t] = offs[c] | flag;
+      for (uint32_t t = 0; t < nw; ++t) h_tasks[first[c] + t] = offs[c] | flag;
     }
   }
   if (int rc = ensure_pool(e, s)) return rc;
-  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, ((size_t)ncls * shards + 3 * (size_t)ncls) * 4, hipMemcpyHostToDevice, s));
-  if (n_host_tasks) HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, (size_t)n_host_tasks * 4, hipMemcpyHostToDevice, s));
+  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, (block_words + (tasks_in_block ? n_host_tasks : 0u)) * 4, hipMemcpyHostToDevice, s));
+  if (n_host_tasks && !tasks_in_block) HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, (size_t)n_host_tasks * 4, hipMemcpyHostToDevice, s));
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
   hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
@@ -873,7 +876,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
   EvalLaunch L;
   L.P = e->dP; L.vert = plans->vert; L.head = plans->head; L.stride = plans->stride;
-  L.perm = e->d_perm; L.wave_cls = e->d_cls; L.pool = e->d_pool; L.ws = e->d_ws;
+  L.perm = e->d_perm; L.wave_cls = tasks_in_block && !one ? e->d_ccount + block_words : e->d_cls; L.pool = e->d_pool; L.ws = e->d_ws;
   L.n_waves = n_waves; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
   L.cls_bytes = (e->max_cls_bytes + 15u) & ~15u;
   // ready-list capacity (a multiple of the scan's batch of 8); classes with more than 4095 nodes or
