@@ -357,6 +357,7 @@ struct rpeg_engine_s {
   double last_ms = -1.0;
   uint64_t stats[7] = {0, 0, 0, 0, 0, 0, 0};
   int n_cu = 256;
+  std::vector<uint32_t> cls_sorted, cls_pos;   // all classes by node count (largest first); place of a class among those of the batch
 };
 
 static int ensure_batch(rpeg_engine_t* e, size_t n) {
@@ -641,6 +642,7 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
   e->cls_sig.clear();
   e->cls_off.clear();
   e->cls_nodes.clear();
+  e->cls_sorted.clear();
   e->tables_for = 0xFFFFFFFFu;
   e->pool.clear();
   e->d_pool_used = 0;
@@ -759,9 +761,19 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   const uint32_t lpw = one ? 1u : ls ? (uint32_t)ls : (uint32_t)WAVE;   // plans per wavefront
   // every class starts on a wavefront boundary; the lanes left over are idle
   // classes with the largest graphs first: their wavefronts run longest and should not start last
-  std::vector<uint32_t> order(counts.size());
-  for (size_t c = 0; c < counts.size(); ++c) order[c] = (uint32_t)c;
-  std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) { return e->cls_nodes[cids[a]] > e->cls_nodes[cids[b]]; });
+  // (the order of all known classes is kept from call to call and only filtered here: a batch of config 3 meets
+  // over ten thousand classes, and sorting them in every call took 0.4 ms)
+  if (e->cls_sorted.size() != ncls) {
+    e->cls_sorted.resize(ncls);
+    for (uint32_t c = 0; c < ncls; ++c) e->cls_sorted[c] = c;
+    std::stable_sort(e->cls_sorted.begin(), e->cls_sorted.end(), [&](uint32_t a, uint32_t b) { return e->cls_nodes[a] > e->cls_nodes[b]; });
+  }
+  e->cls_pos.assign(ncls, 0xFFFFFFFFu);
+  for (size_t c = 0; c < counts.size(); ++c) e->cls_pos[cids[c]] = (uint32_t)c;
+  std::vector<uint32_t> order;
+  order.reserve(counts.size());
+  for (uint32_t g : e->cls_sorted)
+    if (e->cls_pos[g] != 0xFFFFFFFFu) order.push_back(e->cls_pos[g]);
   // first[c]: first wavefront of class c in launch order (first permutation entry for a class of
   // single-plan wavefronts, which follow the others in the permutation and in the task list)
   std::vector<uint32_t> first(counts.size(), 0), clpw(counts.size(), lpw);
