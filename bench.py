@@ -140,8 +140,8 @@ def main():
     ap.add_argument("--sa-steps", type=int, default=2000)
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: every box of this build has one MI355X and the path needs no "
-                 "second one (plans are independent; see DESIGN.md for how it would shard). Use --gpus 1.")
+        sys.exit("bench.py measures one GPU: the path needs no second one (plans are independent: with more GPUs the "
+                 "candidate tensor or the annealing chains would be split evenly across them). Use --gpus 1.")
 
     if args.config == 5:
         return bench_sa(args)
