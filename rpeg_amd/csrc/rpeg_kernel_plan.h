@@ -244,9 +244,14 @@ __device__ inline bool kp_schedule(const ClassView& cv, const int n, const int l
       bool cand = ehi == ghi;
       unsigned long long m = __ballot(cand);
       if (m & (m - 1ull)) {
-        const uint32_t glo = kp_wave_umin(cand ? elo : 0xFFFFFFFFu);
-        cand = cand && elo == glo;
-        m = __ballot(cand);
+        // Lanes that agree in the high word nearly always hold the same time exactly (nodes released by one
+        // finish, or waiting for one device): then the low words need no reduction of their own.
+        const uint32_t lo0 = (uint32_t)__builtin_amdgcn_readlane((int)elo, __builtin_ctzll(m));
+        if (__ballot(cand && elo != lo0) != 0ull) {
+          const uint32_t glo = kp_wave_umin(cand ? elo : 0xFFFFFFFFu);
+          cand = cand && elo == glo;
+          m = __ballot(cand);
+        }
         if (m & (m - 1ull)) {
           const uint32_t go_ = kp_wave_umin(cand ? bo : 0xFFFFFFFFu);
           m = __ballot(cand && bo == go_);
