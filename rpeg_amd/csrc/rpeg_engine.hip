@@ -780,7 +780,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   std::vector<uint8_t> solo(counts.size(), 0);
   if (!ls && !one && !order.empty()) {
     // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
-    // classes with the largest graphs (up to a quarter of the batch) are taken out of it, unless the batch is
+    // classes with the largest graphs (up to 15 % of the batch: beyond that the single-plan kernel would be
+    // the one that ends last) are taken out of it, unless the batch is
     // many rounds of wavefronts deep anyway (then the sum of the work decides, not the slowest): their plans
     // get a wavefront each (k_plan, on a second stream, filling the registers and LDS the main kernel leaves
     // free; graphs of at least six tenths of the largest node count) or, where that kernel does not fit,
@@ -790,7 +791,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     const bool split = e->split_heavy && one_fits;
     // node count from which a class counts as large: the smallest one, not under `floor` percent of the
     // largest, such that the large classes hold at most `share` percent of the batch
-    const uint64_t floor_pct = split ? 60ull : 70ull, share_pct = 25ull;
+    const uint64_t floor_pct = split ? 60ull : 70ull, share_pct = split ? 15ull : 25ull;
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t waves64 = 0;
     for (uint32_t c : counts) waves64 += (c + WAVE - 1) / WAVE;

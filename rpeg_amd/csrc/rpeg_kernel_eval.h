@@ -137,7 +137,7 @@ __device__ inline double ke_dev_max(unsigned m, const double (&lf)[RPEG_MAX_V]) 
 template <int LS>
 __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* lds) {
   constexpr int RW = LS ? LS : KE_WAVE;   // lane stride of the per-lane LDS arrays
-  constexpr int SS = LS ? LS : 1;         // element stride of the per-plan state arrays
+  constexpr int SS = LS ? LS : KE_WAVE;   // element stride of the per-plan state arrays: interleaved by lane
   const int lane = threadIdx.x;
   int first_lane = 0;
   const rpeg_problem_t& P = *L.P;
@@ -177,14 +177,13 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     g_rank = g_time + (size_t)L.ws_nodes * LS;
     g_dur = g_rank + (size_t)L.ws_nodes * LS;
     g_deg = (uint8_t*)((double*)sbase + (2 * (size_t)L.ws_nodes + L.ws_slots) * LS) + lane;
-  } else {   // HBM, one contiguous block per lane: time[nodes] rank[nodes] dur[slots] deg[nodes]
+  } else {   // HBM, the same arrays interleaved by lane: the plans of a wavefront share their class and mostly
+             // work on the same node at the same time, so that their accesses fall into one row
     uint8_t* base = L.ws + (size_t)blockIdx.x * ke_ws_bytes(L.ws_nodes, L.ws_slots);
-    const size_t lane_bytes = ke_ws_bytes(L.ws_nodes, L.ws_slots) / KE_WAVE;
-    uint8_t* lbase = base + (size_t)lane * lane_bytes;
-    g_time = (double*)lbase;
-    g_rank = g_time + L.ws_nodes;
-    g_dur = g_rank + L.ws_nodes;
-    g_deg = (uint8_t*)(g_dur + L.ws_slots);
+    g_time = (double*)base + lane;
+    g_rank = g_time + (size_t)L.ws_nodes * KE_WAVE;
+    g_dur = g_rank + (size_t)L.ws_nodes * KE_WAVE;
+    g_deg = (uint8_t*)((double*)base + (2 * (size_t)L.ws_nodes + L.ws_slots) * KE_WAVE) + lane;
   }
 
   // ---- plan fields -> LDS
