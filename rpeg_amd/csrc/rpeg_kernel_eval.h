@@ -8,11 +8,13 @@
 //         model), the per-vertex memory terms and the ready list: key (est) and a meta word (node, tie-break
 //         class, reserved vertices) per entry.  The arg-min scan, the stale-key update and the removal never
 //         leave LDS.
-//   HBM   (LS = 0) per-plan arrays in a workspace, one contiguous block per lane: ready time and rank per
-//         node, duration per slot, remaining in-degree per node.  The lanes of a wavefront dispatch different
-//         nodes at any moment, so a row-per-node layout would not coalesce either, and a lane's block keeps
-//         its neighbouring nodes in one cache line.  A scheduling step issues all of its loads (duration of
-//         the dispatched node; ready time, in-degree and rank of up to four successors) before it waits.
+//   HBM   (LS = 0) per-plan arrays in a workspace, one block per wavefront, interleaved by lane
+//         (array[row][lane]): ready time and rank per node, duration per slot, remaining in-degree per node.
+//         The 64 plans of a wavefront belong to one class and mostly dispatch the same node at the same
+//         moment, so their accesses fall into one 512-byte row (a contiguous block per lane made every
+//         access touch 64 cache lines: 3.4 times the HBM traffic on GRPO graphs, 1.5 times the run time on
+//         DPO graphs).  A scheduling step issues all of its loads (duration of the dispatched node; ready
+//         time, in-degree and rank of up to four successors) before it waits.
 //         With LS > 0 the same arrays sit in LDS, interleaved by lane.
 #ifndef RPEG_KERNEL_EVAL_H
 #define RPEG_KERNEL_EVAL_H
