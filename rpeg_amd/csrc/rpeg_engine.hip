@@ -672,6 +672,8 @@ int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, u
 
 }  // extern "C"
 
+constexpr uint32_t TINY_CLASS = 16;   // classes of fewer plans go to the single-plan kernel
+
 static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                            double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
   if (!e || !plans) return -1;
@@ -814,6 +816,15 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
           if (split) solo[c] = 1;
           else clpw[c] = heavy_lpw;
         }
+    // A class with a handful of plans would occupy a wavefront of the main kernel with nearly all lanes idle
+    // (on the seeded set of config 3, 46 % of the wavefronts carried 4 % of the plans): its plans get a
+    // wavefront each as well.  Six wavefronts of the main kernel and sixteen of k_plan fit on a compute unit,
+    // and a plan takes k_plan about half as long as a wavefront takes the main kernel: below six plans k_plan
+    // is the cheaper place; the two kernels also run side by side (one waits on latencies, the other issues
+    // vector instructions), and on config 3 any threshold between 8 and 32 plans gives the same step time.
+    if (split)
+      for (size_t c = 0; c < counts.size(); ++c)
+        if (counts[c] < TINY_CLASS) solo[c] = 1;
   }
   uint32_t n_eval_waves = 0, n_solo = 0;
   for (size_t k = 0; k < order.size(); ++k) {
