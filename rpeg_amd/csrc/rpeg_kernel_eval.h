@@ -73,7 +73,10 @@ __host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls, uint3
   const size_t ready = (size_t)rcap * rw * 12;                 // key (8 bytes) and meta (4 bytes) per entry
   const size_t plan = (size_t)nv * RPEG_FIELDS * rw * 2, vmem = (size_t)nv * 4 * rw * 8;
   const size_t top = ready > plan ? (ready > vmem ? ready : vmem) : (plan > vmem ? plan : vmem);
-  return (top + 15) & ~size_t(15);
+  // (2 KB more for the full-width kernel: measured, not derived.  With 1-3 KB of slack behind the ready list the
+  // steps of configs 2, 3 and 4 are 2-3 % shorter on the same machine; from 4 KB on config 3 loses a wavefront
+  // per compute unit and from 6 KB on config 4 does.)
+  return ((top + 15) & ~size_t(15)) + (ls ? 0 : 2048);
 }
 __host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap, uint32_t ls, uint32_t nodes,
                                                uint32_t slots, uint32_t nv) {
@@ -228,15 +231,56 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
 
   KE_STAMP(3);
   // ---- ranks: reverse topological pass, then chain inheritance (scheduler.py:71-100, 367-378)
-  for (int i = n - 1; i >= 0; --i) {
-    const int v = cv.topo[i];
-    const NodeRec nr = cv.node[v];
-    double best = 0.0;
-    for (int j = 0; j < nr.n_succ; ++j) {
-      const double r = g_rank[(cv.succ[nr.succ_begin + j]) * SS];
-      best = r > best ? r : best;
+  if (LS == 0) {
+    // Every rank is read back by the predecessors a few nodes further on, and a round trip through the
+    // workspace per node made this pass a tenth of a long wavefront's time.  The LDS area (free between the
+    // memory model and the ready list) holds the ranks of the last `win` nodes of the order, interleaved by
+    // lane, and the place of every node in the order; a successor further back is read from the workspace.
+    // All lanes carry plans of one class, so the control flow is uniform.
+    const int dyn_bytes = (int)ke_dyn_bytes(L.rcap, 0, L.max_v);
+    int win = (dyn_bytes - ((2 * n + 15) & ~15)) / (KE_WAVE * 8);
+    while (win & (win - 1)) win &= win - 1;   // a power of two: the place in the ring is a mask away
+    uint16_t* l_pos = (uint16_t*)(dyn + (size_t)win * KE_WAVE * 8);
+    double* ring = (double*)dyn + lane;
+    __syncthreads();   // the memory terms in this area are dead
+    if (lane == first_lane)
+      for (int i = 0; i < n; ++i) l_pos[cv.topo[i]] = (uint16_t)i;
+    __syncthreads();
+    // node records and successor lists come from their LDS copies, the order itself one node ahead: the
+    // chain from one rank to the next is LDS reads only
+    auto node_at = [&](int v) { NodeRec r; const uint64_t b = l_node[v]; __builtin_memcpy(&r, &b, 8); return r; };
+    int v_next = n > 0 ? cv.topo[n - 1] : 0;
+    double d_next = n > 0 ? g_dur[(node_at(v_next).slot) * SS] : 0.0;
+    for (int i = n - 1; i >= 0; --i) {
+      const int v = v_next;
+      const NodeRec nr = node_at(v);
+      const double d = d_next;
+      if (i > 0) {   // one node ahead: off the chain
+        v_next = cv.topo[i - 1];
+        d_next = g_dur[(node_at(v_next).slot) * SS];
+      }
+      double best = 0.0;
+      for (int j = 0; j < nr.n_succ; ++j) {
+        const int sx = l_succ[nr.succ_begin + j], px = l_pos[sx];
+        const double r = (win > 0 && px - i <= win) ? ring[(px & (win - 1)) * KE_WAVE] : g_rank[(sx) * SS];
+        best = r > best ? r : best;
+      }
+      const double rk = d + best;
+      g_rank[(v) * SS] = rk;
+      if (win > 0) ring[(i & (win - 1)) * KE_WAVE] = rk;
     }
-    g_rank[(v) * SS] = g_dur[(nr.slot) * SS] + best;
+    __syncthreads();
+  } else {
+    for (int i = n - 1; i >= 0; --i) {
+      const int v = cv.topo[i];
+      const NodeRec nr = cv.node[v];
+      double best = 0.0;
+      for (int j = 0; j < nr.n_succ; ++j) {
+        const double r = g_rank[(cv.succ[nr.succ_begin + j]) * SS];
+        best = r > best ? r : best;
+      }
+      g_rank[(v) * SS] = g_dur[(nr.slot) * SS] + best;
+    }
   }
   for (unsigned g = 0; g < cv.h->n_groups; ++g) {
     const GroupRec gr = cv.group[g];
