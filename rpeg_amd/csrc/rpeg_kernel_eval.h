@@ -356,7 +356,10 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         m[u] = r_nt[(j0 + u) * RW];
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u) r[u] = g_rank[((int)(m[u] & 0xFFFu)) * SS];
+      for (int u = 0; u < 8; ++u) {   // slots past the end of the list hold anything: keep the read inside the plan's rows
+        const uint32_t node = m[u] & 0xFFFu;
+        r[u] = g_rank[(int)(node < L.ws_nodes ? node : 0u) * SS];
+      }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         if (j0 + u >= n_ready) continue;
