@@ -49,9 +49,44 @@ def _edge(e) -> dict:
     return {"src": e.src.id, "dst": e.dst.id, "container": _container(e.container)}
 
 
+_graph_text = {}   # id(rpeg) -> (rpeg, the four fragments of the key text that depend on the template only)
+
+
+def _graph_fragments(rpeg):
+    hit = _graph_text.get(id(rpeg))
+    if hit is not None and hit[0] is rpeg:
+        return hit[1]
+    ends = lambda x: (x["src"], x["dst"])  # noqa: E731
+    dumps = lambda x: json.dumps(x, separators=(",", ":"), sort_keys=True)  # noqa: E731
+    frag = (dumps(sorted((_edge(e) for e in rpeg.data_edges), key=ends)),
+            dumps(sorted((_edge(e) for e in rpeg.pub_edges), key=ends)),
+            dumps({m.value: t for m, t in rpeg.tau.items()}),
+            dumps(sorted((_vertex(v) for v in rpeg.vertices), key=lambda x: x["id"])))
+    if len(_graph_text) >= 64:
+        _graph_text.clear()
+    _graph_text[id(rpeg)] = (rpeg, frag)
+    return frag
+
+
 def config_hash(rpeg, plan) -> str:
     """sha256 of the canonical JSON of (template graph, plan); same payload and key order as the
-    reference, so keys are interchangeable with caches it wrote."""
+    reference (RPEG/search/cache.py:160-185: keys sorted at every level, no blanks), so keys are
+    interchangeable with caches it wrote.  The text is put together from its seven top-level entries in key
+    order; the four that depend on the template alone are kept per template object, since a search hashes
+    thousands of plans of a few templates."""
+    data_edges, pub_edges, tau, vertices = _graph_fragments(rpeg)
+    dumps = lambda x: json.dumps(x, separators=(",", ":"), sort_keys=True)  # noqa: E731
+    sigma = dumps({v.id: {"origin": list(a.origin), "extent": list(a.extent)} for v, a in plan.sigma.items()})
+    pi = dumps({v.id: list(p) for v, p in plan.pi.items()})
+    mb = dumps({v.id: m for v, m in plan.mb.items()})
+    text = ('{"data_edges":' + data_edges + ',"mb":' + mb + ',"pi":' + pi + ',"pub_edges":' + pub_edges +
+            ',"sigma":' + sigma + ',"tau":' + tau + ',"vertices":' + vertices + "}")
+    return hashlib.sha256(text.encode("utf-8")).hexdigest()
+
+
+def _config_hash_plain(rpeg, plan) -> str:
+    """The same key from one json.dumps of the whole payload, as the reference writes it; kept to check the
+    assembled text against."""
     by_id = lambda kv: kv[0].id  # noqa: E731
     ends = lambda x: (x["src"], x["dst"])  # noqa: E731
     payload = {

@@ -186,3 +186,20 @@ def test_structural_settings_in_reference_order():
     assert _ac_penalty(3.0, 0.0) == 3.0 and _ac_penalty(3.0, 0.15) == 3.0 * (1.0 - 0.15)
     assert penalized_score(2.0, None, OptimizerConfig(lambda_ac=0.5), False) == 2.0
     assert penalized_score(2.0, None, OptimizerConfig(lambda_ac=0.5), True) == 1.0
+
+
+def test_cache_key_text_assembled_from_fragments_equals_one_dump():
+    """config_hash puts the key text together from per-template fragments; it must be the text one
+    json.dumps of the whole payload gives (RPEG/search/cache.py:160-185), for every template and staleness of
+    the five configurations, also when two templates alternate."""
+    from rpeg_amd.search.cache import _config_hash_plain, config_hash
+    from tests.helpers import seeded_batch
+    seen = []
+    for c in (1, 2, 3, 4, 5):
+        cfg, batch = seeded_batch(c, 24)
+        for i in range(24):
+            rpeg, plan, _ = batch.configuration(cfg.problem, i)
+            seen.append((rpeg, plan))
+            assert config_hash(rpeg, plan) == _config_hash_plain(rpeg, plan), (c, i)
+    for rpeg, plan in seen[::7]:
+        assert config_hash(rpeg, plan) == _config_hash_plain(rpeg, plan)
