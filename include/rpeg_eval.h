@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define RPEG_ABI_VERSION 2
+#define RPEG_ABI_VERSION 3
 
 #define RPEG_MAX_V 6       /* template vertices per structure                */
 #define RPEG_MAX_E 9       /* within-step data edges                          */
@@ -125,7 +125,8 @@ typedef struct rpeg_problem_s {
   int32_t B, K, S, T;
   int32_t optimizer_stage, ckpt, max_groups;
   int32_t n_phase[RPEG_MAX_SPLIT];
-  int32_t pad;
+  int32_t transfer_both;  /* TransferResourcePolicy (core/types.py:128-200): bit 0 set when weight transfers
+                             reserve both endpoints, bit 1 when activation transfers do; 0 = the default  */
   rpeg_phase_t phase[RPEG_MAX_SPLIT][RPEG_MAX_PH];
   double hw[RPEG_HW_COUNT];
   double cap;             /* (1 - eps_rt) * memory_per_gpu (memory.py:291-298)          */

@@ -1249,18 +1249,19 @@ class DefaultPolicy:
 
 
 def evaluate_plan(rpeg, plan, space, suite, workload, hw, K_eval, policy=None, check_stale=True,
-                  want_trace=False):
+                  want_trace=False, transfer_policy=("destination_only", "destination_only")):
     """One evaluation as `evaluate_cached` computes it on a miss
     (RPEG/search/evaluate.py:235-290, 364-403).  With check_stale=False it is
     `_eval_worker` (:406-442), which omits the stale-layout gate.
 
     Returns a dict: makespan, raw (K_eval*B*K*(S+T)/makespan), peak (worst
     violating device peak, or the max device peak when feasible), cap,
-    feasible, stale_ok, score."""
+    feasible, stale_ok, score.  transfer_policy = (weight, activation) is what the scheduler is given
+    as `transfer_resource_policy` (evaluate.py:280-287)."""
     policy = policy or DefaultPolicy()
     nodes, edges = lower(rpeg, plan, suite, K_eval, workload)
     cost = CostModel(hw, suite, workload, policy.optimizer_stage, policy.activation_checkpointing)
-    start, finish, order = schedule(nodes, edges, cost, space)
+    start, finish, order = schedule(nodes, edges, cost, space, transfer_policy)
     makespan = max(finish.values())
     raw = K_eval * (workload.B * workload.K * (workload.S + workload.T)) / makespan
     mm = make_mem_model(rpeg, suite, workload, hw, policy)

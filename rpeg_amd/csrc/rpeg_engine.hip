@@ -549,7 +549,8 @@ int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
   *out = nullptr;
   if (problem->abi_version != RPEG_ABI_VERSION) return -3;
   if (problem->n_struct < 1 || problem->n_struct > RPEG_MAX_STRUCT || problem->n_split < 1 ||
-      problem->n_split > RPEG_MAX_SPLIT || problem->K_eval < 1)
+      problem->n_split > RPEG_MAX_SPLIT || problem->K_eval < 1 || problem->transfer_both < 0 ||
+      problem->transfer_both > 3)
     return -3;
   for (int s = 0; s < problem->n_struct; ++s) {
     const rpeg_struct_t& st = problem->st[s];

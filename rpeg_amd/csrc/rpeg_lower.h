@@ -298,10 +298,13 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
       r.blocked = (uint8_t)(1u << nd.vertex);
     } else {
       r.ptkey = (uint8_t)nv;  // comm_prio 0, topo_idx = number of template ids (scheduler.py:391-397)
-      // transfer_resources.py:73-148 with the default policy: weights reserve the destination only,
-      // activations also the source unless both adjacent operators use the same dp (a per-plan bit)
-      r.blocked = (uint8_t)(1u << nd.a1);
-      r.cond = nd.weight ? 0 : (uint8_t)(1 + nd.a0 * 8 + nd.a1);
+      // transfer_resources.py:73-148.  "destination_only": weights reserve the destination, activations
+      // also the source unless both adjacent operators use the same dp (a per-plan bit).
+      // "both_endpoints" for the payload class: source and destination, whatever dp is.  A reshard's
+      // two allocations are one and the same.
+      const bool both = nd.kind == 1 && (P.transfer_both >> (nd.weight ? 0 : 1) & 1);
+      r.blocked = (uint8_t)(1u << nd.a1 | (both ? 1u << nd.a0 : 0u));
+      r.cond = nd.weight || both ? 0 : (uint8_t)(1 + nd.a0 * 8 + nd.a1);
     }
     recs[i] = r;
     if (indeg[i] == 0) init.push_back((uint16_t)i);

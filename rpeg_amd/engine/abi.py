@@ -2,7 +2,7 @@
 
 import ctypes as C
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 MAX_V, MAX_E, MAX_PUB, MAX_PAIR, MAX_REL, MAX_PH, MAX_SPLIT, MAX_MODEL, MAX_STRUCT = 6, 9, 2, 4, 13, 6, 7, 5, 3
 FIELDS = 10
 ROLE = {"GEN": 0, "INF": 1, "TRAIN": 2}
@@ -71,7 +71,7 @@ class ProblemT(C.Structure):
                 ("R", C.c_int32), ("N", C.c_int32), ("G", C.c_int32),
                 ("B", C.c_int32), ("K", C.c_int32), ("S", C.c_int32), ("T", C.c_int32),
                 ("optimizer_stage", C.c_int32), ("ckpt", C.c_int32), ("max_groups", C.c_int32),
-                ("n_phase", C.c_int32 * MAX_SPLIT), ("pad", C.c_int32),
+                ("n_phase", C.c_int32 * MAX_SPLIT), ("transfer_both", C.c_int32),
                 ("phase", (PhaseT * MAX_PH) * MAX_SPLIT),
                 ("hw", C.c_double * len(HW_FIELDS)),
                 ("cap", C.c_double), ("group_overhead", C.c_double), ("score_num", C.c_double),

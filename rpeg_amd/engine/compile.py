@@ -142,6 +142,8 @@ def compile_problem(problem: EvalProblem) -> abi.ProblemT:
     P.B, P.K, P.S, P.T = wl.B, wl.K, wl.S, wl.T
     P.optimizer_stage, P.ckpt = pol.optimizer_stage, int(pol.activation_checkpointing)
     P.max_groups = pol.max_worker_groups_per_gpu
+    tp = problem.transfer_resource_policy
+    P.transfer_both = int(tp.weight == "both_endpoints") | int(tp.activation == "both_endpoints") << 1
     for i, name in enumerate(abi.HW_FIELDS):
         P.hw[i] = float(getattr(hw, name))
     for name in ("op_generation_scale", "op_inference_scale", "op_training_scale", "weight_comm_scale",

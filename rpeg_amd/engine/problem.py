@@ -20,7 +20,8 @@ from typing import Callable, FrozenSet, Optional, Sequence, Tuple
 
 import numpy as np
 
-from ..core.types import Allocation, DeviceSpace, Model
+from ..core.types import (Allocation, DeviceSpace, Model, RPEG_TRANSFER_RESOURCE_POLICY,
+                          TransferResourcePolicy)
 from ..ir.plan import ExecutionPlan
 from ..ir.rpeg import RPEG
 from ..ir.ppo import build_PPO_RPEG
@@ -72,6 +73,7 @@ class EvalProblem:
     device_space: DeviceSpace
     K_eval: int
     memory_policy: MemoryPolicy = field(default_factory=MemoryPolicy)
+    transfer_resource_policy: TransferResourcePolicy = RPEG_TRANSFER_RESOURCE_POLICY
 
     def n_splits(self) -> int:
         """Number of generation-split variants: 0 (unsplit) .. Q."""

@@ -91,17 +91,21 @@ _TEMPLATE_IDS = {"ppo": ("g_pi", "i_ref", "i_R", "i_V", "t_pi", "t_V"), "grpo": 
 
 
 def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware, space: DeviceSpace, K_eval: int,
-                policy: MemoryPolicy, more_structures=(), memory_trainable=None):
+                policy: MemoryPolicy, more_structures=(), memory_trainable=None, transfer_policy=None):
     """(engine, structure of `rpeg`): one engine per problem, kept for the life of the process.  The
     structure of `rpeg` is structure 0 of the engine (with `memory_trainable` as the memory model's set of
-    trainable models when that is given and differs from the template's), `more_structures` follow."""
+    trainable models when that is given and differs from the template's), `more_structures` follow.
+    `transfer_policy` (a TransferResourcePolicy, None = the default) is part of the problem: it decides
+    which allocations the lowered transfers reserve."""
     from dataclasses import replace
     from ..engine.runtime import Engine
     st = _structure_of(rpeg)
     if memory_trainable is not None and frozenset(memory_trainable) != frozenset(st.tau_models):
         st = replace(st, memory_trainable=frozenset(memory_trainable))
     structures = (st,) + tuple(more_structures)
-    rest = (tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy)
+    transfer_policy = transfer_policy or RPEG_TRANSFER_RESOURCE_POLICY
+    rest = (tuple(sorted((m.value, s) for m, s in suite.specs.items())), workload, hw, space, K_eval, policy,
+            transfer_policy)
     key = (tuple((s.name, s.memory_trainable) for s in structures),) + rest
     alias = ((st.name, st.memory_trainable), "first") + rest
     hit = key if key in _engines else alias if not more_structures and alias in _engines else None
@@ -111,7 +115,7 @@ def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware,
         _engines[hit] = eng          # most recently used last
         return eng, st
     problem = EvalProblem(structures=structures, suite=suite, workload=workload, hw=hw, device_space=space,
-                          K_eval=K_eval, memory_policy=policy)
+                          K_eval=K_eval, memory_policy=policy, transfer_resource_policy=transfer_policy)
     eng = _engines[key] = Engine(problem)
     _engines.setdefault(alias, eng)
     while len(_engines) > _MAX_ENGINES:      # a long-lived process that sees many problems keeps the recent ones;
@@ -122,9 +126,6 @@ def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware,
 def _check_supported(config: Configuration):
     if config.intra_stage_fusion:
         raise NotImplementedError("intra_stage_fusion=True is not evaluated by this engine")
-    pol = config.transfer_resource_policy or RPEG_TRANSFER_RESOURCE_POLICY
-    if pol != RPEG_TRANSFER_RESOURCE_POLICY:
-        raise NotImplementedError("only the default transfer resource policy is evaluated by this engine")
 
 
 def _pack(configs: Sequence[Configuration], st, workload: Workload) -> PlanBatch:
@@ -158,7 +159,11 @@ def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload
         return BatchResult(z, z, z, np.zeros(0, np.uint8), np.zeros(0, bool))
     for c in configs:
         _check_supported(c)
-    eng, st = _engine_for(configs[0].rpeg, suite, workload, hw, configs[0].device_space, K_eval, memory_policy)
+    pol = configs[0].transfer_resource_policy or RPEG_TRANSFER_RESOURCE_POLICY
+    if any((c.transfer_resource_policy or RPEG_TRANSFER_RESOURCE_POLICY) != pol for c in configs):
+        raise ValueError("the configurations of one batch must share their transfer resource policy")
+    eng, st = _engine_for(configs[0].rpeg, suite, workload, hw, configs[0].device_space, K_eval, memory_policy,
+                          transfer_policy=pol)
     out = eng.eval(_pack(configs, st, workload), gate_stale=gate_stale)
     mask = out["mask"]
     if np.any((mask & abi.MASK_VALID) == 0):
@@ -312,7 +317,8 @@ def evaluate(config: Configuration, suite: ModelSuite, workload: Workload, hw: H
     """unroll -> lower -> cost -> schedule -> score of one configuration (evaluate.py:235-290);
     returns (score, trace, lowered)."""
     _check_supported(config)
-    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy)
+    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy,
+                          transfer_policy=config.transfer_resource_policy)
     batch = _pack([config], st, workload)
     trace, lowered = _trace_of(eng, st, config, batch)
     score = trace.throughput(W_step=workload.B * workload.K * (workload.S + workload.T), K=K_eval)
@@ -353,7 +359,8 @@ def evaluation_cache_key(config: Configuration, memory_policy: MemoryPolicy = Me
 
 def _score_one(config, suite, workload, hw, K_eval, memory_policy, gate_stale):
     _check_supported(config)
-    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy)
+    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy,
+                          transfer_policy=config.transfer_resource_policy)
     batch = _pack([config], st, workload)
     res = evaluate_batch([config], suite, workload, hw, K_eval, memory_policy, gate_stale=gate_stale)
     trace, _ = _trace_of(eng, st, config, batch)

@@ -259,7 +259,8 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
         raise NotImplementedError("deadlines are not part of this engine")
     policy = opt_config.memory_policy()
     more = family_structures(base_config.rpeg, opt_config)
-    eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy, more)
+    eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy, more,
+                          transfer_policy=base_config.transfer_resource_policy)
 
     def directory(structure: int):
         rpeg = eng.problem.template(structure, ())
@@ -325,7 +326,8 @@ class _Utilization:
 def _trace_utilization(config: Configuration, suite, workload, hw, K_eval, policy) -> float:
     """Trace.utilization() of one configuration, folded by the library (rpeg_eval_trace_metrics)."""
     from .evaluate import _pack
-    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, policy)
+    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, policy,
+                          transfer_policy=config.transfer_resource_policy)
     return eng.trace_metrics(_pack([config], st, workload), 0)[0]
 
 

@@ -94,3 +94,15 @@ def check_family_case(p, case, families, res):
     taus = list(case["base_tau"]) if k >= prm.n_variants else [int(prm.tau[k][i]) for i in range(len(st.tau_models))]
     assert taus == case["final_tau"]
     assert rows6(res["best_plan"], len(rpeg.vertices)) == case["final"]
+
+
+# ---- non-default transfer resource policies: golden/ref_transfer_policy.json
+def load_transfer_policy_golden():
+    with open(os.path.join(GOLDEN, "ref_transfer_policy.json")) as f:
+        return json.load(f)
+
+
+def with_transfer_policy(problem, weight, activation):
+    from dataclasses import replace
+    from rpeg_amd.core.types import TransferResourcePolicy
+    return replace(problem, transfer_resource_policy=TransferResourcePolicy(weight=weight, activation=activation))

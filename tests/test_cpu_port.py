@@ -73,3 +73,17 @@ def test_invalid_plans_are_masked():
     out = CpuPort(cfg.problem).eval(batch)
     assert list(out["mask"][1:5] & abi.MASK_VALID) == [0, 0, 0, 0]
     assert out["mask"][0] & abi.MASK_VALID and np.all(np.isnan(out["score"][1:5]))
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_port_transfer_resource_policies_match_reference(c):
+    """The lowering's reserved allocations under the three non-default transfer resource policies: makespans
+    of the host build against the reference scheduler's (tests/golden/ref_transfer_policy.json)."""
+    from tests.helpers import load_transfer_policy_golden, with_transfer_policy
+    gold = load_transfer_policy_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, pol in enumerate(gold["policies"]):
+        out = CpuPort(with_transfer_policy(cfg.problem, *pol)).eval(batch)
+        for i in range(g["n_plans"]):
+            assert float(out["makespan"][i]).hex() == g["rows"][i][k]["makespan"], (i, pol)

@@ -443,3 +443,37 @@ def test_is_valid_drop_in_equals_restatement(c):
             n_view += restated(rpeg, plan, wl, views[0]) != restated(rpeg, plan, wl, views[1])
     assert n_true > 0 and n_false > 0
     print("valid", n_true, "invalid", n_false, "plans on which the two memory views disagree", n_view)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_transfer_resource_policies_equal_reference(c):
+    """Both-endpoints reservations for weights, for activations and for both: makespans of batched launches
+    and, through the drop-in evaluate(), dispatch order, finish times and utilisation against the reference
+    scheduler's (tests/golden/ref_transfer_policy.json)."""
+    from rpeg_amd.core.types import TransferResourcePolicy
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.search.evaluate import Configuration, evaluate
+    from tests.helpers import load_transfer_policy_golden, order_crc, with_transfer_policy
+    gold = load_transfer_policy_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    p = cfg.problem
+    for k, pol in enumerate(gold["policies"]):
+        eng = Engine(with_transfer_policy(p, *pol))
+        out = eng.eval(batch, gate_stale=False)
+        for i in range(g["n_plans"]):
+            assert float(out["makespan"][i]).hex() == g["rows"][i][k]["makespan"], (i, pol)
+            assert not out["mask"][i] & abi.MASK_ERROR
+        for i in range(0, g["n_plans"], 8):
+            util, _ = eng.trace_metrics(batch, i)
+            assert float(util).hex() == g["rows"][i][k]["utilization"], (i, pol)
+        tp = TransferResourcePolicy(weight=pol[0], activation=pol[1])
+        for i in range(0, g["n_plans"], 24):
+            rpeg, plan, wl = batch.configuration(p, i)
+            conf = Configuration(rpeg, plan, p.device_space, transfer_resource_policy=tp)
+            _, trace, _ = evaluate(conf, p.suite, wl, p.hw, p.K_eval, p.memory_policy)
+            want = g["rows"][i][k]
+            assert trace.makespan().hex() == want["makespan"], (i, pol)
+            assert order_crc([n.id for n in trace.start]) == want["order_crc"], (i, pol)
+            assert math.fsum(trace.finish.values()).hex() == want["finish_sum"], (i, pol)
+            assert float(trace.utilization()).hex() == want["utilization"], (i, pol)

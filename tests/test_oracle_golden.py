@@ -55,3 +55,23 @@ def test_node_times_and_peaks_match_reference(c):
             if n.kind == oracle.OP:
                 assert float(mm.peak_bytes(n)).hex() == rec["peak_bytes"], (i, rec["id"])
                 assert [x.hex() for x in cost.breakdown(n)] == rec["breakdown"], (i, rec["id"])
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_transfer_resource_policies_match_reference(c):
+    """Schedules under the three non-default transfer resource policies against the reference scheduler's
+    (tests/golden/make_golden_transfer_policy.py): makespan, dispatch order, finish times, utilisation."""
+    from tests.helpers import load_transfer_policy_golden
+    gold = load_transfer_policy_golden()
+    g = gold["configs"][str(c)]
+    assert g["n_differ_from_default"] > 0
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for i in range(0, g["n_plans"], 1 if c in (1, 4) else 3):
+        for pol, want in zip(gold["policies"], g["rows"][i]):
+            got = oracle_eval(cfg.problem, batch, i, want_trace=True, transfer_policy=tuple(pol))
+            assert got["makespan"].hex() == want["makespan"], (i, pol)
+            assert order_crc(got["order"]) == want["order_crc"], (i, pol)
+            assert math.fsum(got["finish"].values()).hex() == want["finish_sum"], (i, pol)
+            reserved = oracle.reserved_by_node(got["nodes"], got["edges"], tuple(pol))
+            util = oracle.utilization(got["start"], got["finish"], got["order"], reserved)
+            assert float(util).hex() == want["utilization"], (i, pol)
