@@ -477,3 +477,32 @@ def test_transfer_resource_policies_equal_reference(c):
             assert order_crc([n.id for n in trace.start]) == want["order_crc"], (i, pol)
             assert math.fsum(trace.finish.values()).hex() == want["finish_sum"], (i, pol)
             assert float(trace.utilization()).hex() == want["utilization"], (i, pol)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_other_seeds_unroll_depths_and_policies_equal_the_host_build(c):
+    """Away from the shipped problems: unroll depths 1, 2 and 7, both-endpoints reservations and two other
+    seeds of the candidate generator.  Every makespan, peak, score and mask of the batched launch equals the
+    host build of the same arithmetic, whose scheduler is written differently (a push-ordered list, one pop per
+    iteration) and is itself checked against the reference vectors."""
+    from dataclasses import replace
+    from rpeg_amd.core.types import TransferResourcePolicy
+    from rpeg_amd.engine.runtime import Engine
+    cfg = configs.config(c)
+    n = 8192 if c != 5 else 2048
+    for K, pol in ((1, ("destination_only", "destination_only")), (2, ("both_endpoints", "destination_only")),
+                   (7, ("both_endpoints", "both_endpoints"))):
+        p = replace(cfg.problem, K_eval=K, transfer_resource_policy=TransferResourcePolicy(*pol))
+        eng, port = Engine(p), CpuPort(p)
+        for seed in (7, 1234):
+            batch = candidates_of(p, cfg, n, seed, c)
+            got = eng.eval(batch, gate_stale=True)
+            want = port.eval(batch, flags=abi.GATE_STALE, threads=16)
+            for k in ("makespan", "peak", "score"):
+                assert same_bits(got[k], want[k]), (K, pol, seed, k)
+            assert np.array_equal(got["mask"], want["mask"]), (K, pol, seed)
+
+
+def candidates_of(problem, cfg, n, seed, tag):
+    from rpeg_amd.search import candidates
+    return candidates.generate(problem, n, cfg.tau_choices, seed=seed, tag=tag)
