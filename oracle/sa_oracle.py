@@ -428,11 +428,12 @@ class Evaluated:
         self.mem_ok, self.stale_ok, self.mass = mem_ok, stale_ok, mass
 
 
-def oracle_evaluator(rpeg, space, suite, workload, hw, K_eval, policy=None):
+def oracle_evaluator(rpeg, space, suite, workload, hw, K_eval, policy=None,
+                     transfer_policy=("destination_only", "destination_only")):
     """plan -> Evaluated, through the Python restatement of the evaluation path."""
     def run(plan):
         r = O.evaluate_plan(rpeg, plan, space, suite, workload, hw, K_eval, policy, check_stale=False,
-                            want_trace=True)
+                            want_trace=True, transfer_policy=transfer_policy)
         chain = critical_chain(r["nodes"], r["edges"], r["finish"])
         mass = critical_mass(chain, rpeg, r["start"], r["finish"])
         gated = r["score"] if r["stale_ok"] else 0.0

@@ -52,7 +52,14 @@ CASES = [dict(plan=0, stream=(42, 77, 0, 0), E_max=260, E_struct=200, stag_windo
               families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05, memory_per_gpu=1.25e10),
          # utilisation objective (optimizer.py:461-486): throughput x Trace.utilization() above the floor
          dict(plan=0, stream=(42, 77, 5, 0), E_max=330, E_struct=120, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
-              families=True, T_cand=[[0, 1], [0], [0]], base_tau=[0, 0], lambda_ac=0.15, max_throughput_loss=0.10)]
+              families=True, T_cand=[[0, 1], [0], [0]], base_tau=[0, 0], lambda_ac=0.15, max_throughput_loss=0.10),
+         # both-endpoints transfer reservations (core/types.py:200-203), carried by every configuration that
+         # optimize() derives from the base (optimizer.py:596-663, 702-930)
+         dict(plan=0, stream=(42, 77, 7, 0), E_max=260, E_struct=200, stag_window=4, T_init=0.05, T_min=0.05, T_warm=0.10,
+              transfer=["both_endpoints", "both_endpoints"]),
+         dict(plan=2, stream=(42, 77, 8, 0), E_max=300, E_struct=60, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
+              families=True, T_cand=[[0, 1], [0], [1, 0]], base_tau=[1, 0], lambda_ac=0.0,
+              transfer=["destination_only", "both_endpoints"])]
 
 
 PIPELINE = dict(stream=(42, 77, 6, 0), E_max=300, E_struct=60, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
@@ -163,7 +170,9 @@ def main():
             st["log"].append(rows(config))
         unrolled = mods["passes.unroll"].unroll(rpeg, p.K_eval)
         lowered = mods["passes.lower"].lower(rpeg, unrolled, plan, st["suite"], p.K_eval, workload=wl)
-        trace = mods["schedule.scheduler"].schedule(lowered, st["cost"], st["space"])
+        trace = mods["schedule.scheduler"].schedule(   # evaluate.py:280-287
+            lowered, st["cost"], st["space"],
+            transfer_resource_policy=config.transfer_resource_policy or ct.RPEG_TRANSFER_RESOURCE_POLICY)
         raw = trace.throughput(W_step=wl.B * wl.K * (wl.S + wl.T), K=p.K_eval)
         if gate and not O.stale_publication_layout_valid(rpeg, plan):
             return 0.0, trace, False
@@ -174,7 +183,9 @@ def main():
         return raw * max(math.exp(-40.0 * max(0.0, req / cap - 1.0)), 1e-12), trace, False
 
     def evaluation_cache_key(config, memory_policy=None):
-        return rcache.config_hash(config.rpeg, config.plan) + ":mem:fusion=0:transfer=destination_only,destination_only:2:1:0:0:activation_cache=0:groups=0"
+        pol = config.transfer_resource_policy or ct.RPEG_TRANSFER_RESOURCE_POLICY
+        return (rcache.config_hash(config.rpeg, config.plan) + ":mem:fusion=0:transfer=" + ",".join(pol.to_dict().values())
+                + ":2:1:0:0:activation_cache=0:groups=0")
 
     def evaluate_cached(config, cache, suite, workload, hw, K_eval, memory_policy=None):
         h = evaluation_cache_key(config)
@@ -217,6 +228,9 @@ def main():
     real_cpu_count = os.cpu_count
     import dataclasses
     p_config = p
+    def policy_of(case):
+        return ct.TransferResourcePolicy(*case["transfer"]) if "transfer" in case else None
+
     for case in CASES:
         if p is not p_config or "memory_per_gpu" in case:
             p = dataclasses.replace(p_config, hw=dataclasses.replace(
@@ -227,7 +241,7 @@ def main():
         st["families"] = bool(case.get("families"))
         if st["families"]:
             base_rpeg = dataclasses.replace(rpeg0, tau={Model.ACTOR: case["base_tau"][0], Model.CRITIC: case["base_tau"][1]})
-            base = Configuration(base_rpeg, plan, space)
+            base = Configuration(base_rpeg, plan, space, transfer_resource_policy=policy_of(case))
             a, c, s_ = case["T_cand"]
             oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
                                       T_cand={Model.ACTOR: set(a), Model.CRITIC: set(c), Model.AC_SHARE: set(s_)},
@@ -236,7 +250,7 @@ def main():
                                       T_init=case["T_init"], T_warm=case["T_warm"], T_min=case["T_min"],
                                       stag_window=case["stag_window"])
         else:
-            base = Configuration(rpeg0, plan, space)
+            base = Configuration(rpeg0, plan, space, transfer_resource_policy=policy_of(case))
             assert is_valid(base, suite, wl, mm), "the base plan must be valid"
             oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
                                       T_cand={Model.ACTOR: {0}, Model.CRITIC: {0}, Model.AC_SHARE: set()},

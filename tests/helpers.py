@@ -44,6 +44,8 @@ def family_problem(case=None, c=1):
     p = configs.config(c).problem
     if case and "memory_per_gpu" in case:
         p = dataclasses.replace(p, hw=dataclasses.replace(p.hw, memory_per_gpu=case["memory_per_gpu"]))
+    if case and "transfer" in case:
+        p = with_transfer_policy(p, *case["transfer"])
     ppo, ac = STRUCTURES["ppo"], STRUCTURES["ac_share"]
     return dataclasses.replace(p, structures=(ppo, ac, as_seen_from(ac, ppo)))
 

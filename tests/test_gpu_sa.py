@@ -181,7 +181,13 @@ def test_optimize_equals_reference_trajectory():
 
     def rows(r):
         return [[int(x) for x in r[v * 10:(v + 1) * 10]] for v in range(nv)]
+    from rpeg_amd.core.types import TransferResourcePolicy
+    from rpeg_amd.engine.runtime import Engine
+    from tests.helpers import with_transfer_policy
     for case in [c for c in g["cases"] if not c.get("families")]:
+        # a case may ask for both-endpoints transfer reservations: another problem, hence another engine
+        tp = TransferResourcePolicy(*case["transfer"]) if "transfer" in case else None
+        eng = Engine(with_transfer_policy(p, *case["transfer"])) if tp else engine(1)
         _, plan_m, _ = batch.configuration(p, case["plan"])
         by_id = {v.id: v for v in rpeg0.vertices}
         plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
@@ -196,10 +202,10 @@ def test_optimize_equals_reference_trajectory():
         assert log[:8] == case["first"] and res["n_eval_log"] == case["n_eval"]
         assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
         assert res["n_draws"] == case["n_draws"] and rows(res["best_plan"]) == case["final"]
-        base = Configuration(rpeg0, plan, p.device_space)
+        base = Configuration(rpeg0, plan, p.device_space, transfer_resource_policy=tp)
         out = optimize(base, p.suite, p.workload, p.hw, p.K_eval, opt, EvalCache(), seed=case["stream"][0],
                        stream_key=case["stream"][1:])
-        assert rows(plan_row(out.rpeg, out.plan)) == case["final"]
+        assert rows(plan_row(out.rpeg, out.plan)) == case["final"] and out.transfer_resource_policy == tp
         s1, _, f1, _ = evaluate_cached(out, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
         s0, _, _, _ = evaluate_cached(base, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
         assert f1 and s1 >= s0
@@ -308,7 +314,7 @@ def test_optimize_over_structural_families_equals_reference():
     with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
         g = json.load(f)
     cases = [c for c in g["cases"] if c.get("families")]
-    assert len(cases) == 4 and cases[3]["max_throughput_loss"] > 0
+    assert len(cases) == 5 and cases[3]["max_throughput_loss"] > 0 and cases[4]["transfer"][1] == "both_endpoints"
     for case in cases:
         p = family_problem(case)
         eng = Engine(p)
@@ -324,7 +330,8 @@ def test_optimize_over_structural_families_equals_reference():
         check_family_case(p, case, families, res)
 
         base_rpeg = p.template(0, case["base_tau"])
-        base = Configuration(base_rpeg, row_plan(base_rpeg, row), p.device_space)
+        base = Configuration(base_rpeg, row_plan(base_rpeg, row), p.device_space,
+                             transfer_resource_policy=p.transfer_resource_policy if "transfer" in case else None)
         out = optimize(base, p.suite, p.workload, p.hw, p.K_eval, opt, EvalCache(), seed=case["stream"][0],
                        stream_key=case["stream"][1:])
         assert out.rpeg.vertices[0].id == case["final_first_vertex"]

@@ -22,7 +22,8 @@ from rpeg_amd.core.types import Allocation
 from rpeg_amd.engine import abi
 from rpeg_amd.ir.plan import ExecutionPlan
 from rpeg_amd.search.optimizer import OptimizerConfig, plan_row, sa_params
-from tests.helpers import GOLDEN, check_family_case, family_case_setup, family_problem, seeded_batch
+from tests.helpers import (GOLDEN, check_family_case, family_case_setup, family_problem, seeded_batch,
+                           with_transfer_policy)
 
 
 def _directory(p, rpeg0):
@@ -161,8 +162,8 @@ def test_cxx_optimize_matches_reference_optimize():
     rpeg0 = p.template(0, ())
     nv = len(rpeg0.vertices)
     _, _, arrays = _directory(p, rpeg0)
-    port = CpuPort(p)
     for case in [c for c in g["cases"] if not c.get("families")]:
+        port = CpuPort(with_transfer_policy(p, *case["transfer"]) if "transfer" in case else p)
         _, plan_m, _ = batch.configuration(p, case["plan"])
         row = plan_row(rpeg0, ExecutionPlan(sigma={v: plan_m.sigma[u] for v, u in zip(rpeg0.vertices, plan_m.sigma)},
                                             pi={v: plan_m.pi[u] for v, u in zip(rpeg0.vertices, plan_m.pi)},
@@ -228,7 +229,8 @@ def test_cxx_optimize_over_structural_families_matches_reference_optimize():
     with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
         g = json.load(f)
     cases = [c for c in g["cases"] if c.get("families") and not c.get("max_throughput_loss")]   # no traces on this evaluator
-    assert len(cases) == 3
+    assert len(cases) == 4 and cases[3]["transfer"] == ["destination_only", "both_endpoints"]
+    cases = cases[3:] + cases[:3]                 # the lines after the loop are about the tight-memory case
     for case in cases:
         p = family_problem(case)
         port = CpuPort(p)

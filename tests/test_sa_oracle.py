@@ -174,8 +174,11 @@ def test_chain_loop_matches_reference_optimize():
     cfg, batch, rpeg0, cost, mem = _world(1, 8)
     p = cfg.problem
     table, index = S.build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, cost, mem)
-    ev = S.oracle_evaluator(rpeg0, p.device_space, p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
-    for case in [c for c in g["cases"] if not c.get("families")]:
+    cases = [c for c in g["cases"] if not c.get("families")]
+    assert [c.get("transfer") for c in cases] == [None, None, ["both_endpoints", "both_endpoints"]]
+    for case in cases:
+        ev = S.oracle_evaluator(rpeg0, p.device_space, p.suite, p.workload, p.hw, p.K_eval, p.memory_policy,
+                                tuple(case.get("transfer", ("destination_only", "destination_only"))))
         _, plan_m, _ = batch.configuration(p, case["plan"])
         by_id = {v.id: v for v in rpeg0.vertices}
         plan = ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
