@@ -402,3 +402,45 @@ def test_search_from_config_file_writes_loadable_plans(tmp_path):
     # the run is a function of the seed
     again = search_from_config(cfg, hw_overlay=str(hw))
     assert list(plan_row(again.polished.rpeg, again.polished.plan)) == list(plan_row(res.polished.rpeg, res.polished.plan))
+
+
+def test_planner_sequence_of_the_runtime_under_a_transfer_policy():
+    """The calls of the reference's second caller in its order (runtime/job_plan.py:85-213): a base configuration
+    that carries a both-endpoints policy, is_valid, optimize(), then the result lowered and scheduled at another
+    horizon and serialised.  The optimised plan is no worse than the base under that policy, and the schedule at
+    the new horizon equals the oracle's under the same policy (times, dispatch order)."""
+    from rpeg_amd.core.types import CONSERVATIVE_TRANSFER_RESOURCE_POLICY as tp
+    from rpeg_amd.ir import serialize as ser
+    from rpeg_amd.model.memory import NodeMemoryModel
+    from rpeg_amd.search.baselines import build_valid_baseline_plan
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration, _engine_for, evaluate, evaluate_cached, is_valid
+    from rpeg_amd.search.optimizer import optimize
+    from oracle import rpeg_oracle as oracle
+    p = configs.config(1).problem
+    rpeg = p.template(0, ())
+    eng, _ = _engine_for(rpeg, p.suite, p.workload, p.hw, p.device_space, p.K_eval, p.memory_policy, transfer_policy=tp)
+    plan = build_valid_baseline_plan(rpeg, p.device_space, p.suite, p.workload, eng)
+    base = Configuration(rpeg, plan, p.device_space, transfer_resource_policy=tp)
+    mm = NodeMemoryModel.from_policy(p.hw, p.suite, p.workload, p.memory_policy, trainable=frozenset(rpeg.trainable))
+    assert is_valid(base, p.suite, p.workload, mm)
+    opt = OptimizerConfig(K_x=6, T_max=50, E_max=150, E_struct=150, T_cand={m: {0} for m in rpeg.tau},
+                          structural_candidates=frozenset({"separate"}))
+    cache = EvalCache()
+    best = optimize(base, p.suite, p.workload, p.hw, p.K_eval, opt, cache, seed=5)
+    assert best.transfer_resource_policy == tp
+    s0 = evaluate_cached(base, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)[0]
+    s1, _, feasible, _ = evaluate_cached(best, EvalCache(), p.suite, p.workload, p.hw, p.K_eval, p.memory_policy)
+    assert feasible and s1 >= s0
+    for config, score in ((base, s0), (best, s1)):   # the scores are the oracle's under that policy, not the default's
+        want = oracle.evaluate_plan(config.rpeg, config.plan, p.device_space, p.suite, p.workload, p.hw, p.K_eval,
+                                    p.memory_policy, transfer_policy=(tp.weight, tp.activation))
+        assert score == want["score"]
+    horizon = 3
+    _, trace, lowered = evaluate(best, p.suite, p.workload, p.hw, horizon, p.memory_policy)
+    want = oracle.evaluate_plan(best.rpeg, best.plan, p.device_space, p.suite, p.workload, p.hw, horizon,
+                                p.memory_policy, want_trace=True, transfer_policy=(tp.weight, tp.activation))
+    doc = ser.execution_schedule_to_dict(trace, horizon=horizon)
+    assert doc["horizon"] == horizon and doc["predicted_makespan_s"] == want["makespan"]
+    assert [n["node_id"] for n in doc["nodes"]] == list(want["order"])
+    assert [n["predicted_finish_s"] for n in doc["nodes"]] == [want["finish"][i] for i in want["order"]]
