@@ -108,3 +108,15 @@ def with_transfer_policy(problem, weight, activation):
     from dataclasses import replace
     from rpeg_amd.core.types import TransferResourcePolicy
     return replace(problem, transfer_resource_policy=TransferResourcePolicy(weight=weight, activation=activation))
+
+
+# ---- non-default memory policies: golden/ref_memory_policy.json
+def load_memory_policy_golden():
+    with open(os.path.join(GOLDEN, "ref_memory_policy.json")) as f:
+        return json.load(f)
+
+
+def with_memory_policy(problem, fields):
+    from dataclasses import replace
+    from rpeg_amd.model.memory import MemoryPolicy
+    return replace(problem, memory_policy=MemoryPolicy(**fields))

@@ -87,3 +87,21 @@ def test_port_transfer_resource_policies_match_reference(c):
         out = CpuPort(with_transfer_policy(cfg.problem, *pol)).eval(batch)
         for i in range(g["n_plans"]):
             assert float(out["makespan"][i]).hex() == g["rows"][i][k]["makespan"], (i, pol)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_port_memory_policies_match_reference(c):
+    """Non-default memory policies on the host build of the kernels' arithmetic against the reference's
+    evaluations (tests/golden/ref_memory_policy.json), every plan of the vectors."""
+    from tests.helpers import load_memory_policy_golden, with_memory_policy
+    gold = load_memory_policy_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, pol in enumerate(gold["policies"]):
+        out = CpuPort(with_memory_policy(cfg.problem, pol)).eval(batch)
+        for i in range(g["n_plans"]):
+            want = g["rows"][i][k]
+            assert float(out["makespan"][i]).hex() == want["makespan"], (i, pol)
+            assert float(out["peak"][i]).hex() == want["peak"], (i, pol)
+            assert float(out["score"][i]).hex() == want["score"], (i, pol)
+            assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, pol)

@@ -506,3 +506,34 @@ def test_other_seeds_unroll_depths_and_policies_equal_the_host_build(c):
 def candidates_of(problem, cfg, n, seed, tag):
     from rpeg_amd.search import candidates
     return candidates.generate(problem, n, cfg.tau_choices, seed=seed, tag=tag)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_memory_policies_equal_reference(c):
+    """Optimizer stages 0-2, checkpointing off, runtime overhead fraction, per-worker overhead and cache bytes and
+    the worker-group limit: batched launches, and evaluate_cached() with the policy as its argument, against the
+    reference's evaluations (tests/golden/ref_memory_policy.json)."""
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.model.memory import MemoryPolicy
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration, evaluate_cached
+    from tests.helpers import load_memory_policy_golden, with_memory_policy
+    gold = load_memory_policy_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, pol in enumerate(gold["policies"]):
+        p = with_memory_policy(cfg.problem, pol)
+        out = Engine(p).eval(batch, gate_stale=False)
+        for i in range(g["n_plans"]):
+            want = g["rows"][i][k]
+            assert float(out["makespan"][i]).hex() == want["makespan"], (i, pol)
+            assert float(out["peak"][i]).hex() == want["peak"], (i, pol)
+            assert float(out["score"][i]).hex() == want["score"], (i, pol)
+            assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, pol)
+        for i in range(0, g["n_plans"], 16):
+            rpeg, plan, wl = batch.configuration(p, i)
+            if not oracle.stale_publication_layout_valid(rpeg, plan):
+                continue                      # evaluate_cached gates those to 0 (evaluate.py:364-376)
+            s, _, feasible, _ = evaluate_cached(Configuration(rpeg, plan, p.device_space), EvalCache(), p.suite, wl,
+                                                p.hw, p.K_eval, MemoryPolicy(**pol))
+            assert float(s).hex() == g["rows"][i][k]["score"] and feasible == g["rows"][i][k]["feasible"], (i, pol)

@@ -75,3 +75,22 @@ def test_transfer_resource_policies_match_reference(c):
             reserved = oracle.reserved_by_node(got["nodes"], got["edges"], tuple(pol))
             util = oracle.utilization(got["start"], got["finish"], got["order"], reserved)
             assert float(util).hex() == want["utilization"], (i, pol)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_memory_policies_match_reference(c):
+    """Optimizer stages 0-2, checkpointing off, runtime overhead fraction, per-worker overhead and cache bytes
+    and the worker-group limit (inf peaks) against the reference's evaluations
+    (tests/golden/make_golden_memory_policy.py): makespan, worst peak, feasibility, penalised score."""
+    from tests.helpers import load_memory_policy_golden, with_memory_policy
+    gold = load_memory_policy_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, pol in enumerate(gold["policies"]):
+        p = with_memory_policy(cfg.problem, pol)
+        for i in range(0, g["n_plans"], 1 if c in (1, 4) else 3):
+            want = g["rows"][i][k]
+            got = oracle_eval(p, batch, i)
+            assert got["makespan"].hex() == want["makespan"], (i, pol)
+            assert float(got["peak"]).hex() == want["peak"], (i, pol)
+            assert got["feasible"] == want["feasible"] and got["score"].hex() == want["score"], (i, pol)
