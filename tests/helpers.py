@@ -120,3 +120,14 @@ def with_memory_policy(problem, fields):
     from dataclasses import replace
     from rpeg_amd.model.memory import MemoryPolicy
     return replace(problem, memory_policy=MemoryPolicy(**fields))
+
+
+# ---- calibrated hardware records: golden/ref_hardware.json
+def load_hardware_golden():
+    with open(os.path.join(GOLDEN, "ref_hardware.json")) as f:
+        return json.load(f)
+
+
+def with_hardware(problem, fields):
+    from dataclasses import replace
+    return replace(problem, hw=replace(problem.hw, **fields))

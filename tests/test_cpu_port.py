@@ -105,3 +105,21 @@ def test_port_memory_policies_match_reference(c):
             assert float(out["peak"][i]).hex() == want["peak"], (i, pol)
             assert float(out["score"][i]).hex() == want["score"], (i, pol)
             assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, pol)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_port_calibrated_hardware_matches_reference(c):
+    """Calibrated hardware records on the host build of the kernels' arithmetic against the reference's
+    evaluations (tests/golden/ref_hardware.json), every plan of the vectors."""
+    from tests.helpers import load_hardware_golden, with_hardware
+    gold = load_hardware_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, ov in enumerate(gold["overlays"]):
+        out = CpuPort(with_hardware(cfg.problem, ov)).eval(batch)
+        for i in range(g["n_plans"]):
+            want = g["rows"][i][k]
+            assert float(out["makespan"][i]).hex() == want["makespan"], (i, k)
+            assert float(out["peak"][i]).hex() == want["peak"], (i, k)
+            assert float(out["score"][i]).hex() == want["score"], (i, k)
+            assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, k)

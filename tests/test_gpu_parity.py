@@ -537,3 +537,23 @@ def test_memory_policies_equal_reference(c):
             s, _, feasible, _ = evaluate_cached(Configuration(rpeg, plan, p.device_space), EvalCache(), p.suite, wl,
                                                 p.hw, p.K_eval, MemoryPolicy(**pol))
             assert float(s).hex() == g["rows"][i][k]["score"] and feasible == g["rows"][i][k]["feasible"], (i, pol)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_calibrated_hardware_equals_reference(c):
+    """Per-role operator scales, weight-transfer and reshard scales, the fixed activation-transfer overhead,
+    gemm_k_half and other link / efficiency parameters: batched launches against the reference's evaluations
+    (tests/golden/ref_hardware.json)."""
+    from rpeg_amd.engine.runtime import Engine
+    from tests.helpers import load_hardware_golden, with_hardware
+    gold = load_hardware_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, ov in enumerate(gold["overlays"]):
+        out = Engine(with_hardware(cfg.problem, ov)).eval(batch, gate_stale=False)
+        for i in range(g["n_plans"]):
+            want = g["rows"][i][k]
+            assert float(out["makespan"][i]).hex() == want["makespan"], (i, k)
+            assert float(out["peak"][i]).hex() == want["peak"], (i, k)
+            assert float(out["score"][i]).hex() == want["score"], (i, k)
+            assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, k)

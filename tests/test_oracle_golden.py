@@ -94,3 +94,23 @@ def test_memory_policies_match_reference(c):
             assert got["makespan"].hex() == want["makespan"], (i, pol)
             assert float(got["peak"]).hex() == want["peak"], (i, pol)
             assert got["feasible"] == want["feasible"] and got["score"].hex() == want["score"], (i, pol)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
+def test_calibrated_hardware_matches_reference(c):
+    """Per-role operator scales, weight-transfer and reshard scales, the fixed activation-transfer overhead,
+    gemm_k_half and other link / efficiency parameters against the reference's evaluations
+    (tests/golden/make_golden_hardware.py): makespan, dispatch order, worst peak, feasibility, score."""
+    from tests.helpers import load_hardware_golden, with_hardware
+    gold = load_hardware_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    for k, ov in enumerate(gold["overlays"]):
+        p = with_hardware(cfg.problem, ov)
+        for i in range(0, g["n_plans"], 1 if c in (1, 4) else 3):
+            want = g["rows"][i][k]
+            got = oracle_eval(p, batch, i, want_trace=True)
+            assert got["makespan"].hex() == want["makespan"], (i, k)
+            assert order_crc(got["order"]) == want["order_crc"], (i, k)
+            assert float(got["peak"]).hex() == want["peak"], (i, k)
+            assert got["feasible"] == want["feasible"] and got["score"].hex() == want["score"], (i, k)
