@@ -131,3 +131,19 @@ def load_hardware_golden():
 def with_hardware(problem, fields):
     from dataclasses import replace
     return replace(problem, hw=replace(problem.hw, **fields))
+
+
+# ---- problems away from the shipped configurations: golden/ref_variants.json
+def variant_cases():
+    """[(name, problem, seeded batch, reference rows)]"""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_golden_variants", os.path.join(GOLDEN, "make_golden_variants.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    with open(os.path.join(GOLDEN, "ref_variants.json")) as f:
+        gold = json.load(f)
+    out = []
+    for name, problem, tau_choices, tag in mod.variant_problems():
+        batch = candidates.generate(problem, gold["n_plans"], tau_choices, seed=gold["seed"], tag=tag)
+        out.append((name, problem, batch, gold["problems"][name]))
+    return out

@@ -123,3 +123,15 @@ def test_port_calibrated_hardware_matches_reference(c):
             assert float(out["peak"][i]).hex() == want["peak"], (i, k)
             assert float(out["score"][i]).hex() == want["score"], (i, k)
             assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, k)
+
+
+def test_port_problems_away_from_the_shipped_configurations_match_reference():
+    """The host build on the problems of tests/golden/ref_variants.json, every plan of the vectors."""
+    from tests.helpers import variant_cases
+    for name, p, batch, rows in variant_cases():
+        out = CpuPort(p).eval(batch)
+        for i, want in enumerate(rows):
+            assert float(out["makespan"][i]).hex() == want["makespan"], (name, i)
+            assert float(out["peak"][i]).hex() == want["peak"], (name, i)
+            assert float(out["score"][i]).hex() == want["score"], (name, i)
+            assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (name, i)

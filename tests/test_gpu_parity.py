@@ -557,3 +557,27 @@ def test_calibrated_hardware_equals_reference(c):
             assert float(out["peak"][i]).hex() == want["peak"], (i, k)
             assert float(out["score"][i]).hex() == want["score"], (i, k)
             assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (i, k)
+
+
+def test_problems_away_from_the_shipped_configurations_equal_reference():
+    """PPO and GRPO without generation quantiles, one and six quantiles, K > 1, meshes with 2 and 8 devices per
+    node, 4-byte elements, another head size, a stated parameter count: batched launches against the reference's
+    evaluations (tests/golden/ref_variants.json), and 4,096 further plans of each against the host build."""
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.search import candidates
+    from tests.golden.make_golden_variants import variant_problems
+    from tests.helpers import variant_cases
+    for name, p, batch, rows in variant_cases():
+        eng = Engine(p)
+        out = eng.eval(batch, gate_stale=False)
+        for i, want in enumerate(rows):
+            assert float(out["makespan"][i]).hex() == want["makespan"], (name, i)
+            assert float(out["peak"][i]).hex() == want["peak"], (name, i)
+            assert float(out["score"][i]).hex() == want["score"], (name, i)
+            assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (name, i)
+    for name, p, tau_choices, tag in variant_problems():
+        more = candidates.generate(p, 4096, tau_choices, seed=9, tag=tag)
+        got, want = Engine(p).eval(more, gate_stale=True), CpuPort(p).eval(more, flags=abi.GATE_STALE, threads=16)
+        for k in ("makespan", "peak", "score"):
+            assert same_bits(got[k], want[k]), (name, k)
+        assert np.array_equal(got["mask"], want["mask"]), name

@@ -114,3 +114,19 @@ def test_calibrated_hardware_matches_reference(c):
             assert order_crc(got["order"]) == want["order_crc"], (i, k)
             assert float(got["peak"]).hex() == want["peak"], (i, k)
             assert got["feasible"] == want["feasible"] and got["score"].hex() == want["score"], (i, k)
+
+
+def test_problems_away_from_the_shipped_configurations_match_reference():
+    """PPO and GRPO without generation quantiles, one and six quantiles, K > 1, meshes with 2 and 8 devices per
+    node, 4-byte elements, another head size, a stated parameter count: the reference's evaluations
+    (tests/golden/make_golden_variants.py) -- graph size, dispatch order, makespan, peak, feasibility, score."""
+    from tests.helpers import variant_cases
+    for name, p, batch, rows in variant_cases():
+        for i in range(0, len(rows), 2):
+            want = rows[i]
+            got = oracle_eval(p, batch, i, want_trace=True)
+            assert (len(got["nodes"]), len(got["edges"])) == (want["n_nodes"], want["n_edges"]), (name, i)
+            assert order_crc(got["order"]) == want["order_crc"], (name, i)
+            assert got["makespan"].hex() == want["makespan"], (name, i)
+            assert float(got["peak"]).hex() == want["peak"], (name, i)
+            assert got["feasible"] == want["feasible"] and got["score"].hex() == want["score"], (name, i)
