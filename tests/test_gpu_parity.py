@@ -481,7 +481,7 @@ def test_transfer_resource_policies_equal_reference(c):
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_other_seeds_unroll_depths_and_policies_equal_the_host_build(c):
-    """Away from the shipped problems: unroll depths 1, 2 and 7, both-endpoints reservations and two other
+    """Away from the shipped problems: unroll depths 1, 2, 7 and (three configurations) 32, both-endpoints reservations and two other
     seeds of the candidate generator.  Every makespan, peak, score and mask of the batched launch equals the
     host build of the same arithmetic, whose scheduler is written differently (a push-ordered list, one pop per
     iteration) and is itself checked against the reference vectors."""
@@ -490,8 +490,11 @@ def test_other_seeds_unroll_depths_and_policies_equal_the_host_build(c):
     from rpeg_amd.engine.runtime import Engine
     cfg = configs.config(c)
     n = 8192 if c != 5 else 2048
-    for K, pol in ((1, ("destination_only", "destination_only")), (2, ("both_endpoints", "destination_only")),
-                   (7, ("both_endpoints", "both_endpoints"))):
+    cases = [(1, ("destination_only", "destination_only")), (2, ("both_endpoints", "destination_only")),
+             (7, ("both_endpoints", "both_endpoints"))]
+    if c in (1, 2, 4):   # a long horizon, as the runtime's planner schedules (runtime/job_plan.py:174-213)
+        cases.append((32, ("destination_only", "destination_only")))
+    for K, pol in cases:
         p = replace(cfg.problem, K_eval=K, transfer_resource_policy=TransferResourcePolicy(*pol))
         eng, port = Engine(p), CpuPort(p)
         for seed in (7, 1234):
