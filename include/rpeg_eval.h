@@ -162,6 +162,25 @@ const char* rpeg_last_error(const rpeg_engine_t* e);
 int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
                     double* makespan, double* peak, double* score, uint8_t* mask, void* stream);
 
+/* rpeg_eval_batch for callers that cannot allocate device memory.  It has no counterpart in the reference; it
+   is there for callers that may not call hipMalloc: code under HIP graph capture, tight serving loops, harnesses
+   that forbid allocation.  Same arguments, same results bit for bit.  Every intermediate of the call (the
+   per-plan task list of the single-plan-per-wavefront kernel and a block of counters) lives in a file-scope
+   device array of RPEG_STATIC_MAX_PLANS * 4 + 256 bytes that each GPU the library runs on holds until the
+   process ends; the call makes no hipMalloc, hipFree or other allocating call.
+     - n above RPEG_STATIC_MAX_PLANS is rejected with status -9.
+     - The lowering classes of the plans must be on the device already, i.e. an earlier rpeg_eval_batch call
+       of this engine has met them: status -10 when the engine's class tables are not on the device (no such
+       call yet, or classes added since by rpeg_eval_host / rpeg_eval_trace), status -11 when plans of the
+       batch belong to classes the engine has not met (those plans get NaN outputs and RPEG_MASK_ERROR, the
+       others their results).  Problems with a class above 384 nodes are rejected with status -8.
+     - All engines on one GPU share that GPU's array and it keeps the last call's contents; the call resets
+       what must start at zero.  Calls that overlap on one GPU (two host threads, two streams) race.
+   Returns after the results are in place (it waits for the stream to read back one counter). */
+#define RPEG_STATIC_MAX_PLANS 32768
+int rpeg_eval_batch_static(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
+                           double* makespan, double* peak, double* score, uint8_t* mask, void* stream);
+
 /* rpeg_eval_batch plus the critical-chain mass of every plan: what move_gen derives from (trace,
    lowered) of the current plan to bias its choice of vertex (_critical_chain and _critical_mass,
    RPEG/search/moves.py:590-642).  mass[i*RPEG_MAX_V + v] = summed finish - start of the operator nodes

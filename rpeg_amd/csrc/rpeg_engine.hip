@@ -18,6 +18,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <unordered_map>
@@ -95,27 +96,14 @@ struct SigPlans {   // the plan fields of one thread's plan, a column of an LDS 
   const int16_t* col;
   __device__ VPlan operator[](int v) const { return ke_vplan<SIG_BLOCK>(col, v); }
 };
-__global__ __launch_bounds__(SIG_BLOCK) void k_signature(
-    const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
-    const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig, double* makespan, double* peak,
-    double* score, uint8_t* mask, double* mass, const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval,
-    uint32_t hmask, uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
-    uint32_t n_classes, uint32_t shards, const uint32_t* __restrict__ need) {
-  // counters met in this block: key, plans of the block, and the block's first arrival index
-  __shared__ uint32_t t_key[SIG_TABLE], t_cnt[SIG_TABLE], t_base[SIG_TABLE];
-  // plan fields: the gate and the signature index the vertices with run-time values, which would put a
-  // per-thread array into scratch memory
-  __shared__ int16_t s_plan[RPEG_MAX_V * RPEG_FIELDS * SIG_BLOCK];
-  constexpr uint32_t NONE = 0xFFFFFFFFu;
-  for (int j = threadIdx.x; j < SIG_TABLE; j += SIG_BLOCK) { t_key[j] = NONE; t_cnt[j] = 0u; }
-  __syncthreads();
-  const uint64_t i = (uint64_t)blockIdx.x * SIG_BLOCK + threadIdx.x;
-  const bool active = i < n;
-  PlanHead h;
-  h.structure = h.split = h.tau0 = h.tau1 = 0;
-  if (active) h = load_head(head, stride, i);
-  // The structure decides which tables the gate and the signature read.  It is made uniform (one pass per
-  // distinct structure among the plans of the wavefront) so that those reads are scalar loads.
+// Validity gate and class signature of the plan of this thread (SIG_INVALID for an inactive thread or a plan
+// that breaks a rule).  s_plan: LDS, [field][thread]; the gate and the signature index the vertices with
+// run-time values, which would put a per-thread array into scratch memory.
+// The structure decides which tables the gate and the signature read.  It is made uniform (one pass per
+// distinct structure among the plans of the wavefront) so that those reads are scalar loads.
+__device__ inline uint64_t sig_of_thread(const rpeg_problem_t* __restrict__ P, const bool active, const uint64_t i,
+                                         const PlanHead h, const int16_t* __restrict__ vert, const uint64_t stride,
+                                         int16_t* s_plan) {
   uint64_t sg = SIG_INVALID;
   const bool known = active && h.structure >= 0 && h.structure < P->n_struct;
   unsigned long long todo = __ballot(known);
@@ -144,6 +132,29 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
       if (nv != 0 && plan_valid(*P, hu, a)) sg = plan_signature(*P, su, h.split, h.tau0, h.tau1, a);
     }
   }
+  return sg;
+}
+
+__global__ __launch_bounds__(SIG_BLOCK) void k_signature(
+    const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
+    const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig, double* makespan, double* peak,
+    double* score, uint8_t* mask, double* mass, const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval,
+    uint32_t hmask, uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
+    uint32_t n_classes, uint32_t shards, const uint32_t* __restrict__ need) {
+  // counters met in this block: key, plans of the block, and the block's first arrival index
+  __shared__ uint32_t t_key[SIG_TABLE], t_cnt[SIG_TABLE], t_base[SIG_TABLE];
+  // plan fields: the gate and the signature index the vertices with run-time values, which would put a
+  // per-thread array into scratch memory
+  __shared__ int16_t s_plan[RPEG_MAX_V * RPEG_FIELDS * SIG_BLOCK];
+  constexpr uint32_t NONE = 0xFFFFFFFFu;
+  for (int j = threadIdx.x; j < SIG_TABLE; j += SIG_BLOCK) { t_key[j] = NONE; t_cnt[j] = 0u; }
+  __syncthreads();
+  const uint64_t i = (uint64_t)blockIdx.x * SIG_BLOCK + threadIdx.x;
+  const bool active = i < n;
+  PlanHead h;
+  h.structure = h.split = h.tau0 = h.tau1 = 0;
+  if (active) h = load_head(head, stride, i);
+  const uint64_t sg = sig_of_thread(P, active, i, h, vert, stride, s_plan);
   uint32_t key = NONE;
   if (active) {
     sig[i] = sg;
@@ -189,6 +200,47 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
   if (blockIdx.x == 0 && threadIdx.x < KE_NEED_SHARDS) count[(size_t)n_classes * shards + 1 + threadIdx.x] = need[threadIdx.x];
 }
 
+// The plan -> class step of the entry point that allocates nothing: validity gate, signature and, through the
+// table of the classes lowered so far, the pool offset of the plan's class blob, written to cls[i] for the
+// single-plan kernel (KP_SKIP for a plan that is not evaluated).  Plans that break a rule get the outputs
+// k_signature gives them; plans of a class that is not on the device yet get NaN outputs, RPEG_MASK_ERROR and
+// are counted in counters[0].
+__global__ __launch_bounds__(SIG_BLOCK) void k_class_direct(
+    const rpeg_problem_t* __restrict__ P, uint64_t n, const int16_t* __restrict__ vert,
+    const uint8_t* __restrict__ head, uint64_t stride, double* makespan, double* peak, double* score, uint8_t* mask,
+    const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hoff, uint32_t hmask, uint32_t* __restrict__ cls,
+    uint32_t* __restrict__ counters) {
+  __shared__ int16_t s_plan[RPEG_MAX_V * RPEG_FIELDS * SIG_BLOCK];
+  const uint64_t i = (uint64_t)blockIdx.x * SIG_BLOCK + threadIdx.x;
+  const bool active = i < n;
+  PlanHead h;
+  h.structure = h.split = h.tau0 = h.tau1 = 0;
+  if (active) h = load_head(head, stride, i);
+  const uint64_t sg = sig_of_thread(P, active, i, h, vert, stride, s_plan);
+  bool unknown = false;
+  if (active) {
+    uint32_t off = KP_SKIP;
+    if (sg != SIG_INVALID) {
+      unknown = true;
+      for (uint32_t slot = (uint32_t)sig_hash(sg) & hmask, probes = 0; probes <= hmask; slot = (slot + 1) & hmask, ++probes) {
+        const uint64_t k = hkey[slot];
+        if (k == sg) { off = hoff[slot]; unknown = false; break; }
+        if (k == SIG_INVALID) break;
+      }
+    }
+    cls[i] = off;
+    if (off == KP_SKIP) {
+      const double nan = __builtin_nan("");
+      if (makespan) makespan[i] = nan;
+      if (peak) peak[i] = nan;
+      if (score) score[i] = nan;
+      if (mask) mask[i] = unknown ? (uint8_t)(RPEG_MASK_VALID | RPEG_MASK_ERROR) : (uint8_t)0;
+    }
+  }
+  const unsigned long long u = __ballot(unknown);
+  if (u && (threadIdx.x & (WAVE - 1)) == 0) atomicAdd(&counters[0], (uint32_t)__builtin_popcountll(u));
+}
+
 // cbase[class * shards + shard]: plans of the class in lower shards; shard as in k_signature.
 __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const uint32_t* __restrict__ kidx,
                           const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
@@ -221,7 +273,9 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(4, 8))) vo
   extern __shared__ uint8_t kp_lds[];
   for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
     const uint64_t pi = L.perm ? L.perm[w] : w;
-    kp_eval_plan(L, w, pi, class_view(L.pool + L.wave_cls[w]), kp_lds);
+    const uint32_t off = L.wave_cls[w];
+    if (off == KP_SKIP) continue;   // uniform: a task without a plan to evaluate
+    kp_eval_plan(L, w, pi, class_view(L.pool + off), kp_lds);
   }
 }
 
@@ -295,6 +349,31 @@ __global__ void k_exp(uint64_t n, const double* x, double* y) {
 
 }  // namespace
 
+// Scratch memory of rpeg_eval_batch_static, the entry point that allocates nothing: per plan the pool offset of
+// its class blob (what the single-plan kernel takes as its task list), then a block of counters.  Every GPU
+// the library runs on holds its own copy of the array until the process ends; the name below is only a
+// host-side handle, the device address is looked up once per device (static_scratch_ptr) and that pointer is
+// what kernels and copies get.
+constexpr size_t STATIC_CLS_BYTES = (size_t)RPEG_STATIC_MAX_PLANS * 4, STATIC_COUNTER_BYTES = 256;
+static __device__ __align__(256) uint8_t scratch[STATIC_CLS_BYTES + STATIC_COUNTER_BYTES];
+constexpr int STATIC_MAX_DEVICES = 64;
+static uint8_t* g_static_ptr[STATIC_MAX_DEVICES];
+static std::mutex g_static_mu;
+
+// device address of `scratch` on the current device `dev`; null on failure (status in *st)
+static uint8_t* static_scratch_ptr(int dev, hipError_t* st) {
+  *st = hipSuccess;
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES) { *st = hipErrorInvalidDevice; return nullptr; }
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[dev]) {
+    void* p = nullptr;
+    *st = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (*st != hipSuccess) return nullptr;
+    g_static_ptr[dev] = (uint8_t*)p;
+  }
+  return g_static_ptr[dev];
+}
+
 struct rpeg_engine_s {
   rpeg_problem_t P;
   rpeg_problem_t* dP = nullptr;
@@ -306,6 +385,7 @@ struct rpeg_engine_s {
   std::vector<uint32_t> cls_off, cls_nodes;
   uint64_t* d_hkey = nullptr;                        // device table signature -> class id
   uint32_t* d_hval = nullptr;
+  uint32_t* d_hoff = nullptr;                        // the same slots -> pool offset of the class blob
   uint32_t hcap = 0, tables_for = 0;                 // table capacity; class count the device tables reflect
   uint32_t ccap = 0;                                 // capacity of the per-class device arrays
   // per-class tables of a call, one block on each side: counters per (class, shard), which become the shards'
@@ -357,6 +437,8 @@ struct rpeg_engine_s {
   double last_ms = -1.0;
   uint64_t stats[7] = {0, 0, 0, 0, 0, 0, 0};
   int n_cu = 256;
+  uint8_t* static_ptr = nullptr;    // this device's copy of the file-scope scratch array (rpeg_eval_batch_static)
+  uint32_t* h_static = nullptr;     // pinned: the counters of that array, read back after a call
   std::vector<uint32_t> cls_sorted, cls_pos;   // all classes by node count (largest first); place of a class among those of the batch
 };
 
@@ -387,22 +469,25 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
   uint32_t hcap = 1024;
   while (hcap < 4 * ncls) hcap *= 2;
   if (hcap != e->hcap) {
-    if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
+    if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); hipFree(e->d_hoff); }
     e->d_hkey = nullptr; e->hcap = 0;
     HIP_TRY(e, hipMalloc(&e->d_hkey, (size_t)hcap * 8));
     HIP_TRY(e, hipMalloc(&e->d_hval, (size_t)hcap * 4));
+    HIP_TRY(e, hipMalloc(&e->d_hoff, (size_t)hcap * 4));
     e->hcap = hcap;
   }
   std::vector<uint64_t> hk(hcap, SIG_INVALID);
-  std::vector<uint32_t> hv(hcap, 0);
+  std::vector<uint32_t> hv(hcap, 0), ho(hcap, 0);
   for (uint32_t c = 0; c < ncls; ++c) {
     uint32_t slot = (uint32_t)sig_hash(e->cls_sig[c]) & (hcap - 1);
     while (hk[slot] != SIG_INVALID) slot = (slot + 1) & (hcap - 1);
     hk[slot] = e->cls_sig[c];
     hv[slot] = c;
+    ho[slot] = e->cls_off[c];
   }
   HIP_TRY(e, hipMemcpy(e->d_hkey, hk.data(), (size_t)hcap * 8, hipMemcpyHostToDevice));
   HIP_TRY(e, hipMemcpy(e->d_hval, hv.data(), (size_t)hcap * 4, hipMemcpyHostToDevice));
+  HIP_TRY(e, hipMemcpy(e->d_hoff, ho.data(), (size_t)hcap * 4, hipMemcpyHostToDevice));
   if (ncls + 1 > e->ccap) {
     const uint32_t cap = std::max<uint32_t>(2 * (ncls + 1), 4096);
     if (e->d_ccount) {
@@ -568,6 +653,14 @@ int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
   e->max_v = 1;
   for (int q = 0; q < e->P.n_struct; ++q) e->max_v = std::max<uint32_t>(e->max_v, (uint32_t)e->P.st[q].n_vertex);
 
+  {  // the device address of the static scratch array, once per device, with that device current
+    hipError_t st;
+    e->static_ptr = static_scratch_ptr(e->device, &st);
+    if (!e->static_ptr || hipHostMalloc(&e->h_static, STATIC_COUNTER_BYTES) != hipSuccess) {
+      delete e;
+      return -2;
+    }
+  }
   if (hipMalloc(&e->dP, sizeof(rpeg_problem_t)) != hipSuccess ||
       hipMemcpy(e->dP, problem, sizeof(rpeg_problem_t), hipMemcpyHostToDevice) != hipSuccess ||
       hipEventCreate(&e->ev0) != hipSuccess || hipEventCreate(&e->ev1) != hipSuccess) {
@@ -585,7 +678,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_pool) hipFree(e->d_pool);
   if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
   if (e->d_need) hipFree(e->d_need);
-  if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); }
+  if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); hipFree(e->d_hoff); }
+  if (e->h_static) hipHostFree(e->h_static);
   if (e->d_ccount) {
     hipFree(e->d_ccount);
     hipHostFree(e->h_ccount);
@@ -996,6 +1090,59 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
 }
 
 extern "C" {
+
+// rpeg_eval_batch for callers that cannot allocate: every intermediate of the call lives in the file-scope
+// scratch array of this device, and the call makes no hipMalloc / hipFree.  One plan per wavefront (k_plan).
+int rpeg_eval_batch_static(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                           double* peak, double* score, uint8_t* mask, void* stream) {
+  if (!e || !plans) return -1;
+  e->err.clear();
+  e->last_ms = -1.0;
+  if (n == 0) return 0;
+  if (n > (uint64_t)RPEG_STATIC_MAX_PLANS) {
+    e->err = "rpeg_eval_batch_static takes at most " + std::to_string(RPEG_STATIC_MAX_PLANS) + " plans per call, got " +
+             std::to_string(n);
+    return -9;
+  }
+  if (!plans->vert || !plans->head || plans->stride < n) { e->err = "bad plan tensors"; return -1; }
+  if (!e->d_hkey || e->tables_for != (uint32_t)e->cls_sig.size() || e->d_pool_used != e->pool.size() || !e->d_pool) {
+    e->err = "the engine's class tables are not on the device: evaluate a batch with these classes through rpeg_eval_batch first";
+    return -10;
+  }
+  if (e->max_nodes > (uint32_t)(WAVE * KP_MAX_NS) || kp_lds_bytes(e->max_nodes, e->max_slots) > 64 * 1024) {
+    e->err = "a class of this problem has too many nodes for one plan per wavefront";
+    return -8;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t* const d_cls = (uint32_t*)e->static_ptr;
+  uint32_t* const d_counters = (uint32_t*)(e->static_ptr + STATIC_CLS_BYTES);
+  // the array keeps what the last call left: the counters start at zero (a fill kernel, so that a caller may
+  // capture the launches), the task list is rewritten for all n plans
+  hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, s, d_counters, (uint64_t)(STATIC_COUNTER_BYTES / 4), 0u);
+  hipLaunchKernelGGL(k_class_direct, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n,
+                     plans->vert, plans->head, plans->stride, makespan, peak, score, mask, e->d_hkey, e->d_hoff,
+                     e->hcap - 1, d_cls, d_counters);
+  HIP_TRY(e, hipGetLastError());
+  EvalLaunch L;
+  L.P = e->dP; L.vert = plans->vert; L.head = plans->head; L.stride = plans->stride;
+  L.perm = nullptr; L.wave_cls = d_cls; L.pool = e->d_pool; L.ws = nullptr;
+  L.n_waves = n; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
+  L.cls_bytes = 0; L.rcap = 0; L.max_v = e->max_v; L.ovf = nullptr; L.need = nullptr;
+  L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
+  L.mass = nullptr; L.prof = nullptr;
+  const size_t lds = kp_lds_bytes(e->max_nodes, e->max_slots);
+  hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n, (uint64_t)e->n_cu * 32)), dim3(WAVE), lds, s, L);
+  HIP_TRY(e, hipGetLastError());
+  HIP_TRY(e, hipMemcpyAsync(e->h_static, d_counters, 4, hipMemcpyDeviceToHost, s));
+  HIP_TRY(e, hipStreamSynchronize(s));
+  e->stats[0] = 0; e->stats[1] = 0; e->stats[2] = n; e->stats[3] = lds; e->stats[4] = 0; e->stats[5] = 1; e->stats[6] = 0;
+  if (e->h_static[0] != 0u) {
+    e->err = std::to_string(e->h_static[0]) + " plans belong to lowering classes the engine has not met: evaluate them through "
+             "rpeg_eval_batch once (their outputs are NaN, their mask has RPEG_MASK_ERROR)";
+    return -11;
+  }
+  return 0;
+}
 
 int rpeg_op_time_batch(rpeg_engine_t* e, uint64_t n, int32_t structure, int32_t vertex, const int16_t* strat,
                        uint64_t stride, double* time, double* peak, void* stream) {

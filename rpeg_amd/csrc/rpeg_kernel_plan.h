@@ -29,6 +29,7 @@ namespace rpeg {
 
 constexpr int KP_MAX_NS = 6;                    // nodes per lane: classes of up to 384 nodes
 constexpr uint32_t KP_TIE_BITS = 23u, KP_TIE_MASK = (1u << KP_TIE_BITS) - 1u;
+constexpr uint32_t KP_SKIP = 0xFFFFFFFFu;        // task -> class blob offset of a task that is skipped (offsets stay below 2^31)
 constexpr int KP_PLAN_I16 = 80;                 // plan fields in LDS (60 used; pair tests may read past them)
 
 // LDS of one wavefront: plan fields, per-vertex memory terms, durations per slot, rank / finish and start

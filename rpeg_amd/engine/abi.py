@@ -10,6 +10,7 @@ MODEL = {"Pi": 0, "V": 1, "Ref": 2, "R": 3, "AC": 4}
 NEED_DISJ, NEED_PI = 1, 2
 MASK_VALID, MASK_STALE_OK, MASK_MEM_OK, MASK_ERROR = 1, 2, 4, 8
 GATE_STALE = 1
+STATIC_MAX_PLANS = 32768
 HW_FIELDS = (
     "flops_per_gpu", "memory_per_gpu", "memory_bandwidth",
     "alpha_coll_g", "beta_coll_g", "alpha_coll_n", "beta_coll_n", "alpha_coll_r", "beta_coll_r",

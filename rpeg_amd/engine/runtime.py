@@ -24,7 +24,7 @@ EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
            "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
-           "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics")
+           "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static")
 
 
 class EngineError(RuntimeError):
@@ -49,6 +49,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_last_error.argtypes = [vp]
     lib.rpeg_eval_batch.restype = C.c_int
     lib.rpeg_eval_batch.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp]
+    lib.rpeg_eval_batch_static.restype = C.c_int
+    lib.rpeg_eval_batch_static.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp]
     lib.rpeg_eval_batch_mass.restype = C.c_int
     lib.rpeg_eval_batch_mass.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp, vp]
     lib.rpeg_eval_host.restype = C.c_int
@@ -220,6 +222,21 @@ class Engine:
                                           out["makespan"].data_ptr(), out["peak"].data_ptr(), out["score"].data_ptr(),
                                           out["mask"].data_ptr(), stream)
         self._check(rc, "rpeg_eval_batch")
+        return out
+
+    def eval_device_static(self, dbatch: DeviceBatch, out=None, gate_stale: bool = True, n: Optional[int] = None):
+        """eval_device through the entry point that allocates nothing (rpeg_eval_batch_static): at most
+        abi.STATIC_MAX_PLANS plans whose lowering classes an earlier eval_device call has met.  `out` must be
+        given by a caller that may not allocate."""
+        torch = _torch()
+        n = dbatch.n if n is None else n
+        out = out or self.alloc_outputs(n)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_eval_batch_static(self._h, n, C.addressof(dbatch.soa), abi.GATE_STALE if gate_stale else 0,
+                                                 out["makespan"].data_ptr(), out["peak"].data_ptr(),
+                                                 out["score"].data_ptr(), out["mask"].data_ptr(), stream)
+        self._check(rc, "rpeg_eval_batch_static")
         return out
 
     def eval(self, batch: PlanBatch, gate_stale: bool = True, mass: bool = False) -> Dict[str, np.ndarray]:
