@@ -59,10 +59,11 @@ def test_python_oracle_beyond_fixtures(c):
         assert bool(out["mask"][i] & abi.MASK_MEM_OK) == (not want["peak"] > want["cap"]), i
 
 
-@pytest.mark.parametrize("c,n", [(1, 4096), (2, 65536), (3, 65536), (4, 262144)])
+@pytest.mark.parametrize("c,n", [(1, 4096), (2, 65536), (3, 262144), (4, 1048576)])
 def test_full_candidate_sets_rank_and_argmax(c, n):
-    """Whole seeded sets: masks, every score, the ranking and the best plan equal the host build of
-    the same arithmetic, which the CPU suite ties to the reference vectors."""
+    """Whole seeded sets at the sizes the workload description names (4,096 / 65,536 / 262,144 / 1,048,576
+    plans): masks, every score, the ranking and the best plan equal the host build of the same arithmetic,
+    which the CPU suite ties to the reference vectors."""
     cfg, batch = seeded_batch(c, n)
     out = engine(c).eval(batch, gate_stale=True)
     ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)

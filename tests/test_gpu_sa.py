@@ -70,7 +70,7 @@ def _variants(p):
 @pytest.mark.parametrize("c,n_chains,n_steps,kw", [
     (1, 64, 200, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
     (2, 32, 100, dict(T_init=0.30, T_min=0.01, T_warm=0.05, stag_window=5, geometric_cooling=True)),
-    (5, 64, 60, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
+    (5, 64, 2000, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),   # the whole run of config 5
 ])
 def test_chains_equal_host_replay(c, n_chains, n_steps, kw):
     """Same counter-based draws, GPU evaluator against CPU evaluator: every decision of every chain,
