@@ -20,14 +20,22 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 FP64_PEAK_TFLOPS = 78.6     # MI355X vector FP64, published
+ISSUE_PEAK = 256 * 4 * 2.4e9   # wave-instructions per second: 256 CUs x 4 SIMDs x 2.4 GHz, one instruction per clock
 # algorithmic bytes per plan: int16 plan fields (10 per vertex) + 4 header bytes in, 3 doubles + 1 mask byte out
 ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
-# HBM bytes per step of the evaluation kernels measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
-# a 256 MiB copy (the counter summary of this workload is committed under profiles/); None where no counter
-# run exists
-MEASURED_TRAFFIC = {2: 243.5e6}
-# algorithmic fp64 operations per plan (cost model + scheduler + memory model of the fully split DAG)
-ALG_FLOPS = {1: 3.7e3, 2: 2.5e3, 3: 6.0e3, 4: 0.83e3, 5: 3.7e3}
+# fp64 operations per plan (additions, multiplications, divisions, comparisons incl. max/min, 2 per fused
+# multiply-add), counted by oracle/flop_count.cpp (the kernels' arithmetic compiled with a counting number
+# type) and averaged over the seeded set of the configuration (config 5: over 4,096 seeded plans);
+# tests/test_cpu_port.py holds these constants to a fresh count
+ALG_FLOPS = {1: 3697.0, 2: 2165.3, 3: 6502.9, 4: 1245.8, 5: 4155.6}
+# Counter figures of one step, taken from the rocprofv3 --pmc summaries under profiles/ and valid only for the
+# kernel layout they were measured on (`layout`: wave tasks, LDS bytes, plans per wavefront with LDS state,
+# single-plan tasks of rpeg_engine_stats): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
+# by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS + VMEM_RD + VMEM_WR of the
+# evaluation kernels / plans).  A run whose layout differs prints null instead of a stale number.
+MEASURED = {
+    2: dict(layout=(9950, 15392, 0, 8915), traffic=243.5e6, instructions_per_plan=4691.0),
+}
 
 
 def cpu_baseline(cfg, batch, seconds=12.0):
@@ -46,17 +54,65 @@ def cpu_baseline(cfg, batch, seconds=12.0):
                 sample=f"first {done} plans of the same seeded set, Python oracle, 1 process, {dt:.1f} s")
 
 
+def _pool_worker(i):
+    from oracle import rpeg_oracle as oracle
+    cfg, batch = _POOL_STATE
+    p = cfg.problem
+    rpeg, plan, wl = batch.configuration(p, i)
+    return oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, p.K_eval, p.memory_policy)["score"]
+
+
+_POOL_STATE = None
+
+
+def cpu_pool_baseline(cfg, batch, seconds=10.0, workers=None):
+    """The same Python oracle behind multiprocessing.Pool(min(6, cores)) with a blocking map over the
+    candidates of a step, as the reference dispatches them (RPEG/search/optimizer.py:414-417, 793-798).
+    Must run before the process touches the GPU (the workers are forked)."""
+    import multiprocessing as mp
+    global _POOL_STATE
+    workers = workers or min(6, os.cpu_count() or 1)
+    _POOL_STATE = (cfg, batch)
+    done, chunk = 0, 6 * workers
+    with mp.get_context("fork").Pool(workers) as pool:
+        pool.map(_pool_worker, range(chunk))          # start-up and imports are not timed
+        t0 = time.perf_counter()
+        while done + chunk <= batch.n and time.perf_counter() - t0 < seconds:
+            pool.map(_pool_worker, range(done, done + chunk))
+            done += chunk
+        dt = time.perf_counter() - t0
+    return dict(value=done / dt, unit="plan evals/s", cores=workers, kind="port",
+                sample=f"first {done} plans, Python oracle behind multiprocessing.Pool({workers}), blocking map of "
+                       f"{chunk} plans at a time, {dt:.1f} s")
+
+
 def cxx_port(cfg, batch, threads):
+    """Host build of the kernels' arithmetic on all host cores; returns the figure and the results."""
     from oracle.cpu_port import CpuPort
+    from rpeg_amd.engine import abi
     port = CpuPort(cfg.problem)
-    n = min(batch.n, 65536)
-    sub = batch.slice(0, n)
-    port.eval(sub.slice(0, 256), threads=threads)
+    port.eval(batch.slice(0, 256), threads=threads)
     t0 = time.perf_counter()
-    port.eval(sub, threads=threads)
+    ref = port.eval(batch, flags=abi.GATE_STALE, threads=threads)
     dt = time.perf_counter() - t0
-    return dict(value=n / dt, unit="plan evals/s", cores=threads,
-                sample=f"first {n} plans, host build of the kernels' arithmetic (OpenMP), lowering included")
+    return dict(value=batch.n / dt, unit="plan evals/s", cores=threads,
+                sample=f"all {batch.n} plans, host build of the kernels' arithmetic (OpenMP), lowering included"), ref
+
+
+def parity_block(out, ref):
+    """The timed GPU results against the host build's on the same plans: masks, every score, ranking, best plan."""
+    import numpy as np
+    ok = np.isfinite(ref["score"]) & np.isfinite(out["score"])
+    rel = np.abs(out["score"][ok] - ref["score"][ok]) / np.maximum(np.abs(ref["score"][ok]), 1e-300)
+    rel_m = np.abs(out["makespan"][ok] - ref["makespan"][ok]) / np.maximum(np.abs(ref["makespan"][ok]), 1e-300)
+    return dict(
+        against="host build of the same arithmetic (oracle/cpu_port.cpp), which the CPU tests tie to the reference's vectors",
+        plans=int(len(ref["score"])),
+        mask_equal=bool(np.array_equal(out["mask"], ref["mask"])),
+        scores_bit_equal=bool(np.array_equal(out["score"].view(np.uint64), ref["score"].view(np.uint64))),
+        ranking_equal=bool(np.array_equal(np.argsort(-out["score"], kind="stable"), np.argsort(-ref["score"], kind="stable"))),
+        argmax_equal=bool(int(np.nanargmax(out["score"])) == int(np.nanargmax(ref["score"]))),
+        max_rel_err=float(max(rel.max() if rel.size else 0.0, rel_m.max() if rel_m.size else 0.0)))
 
 
 def bench_sa(args):
@@ -146,16 +202,22 @@ def main():
     if args.config == 5:
         return bench_sa(args)
 
-    import torch
     from rpeg_amd import configs
-    from rpeg_amd.engine import abi
-    from rpeg_amd.engine.runtime import DeviceBatch, Engine
     from rpeg_amd.search import candidates
 
     c = args.config
     cfg = configs.config(c)
     n = cfg.n_plans
     batch = candidates.generate(cfg.problem, n, cfg.tau_choices, seed=42, tag=c)
+    # the CPU legs first: the pool forks its workers, which must happen before this process touches the GPU
+    cpu = None
+    if not args.no_cpu:
+        cpu = dict(pool=cpu_pool_baseline(cfg, batch), one=cpu_baseline(cfg, batch))
+        cpu["cxx"], cpu["ref"] = cxx_port(cfg, batch, threads=min(16, os.cpu_count() or 1))
+
+    import torch
+    from rpeg_amd.engine import abi
+    from rpeg_amd.engine.runtime import DeviceBatch, Engine
     eng = Engine(cfg.problem, "cuda:0")
     db = DeviceBatch(batch, "cuda:0")
     out = eng.alloc_outputs(n)
@@ -230,8 +292,10 @@ def main():
         eng.eval(batch)
     pcie_ms = (time.perf_counter() - t0) / 3 * 1e3
 
-    mask = out["mask"].cpu().numpy()
-    score = out["score"].cpu().numpy()
+    eng.eval_device(db, out)
+    torch.cuda.synchronize()
+    res = {k: v.cpu().numpy() for k, v in out.items()}
+    mask, score = res["mask"], res["score"]
     valid = (mask & abi.MASK_VALID) != 0
     alg_bytes = ALG_BYTES[c] * n
     # what the timed launch consists of: one plan per wavefront for a batch that would not fill the chip
@@ -244,6 +308,23 @@ def main():
         kernel_name = f"k_eval<{stats['state_lanes']}>"
     achieved_gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
     achieved_tflops = ALG_FLOPS[c] * n / (kernel_ms * 1e-3) / 1e12
+    hbm = {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": achieved_gbs / HBM_PEAK_GBS, "algorithmic_bytes_per_plan": ALG_BYTES[c]}
+    fp64 = {"bound": "fp64_valu", "achieved": achieved_tflops, "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved_tflops / FP64_PEAK_TFLOPS, "algorithmic_flops_per_plan": ALG_FLOPS[c]}
+    # the roofline of the line is the one with the larger fraction: achieved = max(bytes fraction, flops fraction)
+    roofline = dict(fp64 if fp64["frac"] >= hbm["frac"] else hbm)
+    layout = (stats["wave_tasks"], stats["lds_bytes"], stats["state_lanes"], stats["single_plan_tasks"])
+    measured = MEASURED.get(c)
+    same_layout = measured is not None and tuple(measured["layout"]) == layout
+    roofline.update(traffic=measured["traffic"] if same_layout else None, kernel=kernel_name, kernel_ms=kernel_ms,
+                    layout=list(layout))
+    ipp = measured["instructions_per_plan"] if same_layout else None
+    issue = {"instructions_per_plan": ipp, "peak": ISSUE_PEAK, "unit": "wave-instructions/s",
+             "achieved": None if ipp is None else ipp * n / (kernel_ms * 1e-3),
+             "frac": None if ipp is None else ipp * n / (kernel_ms * 1e-3) / ISSUE_PEAK,
+             "note": "instructions issued per plan from the rocprofv3 counter summary under profiles/; "
+                     "null when the kernel layout of this run is not the profiled one"}
     line = {
         "metric": "cost-model plan evals/sec on 1 MI355X",
         "value": value, "unit": "plan evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -252,11 +333,7 @@ def main():
         "config": {"workload": cfg.name, "n_plans": n, "seed": 42, "K_eval": cfg.problem.K_eval,
                    "device_mesh": [cfg.problem.device_space.R, cfg.problem.device_space.N, cfg.problem.device_space.G],
                    "classes": stats["classes"], "inputs": "resident in HBM", "outputs": "left in HBM"},
-        "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(c),
-                     "kernel": kernel_name, "kernel_ms": kernel_ms, "algorithmic_bytes_per_plan": ALG_BYTES[c]},
-        "fp64_valu": {"achieved": achieved_tflops, "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
-                      "frac": achieved_tflops / FP64_PEAK_TFLOPS, "algorithmic_flops_per_plan": ALG_FLOPS[c]},
+        "roofline": roofline, "hbm": hbm, "fp64_valu": fp64, "issue": issue,
         "kernel_only_evals_per_s": n / (kernel_ms * 1e-3),
         "two_stream_evals_per_s": two_stream,
         "pcie_inclusive_ms_per_step": pcie_ms, "pcie_inclusive_evals_per_s": n / (pcie_ms * 1e-3),
@@ -264,12 +341,15 @@ def main():
         "feasible_fraction": float(((mask & abi.MASK_MEM_OK) != 0)[valid].mean()),
         "best_plan": int(score.argmax()), "best_score": float(score.max()),
     }
-    if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(cfg, batch)
-        line["cpu_port_cxx"] = cxx_port(cfg, batch, threads=min(16, os.cpu_count() or 1))
+    if cpu is not None:
+        line["cpu_baseline"] = cpu["one"]
+        line["cpu_baseline_pool"] = cpu["pool"]
+        line["cpu_port_cxx"] = cpu["cxx"]
+        line["parity"] = parity_block(res, cpu["ref"])
         line["host_cores"] = os.cpu_count()
     else:
         line["cpu_baseline"] = None
+        line["parity"] = None
     print(json.dumps(line))
 
 

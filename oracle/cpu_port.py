@@ -192,3 +192,24 @@ def exp_libm(x):
     y = np.empty_like(x)
     lib().port_exp(x.size, x.ctypes.data, y.ctypes.data)
     return y
+
+
+def count_flops(problem, batch, flags=0):
+    """fp64 operations of the plans of `batch`, as the kernels' arithmetic executes them (flop_count.cpp):
+    dict with the per-plan means of add (additions and subtractions), mul, div, fma, cmp (comparisons, max and
+    min included) and `total` = add + mul + div + cmp + 2 fma, plus `plans` (valid plans counted)."""
+    path = _build.FLOPS if os.path.exists(_build.FLOPS) else (_build.build(force=True) and _build.FLOPS)
+    fl = C.CDLL(path)
+    fl.flop_count.restype = C.c_int
+    fl.flop_count.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint32, C.c_void_p]
+    P = compile_problem(problem)
+    vert = np.ascontiguousarray(batch.vert)
+    head = np.ascontiguousarray(batch.head)
+    out = (C.c_uint64 * 6)()
+    rc = fl.flop_count(C.addressof(P), batch.n, vert.ctypes.data, head.ctypes.data, vert.shape[1], flags, out)
+    if rc != 0:
+        raise RuntimeError("flop_count failed")
+    n = max(1, out[5])
+    res = dict(add=out[0] / n, mul=out[1] / n, div=out[2] / n, fma=out[3] / n, cmp=out[4] / n, plans=int(out[5]))
+    res["total"] = res["add"] + res["mul"] + res["div"] + res["cmp"] + 2 * res["fma"]
+    return res

@@ -135,3 +135,17 @@ def test_port_problems_away_from_the_shipped_configurations_match_reference():
             assert float(out["peak"][i]).hex() == want["peak"], (name, i)
             assert float(out["score"][i]).hex() == want["score"], (name, i)
             assert bool(out["mask"][i] & abi.MASK_MEM_OK) == want["feasible"], (name, i)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_bench_flop_constants_follow_a_fresh_count(c):
+    """bench.py prices its FP64 roofline with operation counts frozen from oracle/flop_count.cpp: a fresh
+    count over the first 4,096 seeded plans stays within 3 % of them (the frozen ones are whole-set means)."""
+    import bench
+    from oracle.cpu_port import count_flops
+    cfg, batch = seeded_batch(c, 4096)
+    got = count_flops(cfg.problem, batch)
+    assert got["plans"] == 4096
+    assert abs(got["total"] - bench.ALG_FLOPS[c]) <= 0.03 * bench.ALG_FLOPS[c], (got, bench.ALG_FLOPS[c])
+    # the count is dominated by the scheduler's comparisons, as the kernels' instruction mix is
+    assert got["cmp"] > got["add"] + got["mul"] + got["div"]
