@@ -447,6 +447,34 @@ def test_is_valid_drop_in_equals_restatement(c):
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_gates_equal_reference_verdicts(c):
+    """The drop-in is_valid and evaluate_cached (through the engine: k_signature's gate, the stale rule, the
+    memory fit, the penalty) against what the reference's own functions returned for seeded plans and for
+    plans broken one rule at a time (tests/golden/ref_validity.json)."""
+    import json
+    import os
+    from rpeg_amd.model.memory import NodeMemoryModel
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration, evaluate_cached, is_valid
+    from tests.golden.make_golden_validity import validity_cases
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_validity.json")) as f:
+        rows = json.load(f)["configs"][str(c)]
+    cfg, batch, cases = validity_cases(c)
+    p = cfg.problem
+    n_valid = n_scored = 0
+    for want, (i, rule, rpeg, plan, wl) in zip(rows, cases):
+        config = Configuration(rpeg, plan, p.device_space)
+        mm = NodeMemoryModel.from_policy(p.hw, p.suite, wl, p.memory_policy, trainable=frozenset(rpeg.trainable))
+        assert is_valid(config, p.suite, wl, mm) == want["is_valid"], (i, rule)
+        n_valid += want["is_valid"]
+        if "score" in want and all(want["compatible"]) and rule in (None, 8):
+            score, _, feasible, miss = evaluate_cached(config, EvalCache(), p.suite, wl, p.hw, p.K_eval, p.memory_policy)
+            assert float(score).hex() == want["score"] and feasible == want["feasible"] and miss, (i, rule)
+            n_scored += 1
+    assert n_valid and n_scored
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_transfer_resource_policies_equal_reference(c):
     """Both-endpoints reservations for weights, for activations and for both: makespans of batched launches
     and, through the drop-in evaluate(), dispatch order, finish times and utilisation against the reference
