@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define RPEG_ABI_VERSION 3
+#define RPEG_ABI_VERSION 4
 
 #define RPEG_MAX_V 6       /* template vertices per structure                */
 #define RPEG_MAX_E 9       /* within-step data edges                          */
@@ -257,6 +257,24 @@ typedef struct rpeg_sa_params_s {
                                  floor (1 - loss) x best throughput so far, and by throughput x 1e-12 below
                                  it (optimizer.py:461-486); every evaluated plan is then traced once more
                                  for its utilisation (rpeg_eval_trace_metrics).  rpeg_sa_run ignores it  */
+  /* the ablation switches of OptimizerConfig (RPEG/search/optimizer.py:83-88, 404-410) */
+  int32_t fixed_mb;           /* moves.py:155-156, 182-188: one micro-batch count per (dp, pp) wherever strategies
+                                 are drawn (the candidate directory must be built under the same rule)           */
+  int32_t uniform_vertex;     /* moves.py:157-158, 688: move_gen draws its vertex uniformly                       */
+  int32_t hard_oom;           /* evaluate.py:392, 437: a plan that does not fit scores 0 instead of the soft penalty */
+  int32_t timed;              /* bit 0: deadline_s holds; bit 1: deadline_struct_s holds                          */
+  /* rpeg_sa_optimize*: OptimizerConfig.deadline and .deadline_per_struct (optimizer.py:78-82) as readings of the
+     run's clock.  That clock is `clock` (seconds, any origin; tests drive it) or, when `clock` is null, the
+     steady clock counted from the start of the call, so that the two fields are then seconds from the start.
+     Once the clock reads deadline_s or more the search ends whatever the budgets: the clock is read before
+     every iteration and after every evaluated batch, and the conditions are tested in the reference's order
+     (deadline, E_max, the setting's share, E_struct; :703-720, 848-865).  With a deadline the time left is
+     split evenly among the structural settings still to come, whatever deadline_struct_s says (:571-579);
+     without one, deadline_struct_s bounds every setting alike.  rpeg_sa_run ignores these. */
+  double deadline_s;
+  double deadline_struct_s;
+  double (*clock)(void* ctx);
+  void* clock_ctx;
 } rpeg_sa_params_t;
 
 typedef struct rpeg_sa_result_s {   /* per-chain arrays of n_chains elements, any may be NULL */
@@ -299,7 +317,8 @@ typedef struct rpeg_sa_serial_result_s {
   uint8_t* eval_log_variant; /*   rows of RPEG_MAX_V*RPEG_FIELDS values / their staleness variants       */
   int64_t eval_log_cap, n_eval_log;
   double wall_s;
-  int32_t best_family, pad;  /* family of best_plan (0 from rpeg_sa_optimize)                            */
+  int32_t best_family;       /* family of best_plan (0 from rpeg_sa_optimize)                            */
+  int32_t timed_out;         /* 1: the search ended at its wall-clock deadline                           */
   double* eval_log_score;    /* optional, eval_log_cap entries each: what the run's cache holds for the   */
   uint8_t* eval_log_feasible;/*   logged plan -- score and feasibility as evaluate_cached stores them for a */
   double* eval_log_util;     /*   current plan (stale-layout gate applied) or as the merge of fresh         */

@@ -109,13 +109,18 @@ def valid_dp_degrees(R, N, B, G=1):
     return [d for d in range(1, R * N * G + 1) if B % d == 0]
 
 
+ABLATION_FIXED_MB = False   # moves.py:155-156: tests set it around a directory build
+
+
 def valid_mb_counts(pp, dp, B):
-    """moves.py:148-176 with both ablations off."""
+    """moves.py:162-199."""
     local = B // dp
     if local < MIN_B_LOCAL and dp > 1:
         return []
     if pp == 1:
         return [1]
+    if ABLATION_FIXED_MB:
+        return [1] if local % pp != 0 else [pp]
     max_mb = local // MIN_B_LOCAL
     return [mb for mb in range(pp, min(max_mb, local) + 1) if local % mb == 0]
 

@@ -89,10 +89,17 @@ struct SaSettings {
   double T_init = 0.30, T_warm = 0.05, T_min = 0.01, T_cool = 1.0, alpha_pair = 0.28, score_eps = 1e-4;
   double max_throughput_loss = 0.0;
   uint64_t seed = 42;
+  int hard_oom = 0;                       // OptimizerConfig.hard_oom: a plan that does not fit scores 0 (evaluate.py:392, 437)
+  int timed = 0;                          // bit 0: deadline_s holds, bit 1: deadline_struct_s holds
+  double deadline_s = 0.0, deadline_struct_s = 0.0;   // readings of the clock at which rpeg_sa_optimize* ends the run / a setting
+  double (*clock)(void*) = nullptr;       // seconds; null: the steady clock, zero when the run starts
+  void* clock_ctx = nullptr;
 };
 
 struct SaContext {
   int nv = 0, R = 1, N = 1, G = 1, B = 1;
+  bool fixed_mb = false;         // moves.py:155-156, 182-188: one micro-batch count per (dp, pp)
+  bool uniform_vertex = false;   // moves.py:157-158, 688: no critical-chain bias when a vertex is drawn
   int L[RPEG_MAX_V] = {0};
   std::vector<int> tps, dps;
   std::vector<int> pps[RPEG_MAX_V];
@@ -135,12 +142,13 @@ struct SaContext {
   }
 };
 
-// moves.py:148-176 (ablations off)
-inline void sa_valid_mb(int pp, int dp, int B, std::vector<int>& out) {
+// moves.py:162-199
+inline void sa_valid_mb(int pp, int dp, int B, std::vector<int>& out, bool fixed_mb = false) {
   out.clear();
   const int local = B / dp;
   if (local < 8 && dp > 1) return;
   if (pp == 1) { out.push_back(1); return; }
+  if (fixed_mb) { out.push_back(local % pp != 0 ? 1 : pp); return; }
   const int max_mb = local / 8;
   for (int mb = pp; mb <= std::min(max_mb, local); ++mb)
     if (local % mb == 0) out.push_back(mb);
@@ -157,7 +165,7 @@ inline void sa_sample_origin(SaRng& rng, const SaContext& cx, int re, int ne, in
 inline int sa_move_gen(SaRng& rng, const SaContext& cx, const SaPlan& plan, const double* mass, int K_x, int T_max,
                        double T, double T_init, SaPlan* out, int* fallback = nullptr) {
   int v;
-  if (rng.random() >= 0.4) {
+  if (!cx.uniform_vertex && rng.random() >= 0.4) {   // (no draw at all under uniform_vertex, moves.py:688)
     double w[RPEG_MAX_V];
     for (int x = 0; x < cx.nv; ++x) w[x] = mass[x] + 1e-6;
     v = rng.weighted(w, cx.nv);
@@ -246,7 +254,7 @@ inline bool sa_sample_region(SaRng& rng, const SaContext& cx, int v, int r_lo, i
   const int n_o = rng.below(cx.N / ne) * ne;
   const int g_o = rng.below(cx.G / ge) * ge;
   std::vector<int> mbs;
-  sa_valid_mb(pp, dp, cx.B, mbs);
+  sa_valid_mb(pp, dp, cx.B, mbs, cx.fixed_mb);
   if (mbs.empty()) return false;
   const int mb = mbs[rng.below((int)mbs.size())];
   row[SA_DP] = (int16_t)dp; row[SA_PP] = (int16_t)pp; row[SA_TP] = (int16_t)tp; row[SA_MB] = (int16_t)mb;
@@ -351,6 +359,12 @@ struct SaRun {
     return (m & RPEG_MASK_VALID) && (m & RPEG_MASK_STALE_OK) && (m & RPEG_MASK_MEM_OK) && !(m & RPEG_MASK_ERROR);
   }
   static double gated(const SaEval& e) { return (e.mask & RPEG_MASK_STALE_OK) ? e.score : 0.0; }
+  // OptimizerConfig.hard_oom (evaluate.py:392, 437): a plan that does not fit scores 0
+  void hard_oom(SaEval* ev, int n) const {
+    if (!p.hard_oom) return;
+    for (int i = 0; i < n; ++i)
+      if (!(ev[i].mask & RPEG_MASK_MEM_OK)) ev[i].score = 0.0;
+  }
 
   std::vector<int16_t> fingerprint(const SaPlan& q) const {   // optimizer.py:158-172: pi, origin, mb
     std::vector<int16_t> fp;
@@ -411,6 +425,7 @@ struct SaRun {
     std::vector<SaEval> ev(plans.size());
     if (!plans.empty())
       if (int rc = be.evaluate((int)plans.size(), plans.data(), var.data(), ev.data())) return rc;
+    hard_oom(ev.data(), (int)plans.size());
     for (size_t i = 0; i < who.size(); ++i) {
       SaChain& ch = chains[who[i]];
       // a sampler failure ends the restart where the reference raises; attempts before it still count
@@ -441,6 +456,7 @@ struct SaRun {
         std::vector<SaEval> ev(p.n_chains);
         for (int c = 0; c < p.n_chains; ++c) var[c] = variant(c);
         if (int rc = be.evaluate(p.n_chains, plans.data(), var.data(), ev.data())) return rc;
+        hard_oom(ev.data(), p.n_chains);
         for (int c = 0; c < p.n_chains; ++c) {
           ++chains[c].n_eval;
           base[c].plan = *base_plan; base[c].ev = ev[c];
@@ -492,6 +508,7 @@ struct SaRun {
       first[p.n_chains] = total;
       if (total > 0)
         if (int rc = be.evaluate(total, cand.data(), var.data(), ev.data())) return rc;
+      hard_oom(ev.data(), total);
 
       // ---- best of K, one Metropolis-Hastings step, stagnation
       std::vector<int> random_who;
@@ -661,7 +678,7 @@ struct SaSerial {
         const bool stale_ok = (ev[j].mask & RPEG_MASK_STALE_OK) != 0, mem_ok = (ev[j].mask & RPEG_MASK_MEM_OK) != 0;
         Stored st;
         st.ev = ev[j];
-        st.score = gated && !stale_ok ? 0.0 : ev[j].score;
+        st.score = (gated && !stale_ok) || (p.hard_oom && !mem_ok) ? 0.0 : ev[j].score;
         st.feasible = mem_ok && (stale_ok || !gated);
         cache[key(todo[j], variant)] = st;
         eval_log.push_back(todo[j]);
@@ -706,9 +723,21 @@ struct SaSerial {
   }
 
   // `base` is a plan of family 0's template; base_variant the backend variant of the base configuration
+  // seconds on the run's clock (optimizer.py reads time.perf_counter())
+  std::chrono::steady_clock::time_point t_start = std::chrono::steady_clock::now();
+  double now() const {
+    if (p.clock) return p.clock(p.clock_ctx);
+    return std::chrono::duration<double>(std::chrono::steady_clock::now() - t_start).count();
+  }
+  bool timed_out = false;   // the run ended at its wall-clock deadline
+
   int run(const SaPlan& base, int base_variant) {
     std::vector<Stored> st;
     std::vector<char> miss;
+    const bool timed = (p.timed & 1) != 0, timed_struct = (p.timed & 3) != 0;
+    const double deadline = p.deadline_s;
+    int n_structs = 0, s_idx = 0;
+    for (const SaFamily& f : fam) n_structs += f.n_variants;
     if (int rc = evaluate(1, &base, base_variant, true, st, miss)) return rc;   // optimizer.py:466-478
     best.plan = base; best.ev = st[0].ev; best_score = eff(st[0].score, st[0].ev.util); best_variant = base_variant;
     if (st[0].feasible) {
@@ -722,6 +751,15 @@ struct SaSerial {
       const SaContext& cx = *f.cx;
       const int variant = f.first_variant + k, valid_variant = f.first_valid + k;
       const bool own_template = f.cx == fam[0].cx;
+      // the time left is split evenly among the settings still to come (optimizer.py:571-579)
+      double deadline_struct = p.deadline_struct_s;
+      if (timed) {   // two readings of the clock, as the reference takes them
+        const double left = deadline - now();
+        const int structs_left = n_structs - s_idx;
+        const double t = now();
+        deadline_struct = structs_left > 0 && left > 0.0 ? t + left / structs_left : t;
+      }
+      ++s_idx;
       SaPlan config = base;
       bool ok = false;
       if (own_template)
@@ -766,7 +804,10 @@ struct SaSerial {
         double T = r > 0 ? p.T_warm : p.T_init;
         int rej = 0;
         while (true) {
+          const double t_top = p.timed ? now() : 0.0;   // optimizer.py:703-720: deadline, budget, setting's share, setting's budget
+          if (timed && t_top >= deadline) { timed_out = true; return 0; }
           if (E >= E_max) return 0;
+          if (timed_struct && t_top >= deadline_struct) { exhausted = true; break; }
           if (E_s >= E_struct) { exhausted = true; break; }
           const double frac = std::min(1.0, T / p.T_init);
           int nc = 0;
@@ -787,7 +828,10 @@ struct SaSerial {
               const double sc = note(f, cand[i], st[i], variant);
               if (sc > bs) { bs = sc; bi = i; }
             }
+          const double t_batch = p.timed ? now() : 0.0;   // optimizer.py:848-865
+          if (timed && t_batch >= deadline) { timed_out = true; return 0; }
           if (E >= E_max) return 0;
+          if (timed_struct && t_batch >= deadline_struct) exhausted = true;
           if (E_s >= E_struct) exhausted = true;
           if (bi >= 0 && !exhausted) {
             const double delta = (bs - score_curr) / (std::fabs(score_curr) + 1e-12);
@@ -831,6 +875,8 @@ struct SaFamilySetup {
           prm->n_variants < 1 || prm->n_variants > 8)
         return "bad family parameters";
       cx[f].init(P, prm->structure);
+      cx[f].fixed_mb = prm->fixed_mb != 0;
+      cx[f].uniform_vertex = prm->uniform_vertex != 0;
       for (int v = 0; v < cx[f].nv; ++v) {
         if (prm->dir_n[v] < 0 || (prm->dir_n[v] > 0 && !prm->dir[v])) return "bad candidate directory";
         if (const char* msg = cx[f].set_directory(v, prm->dir[v], prm->dir_n[v])) return msg;
@@ -866,6 +912,8 @@ inline void sa_settings_from(const rpeg_sa_params_t& prm, SaSettings* st) {
   st->n_variants = prm.n_variants; st->T_init = prm.T_init; st->T_warm = prm.T_warm; st->T_min = prm.T_min;
   st->T_cool = prm.T_cool; st->alpha_pair = prm.alpha_pair; st->score_eps = prm.score_eps; st->seed = prm.seed;
   st->max_throughput_loss = prm.max_throughput_loss;
+  st->hard_oom = prm.hard_oom; st->timed = prm.timed; st->deadline_s = prm.deadline_s;
+  st->deadline_struct_s = prm.deadline_struct_s; st->clock = prm.clock; st->clock_ctx = prm.clock_ctx;
 }
 
 inline void sa_run_result(const SaRun& run, rpeg_sa_result_t* res) {
@@ -903,6 +951,7 @@ inline void sa_serial_result(const SaSerial& run, rpeg_sa_serial_result_t* res) 
     }
   res->best_score = feas ? run.best_feasible_score : run.best_score;
   res->best_feasible = feas;
+  res->timed_out = run.timed_out ? 1 : 0;
   res->E = run.E;
   res->n_draws = (int64_t)run.rng.k;
   res->n_uncounted = run.n_uncounted;

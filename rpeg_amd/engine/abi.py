@@ -2,7 +2,7 @@
 
 import ctypes as C
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 MAX_V, MAX_E, MAX_PUB, MAX_PAIR, MAX_REL, MAX_PH, MAX_SPLIT, MAX_MODEL, MAX_STRUCT = 6, 9, 2, 4, 13, 6, 7, 5, 3
 FIELDS = 10
 ROLE = {"GEN": 0, "INF": 1, "TRAIN": 2}
@@ -92,7 +92,13 @@ class SaParamsT(C.Structure):
                 ("T_init", C.c_double), ("T_warm", C.c_double), ("T_min", C.c_double), ("T_cool", C.c_double),
                 ("alpha_pair", C.c_double), ("score_eps", C.c_double),
                 ("seed", C.c_uint64),
-                ("dir_n", C.c_int32 * MAX_V), ("dir", C.c_void_p * MAX_V), ("max_throughput_loss", C.c_double)]
+                ("dir_n", C.c_int32 * MAX_V), ("dir", C.c_void_p * MAX_V), ("max_throughput_loss", C.c_double),
+                ("fixed_mb", C.c_int32), ("uniform_vertex", C.c_int32), ("hard_oom", C.c_int32), ("timed", C.c_int32),
+                ("deadline_s", C.c_double), ("deadline_struct_s", C.c_double), ("clock", C.c_void_p),
+                ("clock_ctx", C.c_void_p)]
+
+
+CLOCK_FN = C.CFUNCTYPE(C.c_double, C.c_void_p)   # rpeg_sa_params_t.clock
 
 
 class SaResultT(C.Structure):
@@ -107,7 +113,7 @@ class SaSerialResultT(C.Structure):
     _fields_ = [("best_plan", C.c_int16 * (MAX_V * FIELDS)), ("best_variant", C.c_int32), ("best_feasible", C.c_int32),
                 ("best_score", C.c_double), ("E", C.c_int64), ("n_draws", C.c_int64), ("n_uncounted", C.c_int64),
                 ("eval_log", C.c_void_p), ("eval_log_variant", C.c_void_p), ("eval_log_cap", C.c_int64),
-                ("n_eval_log", C.c_int64), ("wall_s", C.c_double), ("best_family", C.c_int32), ("pad", C.c_int32),
+                ("n_eval_log", C.c_int64), ("wall_s", C.c_double), ("best_family", C.c_int32), ("timed_out", C.c_int32),
                 ("eval_log_score", C.c_void_p), ("eval_log_feasible", C.c_void_p), ("eval_log_util", C.c_void_p)]
 
 

@@ -133,7 +133,7 @@ def serial_dict(res, log, logv):
                 best_family=res.best_family, n_uncounted=res.n_uncounted, n_eval_log=res.n_eval_log, eval_log=log[:n].copy(),
                 eval_log_variant=logv[:n].copy(), eval_log_score=res._stored[0][:n].copy(),
                 eval_log_feasible=res._stored[1][:n].astype(bool), eval_log_util=res._stored[2][:n].copy(),
-                wall_s=res.wall_s)
+                wall_s=res.wall_s, timed_out=bool(res.timed_out))
 
 
 def _torch():

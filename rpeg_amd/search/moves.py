@@ -34,13 +34,22 @@ def valid_dp_degrees(R: int, N: int, B: int, G: int = 1) -> List[int]:
     return [d for d in range(1, R * N * G + 1) if B % d == 0]
 
 
+# moves.py:155-158: the ablation switches.  optimize() sets them from its OptimizerConfig as the reference does
+# (optimizer.py:408-409), so that a directory built afterwards follows the same micro-batch rule as the
+# proposals drawn inside rpeg_sa_optimize*.
+ABLATION_FIXED_MB = False
+ABLATION_UNIFORM_VERTEX = False
+
+
 def valid_mb_counts(pp: int, dp: int, B: int) -> List[int]:
-    """moves.py:148-176 with the ablation switches off."""
+    """moves.py:162-199."""
     local = B // dp
     if local < MIN_B_LOCAL and dp > 1:
         return []
     if pp == 1:
         return [1]
+    if ABLATION_FIXED_MB:
+        return [1] if local % pp != 0 else [pp]
     max_mb = local // MIN_B_LOCAL
     return [mb for mb in range(pp, min(max_mb, local) + 1) if local % mb == 0]
 

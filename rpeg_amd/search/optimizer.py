@@ -138,7 +138,27 @@ def sa_params(opt: OptimizerConfig, n_chains: int, n_steps: int, variants: Seque
     p.T_init, p.T_warm, p.T_min, p.T_cool = opt.T_init, opt.T_warm, opt.T_min, opt.T_cool
     p.alpha_pair, p.score_eps, p.seed = opt.alpha_pair, opt.score_eps, seed
     p.max_throughput_loss = float(opt.max_throughput_loss)
+    p.fixed_mb, p.uniform_vertex, p.hard_oom = int(opt.fixed_mb), int(opt.uniform_vertex), int(opt.hard_oom)
     return p
+
+
+def set_deadline(params: abi.SaParamsT, opt: OptimizerConfig, clock=None):
+    """Enters OptimizerConfig.deadline / .deadline_per_struct into the parameters of rpeg_sa_optimize*.  Both
+    are readings of time.perf_counter() (optimizer.py:78-82) -- or of `clock` when one is given -- and the
+    library counts its steady clock from the start of the call, so without `clock` they go in as seconds
+    from now.  Returns what must stay alive while the call runs (the callback of `clock`)."""
+    params.timed = (1 if opt.deadline is not None else 0) | (2 if opt.deadline_per_struct is not None else 0)
+    if not params.timed:
+        return None
+    import time
+    now = 0.0 if clock is not None else time.perf_counter()
+    params.deadline_s = (opt.deadline - now) if opt.deadline is not None else 0.0
+    params.deadline_struct_s = (opt.deadline_per_struct - now) if opt.deadline_per_struct is not None else 0.0
+    if clock is None:
+        return None
+    fn = abi.CLOCK_FN(lambda _ctx: float(clock()))
+    params.clock = C.cast(fn, C.c_void_p)
+    return fn
 
 
 def plan_row(rpeg, plan: ExecutionPlan) -> np.ndarray:
@@ -236,7 +256,7 @@ def family_structures(rpeg, opt_config: OptimizerConfig) -> tuple:
 
 def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
              opt_config: OptimizerConfig, cache: Optional[EvalCache] = None, seed: int = 42,
-             stream_key: Sequence[int] = (0, 0, 0)) -> Configuration:
+             stream_key: Sequence[int] = (0, 0, 0), clock=None) -> Configuration:
     """Drop-in for optimize() (RPEG/search/optimizer.py:365-946) on the template of `base_config`.
 
     Runs the reference's loop (rpeg_sa_optimize_families): the structural families one after the other --
@@ -251,12 +271,20 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
     With `max_throughput_loss` > 0 plans are ranked by throughput x utilisation above the throughput floor
     (optimizer.py:461-486); every evaluated plan is then traced once more for its utilisation.
 
-    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused") and deadlines.  The run
-    keeps its own cache (keyed by plan, template and staleness); what it evaluated is put into `cache`
-    afterwards under the reference's keys, entries `cache` held before are not consulted."""
+    `opt_config.deadline` / `.deadline_per_struct` are readings of time.perf_counter() as in the reference
+    (optimizer.py:78-82, 571-579, 703-720, 848-865); `clock`, a callable returning seconds, takes the place of
+    perf_counter for both when given.  The ablation switches `fixed_mb`, `uniform_vertex` and `hard_oom` are
+    turned into the module switches of search.moves and search.evaluate as the reference does
+    (optimizer.py:404-410) and stay set afterwards, as there.
+
+    Not entered: the intra-stage-fusion settings (`structural_candidates` "fused").  The run keeps its own
+    cache (keyed by plan, template and staleness); what it evaluated is put into `cache` afterwards under the
+    reference's keys, entries `cache` held before are not consulted."""
     _check_supported(base_config)
-    if opt_config.deadline is not None:
-        raise NotImplementedError("deadlines are not part of this engine")
+    from . import evaluate as _eval_mod, moves as _moves_mod
+    _moves_mod.ABLATION_FIXED_MB = bool(opt_config.fixed_mb)
+    _moves_mod.ABLATION_UNIFORM_VERTEX = bool(opt_config.uniform_vertex)
+    _eval_mod.ABLATION_HARD_OOM = bool(opt_config.hard_oom)
     policy = opt_config.memory_policy()
     more = family_structures(base_config.rpeg, opt_config)
     eng, st = _engine_for(base_config.rpeg, suite, workload, hw, base_config.device_space, K_eval, policy, more,
@@ -269,10 +297,16 @@ def optimize(base_config: Configuration, suite: ModelSuite, workload: Workload, 
 
     families = optimize_families(eng.problem, opt_config, directory)
     families[0][0].seed = seed
+    keep_clock = set_deadline(families[0][0], opt_config, clock)
+    # evaluations the run can make: its budget, and per structural setting E_struct, the batch that crosses it,
+    # the setting's start plan and the restart that follows the crossing
+    n_settings = sum(f[0].n_variants for f in families)
+    log_cap = min(opt_config.E_max, n_settings * (opt_config.E_struct + 2 * opt_config.K_x + 2)) + 64
     own = [int(base_config.rpeg.tau.get(m, 0)) for m in st.tau_models]
     res = eng.sa_optimize_families(families, own, plan_row(base_config.rpeg, base_config.plan), opt_config.E_max,
                                    opt_config.E_struct, opt_config.R_max, stream_key,
-                                   log_cap=opt_config.E_max + 64 if cache is not None else 0)
+                                   log_cap=log_cap if cache is not None else 0)
+    del keep_clock
     if cache is not None:
         _carry_into(cache, eng.problem, families, res, own, suite, workload, base_config, policy,
                     opt_config.max_throughput_loss > 0.0)

@@ -4,6 +4,7 @@ optimize() over the structural families, polish() on the same cache.  Every step
 
 from __future__ import annotations
 
+import dataclasses
 import time
 from dataclasses import dataclass, field
 from typing import Dict, Optional, Sequence
@@ -44,8 +45,11 @@ class SearchResult:
 def search_plan(suite: ModelSuite, workload: Workload, hw: Hardware, device_space: DeviceSpace, K_eval: int,
                 opt_config: OptimizerConfig, algorithm: Optional[str] = None, tau: Optional[Dict[Model, int]] = None,
                 seed_plan: Optional[ExecutionPlan] = None, cache: Optional[EvalCache] = None, seed: int = 42,
-                stream_key: Sequence[int] = (0, 0, 0), no_polish: bool = False) -> SearchResult:
+                stream_key: Sequence[int] = (0, 0, 0), no_polish: bool = False,
+                time_budget: Optional[float] = None) -> SearchResult:
     """Start plans -> optimize -> polish, in the order and on the shared cache of RPEG/pipeline.py:1412-1560.
+    `time_budget` is the reference's --time (pipeline.py:1351-1366, 1542-1545): the annealing loop ends that many
+    seconds after optimize() is entered and the evaluation budget E_max is lifted; E_struct still bounds a setting.
     The start plans are built and scored on the synchronous template (staleness 0 for every model of `tau`,
     pipeline.py:1398-1410); the optimizer is seeded with the template of staleness `tau` (pipeline.py:1524-1525)."""
     algorithm = algorithm or opt_config.algorithm
@@ -68,6 +72,8 @@ def search_plan(suite: ModelSuite, workload: Workload, hw: Hardware, device_spac
     scores["start"] = evaluate_cached(start, cache, suite, workload, hw, K_eval, policy)[0]
     t2 = time.perf_counter()
     seed_config = Configuration(seed_rpeg, start.plan, device_space)
+    if time_budget is not None:
+        opt_config = dataclasses.replace(opt_config, deadline=time.perf_counter() + time_budget, E_max=10 ** 9)
     optimized = optimize(seed_config, suite, workload, hw, K_eval, opt_config, cache, seed=seed, stream_key=stream_key)
     t3 = time.perf_counter()
     scores["optimized"], _, feasible, _ = evaluate_cached(optimized, cache, suite, workload, hw, K_eval, policy)
@@ -84,7 +90,7 @@ def search_plan(suite: ModelSuite, workload: Workload, hw: Hardware, device_spac
 
 
 def search_from_config(cfg, hw_overlay: Optional[str] = None, seed_plan_file: Optional[str] = None, seed: Optional[int] = None,
-                       stream_key: Sequence[int] = (0, 0, 0)) -> SearchResult:
+                       stream_key: Sequence[int] = (0, 0, 0), time_budget: Optional[float] = None) -> SearchResult:
     """`search_plan` for a configuration in the reference's YAML schema (a path or a loaded dict), with the glue
     of RPEG/pipeline.py:1285-1404, 1431-1436, 1521-1522, 1760-1761: optional calibrated-hardware overlay, algorithm
     and AC-share permission from the policy section, optimizer settings, staleness of the seed template = the first
@@ -109,7 +115,7 @@ def search_from_config(cfg, hw_overlay: Optional[str] = None, seed_plan_file: Op
     seed_plan = load_plan(seed_plan_file, _template(algorithm, suite, workload, tau)) if seed_plan_file else None
     res = search_plan(suite, workload, hw, device_space, o["k_eval"], optim, algorithm=algorithm, tau=tau,
                       seed_plan=seed_plan, seed=seed if seed is not None else out.get("seed") or 42,
-                      stream_key=stream_key, no_polish=optim.no_polish)
+                      stream_key=stream_key, no_polish=optim.no_polish, time_budget=time_budget)
     if out.get("base_plan"):
         save_plan(res.start, out["base_plan"])
     if out.get("opt_plan"):

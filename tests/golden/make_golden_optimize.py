@@ -62,6 +62,31 @@ CASES = [dict(plan=0, stream=(42, 77, 0, 0), E_max=260, E_struct=200, stag_windo
               transfer=["destination_only", "both_endpoints"])]
 
 
+# the ablation switches of OptimizerConfig (optimizer.py:83-88, 404-410) and its wall-clock deadline (:78-82,
+# 571-579, 703-720, 848-865).  Stored under "flag_cases".  A deadline case runs on a clock that advances by one
+# second at every reading (time.perf_counter is replaced while optimize() runs): `deadline` is a reading of it.
+FLAG_CASES = [
+    dict(plan=0, stream=(42, 78, 0, 0), E_max=200, E_struct=200, stag_window=4, T_init=0.05, T_min=0.05, T_warm=0.10,
+         fixed_mb=True),
+    dict(plan=2, stream=(42, 78, 1, 0), E_max=200, E_struct=200, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
+         uniform_vertex=True),
+    dict(plan=0, stream=(42, 78, 2, 0), E_max=360, E_struct=70, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
+         families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05, memory_per_gpu=1.25e10,
+         hard_oom=True),
+    dict(plan=2, stream=(42, 78, 3, 0), E_max=200, E_struct=200, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
+         fixed_mb=True, uniform_vertex=True, hard_oom=True),
+    # deadlines: one setting (ends on the deadline), several settings (each ends on its share, the last on the
+    # deadline), a deadline behind the budget (E_max ends the run), one already past at the start
+    dict(plan=0, stream=(42, 78, 4, 0), E_max=10 ** 9, E_struct=400, stag_window=4, T_init=0.05, T_min=0.05, T_warm=0.10,
+         deadline=61.0),
+    dict(plan=0, stream=(42, 78, 5, 0), E_max=10 ** 9, E_struct=70, stag_window=3, T_init=0.05, T_min=0.05, T_warm=0.10,
+         families=True, T_cand=[[0, 1], [0, 1], [0, 1]], base_tau=[0, 0], lambda_ac=0.05, deadline=150.0),
+    dict(plan=2, stream=(42, 78, 6, 0), E_max=90, E_struct=60, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
+         families=True, T_cand=[[0, 1], [0], [1, 0]], base_tau=[1, 0], lambda_ac=0.0, deadline=1000.0),
+    dict(plan=0, stream=(42, 78, 7, 0), E_max=200, E_struct=200, stag_window=4, T_init=0.05, T_min=0.05, T_warm=0.10,
+         deadline=0.0)]
+
+
 PIPELINE = dict(stream=(42, 77, 6, 0), E_max=300, E_struct=60, stag_window=3, T_init=0.30, T_min=0.03, T_warm=0.05,
                 lambda_ac=0.05)
 
@@ -161,6 +186,11 @@ def main():
         return st["mms"][key]
 
     def _eval(config, gate):
+        out = _eval_inner(config, gate)
+        st.setdefault("scores", []).append(out[0])
+        return out
+
+    def _eval_inner(config, gate):
         p = st["problem"]
         rpeg, plan, wl = config.rpeg, config.plan, st["wl"]
         if st["families"]:
@@ -179,6 +209,8 @@ def main():
         violation = mods["model.memory"].mem_worst_violation(lowered, memory_model(rpeg))
         if violation is None:
             return raw, trace, True
+        if getattr(stub, "ABLATION_HARD_OOM", False):   # evaluate.py:392, 437; optimize() sets it on this module (:410)
+            return 0.0, trace, False
         _, req, cap = violation
         return raw * max(math.exp(-40.0 * max(0.0, req / cap - 1.0)), 1e-12), trace, False
 
@@ -231,7 +263,22 @@ def main():
     def policy_of(case):
         return ct.TransferResourcePolicy(*case["transfer"]) if "transfer" in case else None
 
-    for case in CASES:
+    def ticking_clock():
+        t = [0.0]
+
+        def read():
+            t[0] += 1.0
+            return t[0]
+        return read
+
+    import time
+    for case in CASES + FLAG_CASES:
+        flagged = case in FLAG_CASES
+        if flagged and "flag_cases" not in doc:   # the pipeline case runs between the two lists, as it always has
+            doc["pipeline"] = pipeline_case(args.ref, mods, moves, ropt, rcache, Configuration, st, ct, p_config, rows)
+            doc["flag_cases"] = []
+            st.update(problem=p, suite=suite, wl=wl, hw=hw, space=space, cost=cost, mm=mm, mms={}, log=[])
+        extra = {k: case[k] for k in ("fixed_mb", "uniform_vertex", "hard_oom", "deadline") if k in case}
         if p is not p_config or "memory_per_gpu" in case:
             p = dataclasses.replace(p_config, hw=dataclasses.replace(
                 p_config.hw, memory_per_gpu=case.get("memory_per_gpu", p_config.hw.memory_per_gpu)))
@@ -248,35 +295,44 @@ def main():
                                       structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"],
                                       max_throughput_loss=case.get("max_throughput_loss", 0.0),
                                       T_init=case["T_init"], T_warm=case["T_warm"], T_min=case["T_min"],
-                                      stag_window=case["stag_window"])
+                                      stag_window=case["stag_window"], **extra)
         else:
             base = Configuration(rpeg0, plan, space, transfer_resource_policy=policy_of(case))
             assert is_valid(base, suite, wl, mm), "the base plan must be valid"
             oc = ropt.OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"],
                                       T_cand={Model.ACTOR: {0}, Model.CRITIC: {0}, Model.AC_SHARE: set()},
                                       structural_candidates=frozenset({"separate"}), T_init=case["T_init"],
-                                      T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"])
+                                      T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"], **extra)
         rng = CounterRng(*case["stream"])
         ropt.random = rng
         moves.random = rng
-        st["log"] = []
+        st["log"], st["scores"] = [], []
         os.cpu_count = lambda: 1
+        real_clock = time.perf_counter
+        if "deadline" in case:
+            time.perf_counter = ticking_clock()
         try:
             out = ropt.optimize(base, suite, wl, hw, p.K_eval, oc, rcache.EvalCache())
         finally:
             os.cpu_count = real_cpu_count
+            clock_reads = int(time.perf_counter()) - 1 if "deadline" in case else 0
+            time.perf_counter = real_clock
         log = st["log"]
-        doc["cases"].append(dict(case, stream=list(case["stream"]), T_cool=oc.T_cool.hex(), n_eval=len(log),
+        where = doc["flag_cases"] if flagged else doc["cases"]
+        if flagged:
+            case = dict(case, clock_reads=clock_reads, eval_scores_crc=zlib.crc32(
+                json.dumps([float(x).hex() for x in st["scores"]]).encode()))
+        where.append(dict(case, stream=list(case["stream"]), T_cool=oc.T_cool.hex(), n_eval=len(log),
                                  n_draws=rng.k, eval_crc=zlib.crc32(json.dumps(log, separators=(",", ":")).encode()),
                                  first=log[:8], final=rows(out), final_first_vertex=out.rpeg.vertices[0].id,
                                  final_tau=[out.rpeg.tau[m] for m in sorted(out.rpeg.tau, key=lambda m: m.value)]))
         if st["families"]:
             import collections
-            doc["cases"][-1]["per_setting"] = [[k[0], list(k[1]), n] for k, n in collections.Counter(
+            where[-1]["per_setting"] = [[k[0], list(k[1]), n] for k, n in collections.Counter(
                 (e[0], tuple(e[1])) for e in log).items()]
-        print("case", case["plan"], "evaluations", len(log), "draws", rng.k, doc["cases"][-1].get("per_setting", ""),
-              "->", doc["cases"][-1]["final_first_vertex"], doc["cases"][-1]["final_tau"])
-    doc["pipeline"] = pipeline_case(args.ref, mods, moves, ropt, rcache, Configuration, st, ct, p_config, rows)
+        print("case", case["plan"], extra, "evaluations", len(log), "draws", rng.k, where[-1].get("per_setting", ""),
+              "->", where[-1]["final_first_vertex"], where[-1]["final_tau"], flush=True)
+    moves.ABLATION_FIXED_MB = moves.ABLATION_UNIFORM_VERTEX = stub.ABLATION_HARD_OOM = False
     path = os.path.join(HERE, "ref_optimize.json")
     with open(path, "w") as f:
         json.dump(doc, f, separators=(",", ":"))

@@ -10,7 +10,8 @@ lies, compiles the text up to the line `def _eval_worker(` as the module `search
 into this repository, nothing else is altered) and records what the reference's own
 
     is_compatible, allocations_overlap, stale_publication_layout_valid, is_valid,
-    evaluation_cache_key, evaluate_cached (score, feasibility: the penalty arithmetic of :388-401)
+    evaluation_cache_key, evaluate_cached (score, feasibility: the penalty arithmetic of :388-401, and the score
+    under ABLATION_HARD_OOM for the plans that do not fit)
 
 return for seeded plans of all five configurations (every template: PPO, GRPO, DPO and AC-share) and for the
 same plans broken one rule at a time.  Inputs are regenerated from the seed by the tests through
@@ -147,6 +148,13 @@ def main():
                 try:
                     score, _, feasible, miss = ev.evaluate_cached(config, EvalCache(), suite, wl, hw, p.K_eval, pol)
                     row.update(score=float(score).hex(), feasible=bool(feasible), miss=bool(miss))
+                    if not feasible:   # the hard-OOM switch (evaluate.py:297-298, 392) on the reference's own function
+                        ev.ABLATION_HARD_OOM = True
+                        try:
+                            hard = ev.evaluate_cached(config, EvalCache(), suite, wl, hw, p.K_eval, pol)
+                        finally:
+                            ev.ABLATION_HARD_OOM = False
+                        row.update(score_hard_oom=float(hard[0]).hex(), feasible_hard_oom=bool(hard[2]))
                 except (ZeroDivisionError, KeyError, ValueError) as e:
                     row.update(raises=type(e).__name__)
             rows.append(row)

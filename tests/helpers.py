@@ -50,7 +50,7 @@ def family_problem(case=None, c=1):
     return dataclasses.replace(p, structures=(ppo, ac, as_seen_from(ac, ppo)))
 
 
-def family_case_setup(p, case, directory_of):
+def family_case_setup(p, case, directory_of, **more):
     """(families, base row, OptimizerConfig) of one family case of tests/golden/ref_optimize.json."""
     from rpeg_amd.core.types import Model
     from rpeg_amd.ir.plan import ExecutionPlan
@@ -66,7 +66,7 @@ def family_case_setup(p, case, directory_of):
                           T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"],
                           T_cand={Model.ACTOR: set(a), Model.CRITIC: set(c_), Model.AC_SHARE: set(s_)},
                           structural_candidates=frozenset({"separate", "ac_share"}), lambda_ac=case["lambda_ac"],
-                          max_throughput_loss=case.get("max_throughput_loss", 0.0))
+                          max_throughput_loss=case.get("max_throughput_loss", 0.0), **more)
     assert opt.T_cool.hex() == case["T_cool"]
     families = optimize_families(p, opt, directory_of)
     families[0][0].seed = case["stream"][0]

@@ -455,13 +455,14 @@ def test_gates_equal_reference_verdicts(c):
     import os
     from rpeg_amd.model.memory import NodeMemoryModel
     from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search import evaluate as evaluate_mod
     from rpeg_amd.search.evaluate import Configuration, evaluate_cached, is_valid
     from tests.golden.make_golden_validity import validity_cases
     with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_validity.json")) as f:
         rows = json.load(f)["configs"][str(c)]
     cfg, batch, cases = validity_cases(c)
     p = cfg.problem
-    n_valid = n_scored = 0
+    n_valid = n_scored = n_hard = 0
     for want, (i, rule, rpeg, plan, wl) in zip(rows, cases):
         config = Configuration(rpeg, plan, p.device_space)
         mm = NodeMemoryModel.from_policy(p.hw, p.suite, wl, p.memory_policy, trainable=frozenset(rpeg.trainable))
@@ -471,7 +472,15 @@ def test_gates_equal_reference_verdicts(c):
             score, _, feasible, miss = evaluate_cached(config, EvalCache(), p.suite, wl, p.hw, p.K_eval, p.memory_policy)
             assert float(score).hex() == want["score"] and feasible == want["feasible"] and miss, (i, rule)
             n_scored += 1
-    assert n_valid and n_scored
+            if "score_hard_oom" in want:     # the hard-OOM switch, as the reference's evaluate_cached applies it
+                evaluate_mod.ABLATION_HARD_OOM = True
+                try:
+                    hard = evaluate_cached(config, EvalCache(), p.suite, wl, p.hw, p.K_eval, p.memory_policy)
+                finally:
+                    evaluate_mod.ABLATION_HARD_OOM = False
+                assert float(hard[0]).hex() == want["score_hard_oom"] and hard[2] == want["feasible_hard_oom"], (i, rule)
+                n_hard += 1
+    assert n_valid and n_scored and n_hard
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])

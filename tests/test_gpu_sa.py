@@ -444,3 +444,123 @@ def test_planner_sequence_of_the_runtime_under_a_transfer_policy():
     assert doc["horizon"] == horizon and doc["predicted_makespan_s"] == want["makespan"]
     assert [n["node_id"] for n in doc["nodes"]] == list(want["order"])
     assert [n["predicted_finish_s"] for n in doc["nodes"]] == [want["finish"][i] for i in want["order"]]
+
+
+@pytest.mark.parametrize("k", range(8))
+def test_optimize_ablations_and_deadlines_equal_reference(k):
+    """OptimizerConfig's ablation switches and wall-clock deadline on the GPU evaluator, through
+    rpeg_sa_optimize / rpeg_sa_optimize_families and through the drop-in optimize(), against the reference's own
+    optimize() run with the same switches, generator and ticking clock (the flag cases of
+    tests/golden/make_golden_optimize.py): every evaluated plan and its score in order, the draws, the number
+    of clock readings, the returned configuration."""
+    import ctypes as C
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.search import evaluate as evaluate_mod, moves as moves_mod
+    from rpeg_amd.search.cache import EvalCache
+    from rpeg_amd.search.evaluate import Configuration
+    from rpeg_amd.search.optimizer import optimize, plan_row, row_plan
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        case = json.load(f)["flag_cases"][k]
+    flags = {name: bool(case.get(name)) for name in ("fixed_mb", "uniform_vertex", "hard_oom")}
+
+    class Ticking:
+        def __init__(self):
+            self.reads = 0
+            self.fn = abi.CLOCK_FN(lambda _ctx: self())
+
+        def __call__(self):
+            self.reads += 1
+            return float(self.reads)
+
+    def timed(params, clock):
+        if "deadline" in case:
+            params.timed, params.deadline_s, params.clock = 1, case["deadline"], C.cast(clock.fn, C.c_void_p)
+
+    p = family_problem(case) if case.get("families") else configs.config(1).problem
+    eng = Engine(p)
+    moves_mod.ABLATION_FIXED_MB = flags["fixed_mb"]
+    try:
+        def directory_of(structure):
+            rpeg = p.template(structure, ())
+            return directory_arrays(rpeg, build_candidate_directory(rpeg, p.suite, p.device_space, p.workload, eng,
+                                                                    structure)[0])
+        clock = Ticking()
+        if case.get("families"):
+            families, row, opt = family_case_setup(p, case, directory_of, **flags)
+            timed(families[0][0], clock)
+            res = eng.sa_optimize_families(families, case["base_tau"], row, case["E_max"], case["E_struct"],
+                                           stream_key=case["stream"][1:], log_cap=4096)
+            check_family_case(p, case, families, res)
+            base_tau = case["base_tau"]
+        else:
+            _, batch = seeded_batch(1, 8)
+            rpeg0 = p.template(0, ())
+            nv = len(rpeg0.vertices)
+            _, plan_m, _ = batch.configuration(p, case["plan"])
+            by_id = {v.id: v for v in rpeg0.vertices}
+            from rpeg_amd.ir.plan import ExecutionPlan
+            row = plan_row(rpeg0, ExecutionPlan(sigma={by_id[v.id]: a for v, a in plan_m.sigma.items()},
+                                                pi={by_id[v.id]: x for v, x in plan_m.pi.items()},
+                                                mb={by_id[v.id]: x for v, x in plan_m.mb.items()}))
+            opt = OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"], T_init=case["T_init"],
+                                  T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"],
+                                  T_cand={m: {0} for m in rpeg0.tau}, structural_candidates=frozenset({"separate"}), **flags)
+            params = sa_params(opt, 1, 1, [(0, 0)], 0, 1, case["stream"][0])
+            timed(params, clock)
+            res = eng.sa_optimize(params, directory_of(0), row, case["E_max"], case["E_struct"],
+                                  stream_key=case["stream"][1:], log_cap=4096)
+            log = [[[int(x) for x in r[v * 10:(v + 1) * 10]] for v in range(nv)] for r in res["eval_log"]]
+            assert log[:8] == case["first"] and res["n_eval_log"] == case["n_eval"] == len(log)
+            assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
+            assert res["n_draws"] == case["n_draws"]
+            base_tau = [0, 0]
+        scores = [float(x).hex() for x in res["eval_log_score"]]
+        assert zlib.crc32(json.dumps(scores).encode()) == case["eval_scores_crc"]
+        assert clock.reads == case["clock_reads"]
+        assert res["timed_out"] == ("deadline" in case and case["n_eval"] < case["E_max"])
+
+        # the drop-in: switches and deadline from the OptimizerConfig, the clock in perf_counter's place
+        import dataclasses
+        clock = Ticking()
+        moves_mod.ABLATION_FIXED_MB = False
+        base_rpeg = p.template(0, base_tau)
+        base = Configuration(base_rpeg, row_plan(base_rpeg, row), p.device_space)
+        out = optimize(base, p.suite, p.workload, p.hw, p.K_eval, dataclasses.replace(opt, deadline=case.get("deadline")),
+                       EvalCache(), seed=case["stream"][0], stream_key=case["stream"][1:],
+                       clock=clock if "deadline" in case else None)
+        assert (moves_mod.ABLATION_FIXED_MB, moves_mod.ABLATION_UNIFORM_VERTEX, evaluate_mod.ABLATION_HARD_OOM) == \
+            (flags["fixed_mb"], flags["uniform_vertex"], flags["hard_oom"])       # optimizer.py:408-410
+        assert out.rpeg.vertices[0].id == case["final_first_vertex"]
+        assert [out.rpeg.tau[m] for m in sorted(out.rpeg.tau, key=lambda m: m.value)] == case["final_tau"]
+        got = plan_row(out.rpeg, out.plan)
+        assert [[int(x) for x in got[v * 10:(v + 1) * 10]] for v in range(len(out.rpeg.vertices))] == case["final"]
+        assert clock.reads == case["clock_reads"]
+    finally:
+        moves_mod.ABLATION_FIXED_MB = moves_mod.ABLATION_UNIFORM_VERTEX = False
+        evaluate_mod.ABLATION_HARD_OOM = False
+        eng.close()
+
+
+def test_time_budget_ends_the_search_on_the_wall_clock():
+    """--time of the reference's pipeline (RPEG/pipeline.py:1351-1366, 1542-1545) on the real clock: with the
+    evaluation budget lifted, a budget of a fraction of a second ends optimize() shortly after it (one batch of
+    K_x evaluations may be under way), a budget of zero leaves the start plan, and more time never gives a
+    worse plan on the same generator."""
+    import time
+    from rpeg_amd.search.pipeline import search_plan
+    p = configs.config(1).problem
+    opt = OptimizerConfig(K_x=6, T_max=50, E_max=100, E_struct=10 ** 6, structural_candidates=frozenset({"separate"}),
+                          T_cand={m: {0} for m in p.template(0, ()).tau})
+    search_plan(p.suite, p.workload, p.hw, p.device_space, p.K_eval, opt, algorithm="ppo", no_polish=True)   # warm-up
+    got = {}
+    for budget in (0.0, 0.05, 0.4):
+        t0 = time.perf_counter()
+        res = search_plan(p.suite, p.workload, p.hw, p.device_space, p.K_eval, opt, algorithm="ppo", no_polish=True,
+                          time_budget=budget)
+        got[budget] = res
+        # (optimize() also enters what the run evaluated into the shared cache afterwards: host work per evaluation)
+        assert budget <= res.seconds["optimize"] < budget + 0.1 + 2e-3 * res.cache.misses, (budget, res.seconds)
+        assert time.perf_counter() - t0 < budget + 5.0
+    assert got[0.0].scores["optimized"] == got[0.0].scores["start"]
+    assert got[0.0].scores["optimized"] <= got[0.05].scores["optimized"] <= got[0.4].scores["optimized"]
+    assert got[0.4].cache.misses > got[0.05].cache.misses > got[0.0].cache.misses

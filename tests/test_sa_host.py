@@ -8,6 +8,7 @@ scheduler code, run through the CPU build of the kernels' headers:
   trajectories, step by step.
 """
 
+import ctypes as C
 import json
 import os
 
@@ -246,3 +247,92 @@ def test_cxx_optimize_over_structural_families_matches_reference_optimize():
     res = port.sa_optimize_families(families, case["base_tau"], row, case["E_max"], case["E_struct"],
                                     stream_key=case["stream"][1:], log_cap=4096, threads=4)
     assert res["n_draws"] != case["n_draws"]
+
+
+class _TickingClock:
+    """A clock that advances by one second at every reading, as the one the deadline cases of
+    tests/golden/make_golden_optimize.py put in perf_counter's place."""
+
+    def __init__(self):
+        self.reads = 0
+        self.fn = abi.CLOCK_FN(self._read)
+
+    def _read(self, _ctx):
+        self.reads += 1
+        return float(self.reads)
+
+    def install(self, params, deadline):
+        params.timed, params.deadline_s = 1, float(deadline)
+        params.clock = C.cast(self.fn, C.c_void_p)
+
+
+def flag_cases():
+    with open(os.path.join(GOLDEN, "ref_optimize.json")) as f:
+        return json.load(f)["flag_cases"]
+
+
+def flag_config(case, **kw):
+    return OptimizerConfig(K_x=6, T_max=50, E_max=case["E_max"], E_struct=case["E_struct"], T_init=case["T_init"],
+                           T_warm=case["T_warm"], T_min=case["T_min"], stag_window=case["stag_window"],
+                           fixed_mb=case.get("fixed_mb", False), uniform_vertex=case.get("uniform_vertex", False),
+                           hard_oom=case.get("hard_oom", False), **kw)
+
+
+def check_flag_case_scores(case, res):
+    import zlib
+    got = [float(x).hex() for x in res["eval_log_score"]]
+    assert zlib.crc32(json.dumps(got).encode()) == case["eval_scores_crc"]
+
+
+@pytest.mark.parametrize("k", range(8))
+def test_cxx_optimize_ablations_and_deadlines_match_reference_optimize(k):
+    """OptimizerConfig's ablation switches (fixed_mb, uniform_vertex, hard_oom; RPEG/search/optimizer.py:404-410,
+    moves.py:182-188, 688, evaluate.py:392, 437) and its wall-clock deadline (optimizer.py:571-579, 703-720,
+    848-865) in the shipped loop, against the reference's own optimize() run with the same switches on the same
+    generator and -- for the deadlines -- the same ticking clock: same plans in the same order, same scores,
+    same number of draws and of clock readings, same returned configuration."""
+    import zlib
+    case = flag_cases()[k]
+    S.ABLATION_FIXED_MB = bool(case.get("fixed_mb"))
+    try:
+        clock = _TickingClock()
+        if case.get("families"):
+            p = family_problem(case)
+            port = CpuPort(p)
+            families, row, opt = family_case_setup(p, case, lambda s: _directory(p, p.template(s, ()))[2],
+                                                   fixed_mb=case.get("fixed_mb", False), hard_oom=case.get("hard_oom", False),
+                                                   uniform_vertex=case.get("uniform_vertex", False))
+            if "deadline" in case:
+                clock.install(families[0][0], case["deadline"])
+            res = port.sa_optimize_families(families, case["base_tau"], row, case["E_max"], case["E_struct"],
+                                            stream_key=case["stream"][1:], log_cap=4096, threads=4)
+            check_family_case(p, case, families, res)
+        else:
+            cfg, batch = seeded_batch(1, 8)
+            p = cfg.problem
+            rpeg0 = p.template(0, ())
+            nv = len(rpeg0.vertices)
+            port = CpuPort(p)
+            _, plan_m, _ = batch.configuration(p, case["plan"])
+            row = plan_row(rpeg0, ExecutionPlan(sigma={v: plan_m.sigma[u] for v, u in zip(rpeg0.vertices, plan_m.sigma)},
+                                                pi={v: plan_m.pi[u] for v, u in zip(rpeg0.vertices, plan_m.pi)},
+                                                mb={v: plan_m.mb[u] for v, u in zip(rpeg0.vertices, plan_m.mb)}))
+            opt = flag_config(case)
+            assert opt.T_cool.hex() == case["T_cool"]
+            params = sa_params(opt, 1, 1, [(0, 0)], 0, 1, case["stream"][0])
+            if "deadline" in case:
+                clock.install(params, case["deadline"])
+            res = port.sa_optimize(params, _directory(p, rpeg0)[2], row, case["E_max"], case["E_struct"],
+                                   stream_key=case["stream"][1:], log_cap=4096, threads=4)
+            log = [_rows6(r, nv) for r in res["eval_log"]]
+            assert log[:8] == case["first"]
+            assert res["n_eval_log"] == case["n_eval"] == len(log)
+            assert zlib.crc32(json.dumps(log, separators=(",", ":")).encode()) == case["eval_crc"]
+            assert res["n_draws"] == case["n_draws"]
+            assert _rows6(res["best_plan"], nv) == case["final"]
+    finally:
+        S.ABLATION_FIXED_MB = False
+    check_flag_case_scores(case, res)
+    assert clock.reads == case["clock_reads"]
+    # the run ended on its deadline exactly when the deadline, not the budget, is what stopped the reference
+    assert res["timed_out"] == ("deadline" in case and case["n_eval"] < case["E_max"])
