@@ -44,8 +44,12 @@ enum {
   RPEG_MASK_VALID = 1,     /* integer validity rules of is_valid (evaluate.py:172-196) hold   */
   RPEG_MASK_STALE_OK = 2,  /* stale_publication_layout_valid (evaluate.py:115-140)            */
   RPEG_MASK_MEM_OK = 4,    /* no device peak above capacity (memory.py:864-887)               */
-  RPEG_MASK_ERROR = 8      /* the reference would raise (division by zero, cycle) or an engine
+  RPEG_MASK_ERROR = 8,     /* the reference would raise (division by zero, cycle) or an engine
                               limit was hit; the numeric outputs of this plan are NaN           */
+  RPEG_MASK_LIMIT = 16     /* set with RPEG_MASK_ERROR when the cause is a limit of this engine
+                              (more than 31 ready nodes at once, a node that reserves more than
+                              two vertex allocations, more than 2^23 heap pushes): the reference
+                              would have evaluated the plan                                      */
 };
 
 /* eval flags */
@@ -375,6 +379,13 @@ int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
    up to 384 nodes).  lanes = -1 (default): chosen per batch from its size.
    Results do not depend on the setting. */
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
+
+/* Ready-list entries per plan in the main kernel: 8, 16, 24 or 32 (default).  A plan with that many nodes
+   ready at once is not evaluated: NaN outputs, RPEG_MASK_ERROR | RPEG_MASK_LIMIT (the reference's heap has no
+   such bound; the longest list seen on the shipped problems is 24).  Fewer entries take less LDS per wavefront.
+   The kernel that runs one plan per wavefront (small batches) keeps its ready set in registers and has no
+   such bound.  No reference counterpart: tests use it to reach the limit. */
+int rpeg_engine_set_ready_cap(rpeg_engine_t* e, int32_t entries);
 
 /* Forgets every lowered class, so that the next rpeg_eval_batch lowers all the classes of its batch
    again (used to measure a cold call). */

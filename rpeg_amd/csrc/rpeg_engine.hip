@@ -420,6 +420,7 @@ struct rpeg_engine_s {
   // kernel, read back with the class counts of the next call); plans that outgrow it are flagged and redone
   // with the full capacity by a second launch.
   uint8_t* d_ovf = nullptr;
+  uint32_t ready_cap = 32;      // ready-list entries per plan in the main kernel (rpeg_engine_set_ready_cap)
   uint32_t* d_need = nullptr;
   uint32_t need = 0;
   uint32_t max_v = RPEG_MAX_V;   // largest vertex count of the problem's structures
@@ -452,6 +453,8 @@ static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (!e->d_need) {
     HIP_TRY(e, hipMalloc(&e->d_need, (KE_NEED_SHARDS + 1) * 4));
     HIP_TRY(e, hipMemset(e->d_need, 0, (KE_NEED_SHARDS + 1) * 4));
+  } else {
+    HIP_TRY(e, hipMemset(e->d_need + KE_NEED_SHARDS, 0, 4));   // the count of flagged plans belongs to the flags just replaced
   }
   HIP_TRY(e, hipMalloc(&e->d_sig, cap * 8));
   HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
@@ -730,6 +733,16 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
   return 0;
 }
 
+int rpeg_engine_set_ready_cap(rpeg_engine_t* e, int32_t entries) {
+  if (!e) return -1;
+  if (entries != 8 && entries != 16 && entries != 24 && entries != 32) {
+    e->err = "the ready-list capacity must be 8, 16, 24 or 32";
+    return -1;
+  }
+  e->ready_cap = (uint32_t)entries;
+  return 0;
+}
+
 int rpeg_engine_reset_classes(rpeg_engine_t* e) {
   if (!e) return -1;
   hipDeviceSynchronize();
@@ -964,7 +977,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // lists of a full wavefront do
   // Ready-list capacity: the full 32 entries until the longest list of earlier launches is known, then a
   // short list (less LDS, more wavefronts per compute unit); plans that outgrow it are redone below.
-  const uint32_t rcap_full = 32;
+  const uint32_t rcap_full = e->ready_cap;
   const bool short_list = !ls && !one && e->need > 0 && ((e->need + 2 + 7) & ~7u) < rcap_full;
   const uint32_t rcap = short_list ? std::max(8u, (e->need + 2 + 7) & ~7u) : rcap_full;
   const bool few_in_lds = !ls && !one &&
@@ -1003,7 +1016,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (e->max_nodes > 4095) { e->err = "class with more than 4095 nodes"; return -8; }
   L.rcap = rcap;
   L.max_v = e->max_v;
-  L.ovf = !ls && !one ? e->d_ovf : nullptr;
+  // Overflow flags are written only by a launch that a fix-up launch follows (the short list): with the full list
+  // an overflow is final (RPEG_MASK_LIMIT), and a flag left standing would be redone by a later call's fix-up.
+  L.ovf = short_list ? e->d_ovf : nullptr;
   L.need = !ls && !one ? e->d_need : nullptr;
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
@@ -1179,6 +1194,10 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   int64_t off = class_offset(e, sg, nullptr);
   if (off < 0) return -5;
   hipStream_t s = nullptr;
+  // This call works on the null stream and reuses the engine's task, lane and state buffers.  A batched call
+  // returns without waiting for its stream, and a stream created as non-blocking does not order itself against
+  // the null stream: wait for everything the device still runs before those buffers are written.
+  HIP_TRY(e, hipDeviceSynchronize());
   if (int rc = ensure_pool(e, s)) return rc;
   if (int rc = ensure_perm(e, WAVE, 1)) return rc;
   if (int rc = ensure_ws(e, wave_ws_bytes(e->max_nodes, e->max_slots), s)) return rc;

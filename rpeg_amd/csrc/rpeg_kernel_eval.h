@@ -318,7 +318,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
 #pragma unroll
   for (int x = 0; x < RPEG_MAX_V; ++x) lf[x] = 0.0;
   int n_ready = 0, done = 0, max_ready = 0;
-  bool ovf = false;
+  bool ovf = false, limit = false;
   const int rcap = (int)L.rcap;   // a multiple of eight
   const double inf = __builtin_inf();
   constexpr uint32_t SAME = 1u << 22;
@@ -331,7 +331,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     const unsigned x = (unsigned)__builtin_ctz(blk | 0x100u);
     const unsigned rest = blk & (blk - 1u);
     const unsigned y = rest ? (unsigned)__builtin_ctz(rest) : x;
-    if (rest & (rest - 1u)) err = true;   // more than two reserved vertices cannot be packed
+    if (rest & (rest - 1u)) err = limit = true;   // more than two reserved vertices cannot be packed
     return (uint32_t)v | ((uint32_t)r.ptkey << 12) | (x << 16) | (y << 19);
   };
   // Up to NQ pushes at once, with the result of pushing them one after the other: a stable merge in
@@ -592,6 +592,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   if (err || makespan == 0.0) {
     out_makespan = out_score = __builtin_nan("");
     mask |= RPEG_MASK_ERROR;
+    if (ovf || limit) mask |= RPEG_MASK_LIMIT;
   } else {
     double score = P.score_num / makespan;
     if (!mem_ok) score = score * oom_penalty(peak, P.cap);

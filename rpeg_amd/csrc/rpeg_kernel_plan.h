@@ -87,9 +87,9 @@ __device__ inline bool kp_is_inf(double v) {   // on the bits, so that a uniform
 
 // Ranks, tie-break classes and the list scheduler for a class of at most 64 * NS nodes.  l_rank holds the
 // ranks while they are computed and the finish times afterwards; nd is the index of the neutral element.
-// Returns false on a broken class (cycle).
+// Returns 0, 1 on a broken class (cycle), 2 when the push counter outgrew its field (a limit of this kernel).
 template <int NS>
-__device__ inline bool kp_schedule(const ClassView& cv, const int n, const int lane, const uint64_t ovl,
+__device__ inline int kp_schedule(const ClassView& cv, const int n, const int lane, const uint64_t ovl,
                                    const uint64_t dpne, const int nd, const double* l_dur, double* l_rank,
                                    double* l_start, uint8_t* l_pt, const bool keep_trace, double* out_makespan,
                                    long* out_pops, unsigned long long* stamp) {
@@ -406,11 +406,11 @@ __device__ inline bool kp_schedule(const ClassView& cv, const int n, const int l
       ++ctr;
     }
   }
-  if (ctr > KP_TIE_MASK) ok = false;
   if (done != n) ok = false;
   *out_makespan = makespan;
   *out_pops = (slow_decisions << 20) | pops;
-  return ok;
+  if (ctr > KP_TIE_MASK) return 2;   // the push counter outgrew its field of the packed order: a limit of this kernel
+  return ok ? 0 : 1;
 }
 
 // Pair relations and vertex sets of one plan by POSITION in the order of first appearance (bit 8i+j of a
@@ -527,7 +527,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   KE_STAMP(1);
 
   // ---- durations of the class's slots, one slot per lane
-  bool err = cv.h->error != 0, zero_div = false;
+  bool err = cv.h->error != 0, zero_div = false, limit = false;
   const int split = (int)cv.h->split;
   for (int s = lane; s < n_slots; s += KE_WAVE) l_dur[s] = ke_slot_duration<1>(P, st, split, cv.slot[s], l_plan, &zero_div);
   err = err || __ballot(zero_div) != 0ull;
@@ -587,14 +587,15 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   double makespan = 0.0;
   long pops = 0;
   if (!err) {
-    bool ok;
+    int ok;
     if (n <= 64) ok = kp_schedule<1>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
     else if (n <= 128) ok = kp_schedule<2>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
     else if (n <= 192) ok = kp_schedule<3>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
     else if (n <= 256) ok = kp_schedule<4>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
     else if (n <= 320) ok = kp_schedule<5>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
     else ok = kp_schedule<6>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
-    err = !ok;
+    err = ok != 0;
+    limit = ok == 2;
   }
   KE_STAMP(5);
   if (L.prof && lane == 0) L.prof[w * 8 + 7] = ((unsigned long long)n << 32) | (unsigned long long)pops;
@@ -607,6 +608,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   if (err || makespan == 0.0) {
     out_makespan = out_score = __builtin_nan("");
     mask |= RPEG_MASK_ERROR;
+    if (limit) mask |= RPEG_MASK_LIMIT;
   } else {
     double score = P.score_num / makespan;
     if (!mem_ok) score = score * oom_penalty(peak, P.cap);

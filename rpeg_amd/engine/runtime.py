@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
            "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static")
 
 
@@ -75,6 +75,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_last_kernel_ms.argtypes = [vp]
     lib.rpeg_engine_set_state_lanes.restype = C.c_int
     lib.rpeg_engine_set_state_lanes.argtypes = [vp, i32]
+    lib.rpeg_engine_set_ready_cap.restype = C.c_int
+    lib.rpeg_engine_set_ready_cap.argtypes = [vp, i32]
     lib.rpeg_engine_reset_classes.restype = C.c_int
     lib.rpeg_engine_reset_classes.argtypes = [vp]
     lib.rpeg_engine_profile.restype = C.c_int
@@ -190,6 +192,10 @@ class Engine:
     def set_state_lanes(self, lanes: int):
         """-1 automatic; 0 scheduler state in HBM (64 plans per wavefront); 8/16/32/64 state in LDS."""
         self._check(self.lib.rpeg_engine_set_state_lanes(self._h, int(lanes)), "rpeg_engine_set_state_lanes")
+
+    def set_ready_cap(self, entries: int):
+        """Ready-list entries per plan in the main kernel (8, 16, 24 or 32); plans that need more get MASK_LIMIT."""
+        self._check(self.lib.rpeg_engine_set_ready_cap(self._h, int(entries)), "rpeg_engine_set_ready_cap")
 
     def reset_classes(self):
         self.lib.rpeg_engine_reset_classes(self._h)

@@ -185,6 +185,50 @@ def test_plans_that_outgrow_the_learned_ready_list_are_redone():
     eng.close()
 
 
+def test_ready_list_limit_is_reported_and_leaves_nothing_behind():
+    """A plan that outgrows the FULL ready list is not evaluated: NaN outputs, MASK_ERROR | MASK_LIMIT, the other
+    plans of the batch unaffected.  The limit is 32 entries, above every list of the shipped problems, so the test
+    lowers it to 8.  Afterwards, with the limit back at 32, the same engine evaluates the set exactly again -- in
+    the launch that learns the short capacity and in the next one, whose fix-up launch must find no flag or count
+    left over from the overflowing call -- and the drop-in reports the condition under its own name."""
+    from rpeg_amd.engine.runtime import Engine
+    from rpeg_amd.search import evaluate as ev
+    n = 40000
+    cfg, batch = seeded_batch(2, n)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    eng = Engine(cfg.problem)
+    eng.set_ready_cap(8)
+    out = eng.eval_resident(batch)
+    limit = (out["mask"] & abi.MASK_LIMIT) != 0
+    assert 0 < limit.sum() < (ref["mask"] & abi.MASK_VALID).sum()
+    assert np.all(out["mask"][limit] & abi.MASK_ERROR) and np.all(np.isnan(out["score"][limit]))
+    assert np.all(np.isnan(out["makespan"][limit]))
+    assert np.array_equal(out["mask"][~limit], ref["mask"][~limit])
+    assert same_bits(out["score"][~limit], ref["score"][~limit]) and same_bits(out["makespan"][~limit], ref["makespan"][~limit])
+    eng.set_ready_cap(32)
+    for _ in range(3):
+        out = eng.eval_resident(batch)
+        assert np.array_equal(out["mask"], ref["mask"]) and same_bits(out["score"], ref["score"])
+    with pytest.raises(Exception, match="8, 16, 24 or 32"):
+        eng.set_ready_cap(12)
+    eng.close()
+
+    class Limited:                       # evaluate_batch names the condition instead of a division by zero
+        def eval(self, b, gate_stale=True):
+            m = np.full(b.n, abi.MASK_VALID | abi.MASK_ERROR | abi.MASK_LIMIT, np.uint8)
+            nan = np.full(b.n, np.nan)
+            return dict(mask=m, score=nan, makespan=nan, peak=nan)
+    p = cfg.problem
+    rpeg, plan, wl = batch.configuration(p, 0)
+    real = ev._engine_for
+    ev._engine_for = lambda *a, **k: (Limited(), real(*a, **k)[1])
+    try:
+        with pytest.raises(ev.EngineLimitError):
+            ev.evaluate_batch([ev.Configuration(rpeg, plan, p.device_space)], p.suite, wl, p.hw, p.K_eval, p.memory_policy)
+    finally:
+        ev._engine_for = real
+
+
 def test_mixed_structures_config3():
     cfg, batch = seeded_batch(3, 2000, start=500_000)
     out = engine(3).eval(batch)
