@@ -363,6 +363,20 @@ int rpeg_sa_optimize_families(rpeg_engine_t* e, int32_t n_families, const rpeg_s
                               uint64_t stream_a, uint64_t stream_b, uint64_t stream_c, const int16_t* base_plan,
                               rpeg_sa_serial_result_t* result, void* stream);
 
+/* One draw of the proposal kernels that the annealing loops run, for callers that drive the loop themselves
+   (host arithmetic only, no launch).  what = 0: move_gen (RPEG/search/moves.py:645-826) for the plan `plan` with
+   critical-chain masses `mass` (RPEG_MAX_V doubles, rpeg_eval_batch_mass) at temperature T: up to K_x plans of
+   RPEG_MAX_V*RPEG_FIELDS values each into `out`; *fallback = 1 when the current strategy was not in the
+   directory (moves.py:554-587).  what = 1: multi_move_pair (moves.py:845-1010): one plan or none.  what = 2:
+   sample_expl_in_region (moves.py:202-296) for vertex `vertex` on racks [r_lo, r_hi): RPEG_FIELDS values or none.
+   The draws are words *draws+1, ... of the stream (prm->seed, stream_a, stream_b, stream_c); *draws is advanced
+   by the words used, so that successive calls continue one stream.  Of `prm` the structure, K_x, T_max, T_init,
+   the directory and the ablation switches are read.  Returns the number of plans (rows) written, negative on
+   bad arguments. */
+int rpeg_sa_propose(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t what, uint64_t stream_a, uint64_t stream_b,
+                    uint64_t stream_c, const int16_t* plan, const double* mass, double T, int32_t vertex, int32_t r_lo,
+                    int32_t r_hi, int16_t* out, int64_t* draws, int32_t* fallback);
+
 /* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,
    [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace; 1: one plan per

@@ -1702,6 +1702,52 @@ int rpeg_sa_optimize(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t E_ma
                                    base_plan, res, stream);
 }
 
+int rpeg_sa_propose(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t what, uint64_t stream_a, uint64_t stream_b,
+                    uint64_t stream_c, const int16_t* plan, const double* mass, double T, int32_t vertex, int32_t r_lo,
+                    int32_t r_hi, int16_t* out, int64_t* draws, int32_t* fallback) {
+  if (!e || !prm || !out || what < 0 || what > 2) return -1;
+  e->err.clear();
+  if (prm->structure < 0 || prm->structure >= e->P.n_struct || prm->K_x < 1 || prm->K_x > 16 || !(prm->T_init > 0.0) ||
+      prm->T_max < 0 || (what < 2 && !plan) || (what == 0 && !mass)) {
+    e->err = "bad proposal parameters";
+    return -1;
+  }
+  SaContext cx;
+  cx.init(e->P, prm->structure);
+  cx.fixed_mb = prm->fixed_mb != 0;
+  cx.uniform_vertex = prm->uniform_vertex != 0;
+  for (int v = 0; v < cx.nv; ++v) {
+    if (prm->dir_n[v] < 0 || (prm->dir_n[v] > 0 && !prm->dir[v])) { e->err = "bad candidate directory"; return -1; }
+    if (const char* msg = cx.set_directory(v, prm->dir[v], prm->dir_n[v])) { e->err = msg; return -1; }
+  }
+  if (what == 2 && (vertex < 0 || vertex >= cx.nv || r_lo < 0 || r_hi > cx.R || r_lo >= r_hi)) {
+    e->err = "bad vertex or rack range";
+    return -1;
+  }
+  if (what == 0)
+    for (int v = 0; v < cx.nv; ++v)
+      if (prm->dir_n[v] == 0) { e->err = "empty candidate table"; return -1; }   // the reference's move_gen raises on one
+  SaRng rng(prm->seed, stream_a, stream_b, stream_c);
+  if (draws) rng.k = (uint64_t)*draws;
+  SaPlan cur;
+  if (plan) std::memcpy(&cur, plan, sizeof cur);
+  int n = 0, fb = 0;
+  if (what == 0) {
+    std::vector<SaPlan> o(prm->K_x);
+    n = sa_move_gen(rng, cx, cur, mass, prm->K_x, prm->T_max, T, prm->T_init, o.data(), &fb);
+    std::memcpy(out, o.data(), sizeof(SaPlan) * n);
+  } else if (what == 1) {
+    SaPlan o;
+    n = sa_move_pair(rng, cx, cur, &o) ? 1 : 0;
+    if (n) std::memcpy(out, &o, sizeof o);
+  } else {
+    n = sa_sample_region(rng, cx, vertex, r_lo, r_hi, out) ? 1 : 0;
+  }
+  if (draws) *draws = (int64_t)rng.k;
+  if (fallback) *fallback = fb;
+  return n;
+}
+
 int rpeg_device_exp(rpeg_engine_t* e, uint64_t n, const double* x, double* y, void* stream) {
   if (!e || !x || !y) return -1;
   if (n == 0) return 0;

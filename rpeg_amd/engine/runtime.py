@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_engine_set_state_lanes", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_engine_set_state_lanes", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
            "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static")
 
 
@@ -81,6 +81,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_reset_classes.argtypes = [vp]
     lib.rpeg_engine_profile.restype = C.c_int
     lib.rpeg_engine_profile.argtypes = [vp, i32, vp, u64]
+    lib.rpeg_sa_propose.restype = C.c_int
+    lib.rpeg_sa_propose.argtypes = [vp, vp, i32, u64, u64, u64, vp, vp, C.c_double, i32, i32, i32, vp, vp, vp]
     lib.rpeg_device_exp.restype = C.c_int
     lib.rpeg_device_exp.argtypes = [vp, u64, vp, vp, vp]
     if path is None:
@@ -359,6 +361,26 @@ class Engine:
         self._check(rc, "rpeg_sa_optimize_families")
         del keep
         return serial_dict(res, log, logv)
+
+    def sa_propose(self, params: "abi.SaParamsT", directory, what: int, stream_key=(0, 0, 0), plan=None, mass=None,
+                   T: float = 0.0, v: int = 0, r_lo: int = 0, r_hi: int = 0, skip: int = 0):
+        """One draw of a proposal kernel (rpeg_sa_propose) on the stream (params.seed, *stream_key), continued
+        after `skip` words: what = 0 move_gen, 1 donor/receiver pair, 2 region sample of vertex v on racks
+        [r_lo, r_hi).  Returns (rows [n, MAX_V*10] -- [n, 10] for what = 2 --, words drawn so far, fallback)."""
+        keep = set_directory(params, directory)
+        W = abi.MAX_V * abi.FIELDS
+        out = np.zeros((max(params.K_x, 1), W), np.int16)
+        draws, fb = C.c_int64(skip), C.c_int32(0)
+        p = None if plan is None else np.ascontiguousarray(plan, dtype=np.int16).reshape(W)
+        m = None if mass is None else np.ascontiguousarray(mass, dtype=np.float64)
+        n = self.lib.rpeg_sa_propose(self._h, C.addressof(params), what, *[int(x) for x in stream_key],
+                                     p.ctypes.data if p is not None else None, m.ctypes.data if m is not None else None,
+                                     float(T), v, r_lo, r_hi, out.ctypes.data, C.addressof(draws), C.addressof(fb))
+        self._check(n, "rpeg_sa_propose")
+        del keep
+        if what == 2:
+            return out.reshape(-1)[:abi.FIELDS * n].reshape(n, abi.FIELDS), draws.value, fb.value
+        return out[:n], draws.value, fb.value
 
     def op_time(self, structure: int, vertex: int, strat: np.ndarray):
         """time() and peak_bytes() of mock nodes: strat is int16 [7, n] = dp pp tp mb r_ext n_ext g_ext."""

@@ -128,6 +128,29 @@ def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware,
     return eng, st
 
 
+def _engine_like(rpeg, space: DeviceSpace, suite=None, workload=None, vertex=None):
+    """The most recently used engine that holds the template of `rpeg` as a structure on device space `space`
+    (and, when given, for these models and this workload), with the index of that structure -- for calls of the
+    reference's API that name neither the hardware nor the horizon (the proposal functions of search.moves),
+    whose results depend on neither.  With `vertex` in place of `rpeg`: an engine with a template that holds that
+    vertex, the structure and the vertex's slot in it."""
+    want = None if rpeg is None else _structure_of(rpeg).name
+    for eng in reversed(list(_engines.values())):
+        p = eng.problem
+        if p.device_space != space or (suite is not None and p.suite.specs != suite.specs) or \
+                (workload is not None and p.workload != workload):
+            continue
+        for k, st in enumerate(p.structures):
+            if vertex is not None:
+                ids = [v.id for v in p.template(k, ()).vertices]
+                if vertex.id in ids and st.memory_trainable is None:
+                    return eng, k, ids.index(vertex.id)
+            elif st.name == want and st.memory_trainable is None:
+                return eng, k
+    raise LookupError("no evaluation engine for this template and device space yet: evaluate a configuration of it "
+                      "(evaluate, evaluate_cached, evaluate_batch) before asking for proposals")
+
+
 def _check_supported(config: Configuration):
     if config.intra_stage_fusion:
         raise NotImplementedError("intra_stage_fusion=True is not evaluated by this engine")
