@@ -26,6 +26,9 @@ def hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
+PROFILE_LIB = os.path.join(HERE, "librpeg_eval_prof.so")   # the same library with the scheduling loop's section clocks
+
+
 def build(force: bool = True, verbose: bool = False) -> str:
     if not force and os.path.exists(LIB) and all(os.path.getmtime(LIB) >= os.path.getmtime(f) for f in SOURCES + HEADERS):
         return LIB
@@ -36,5 +39,16 @@ def build(force: bool = True, verbose: bool = False) -> str:
     return LIB
 
 
+def build_profile(verbose: bool = False) -> str:
+    """The measurement build (-DKE_FINE_PROF): k_eval sums the shader clocks of the four sections of its
+    scheduling loop per wavefront (rpeg_amd.engine.profile --sections reads them).  Not loaded by anything else."""
+    cmd = [hipcc()] + FLAGS + ["-DKE_FINE_PROF", "-o", PROFILE_LIB] + SOURCES
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.run(cmd, check=True)
+    return PROFILE_LIB
+
+
 if __name__ == "__main__":
-    print(build(force=True, verbose=True))
+    import sys
+    print(build_profile(verbose=True) if "--profile" in sys.argv else build(force=True, verbose=True))

@@ -135,7 +135,11 @@ __device__ inline double ke_dev_max(unsigned m, const double (&lf)[RPEG_MAX_V]) 
   return d;
 }
 
+#ifdef KE_FINE_PROF
+#define KE_STAMP(k) do { if (L.prof && lane == first_lane && ((k) == 0 || (k) >= 5)) L.prof[w * 8 + (k)] = wall_clock64(); } while (0)
+#else
 #define KE_STAMP(k) do { if (L.prof && lane == first_lane) L.prof[w * 8 + (k)] = wall_clock64(); } while (0)
+#endif
 
 // LS = 0: 64 plans per wavefront, per-plan state in the HBM workspace.  LS > 0: LS plans per wavefront
 // (lanes LS..63 only help to stage the class tables), per-plan state in LDS.
@@ -407,11 +411,22 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   double makespan = 0.0;
   const long guard_max = (long)n * n + 64;
   long guard_total = 0;
+  // KE_FINE_PROF (a build of its own, for measurements): shader clocks of the four sections of the loop, summed
+  // over the dispatches of the wavefront, in place of the phase stamps 1-4 of the profile row
+#ifdef KE_FINE_PROF
+  long long fp_pop = 0, fp_rm = 0, fp_succ = 0, fp_push = 0, fp_t = 0;
+#define FP_MARK(acc) do { const long long _t = clock64(); acc += _t - fp_t; fp_t = _t; } while (0)
+#else
+#define FP_MARK(acc) do {} while (0)
+#endif
   for (long guard = 0; !err && done < n && guard < guard_max; ++guard) {
     ++guard_total;
     if (n_ready == 0) { err = true; break; }
     int bj = 0;
     double est = 0.0;
+#ifdef KE_FINE_PROF
+    fp_t = clock64();
+#endif
     for (long inner = 0; inner < guard_max; ++inner) {
       double bk = inf;
       bj = 0;
@@ -454,6 +469,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         }
       }
     }
+    FP_MARK(fp_pop);
     const uint32_t bm = r_nt[bj * RW];
     const int bv = (int)(bm & 0xFFFu);
     const unsigned blocked = (1u << ((bm >> 16) & 7u)) | (1u << ((bm >> 19) & 7u));
@@ -496,6 +512,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
       }
     }
     r_key[n_ready * RW] = inf;
+    FP_MARK(fp_rm);
     const double fin = est + d;
     makespan = fin > makespan ? fin : makespan;
     ++done;
@@ -549,6 +566,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         }
       }
       if (n_ready + cnt >= rcap) { err = ovf = true; break; }
+      FP_MARK(fp_succ);
       // the widest push of the wavefront selects the code: most dispatches release one or two successors
       if (__ballot(cnt > 2)) {
         if (cnt) push_many(std::integral_constant<int, 4>{}, cnt, nm, nk, nrk);
@@ -557,8 +575,14 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
       } else if (cnt) {
         push_many(std::integral_constant<int, 1>{}, cnt, nm, nk, nrk);
       }
+      FP_MARK(fp_push);
     }
   }
+#ifdef KE_FINE_PROF
+  if (L.prof && lane == first_lane) {
+    L.prof[w * 8 + 1] = fp_pop; L.prof[w * 8 + 2] = fp_rm; L.prof[w * 8 + 3] = fp_succ; L.prof[w * 8 + 4] = fp_push;
+  }
+#endif
   if (done != n) err = true;
   if (L.ovf) {
     const bool fix = (L.flags & KE_FIXUP) != 0;
