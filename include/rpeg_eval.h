@@ -206,6 +206,17 @@ int rpeg_eval_batch_mass(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* pl
 int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                    double* peak, double* score, uint8_t* mask, double* mass, void* stream);
 
+/* rpeg_eval_host with Trace.utilization() (RPEG/schedule/trace.py:53-101) of every plan as a further output,
+   computed in the same launch from the schedule the kernel has just built: the mean over the devices that any
+   node reserved of busy time / makespan, summed in the order in which the reference's trace first meets the
+   devices, hence equal to the reference's number bit for bit (NaN for a plan with RPEG_MASK_ERROR or an
+   invalid one).  This is the second factor of the utilisation objective of optimize() and polish()
+   (RPEG/search/optimizer.py:461-486, 1021-1044), which then costs no launch of its own.  At most 1,024 plans per
+   call, one plan per wavefront (status -8 beyond that, and for problems with a class above 384 nodes);
+   rpeg_eval_trace_metrics gives the same number for a single plan of any size. */
+int rpeg_eval_host_util(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                        double* peak, double* score, uint8_t* mask, double* utilization, void* stream);
+
 /* Single-node durations and isolated peaks: the batched form of the candidate-directory loop
    (RPEG/search/moves.py:532-549): for strategy i, time = NodeCostModel.time(mock node) and
    peak = NodeMemoryModel.peak_bytes(mock node) of vertex `vertex` of structure `structure` placed at

@@ -1327,7 +1327,7 @@ int rpeg_eval_trace_metrics(rpeg_engine_t* e, const int16_t* vert_fields, const 
 namespace {
 
 constexpr size_t HS_IN_BYTES = (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 + 4 + 4;   // per plan: fields, header, class offset
-constexpr size_t HS_OUT_BYTES = 3 * 8 + (size_t)RPEG_MAX_V * 8 + 8;            // makespan, peak, score, mass, mask (padded)
+constexpr size_t HS_OUT_BYTES = 3 * 8 + (size_t)RPEG_MAX_V * 8 + 8 + 8;        // makespan, peak, score, mass, utilisation, mask (padded)
 
 int ensure_host_stage(rpeg_engine_t* e, size_t n, hipStream_t s) {
   if (n <= e->hs_cap) return 0;
@@ -1350,7 +1350,7 @@ int ensure_host_stage(rpeg_engine_t* e, size_t n, hipStream_t s) {
 // eligible (a class too large for k_plan); the caller then takes the device path.  Output arrays may be null.
 template <class GET>
 int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, double* makespan, double* peak, double* score,
-                    uint8_t* mask, double* mass, hipStream_t s) {
+                    uint8_t* mask, double* mass, hipStream_t s, double* util = nullptr) {
   e->last_ms = -1.0;
   if (n == 0) return 0;
   const size_t stride = ((size_t)n + 63) & ~size_t(63);
@@ -1373,6 +1373,7 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
       if (mask) mask[i] = 0;
       if (mass)
         for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
+      if (util) util[i] = nan;
       continue;
     }
     bool is_new = false;
@@ -1401,7 +1402,8 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
   double* o_peak = o_makespan + stride;
   double* o_score = o_peak + stride;
   double* o_mass = o_score + stride;
-  uint8_t* o_mask = (uint8_t*)(o_mass + (size_t)RPEG_MAX_V * stride);
+  double* o_util = o_mass + (size_t)RPEG_MAX_V * stride;
+  uint8_t* o_mask = (uint8_t*)(o_util + stride);
   EvalLaunch L;
   L.P = e->dP;
   L.vert = (const int16_t*)e->ds_in;
@@ -1414,6 +1416,7 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
   L.cls_bytes = 0; L.rcap = 0; L.max_v = e->max_v; L.ovf = nullptr; L.need = nullptr;
   L.flags = flags; L.makespan = o_makespan; L.peak = o_peak; L.score = o_score; L.mask = o_mask;
   L.mass = mass ? o_mass : nullptr;
+  L.util = util ? o_util : nullptr;
   L.prof = nullptr;
   const size_t lds = kp_lds_bytes(e->max_nodes, e->max_slots);
   const unsigned grid = (unsigned)std::min<uint64_t>(m, (uint64_t)e->n_cu * 32);
@@ -1436,6 +1439,7 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
     if (mask) mask[i] = o_mask[j];
     if (mass)
       for (int x = 0; x < RPEG_MAX_V; ++x) mass[(size_t)i * RPEG_MAX_V + x] = o_mass[j * RPEG_MAX_V + x];
+    if (util) util[i] = o_util[j];
   }
   return 0;
 }
@@ -1528,7 +1532,7 @@ struct GpuSaBackend : SaBackend {
   uint8_t head_of[256][4] = {};
   int16_t *h_vert = nullptr, *d_vert = nullptr;
   uint8_t *h_head = nullptr, *d_head = nullptr, *h_mask = nullptr, *d_mask = nullptr;
-  double *h_score = nullptr, *d_score = nullptr, *h_mass = nullptr, *d_mass = nullptr;
+  double *h_score = nullptr, *d_score = nullptr, *h_mass = nullptr, *d_mass = nullptr, *h_util = nullptr;
   double eval_s = 0.0;
   long n_launch = 0, n_plans = 0;
   int rc_alloc = 0;
@@ -1540,7 +1544,8 @@ struct GpuSaBackend : SaBackend {
               hipHostMalloc(&h_mask, cap) == hipSuccess && hipMalloc(&d_mask, cap) == hipSuccess &&
               hipHostMalloc(&h_score, 8 * (size_t)cap) == hipSuccess && hipMalloc(&d_score, 8 * (size_t)cap) == hipSuccess &&
               hipHostMalloc(&h_mass, 8 * (size_t)cap * RPEG_MAX_V) == hipSuccess &&
-              hipMalloc(&d_mass, 8 * (size_t)cap * RPEG_MAX_V) == hipSuccess;
+              hipMalloc(&d_mass, 8 * (size_t)cap * RPEG_MAX_V) == hipSuccess &&
+              hipHostMalloc(&h_util, 8 * (size_t)cap) == hipSuccess;
     if (!ok) { rc_alloc = -2; e->err = "out of memory for the annealing buffers"; }
     else std::memset(h_vert, 0, V * cap * 2);
   }
@@ -1556,13 +1561,18 @@ struct GpuSaBackend : SaBackend {
     if (d_score) hipFree(d_score);
     if (h_mass) hipHostFree(h_mass);
     if (d_mass) hipFree(d_mass);
+    if (h_util) hipHostFree(h_util);
   }
 
   int utilization(const SaPlan& plan, uint8_t variant, double* out) override {
     return rpeg_eval_trace_metrics(e, &plan.f[0][0], head_of[variant], out, nullptr);
   }
 
-  int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override {
+  int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override { return evaluate(n, plans, variant, out, false); }
+
+  // with_util: Trace.utilization() of every plan from the same launch (out[i].util); 1 when this batch cannot
+  // take that path (the caller then asks per plan)
+  int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out, bool with_util) override {
     if (n > cap) { e->err = "annealing batch exceeds its buffers"; return -1; }
     {  // a step's proposals are a small batch: one copy, one launch (eval_host_small)
       const auto t0 = std::chrono::steady_clock::now();
@@ -1577,13 +1587,15 @@ struct GpuSaBackend : SaBackend {
           a[v].e[0] = f[7]; a[v].e[1] = f[8]; a[v].e[2] = f[9];
         }
       };
-      const int rc = eval_host_small(e, (uint64_t)n, get, 0u, nullptr, nullptr, h_score, h_mask, h_mass, s);
+      const int rc = eval_host_small(e, (uint64_t)n, get, 0u, nullptr, nullptr, h_score, h_mask, h_mass, s,
+                                     with_util ? h_util : nullptr);
       if (rc < 0) return rc;
       if (rc == 0) {
         for (int i = 0; i < n; ++i) {
           out[i].score = h_score[i];
           out[i].mask = h_mask[i];
           for (int x = 0; x < RPEG_MAX_V; ++x) out[i].mass[x] = h_mass[(size_t)i * RPEG_MAX_V + x];
+          if (with_util) out[i].util = h_util[i];
         }
         eval_s += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
         ++n_launch;
@@ -1591,6 +1603,7 @@ struct GpuSaBackend : SaBackend {
         return 0;
       }
     }
+    if (with_util) return 1;   // the staged path has no utilisation output
     const auto t0 = std::chrono::steady_clock::now();
     const size_t V = RPEG_MAX_V * RPEG_FIELDS;
     for (int i = 0; i < n; ++i) {
@@ -1621,6 +1634,30 @@ struct GpuSaBackend : SaBackend {
 }  // namespace
 
 extern "C" {
+
+int rpeg_eval_host_util(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
+                        double* peak, double* score, uint8_t* mask, double* utilization, void* stream) {
+  if (!e || !plans || !utilization) return -1;
+  e->err.clear();
+  e->last_ms = -1.0;
+  if (n == 0) return 0;
+  if (!plans->vert || !plans->head || plans->stride < n) { e->err = "bad plan tensors"; return -1; }
+  if (n > (uint64_t)e->host_small_max) {
+    e->err = "rpeg_eval_host_util takes at most " + std::to_string(e->host_small_max) + " plans per call";
+    return -8;
+  }
+  const int16_t* vert = plans->vert;
+  const uint8_t* head = plans->head;
+  const uint64_t stride = plans->stride;
+  auto get = [&](uint64_t i, PlanHead& h, VPlan (&a)[RPEG_MAX_V]) {
+    h = load_head(head, stride, i);
+    const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;
+    for (int v = 0; v < nv; ++v) load_vertex(vert, stride, i, v, &a[v]);
+  };
+  const int rc = eval_host_small(e, n, get, flags, makespan, peak, score, mask, nullptr, (hipStream_t)stream, utilization);
+  if (rc == 1) { e->err = "a class of this problem has too many nodes for one plan per wavefront"; return -8; }
+  return rc;
+}
 
 int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* base_plan, rpeg_sa_result_t* res,
                 void* stream) {

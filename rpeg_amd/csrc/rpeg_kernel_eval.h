@@ -50,6 +50,7 @@ struct EvalLaunch {              // uniform launch parameters
   double* score;
   uint8_t* mask;
   double* mass;                  // optional critical-chain mass, [plan][RPEG_MAX_V], or null
+  double* util = nullptr;        // optional Trace.utilization() per plan (k_plan only), or null
   unsigned long long* prof;      // optional per-wavefront phase clocks (8 per wavefront), or null
   uint8_t* ovf;                  // per plan: its ready list outgrew rcap (set by a launch with a short list,
                                  // consumed by the KE_FIXUP launch with the full one), or null

@@ -33,9 +33,11 @@ constexpr uint32_t KP_SKIP = 0xFFFFFFFFu;        // task -> class blob offset of
 constexpr int KP_PLAN_I16 = 80;                 // plan fields in LDS (60 used; pair tests may read past them)
 
 // LDS of one wavefront: plan fields, per-vertex memory terms, durations per slot, rank / finish and start
-// per node (plus one neutral element each), tie-break class per node.
+// per node (plus one neutral element each), tie-break class per node; busy-time table and dispatch order.
 __host__ __device__ inline size_t kp_lds_bytes(uint32_t nodes, uint32_t slots) {
-  return ((size_t)KP_PLAN_I16 * 2 + (size_t)RPEG_MAX_V * 4 * 8 + 8ull * slots + 16ull * (nodes + 1) + nodes + 15) & ~size_t(15);
+  const size_t base = ((size_t)KP_PLAN_I16 * 2 + (size_t)RPEG_MAX_V * 4 * 8 + 8ull * slots + 16ull * (nodes + 1) + nodes + 7) & ~size_t(7);
+  // then, for the utilisation: busy time by allocation set (64 doubles) and the dispatch order (2 bytes per node)
+  return (base + 64 * 8 + 2ull * nodes + 15) & ~size_t(15);
 }
 
 #if defined(__HIPCC__)
@@ -91,8 +93,8 @@ __device__ inline bool kp_is_inf(double v) {   // on the bits, so that a uniform
 template <int NS>
 __device__ inline int kp_schedule(const ClassView& cv, const int n, const int lane, const uint64_t ovl,
                                    const uint64_t dpne, const int nd, const double* l_dur, double* l_rank,
-                                   double* l_start, uint8_t* l_pt, const bool keep_trace, double* out_makespan,
-                                   long* out_pops, unsigned long long* stamp) {
+                                   double* l_start, uint8_t* l_pt, const bool keep_trace, uint16_t* l_order,
+                                   double* out_makespan, long* out_pops, unsigned long long* stamp) {
   const double inf = __builtin_inf();
   double key[NS], tm[NS], dvc[NS], dur[NS], rk[NS];
   uint32_t ord[NS], info[NS], deg[NS], sxl[NS], sxh[NS], pt[NS];
@@ -385,6 +387,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
     if (keep_trace && mine) {
       l_rank[ws * 64 + wl] = fin;
       l_start[ws * 64 + wl] = gk;
+      if (l_order) l_order[done - 1] = (uint16_t)(ws * 64 + wl);
     }
     // successors in adjacency order; a node whose last predecessor this was becomes ready
     const int ns = (int)((binfo >> 8) & 0xFFu), sb = (int)(binfo >> 16);
@@ -489,6 +492,114 @@ __device__ inline double kp_class_peak(const rpeg_problem_t& P, const rpeg_struc
   return peak;
 }
 
+// Trace.utilization() (RPEG/schedule/trace.py:53-101) of the plan just scheduled: the mean over the devices that
+// any node reserved of busy time / makespan, where a device's busy time is the measure of the union of the
+// (start, finish) spans of the nodes whose reserved allocations hold it, merged in sorted order, and the mean is
+// a running sum over the devices in the order in which the trace first met them (dispatch order of the nodes;
+// within a node the source allocation before the destination; within an allocation rack-major) divided by
+// their number.  The additions are done in exactly that order: the result equals the reference's bit for bit.
+//
+// All devices held by the same set of vertex allocations have the same spans, so the busy time is computed once
+// per set (lane m takes the set with bit pattern m) over the nodes in dispatch order -- on one device that is
+// the sorted order, because a node starts no earlier than the nodes dispatched before it on its devices ended.
+// Then the vertices are taken in the order of their first reservation, and the devices of each allocation that
+// no earlier one holds are added 64 at a time: the lanes find set and value of their device, one running sum
+// takes the values in lane order.  l_start / l_fin: per node; l_order: node dispatched k-th; l_tab: 64 doubles.
+__device__ inline double kp_utilization(const ClassView& cv, const int n, const int lane, const int nv, const int16_t* l_plan,
+                                        const uint64_t dpne, const double* l_start, const double* l_fin,
+                                        const uint16_t* l_order, double* l_tab, const double ms) {
+  if (!(ms > 0.0) || n == 0) return 0.0;
+  {
+    const unsigned mine = (unsigned)lane;
+    double merged = 0.0, cs = 0.0, ce = 0.0;
+    bool open = false;
+    for (int k = 0; k < n; ++k) {
+      const int i = (int)l_order[k];
+      const uint64_t bits = ((const uint64_t*)cv.node)[i];
+      NodeRec nr;
+      __builtin_memcpy(&nr, &bits, 8);
+      const unsigned b = blocked_mask(nr, dpne);
+      const double s = l_start[i], f = l_fin[i];
+      if (b & mine) {
+        if (!open || s > ce) {
+          if (open) merged += ce - cs;
+          cs = s;
+          ce = f;
+          open = true;
+        } else {
+          ce = f > ce ? f : ce;
+        }
+      }
+    }
+    if (open) merged += ce - cs;
+    l_tab[lane] = merged / ms;
+  }
+  __syncthreads();
+  // vertices by first reservation, four bits each
+  uint32_t order = 0u;
+  int n_ev = 0;
+  {
+    unsigned seen = 0u;
+    for (int k = 0; k < n && n_ev < nv; ++k) {
+      const int i = __builtin_amdgcn_readfirstlane((int)l_order[k]);
+      const uint64_t bits = ((const uint64_t*)cv.node)[i];
+      NodeRec nr;
+      __builtin_memcpy(&nr, &bits, 8);
+      unsigned b = blocked_mask(nr, dpne) & ~seen;
+      if (nr.cond) {   // a transfer: source before destination
+        const unsigned src = (nr.cond - 1u) >> 3;
+        if ((b >> src) & 1u) {
+          order |= src << (4 * n_ev);
+          ++n_ev;
+          seen |= 1u << src;
+          b &= ~(1u << src);
+        }
+      }
+      while (b) {
+        const unsigned v = (unsigned)__builtin_ctz(b);
+        b &= b - 1u;
+        order |= v << (4 * n_ev);
+        ++n_ev;
+        seen |= 1u << v;
+      }
+    }
+  }
+  double total = 0.0;
+  int count = 0;
+  unsigned earlier = 0u;
+  for (int e = 0; e < n_ev; ++e) {
+    const int v = (int)((order >> (4 * e)) & 15u);
+    const int16_t* bx = l_plan + v * RPEG_FIELDS;
+    const int ro = bx[4], qo = bx[5], go = bx[6], re = bx[7], qe = bx[8], ge = bx[9];
+    const uint32_t ng = (uint32_t)(qe * ge), cnt = (uint32_t)re * ng;
+    const uint32_t m_ng = 0xFFFFFFFFu / ng + 1u, m_g = 0xFFFFFFFFu / (uint32_t)ge + 1u;   // exact quotients below 2^16
+    for (uint32_t base = 0; base < cnt; base += 64u) {
+      const uint32_t idx = base + (uint32_t)lane;
+      const uint32_t r = ng == 1u ? idx : __umulhi(idx, m_ng);
+      const uint32_t rem = idx - r * ng;
+      const uint32_t q = ge == 1 ? rem : __umulhi(rem, m_g);
+      const int R = ro + (int)r, Q = qo + (int)q, G = go + (int)(rem - q * (uint32_t)ge);
+      unsigned M = 0u;
+#pragma unroll
+      for (int x = 0; x < RPEG_MAX_V; ++x) {
+        const int16_t* p = l_plan + x * RPEG_FIELDS;
+        const bool in = x < nv && R >= p[4] && R < p[4] + p[7] && Q >= p[5] && Q < p[5] + p[8] && G >= p[6] && G < p[6] + p[9];
+        M |= in ? 1u << x : 0u;
+      }
+      const double val = l_tab[M & 63u];
+      unsigned long long fresh = __ballot(idx < cnt && (M & earlier) == 0u);
+      count += (int)__builtin_popcountll(fresh);
+      while (fresh) {
+        const int j = __builtin_ctzll(fresh);
+        fresh &= fresh - 1ull;
+        total += kp_readlane(val, j);
+      }
+    }
+    earlier |= 1u << v;
+  }
+  return count ? total / (double)count : 0.0;
+}
+
 // One plan, evaluated by the whole wavefront.  pi: plan index (uniform).
 __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const uint64_t pi, const ClassView cv,
                                     uint8_t* lds) {
@@ -505,6 +616,8 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   double* l_rank = l_dur + L.ws_slots;
   double* l_start = l_rank + (L.ws_nodes + 1);
   uint8_t* l_pt = (uint8_t*)(l_start + (L.ws_nodes + 1));
+  double* l_tab = (double*)(((uintptr_t)(l_pt + L.ws_nodes) + 7) & ~(uintptr_t)7);
+  uint16_t* l_ord = (uint16_t*)(l_tab + 64);
 
   __syncthreads();   // the previous plan of this wavefront is done with LDS
   KE_STAMP(0);
@@ -586,14 +699,16 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   // ---- ranks and list scheduling
   double makespan = 0.0;
   long pops = 0;
+  const bool keep = L.mass != nullptr || L.util != nullptr;
+  uint16_t* const l_order = L.util ? l_ord : nullptr;
   if (!err) {
     int ok;
-    if (n <= 64) ok = kp_schedule<1>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
-    else if (n <= 128) ok = kp_schedule<2>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
-    else if (n <= 192) ok = kp_schedule<3>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
-    else if (n <= 256) ok = kp_schedule<4>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
-    else if (n <= 320) ok = kp_schedule<5>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
-    else ok = kp_schedule<6>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, L.mass != nullptr, &makespan, &pops, stamp);
+    if (n <= 64) ok = kp_schedule<1>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
+    else if (n <= 128) ok = kp_schedule<2>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
+    else if (n <= 192) ok = kp_schedule<3>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
+    else if (n <= 256) ok = kp_schedule<4>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
+    else if (n <= 320) ok = kp_schedule<5>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
+    else ok = kp_schedule<6>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
     err = ok != 0;
     limit = ok == 2;
   }
@@ -626,7 +741,13 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
       critical_mass(cv, [&](int i) { return l_rank[i]; }, [&](int i) { return l_start[i]; }, m);
     }
   }
+  double util = 0.0;
+  if (L.util) {
+    __syncthreads();
+    util = err ? __builtin_nan("") : kp_utilization(cv, n, lane, nv, l_plan, pm.dpne, l_start, l_rank, l_ord, l_tab, makespan);
+  }
   if (lane == 0) {
+    if (L.util) L.util[pi] = util;
     if (L.makespan) L.makespan[pi] = out_makespan;
     if (L.peak) L.peak[pi] = peak;
     if (L.score) L.score[pi] = out_score;

@@ -304,7 +304,9 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
       // two allocations are one and the same.
       const bool both = nd.kind == 1 && (P.transfer_both >> (nd.weight ? 0 : 1) & 1);
       r.blocked = (uint8_t)(1u << nd.a1 | (both ? 1u << nd.a0 : 0u));
-      r.cond = nd.weight || both ? 0 : (uint8_t)(1 + nd.a0 * 8 + nd.a1);
+      // (with both endpoints reserved the condition adds nothing to `blocked`; it is kept as the record of which
+      // endpoint is the source: the utilisation lists a transfer's source devices before its destination's)
+      r.cond = nd.weight && !both ? 0 : (uint8_t)(1 + nd.a0 * 8 + nd.a1);
     }
     recs[i] = r;
     if (indeg[i] == 0) init.push_back((uint16_t)i);

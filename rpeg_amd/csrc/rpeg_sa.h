@@ -79,6 +79,12 @@ struct SaBackend {
   virtual ~SaBackend() {}
   // evaluates n plans; variant[i] selects the staleness variant of plan i
   virtual int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) = 0;
+  // the same with Trace.utilization() of every plan (out[i].util) from the same evaluation when with_util is set;
+  // returns 1 when the backend cannot do that for this batch (the caller then asks plan by plan)
+  virtual int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out, bool with_util) {
+    if (with_util) return 1;
+    return evaluate(n, plans, variant, out);
+  }
   // Trace.utilization() of one plan (trace.py:53-101); backends without traces refuse
   virtual int utilization(const SaPlan& plan, uint8_t variant, double* out) { (void)plan; (void)variant; (void)out; return -1; }
 };
@@ -670,10 +676,14 @@ struct SaSerial {
     if (!todo.empty()) {
       std::vector<uint8_t> var(todo.size(), (uint8_t)variant);
       std::vector<SaEval> ev(todo.size());
-      if (int rc = be.evaluate((int)todo.size(), todo.data(), var.data(), ev.data())) return rc;
-      if (p.max_throughput_loss > 0.0)
+      const bool with_util = p.max_throughput_loss > 0.0;
+      int rc = be.evaluate((int)todo.size(), todo.data(), var.data(), ev.data(), with_util);
+      if (rc == 1 && with_util) {   // no utilisation from the batched evaluation: one trace per plan
+        if ((rc = be.evaluate((int)todo.size(), todo.data(), var.data(), ev.data())) != 0) return rc;
         for (size_t j = 0; j < todo.size(); ++j)
-          if (int rc = be.utilization(todo[j], (uint8_t)variant, &ev[j].util)) return rc;
+          if ((rc = be.utilization(todo[j], (uint8_t)variant, &ev[j].util)) != 0) return rc;
+      }
+      if (rc) return rc;
       for (size_t j = 0; j < todo.size(); ++j) {
         const bool stale_ok = (ev[j].mask & RPEG_MASK_STALE_OK) != 0, mem_ok = (ev[j].mask & RPEG_MASK_MEM_OK) != 0;
         Stored st;

@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_engine_set_state_lanes", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
            "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static")
 
 
@@ -81,6 +81,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_reset_classes.argtypes = [vp]
     lib.rpeg_engine_profile.restype = C.c_int
     lib.rpeg_engine_profile.argtypes = [vp, i32, vp, u64]
+    lib.rpeg_eval_host_util.restype = C.c_int
+    lib.rpeg_eval_host_util.argtypes = [vp, u64, vp, u32, vp, vp, vp, vp, vp, vp]
     lib.rpeg_sa_propose.restype = C.c_int
     lib.rpeg_sa_propose.argtypes = [vp, vp, i32, u64, u64, u64, vp, vp, C.c_double, i32, i32, i32, vp, vp, vp]
     lib.rpeg_device_exp.restype = C.c_int
@@ -265,6 +267,24 @@ class Engine:
                                          out["makespan"].ctypes.data, out["peak"].ctypes.data, out["score"].ctypes.data,
                                          out["mask"].ctypes.data, out["mass"].ctypes.data if mass else None, stream)
         self._check(rc, "rpeg_eval_host")
+        return out
+
+    def eval_util(self, batch: PlanBatch, gate_stale: bool = False) -> Dict[str, np.ndarray]:
+        """`eval` plus Trace.utilization() of every plan from the same launch (rpeg_eval_host_util; at most 1,024
+        plans): the dict of `eval` with "util", float64 [n]."""
+        torch = _torch()
+        n = batch.n
+        out = dict(makespan=np.empty(n), peak=np.empty(n), score=np.empty(n), mask=np.empty(n, np.uint8), util=np.empty(n))
+        if n == 0:
+            return out
+        vert, head = np.ascontiguousarray(batch.vert), np.ascontiguousarray(batch.head)
+        soa = abi.PlanSoaT(vert.ctypes.data, head.ctypes.data, vert.shape[1])
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        with torch.cuda.device(self.device):
+            rc = self.lib.rpeg_eval_host_util(self._h, n, C.addressof(soa), abi.GATE_STALE if gate_stale else 0,
+                                              out["makespan"].ctypes.data, out["peak"].ctypes.data, out["score"].ctypes.data,
+                                              out["mask"].ctypes.data, out["util"].ctypes.data, stream)
+        self._check(rc, "rpeg_eval_host_util")
         return out
 
     def eval_mass(self, batch: PlanBatch, gate_stale: bool = False) -> Dict[str, np.ndarray]:

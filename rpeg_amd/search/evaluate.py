@@ -177,11 +177,14 @@ class BatchResult:
     peak: np.ndarray
     mask: np.ndarray
     feasible: np.ndarray   # memory-feasible and stale-layout valid
+    util: Optional[np.ndarray] = None   # Trace.utilization() per configuration, when asked for
 
 
 def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload: Workload, hw: Hardware,
-                   K_eval: int, memory_policy: MemoryPolicy = MemoryPolicy(), gate_stale: bool = True) -> BatchResult:
-    """Scores many configurations of ONE template structure in one GPU launch."""
+                   K_eval: int, memory_policy: MemoryPolicy = MemoryPolicy(), gate_stale: bool = True,
+                   with_util: bool = False) -> BatchResult:
+    """Scores many configurations of ONE template structure in one GPU launch.  `with_util`: also
+    Trace.utilization() of each (trace.py:53-101) from the same launch, 1,024 configurations at a time."""
     if not configs:
         z = np.zeros(0)
         return BatchResult(z, z, z, np.zeros(0, np.uint8), np.zeros(0, bool))
@@ -192,7 +195,12 @@ def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload
         raise ValueError("the configurations of one batch must share their transfer resource policy")
     eng, st = _engine_for(configs[0].rpeg, suite, workload, hw, configs[0].device_space, K_eval, memory_policy,
                           transfer_policy=pol)
-    out = eng.eval(_pack(configs, st, workload), gate_stale=gate_stale)
+    batch = _pack(configs, st, workload)
+    if with_util:
+        parts = [eng.eval_util(batch.slice(a, min(a + 1024, batch.n)), gate_stale=gate_stale) for a in range(0, batch.n, 1024)]
+        out = {k: np.concatenate([q[k] for q in parts]) for k in parts[0]}
+    else:
+        out = eng.eval(batch, gate_stale=gate_stale)
     mask = out["mask"]
     if np.any((mask & abi.MASK_VALID) == 0):
         raise ValueError("a configuration violates the integer validity rules of is_valid")
@@ -206,7 +214,7 @@ def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload
     score = out["score"].copy()
     if ABLATION_HARD_OOM:
         score[(mask & abi.MASK_MEM_OK) == 0] = 0.0
-    return BatchResult(score, out["makespan"], out["peak"], mask, feasible)
+    return BatchResult(score, out["makespan"], out["peak"], mask, feasible, out.get("util"))
 
 
 # ----------------------------------------------------------------------------- trace objects

@@ -357,14 +357,6 @@ class _Utilization:
         return self.value
 
 
-def _trace_utilization(config: Configuration, suite, workload, hw, K_eval, policy) -> float:
-    """Trace.utilization() of one configuration, folded by the library (rpeg_eval_trace_metrics)."""
-    from .evaluate import _pack
-    eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, policy,
-                          transfer_policy=config.transfer_resource_policy)
-    return eng.trace_metrics(_pack([config], st, workload), 0)[0]
-
-
 def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw: Hardware, K_eval: int,
            opt_config: OptimizerConfig, cache: EvalCache, table, index, ac_share: bool = False,
            max_rounds: int = 50) -> Configuration:
@@ -423,11 +415,12 @@ def polish(best_config: Configuration, suite: ModelSuite, workload: Workload, hw
                     misses.append((nb, h))
             fresh = []
             if misses:
-                res = evaluate_batch([nb for nb, _ in misses], suite, workload, hw, K_eval, policy, gate_stale=False)
-                for (nb, h), s, m in zip(misses, res.score, res.mask):
+                res = evaluate_batch([nb for nb, _ in misses], suite, workload, hw, K_eval, policy, gate_stale=False,
+                                     with_util=delta > 0.0)
+                for j, ((nb, h), s, m) in enumerate(zip(misses, res.score, res.mask)):
                     f = bool(m & abi.MASK_MEM_OK)
-                    # the utilisation objective reads one number of a candidate's trace: keep that
-                    t = _Utilization(_trace_utilization(nb, suite, workload, hw, K_eval, policy)) if delta > 0.0 else None
+                    # the utilisation objective reads one number of a candidate's trace: keep that (same launch)
+                    t = _Utilization(float(res.util[j])) if delta > 0.0 else None
                     cache.put(h, float(s), t, f)
                     fresh.append((nb, float(s), t, f))
             for nb, s, t, f in hits + fresh:

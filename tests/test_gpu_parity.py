@@ -562,6 +562,43 @@ def test_transfer_resource_policies_equal_reference(c):
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+def test_utilization_from_the_batched_launch_equals_reference(c):
+    """Trace.utilization() as a further output of the batched launch (rpeg_eval_host_util, folded inside k_plan)
+    against the reference's own numbers for every plan of tests/golden/ref_transfer_policy.json under the three
+    transfer-reservation policies, against the single-plan trace path for other seeded plans, and NaN / mask for
+    plans that are not evaluated; the other outputs are those of the plain launch."""
+    from rpeg_amd.engine.runtime import Engine, EngineError
+    from tests.helpers import load_transfer_policy_golden, with_transfer_policy
+    gold = load_transfer_policy_golden()
+    g = gold["configs"][str(c)]
+    cfg, batch = seeded_batch(c, g["n_plans"])
+    p = cfg.problem
+    for k, pol in enumerate(gold["policies"]):
+        eng = Engine(with_transfer_policy(p, *pol))
+        out = eng.eval_util(batch, gate_stale=False)
+        plain = eng.eval(batch, gate_stale=False)
+        for key in ("makespan", "peak", "score"):
+            assert same_bits(out[key], plain[key]), (pol, key)
+        assert np.array_equal(out["mask"], plain["mask"])
+        for i in range(g["n_plans"]):
+            assert float(out["util"][i]).hex() == g["rows"][i][k]["utilization"], (i, pol)
+        eng.close()
+    eng = engine(c)
+    _, more = seeded_batch(c, 300, start=700_000)
+    out = eng.eval_util(more)
+    valid = np.flatnonzero((out["mask"] & abi.MASK_VALID) != 0)
+    assert len(valid) > 100
+    for i in valid[::7]:
+        assert float(out["util"][i]).hex() == float(eng.trace_metrics(more, int(i))[0]).hex(), i
+    assert np.all((out["util"][valid] > 0.0) & (out["util"][valid] <= 1.0))
+    more.vert[0, 3] = 3           # tp = 3 divides no G: not evaluated
+    bad = eng.eval_util(more.slice(0, 8))
+    assert bad["mask"][3] == 0 and np.isnan(bad["util"][3]) and not np.isnan(bad["util"][2])
+    with pytest.raises(EngineError, match="at most 1024"):
+        eng.eval_util(seeded_batch(c, 1025)[1])
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_other_seeds_unroll_depths_and_policies_equal_the_host_build(c):
     """Away from the shipped problems: unroll depths 1, 2, 7 and (three configurations) 32, both-endpoints reservations and two other
     seeds of the candidate generator.  Every makespan, peak, score and mask of the batched launch equals the
