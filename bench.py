@@ -119,6 +119,7 @@ def bench_sa(args):
     """Config 5: 64 chains x 2000 steps of batched simulated annealing.  Prints one JSON line whose value
     is the wall-clock of the whole run (directory build excluded and reported beside it)."""
     import zlib
+    import numpy as np
     import torch
     from rpeg_amd import configs
     from rpeg_amd.engine.runtime import Engine
@@ -161,9 +162,33 @@ def bench_sa(args):
         "restarts": int(cold.restarts.sum()), "dead_chains": int(cold.dead.sum()),
         "feasible_chains": int(cold.best_feasible.sum()),
     }
+    # optimize() as the reference runs it (one chain at a time, cache, restarts), under a wall-clock deadline as
+    # `pipeline.py --time` sets it: the best score reached within t seconds, on the GPU evaluator and -- the same
+    # loop, the same generator -- on the host build of the evaluator
+    from rpeg_amd.engine import abi
+    from rpeg_amd.search import candidates
+    seeds = candidates.generate(p, 64, cfg.tau_choices, seed=42, tag=5)
+    verdict = eng.eval(seeds)["mask"]
+    start = next(i for i in range(seeds.n) if verdict[i] & abi.MASK_VALID and verdict[i] & abi.MASK_MEM_OK)
+    row = np.ascontiguousarray(seeds.vert[:, start])
+    split = 1 if p.workload.gen_quantiles else 0
+
+    def timed(seconds):
+        prm = sa_params(opt, 1, 1, [(0, 0)], 0, split, 42)
+        prm.timed, prm.deadline_s = 1, seconds
+        return prm
+    line["within_deadline"] = []
+    for seconds in (0.1, 0.3, 1.0):
+        r = eng.sa_optimize(timed(seconds), arrays, row, 10 ** 9, 10 ** 9, stream_key=(5, 0, 0))
+        line["within_deadline"].append(dict(seconds=seconds, best_score=r["best_score"], best_feasible=r["best_feasible"],
+                                            evaluations=r["E"], timed_out=r["timed_out"]))
     if not args.no_cpu:
         # the same host logic over the CPU build of the evaluator, all host cores, on a bounded number of steps
         from oracle.cpu_port import CpuPort
+        for rec in line["within_deadline"]:
+            r = CpuPort(p).sa_optimize(timed(rec["seconds"]), arrays, row, 10 ** 9, 10 ** 9, stream_key=(5, 0, 0),
+                                       threads=min(16, os.cpu_count() or 1))
+            rec.update(cpu_port_best_score=r["best_score"], cpu_port_evaluations=r["E"])
         threads = min(16, os.cpu_count() or 1)
         steps = max(1, min(args.sa_steps, 40))
         split = 1 if p.workload.gen_quantiles else 0

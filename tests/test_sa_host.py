@@ -336,3 +336,44 @@ def test_cxx_optimize_ablations_and_deadlines_match_reference_optimize(k):
     assert clock.reads == case["clock_reads"]
     # the run ended on its deadline exactly when the deadline, not the budget, is what stopped the reference
     assert res["timed_out"] == ("deadline" in case and case["n_eval"] < case["E_max"])
+
+
+def test_a_deadline_run_is_a_prefix_of_the_budget_run():
+    """With one structural setting the wall clock only ends the search: what a run under a deadline evaluates is
+    the beginning of what the same run evaluates under its budgets alone, whatever the deadline; and its result is
+    the best of that beginning."""
+    cfg, batch = seeded_batch(1, 8)
+    p = cfg.problem
+    rpeg0 = p.template(0, ())
+    port = CpuPort(p)
+    _, plan_m, _ = batch.configuration(p, 0)
+    row = plan_row(rpeg0, ExecutionPlan(sigma={v: plan_m.sigma[u] for v, u in zip(rpeg0.vertices, plan_m.sigma)},
+                                        pi={v: plan_m.pi[u] for v, u in zip(rpeg0.vertices, plan_m.pi)},
+                                        mb={v: plan_m.mb[u] for v, u in zip(rpeg0.vertices, plan_m.mb)}))
+    arrays = _directory(p, rpeg0)[2]
+    opt = OptimizerConfig(K_x=6, T_max=50, E_max=400, E_struct=10 ** 6, T_init=0.05, T_warm=0.10, T_min=0.05, stag_window=4)
+
+    def run(deadline=None):
+        params = sa_params(opt, 1, 1, [(0, 0)], 0, 1, 42)
+        clock = _TickingClock()
+        if deadline is not None:
+            clock.install(params, deadline)
+        res = port.sa_optimize(params, arrays, row, opt.E_max, opt.E_struct, stream_key=(78, 9, 0), log_cap=4096, threads=4)
+        return res, clock
+    full, clock = run()
+    assert clock.reads == 0 and not full["timed_out"] and full["n_eval_log"] >= opt.E_max
+    seen = []
+    for deadline in (0.0, 3.0, 40.0, 41.0, 97.0, 10 ** 6):
+        res, clock = run(deadline)
+        n = res["n_eval_log"]
+        assert np.array_equal(res["eval_log"], full["eval_log"][:n])
+        assert np.array_equal(res["eval_log_score"].view(np.uint64), full["eval_log_score"][:n].view(np.uint64))
+        assert res["timed_out"] == (deadline < 10 ** 6) and (res["timed_out"] or n == full["n_eval_log"])
+        # the clock is read before every iteration and after every evaluated batch: the run ends on the reading that
+        # reaches the deadline
+        assert clock.reads == (deadline if 1.0 <= deadline < 10 ** 6 else clock.reads)
+        feasible = res["eval_log_feasible"]
+        if feasible.any():
+            assert res["best_feasible"] and res["best_score"] == res["eval_log_score"][feasible].max()
+        seen.append(n)
+    assert seen == sorted(seen) and seen[0] == 1 and seen[1] < seen[3] < seen[4] < seen[5]
