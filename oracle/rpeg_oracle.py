@@ -974,10 +974,9 @@ def alloc_devices(a):
 
 
 def device_peaks(nodes, mm):
-    """RPEG/model/memory.py:608-841, worker-liveness branch (trainable non-empty),
-    no fusion groups.  Returns {device: peak bytes} in first-touch order."""
-    if not mm.trainable:
-        raise NotImplementedError("oracle covers the worker-liveness model only (trainable non-empty)")
+    """RPEG/model/memory.py:608-841 without fusion groups: the worker-liveness model, or -- for a memory model
+    without trainable models -- the co-resident sum model (:706-742).  Returns {device: peak bytes} in first-touch
+    order."""
     per_dev = defaultdict(list)
     ops = []
     for nd in nodes:
@@ -996,6 +995,32 @@ def device_peaks(nodes, mm):
         overhead = len(keys) * (mm.worker_overhead + mm.act_cache)
         if mm.max_groups > 0 and len(keys) > mm.max_groups:
             peaks[dev] = math.inf
+            continue
+        if not mm.trainable:
+            # every model present keeps its static footprint (the largest shard among its nodes; optimizer state
+            # and gradients too where a training node of the model is present, at that node's dp), the nodes
+            # share the room for their transients
+            info = {}
+            for n in here:
+                trained = _role(n.tpl) == TRAIN
+                if n.model not in info:
+                    info[n.model] = [ws[id(n)], trained, n.pi[0]]
+                else:
+                    rec = info[n.model]
+                    rec[0] = max(rec[0], ws[id(n)])
+                    if trained:
+                        rec[1], rec[2] = True, n.pi[0]
+            static = 0
+            for m, (w, trained, dp) in info.items():
+                sb = mm.suite.specs[m].dtype_bytes
+                if trained:
+                    static = static + (sb * w + 12 * w / (dp if mm.stage >= 1 else 1) + sb * w / (dp if mm.stage >= 2 else 1))
+                else:
+                    static = static + sb * w
+            transient = 0.0
+            for n in here:
+                transient = max(transient, extra[id(n)])
+            peaks[dev] = overhead + static + transient
             continue
         opt = {}
         train_keys = defaultdict(set)

@@ -380,7 +380,9 @@ RPEG_HD int isqrt_small(int n) {
   return r;
 }
 
-RPEG_HD VMem vertex_memory(const rpeg_problem_t& P, const rpeg_vertex_t& vx, const VPlan& a) {
+// `dp_for_opt`: the co-resident sum model (memory.py:706-742) needs the vertex's dp where the worker-liveness model
+// needs its optimizer shard; the record then carries (double)dp in `opt`.
+RPEG_HD VMem vertex_memory(const rpeg_problem_t& P, const rpeg_vertex_t& vx, const VPlan& a, bool dp_for_opt = false) {
   const rpeg_model_t& md = P.model[vx.model];
   const int dp = a.dp, pp = a.pp, tp = a.tp;
   const int64_t emb = (int64_t)md.V * md.d, head = md.d;
@@ -396,7 +398,7 @@ RPEG_HD VMem vertex_memory(const rpeg_problem_t& P, const rpeg_vertex_t& vx, con
   const double sb = (double)md.sb;
   r.mem_w = (double)(r.w_shard * md.sb);
   int odp = P.optimizer_stage >= 1 ? dp : 1;
-  r.opt = (double)(12 * r.w_shard) / (double)odp;
+  r.opt = dp_for_opt ? (double)dp : (double)(12 * r.w_shard) / (double)odp;
   const double d = (double)md.d;
   const int64_t BK = (int64_t)P.B * P.K;
   const double b_local = (double)BK / (double)((int64_t)dp * a.mb);
@@ -459,7 +461,14 @@ struct StructMasks {
   uint8_t train_same[RPEG_MAX_V];   // TRAIN vertices of v's model
   uint8_t before[RPEG_MAX_V];       // vertices that precede order[i] in first-appearance order
   uint8_t train, trainable;         // TRAIN vertices; vertices of trainable models
+  bool coresident;                  // the memory model lists no trainable model at all: co-resident sum model
 };
+// NodeMemoryModel.trainable is empty (memory.py:647: `use_worker_liveness_model = len(mem_model.trainable) > 0`)
+RPEG_HD bool struct_coresident(const rpeg_struct_t& st) {
+  bool any = false;
+  for (unsigned m = 0; m < sizeof(st.mem_trainable); ++m) any = any || st.mem_trainable[m] != 0;
+  return !any;
+}
 RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) {
   StructMasks m;
   m.train = m.trainable = 0;
@@ -475,6 +484,7 @@ RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) 
       }
   }
   for (int i = 0; i < st.n_vertex; ++i) { m.before[i] = (uint8_t)seen; seen |= 1u << order[i]; }
+  m.coresident = struct_coresident(st);
   return m;
 }
 
@@ -508,6 +518,35 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
     const int v = order[i];
     if (!((M >> v) & 1u)) continue;
     if ((mask_row(pm.eq, v) & M & sm.same_model[v] & sm.before[i]) == 0) ++groups;
+  }
+  if (sm.coresident) {
+    // memory.py:706-742: every model present keeps its static footprint -- its largest shard among the vertices
+    // here; with a training vertex of the model here also optimizer state and gradients at that vertex's dp (the
+    // last such vertex in node order) -- summed in order of first appearance; the transients share their room.
+    // vm.opt(v) carries dp of vertex v in this mode.
+    double stat = 0.0, transient = 0.0;
+    for (int i = 0; i < nv; ++i) {
+      const int v = order[i];
+      if (!((M >> v) & 1u)) continue;
+      transient = dmax(transient, vm.extra(v));
+      const unsigned same = M & sm.same_model[v];
+      if (same & sm.before[i]) continue;   // the model's entry exists
+      double wmax = 0.0, dp = vm.opt(v);
+      bool trained = false;
+      for (int j = 0; j < nv; ++j) {
+        const int w = order[j];
+        if (!((same >> w) & 1u)) continue;
+        wmax = dmax(wmax, vm.w_shard(w));
+        if ((sm.train >> w) & 1u) { trained = true; dp = vm.opt(w); }
+      }
+      const double sbw = (double)P.model[st.vertex[v].model].sb * wmax;
+      double x = sbw;
+      if (trained) x = (sbw + 12.0 * wmax / (P.optimizer_stage >= 1 ? dp : 1.0)) + sbw / (P.optimizer_stage >= 2 ? dp : 1.0);
+      stat += x;
+    }
+    double peak = ((double)groups * P.group_overhead + stat) + transient;
+    if (P.max_groups > 0 && groups > P.max_groups) peak = __builtin_inf();
+    return peak;
   }
   for (int i = 0; i < nv; ++i) {  // optimizer shards of the training vertices
     const int v = order[i];

@@ -220,10 +220,11 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
 
   KE_STAMP(2);
   // ---- memory model and gates (plan fields in LDS are dead after this point)
+  const bool coresident = struct_coresident(st);
 #pragma unroll
   for (int v = 0; v < RPEG_MAX_V; ++v)
     if (v < nv) {
-      const VMem m = vertex_memory(P, st.vertex[v], a[v]);
+      const VMem m = vertex_memory(P, st.vertex[v], a[v], coresident);
       l_vm[(v * 4 + 0) * RW] = (double)m.w_shard;
       l_vm[(v * 4 + 1) * RW] = m.mem_w;
       l_vm[(v * 4 + 2) * RW] = m.opt;

@@ -421,6 +421,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
 struct KpOrdered {
   unsigned long long ovl, eq, same_model, train_same;
   unsigned train, trainable;
+  bool coresident;
 };
 __device__ inline unsigned kp_row(unsigned long long m, int i) { return (unsigned)(m >> (8 * i)) & 0xFFu; }
 
@@ -448,6 +449,31 @@ __device__ inline double kp_class_peak(const rpeg_problem_t& P, const rpeg_struc
   for (int i = 0; i < RPEG_MAX_V; ++i) {   // distinct (model, allocation) worker keys
     if (!((M >> i) & 1u)) continue;
     if ((kp_row(om.eq, i) & M & kp_row(om.same_model, i) & ((1u << i) - 1u)) == 0) ++groups;
+  }
+  if (om.coresident) {   // the co-resident sum model, as in device_class_peak (vm[i * 4 + 2] carries dp)
+    double stat = 0.0, transient = 0.0;
+#pragma unroll
+    for (int i = 0; i < RPEG_MAX_V; ++i) {
+      if (!((M >> i) & 1u)) continue;
+      transient = dmax(transient, vm[i * 4 + 3]);
+      const unsigned same = M & kp_row(om.same_model, i);
+      if (same & ((1u << i) - 1u)) continue;
+      double wmax = 0.0, dp = vm[i * 4 + 2];
+      bool trained = false;
+#pragma unroll
+      for (int q = 0; q < RPEG_MAX_V; ++q) {
+        if (!((same >> q) & 1u)) continue;
+        wmax = dmax(wmax, vm[q * 4 + 0]);
+        if ((om.train >> q) & 1u) { trained = true; dp = vm[q * 4 + 2]; }
+      }
+      const double sbw = (double)P.model[st.vertex[order[i]].model].sb * wmax;
+      double x = sbw;
+      if (trained) x = (sbw + 12.0 * wmax / (P.optimizer_stage >= 1 ? dp : 1.0)) + sbw / (P.optimizer_stage >= 2 ? dp : 1.0);
+      stat += x;
+    }
+    double peak = ((double)groups * P.group_overhead + stat) + transient;
+    if (P.max_groups > 0 && groups > P.max_groups) peak = __builtin_inf();
+    return peak;
   }
 #pragma unroll
   for (int i = 0; i < RPEG_MAX_V; ++i)     // optimizer shards of the training vertices
@@ -651,9 +677,10 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   // One vertex per lane, then one vertex subset per lane tests whether it is a device class (a maximal clique
   // of the overlap graph); the few that are get evaluated one after the other with uniform control flow.
   const uint8_t* order = cv.h->vorder;
+  const bool coresident = struct_coresident(st);
   if (lane < nv) {
     const int v = order[lane];
-    const VMem m = vertex_memory(P, st.vertex[v], ke_vplan<1>(l_plan, v));
+    const VMem m = vertex_memory(P, st.vertex[v], ke_vplan<1>(l_plan, v), coresident);
     l_vm[lane * 4 + 0] = (double)m.w_shard;
     l_vm[lane * 4 + 1] = m.mem_w;
     l_vm[lane * 4 + 2] = m.opt;
@@ -673,6 +700,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     const unsigned long long t = __ballot(valid && j == 0 && xi.role == RPEG_ROLE_TRAIN),
                              tr = __ballot(valid && j == 0 && st.mem_trainable[xi.model] != 0);   // bit 8i: position i
     om.train = om.trainable = 0u;
+    om.coresident = coresident;
 #pragma unroll
     for (int q = 0; q < RPEG_MAX_V; ++q) {
       om.train |= (unsigned)((t >> (8 * q)) & 1ull) << q;

@@ -97,7 +97,8 @@ RPEG_HD PlanOut eval_plan(const rpeg_problem_t& P, const ClassView& c, const Pla
   double makespan = 0.0;
   if (!err) makespan = list_schedule(c, mem, ovl, pm.dpne, st.n_vertex, ready_cap, &err);
   VMem vm[RPEG_MAX_V];
-  for (int v = 0; v < st.n_vertex; ++v) vm[v] = vertex_memory(P, st.vertex[v], a[v]);
+  const bool coresident = struct_coresident(st);
+  for (int v = 0; v < st.n_vertex; ++v) vm[v] = vertex_memory(P, st.vertex[v], a[v], coresident);
   const VMemArray vma{vm};
   const double peak = device_peak_max(P, st, c.h->vorder, pm, vma);
   const bool stale_ok = stale_layout_ok(st, h, pm.ovl);

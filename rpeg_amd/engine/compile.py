@@ -136,8 +136,10 @@ def compile_problem(problem: EvalProblem) -> abi.ProblemT:
     P.n_struct, P.n_split, P.K_eval = len(problem.structures), problem.n_splits(), problem.K_eval
     if P.n_split > abi.MAX_SPLIT:
         raise ValueError(f"at most {abi.MAX_PH} generation quantiles are supported")
-    if problem.K_eval < 1 or problem.K_eval > 64:
-        raise ValueError("K_eval must be in 1..64")
+    if problem.K_eval < 1 or problem.K_eval > 4095:
+        # (what bounds the horizon is the size of a lowered graph: 4,095 nodes per class, reported by the engine
+        # when a plan's class exceeds it -- a few hundred steps, depending on the template)
+        raise ValueError("K_eval must be in 1..4095")
     P.R, P.N, P.G = sp.R, sp.N, sp.G
     P.B, P.K, P.S, P.T = wl.B, wl.K, wl.S, wl.T
     P.optimizer_stage, P.ckpt = pol.optimizer_stage, int(pol.activation_checkpointing)

@@ -375,8 +375,7 @@ def is_valid(config: Configuration, suite: ModelSuite, workload: Workload, mem_m
     for v in config.rpeg.vertices:
         if v not in plan.sigma or v not in plan.pi or v not in plan.mb:
             return False
-    if not mem_model.trainable:
-        raise NotImplementedError("the co-resident memory model (no trainable model) is not part of this engine")
+    # (a memory model without trainable models is the reference's co-resident sum model, memory.py:706-742)
     eng, st = _engine_for(config.rpeg, suite, workload, mem_model.hw, config.device_space, 1, mem_model.policy,
                           memory_trainable=mem_model.trainable)
     mask = int(eng.eval(_pack([config], st, workload), gate_stale=False)["mask"][0])

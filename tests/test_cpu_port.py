@@ -149,3 +149,23 @@ def test_bench_flop_constants_follow_a_fresh_count(c):
     assert abs(got["total"] - bench.ALG_FLOPS[c]) <= 0.03 * bench.ALG_FLOPS[c], (got, bench.ALG_FLOPS[c])
     # the count is dominated by the scheduler's comparisons, as the kernels' instruction mix is
     assert got["cmp"] > got["add"] + got["mul"] + got["div"]
+
+
+@pytest.mark.parametrize("c,K", [(1, 100), (2, 100), (4, 128)])
+def test_port_matches_oracle_at_long_horizons(c, K):
+    """Horizons as the runtime's planner asks for them (runtime/job_plan.py:170-214): the host build of the kernels'
+    arithmetic against the Python restatement on graphs of 800-3,000 lowered nodes (for DPO with 128 entries ready at
+    once: the host build's list is not bounded as the GPU's is)."""
+    import dataclasses
+    cfg, batch = seeded_batch(c, 6, start=300_000)
+    p = dataclasses.replace(cfg.problem, K_eval=K)
+    out = CpuPort(p).eval(batch, flags=abi.GATE_STALE)
+    n_checked = 0
+    for i in range(6):
+        if not out["mask"][i] & abi.MASK_VALID:
+            continue
+        rpeg, plan, wl = batch.configuration(p, i)
+        want = oracle.evaluate_plan(rpeg, plan, p.device_space, p.suite, wl, p.hw, K, p.memory_policy, check_stale=True)
+        assert out["makespan"][i] == want["makespan"] and out["peak"][i] == want["peak"] and out["score"][i] == want["score"], i
+        n_checked += 1
+    assert n_checked >= 2

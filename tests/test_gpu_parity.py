@@ -561,6 +561,29 @@ def test_transfer_resource_policies_equal_reference(c):
             assert float(trace.utilization()).hex() == want["utilization"], (i, pol)
 
 
+def test_a_horizon_beyond_the_ready_list_is_reported_as_a_limit():
+    """DPO's unrolled steps are independent of each other, so every step's first node is ready at time zero: at a
+    horizon of 128 steps the ready list would need 128 entries.  The engine says so (MASK_ERROR | MASK_LIMIT, NaN),
+    it does not return a number; the host build, whose list is unbounded in this range, evaluates the plans."""
+    from dataclasses import replace
+    from rpeg_amd.engine.runtime import Engine
+    cfg, batch = seeded_batch(4, 2048)
+    for K, limited in ((24, False), (128, True)):
+        p = replace(cfg.problem, K_eval=K)
+        eng = Engine(p)
+        out = eng.eval(batch)
+        valid = (out["mask"] & abi.MASK_VALID) != 0
+        assert valid.sum() > 1000
+        assert np.all(((out["mask"][valid] & abi.MASK_LIMIT) != 0) == limited)
+        assert np.all(np.isnan(out["score"][valid]) == limited)
+        if not limited:
+            ref = CpuPort(p).eval(batch, flags=abi.GATE_STALE, threads=16)
+            assert same_bits(out["score"], ref["score"]) and np.array_equal(out["mask"], ref["mask"])
+        eng.close()
+    with pytest.raises(ValueError, match="K_eval"):
+        Engine(replace(cfg.problem, K_eval=5000))
+
+
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_utilization_from_the_batched_launch_equals_reference(c):
     """Trace.utilization() as a further output of the batched launch (rpeg_eval_host_util, folded inside k_plan)
@@ -613,6 +636,8 @@ def test_other_seeds_unroll_depths_and_policies_equal_the_host_build(c):
              (7, ("both_endpoints", "both_endpoints"))]
     if c in (1, 2, 4):   # a long horizon, as the runtime's planner schedules (runtime/job_plan.py:174-213)
         cases.append((32, ("destination_only", "destination_only")))
+    if c in (1, 2, 3):   # and a longer one: graphs of 1,500-3,000 lowered nodes
+        cases.append((100, ("destination_only", "destination_only")))
     for K, pol in cases:
         p = replace(cfg.problem, K_eval=K, transfer_resource_policy=TransferResourcePolicy(*pol))
         eng, port = Engine(p), CpuPort(p)
