@@ -728,3 +728,17 @@ def test_problems_away_from_the_shipped_configurations_equal_reference():
         for k in ("makespan", "peak", "score"):
             assert same_bits(got[k], want[k]), (name, k)
         assert np.array_equal(got["mask"], want["mask"]), name
+
+
+def test_profile_tool_runs(capsys):
+    """python -m rpeg_amd.engine.profile: the per-wavefront clocks of both kernels on a small seeded set."""
+    import sys
+    from rpeg_amd.engine import profile
+    argv = sys.argv
+    sys.argv = ["profile", "--config", "2", "--plans", "40000"]
+    try:
+        profile.main()
+    finally:
+        sys.argv = argv
+    text = capsys.readouterr().out
+    assert "k_eval:" in text and "k_plan:" in text and "phases, mean us per task" in text and "longest tasks" in text
