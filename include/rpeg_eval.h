@@ -392,7 +392,7 @@ int rpeg_sa_propose(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t what,
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,
    [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace; 1: one plan per
    wavefront), [6] plans of a large batch that ran one per wavefront beside the main kernel (included
-   in [2]). */
+   in [2]), [7] wave tasks of the four-lanes-per-plan kernel (included in [2]). */
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
 
 /* Where the evaluation kernel keeps the scheduler state of a plan (ready time, rank and remaining
@@ -401,9 +401,19 @@ int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
    layout: a batch too small to fill the chip finishes sooner); fails at the next call when the state
    of the problem's largest class does not fit.  lanes = 1: one plan per wavefront, its nodes spread
    over the lanes (the layout of lowest latency, for batches of a few thousand plans at most; classes of
-   up to 384 nodes).  lanes = -1 (default): chosen per batch from its size.
+   up to 384 nodes).  lanes = 4: four lanes per plan, sixteen plans per wavefront, the ready entries (at most 32
+   at once) in the registers of the four lanes (the layout for dense graphs, whose plan-per-lane wavefronts end
+   last).
+   lanes = -1 (default): chosen per batch from its size.
    Results do not depend on the setting. */
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
+
+/* With lanes = -1 and a batch that fills the chip in one round of wavefronts: the largest share of the batch's
+   plans, in percent, that the four-lanes-per-plan kernel may take on a stream of its own (default 25; 0: none).
+   Which classes it takes is learned: the main kernel records, per class, how long its slowest wavefront ran and how
+   many heap pops per dispatch it needed, and from the second call on the classes that would end last there (dense
+   graphs) are moved.  Results do not depend on the setting.  No reference counterpart (a tuning knob). */
+int rpeg_engine_set_quad_share(rpeg_engine_t* e, int32_t percent);
 
 /* Ready-list entries per plan in the main kernel: 8, 16, 24 or 32 (default).  A plan with that many nodes
    ready at once is not evaluated: NaN outputs, RPEG_MASK_ERROR | RPEG_MASK_LIMIT (the reference's heap has no

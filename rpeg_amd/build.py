@@ -11,7 +11,7 @@ LIB = os.path.join(HERE, "librpeg_eval.so")
 SOURCES = [os.path.join(HERE, "csrc", "rpeg_engine.hip")]
 HEADERS = [os.path.join(HERE, "csrc", f) for f in
            ("rpeg_core.h", "rpeg_class.h", "rpeg_lower.h", "rpeg_plan.h", "rpeg_sa.h", "rpeg_kernel_eval.h",
-            "rpeg_kernel_plan.h", "rpeg_exp_table.inc")] + \
+            "rpeg_kernel_plan.h", "rpeg_kernel_quad.h", "rpeg_exp_table.inc")] + \
           [os.path.join(HERE, "..", "include", "rpeg_eval.h")]
 
 # -ffp-contract=off: scores must equal the reference's Python floats, which never fuse a*b+c.

@@ -81,6 +81,7 @@ struct ClassHdr {
   uint32_t off_pbeg, off_pred;       // predecessor lists in edge order: pred[pbeg[v] .. pbeg[v+1])
   uint32_t bytes;
   uint32_t structure, split, error;  // error != 0: the reference would raise for this class
+  uint32_t id;                       // index of the class in the tables of the engine that holds it (0 elsewhere)
   uint8_t vorder[8];                 // vertices by first appearance among the lowered operator nodes
 };
 

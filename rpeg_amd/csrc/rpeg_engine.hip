@@ -26,6 +26,7 @@
 
 #include "rpeg_kernel_eval.h"
 #include "rpeg_kernel_plan.h"
+#include "rpeg_kernel_quad.h"
 #include "rpeg_lower.h"
 #include "rpeg_plan.h"
 #include "rpeg_sa.h"
@@ -268,6 +269,14 @@ __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
   }
 }
 
+// Four lanes per plan, sixteen plans per wavefront (rpeg_kernel_quad.h); tasks and permutation as for k_eval.
+// At most 128 vector registers, so that a wavefront of it fits beside one of the main kernel and one of k_plan on a
+// SIMD (the cost model spills a little; the scheduling loop does not).
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(4, 8))) void k_quad(const EvalLaunch L) {
+  extern __shared__ uint8_t kq_lds[];
+  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) kq_eval_wave(L, w, kq_lds);
+}
+
 // One plan per wavefront (rpeg_kernel_plan.h); perm[w] is the plan of wavefront task w.
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(4, 8))) void k_plan(const EvalLaunch L) {
   extern __shared__ uint8_t kp_lds[];
@@ -382,7 +391,13 @@ struct rpeg_engine_s {
   // lowering classes
   std::unordered_map<uint64_t, uint32_t> class_off;  // signature -> byte offset in the pool
   std::vector<uint64_t> cls_sig;                     // class id -> signature / pool offset / node count
-  std::vector<uint32_t> cls_off, cls_nodes;
+  std::vector<uint32_t> cls_off, cls_nodes, cls_slots;
+  std::vector<uint32_t> cls_pops16;                  // learned, of the slowest full wavefront of the class in the main kernel:
+                                                     // microseconds << 12 | heap pops per dispatch in sixteenths
+  uint32_t* d_cstat = nullptr;                       // the device's copy, written by the main kernel
+  uint32_t cstat_cap = 0;
+  uint32_t learn_calls = 0;                          // calls left after which the statistic is read back
+  uint64_t batch_calls = 0;
   uint64_t* d_hkey = nullptr;                        // device table signature -> class id
   uint32_t* d_hval = nullptr;
   uint32_t* d_hoff = nullptr;                        // the same slots -> pool offset of the class blob
@@ -426,6 +441,10 @@ struct rpeg_engine_s {
   uint32_t max_v = RPEG_MAX_V;   // largest vertex count of the problem's structures
   hipStream_t s2 = nullptr;                     // second stream: single-plan wavefronts of a large batch run beside the others
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  hipStream_t s3 = nullptr;                     // third stream: the four-lanes-per-plan wavefronts (k_quad)
+  hipEvent_t ev_join3 = nullptr;
+  uint32_t quad_share_pct = 25;                 // share of a full batch that k_quad takes (rpeg_engine_set_quad_share)
+  bool quad_attr_set = false;
   int split_heavy = 1;                          // 0: the classes with the largest graphs stay in the main kernel
   uint64_t* d_sig = nullptr;
   uint64_t* h_sig = nullptr;
@@ -436,7 +455,7 @@ struct rpeg_engine_s {
   bool timing = false;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   double last_ms = -1.0;
-  uint64_t stats[7] = {0, 0, 0, 0, 0, 0, 0};
+  uint64_t stats[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   int n_cu = 256;
   uint8_t* static_ptr = nullptr;    // this device's copy of the file-scope scratch array (rpeg_eval_batch_static)
   uint32_t* h_static = nullptr;     // pinned: the counters of that array, read back after a call
@@ -502,6 +521,15 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
     HIP_TRY(e, hipHostMalloc(&e->h_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4));
     e->ccap = cap;
   }
+  if (ncls > e->cstat_cap) {   // the per-class statistic keeps what it has learned
+    const uint32_t cap = std::max<uint32_t>(2 * ncls, 4096);
+    if (e->d_cstat) hipFree(e->d_cstat);
+    e->d_cstat = nullptr; e->cstat_cap = 0;
+    HIP_TRY(e, hipMalloc(&e->d_cstat, (size_t)cap * 4));
+    HIP_TRY(e, hipMemset(e->d_cstat, 0, (size_t)cap * 4));
+    HIP_TRY(e, hipMemcpy(e->d_cstat, e->cls_pops16.data(), (size_t)ncls * 4, hipMemcpyHostToDevice));
+    e->cstat_cap = cap;
+  }
   e->tables_for = ncls;
   return 0;
 }
@@ -558,10 +586,14 @@ static int64_t class_append(rpeg_engine_t* e, uint64_t sig, const LoweredClass& 
   if (e->pool.size() + lc.blob.size() >= (1ull << 31)) { e->err = "class pool exceeds 2 GiB"; return -1; }   // bit 31 of an offset is a flag
   uint32_t off = (uint32_t)e->pool.size();
   e->pool.insert(e->pool.end(), lc.blob.begin(), lc.blob.end());
+  ((ClassHdr*)(e->pool.data() + off))->id = (uint32_t)e->cls_sig.size();
   e->class_off.emplace(sig, off);
   e->cls_sig.push_back(sig);
   e->cls_off.push_back(off);
   e->cls_nodes.push_back(h->n_nodes);
+  e->cls_slots.push_back(h->n_slots);
+  e->cls_pops16.push_back(0);
+  e->learn_calls = 3;
   return off;
 }
 
@@ -681,6 +713,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_pool) hipFree(e->d_pool);
   if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
   if (e->d_need) hipFree(e->d_need);
+  if (e->d_cstat) hipFree(e->d_cstat);
   if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); hipFree(e->d_hoff); }
   if (e->h_static) hipHostFree(e->h_static);
   if (e->d_ccount) {
@@ -690,6 +723,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_perm) hipFree(e->d_perm);
   if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
   if (e->s2) { hipStreamDestroy(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
+  if (e->s3) { hipStreamDestroy(e->s3); hipEventDestroy(e->ev_join3); }
   if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
   if (e->d_stage) hipFree(e->d_stage);
   if (e->h_stage) hipHostFree(e->h_stage);
@@ -725,11 +759,18 @@ int rpeg_engine_profile(rpeg_engine_t* e, int32_t enable, unsigned long long* ou
 
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
   if (!e) return -1;
-  if (lanes != -1 && lanes != 0 && lanes != 1 && lanes != 8 && lanes != 16 && lanes != 32 && lanes != 64) {
-    e->err = "state lanes must be -1, 0, 1, 8, 16, 32 or 64";
+  if (lanes != -1 && lanes != 0 && lanes != 1 && lanes != 4 && lanes != 8 && lanes != 16 && lanes != 32 && lanes != 64) {
+    e->err = "state lanes must be -1, 0, 1, 4, 8, 16, 32 or 64";
     return -1;
   }
   e->state_lanes = lanes;
+  return 0;
+}
+
+int rpeg_engine_set_quad_share(rpeg_engine_t* e, int32_t percent) {
+  if (!e) return -1;
+  if (percent < 0 || percent > 100) { e->err = "the share is a percentage"; return -1; }
+  e->quad_share_pct = (uint32_t)percent;
   return 0;
 }
 
@@ -750,6 +791,9 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
   e->cls_sig.clear();
   e->cls_off.clear();
   e->cls_nodes.clear();
+  e->cls_slots.clear();
+  e->cls_pops16.clear();
+  if (e->d_cstat) { hipFree(e->d_cstat); e->d_cstat = nullptr; e->cstat_cap = 0; }
   e->cls_sorted.clear();
   e->tables_for = 0xFFFFFFFFu;
   e->pool.clear();
@@ -759,7 +803,7 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
 
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n) {
   if (!e || !out) return -1;
-  for (int i = 0; i < n && i < 7; ++i) out[i] = e->stats[i];
+  for (int i = 0; i < n && i < 8; ++i) out[i] = e->stats[i];
   return 0;
 }
 
@@ -811,7 +855,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
                        e->d_kidx, e->d_ccount, ncls, shards, e->d_need);
     HIP_TRY(e, hipGetLastError());
     HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, (n_count + KE_NEED_SHARDS) * 4, hipMemcpyDeviceToHost, s));
+    // what earlier launches of the main kernel learned about the classes (pops per dispatch): read in the calls
+    // that follow new classes, and now and then afterwards
+    const bool read_stat = round == 0 && e->quad_share_pct && ncls && (e->learn_calls > 0 || (e->batch_calls & 63) == 0);
+    if (read_stat) HIP_TRY(e, hipMemcpyAsync(e->cls_pops16.data(), e->d_cstat, (size_t)ncls * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
+    if (read_stat && e->learn_calls > 0) --e->learn_calls;
     for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_ccount[n_count + q]);
     if (e->h_ccount[n_count - 1] == 0) break;
     if (round >= 2) { e->err = "class table did not converge"; return -5; }
@@ -827,6 +876,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     }
     if (int rc = lower_new_classes(e, sigs, &n_new)) return rc;
   }
+  ++e->batch_calls;
   std::vector<uint32_t> offs, counts, cids;   // the classes present in this batch
   for (uint32_t c = 0; c < ncls; ++c) {   // per-shard counts become the shards' offsets within the class
     uint32_t total = 0;
@@ -842,6 +892,14 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // wavefronts of fewer plans whose state fits in LDS, which shortens every scheduler step.
   int ls = e->state_lanes;
   bool one = false;   // one plan per wavefront (k_plan)
+  const bool quad_all = ls == 4;   // every class in the four-lanes-per-plan kernel (k_quad)
+  if (quad_all) {
+    ls = 0;
+    if (kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, e->max_nodes, e->max_slots, e->max_v, (uint32_t)KQ_PLANS) > 160 * 1024) {
+      e->err = "per-plan state of this problem does not fit in LDS with sixteen plans per wavefront";
+      return -8;
+    }
+  }
   {
     auto waves_for = [&](uint32_t per) { uint64_t t = 0; for (uint32_t c : counts) t += (c + per - 1) / per; return t; };
     auto fits = [&](int l) {
@@ -887,8 +945,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // first[c]: first wavefront of class c in launch order (first permutation entry for a class of
   // single-plan wavefronts, which follow the others in the permutation and in the task list)
   std::vector<uint32_t> first(counts.size(), 0), clpw(counts.size(), lpw);
-  std::vector<uint8_t> solo(counts.size(), 0);
-  if (!ls && !one && !order.empty()) {
+  std::vector<uint8_t> solo(counts.size(), 0), quad(counts.size(), quad_all ? 1 : 0);
+  uint32_t quad_nodes = quad_all ? e->max_nodes : 0, quad_slots = quad_all ? e->max_slots : 0;
+  if (!ls && !one && !quad_all && !order.empty()) {
     // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
     // classes with the largest graphs (up to 15 % of the batch: beyond that the single-plan kernel would be
     // the one that ends last) are taken out of it, unless the batch is
@@ -901,7 +960,14 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     const bool split = e->split_heavy && one_fits;
     // node count from which a class counts as large: the smallest one, not under `floor` percent of the
     // largest, such that the large classes hold at most `share` percent of the batch
-    const uint64_t floor_pct = split ? 60ull : 70ull, share_pct = split ? 15ull : 25ull;
+    // (ten percent when k_quad takes the dense classes: a plan costs k_plan four times the instructions)
+    const uint64_t floor_pct = split ? 60ull : 70ull;
+    uint64_t share_pct = split ? 15ull : 25ull;
+    {
+      uint64_t w64 = 0;
+      for (uint32_t c : counts) w64 += (c + WAVE - 1) / WAVE;
+      if (split && e->quad_share_pct && w64 <= (uint64_t)e->n_cu * 6) share_pct = 10;
+    }
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t waves64 = 0;
     for (uint32_t c : counts) waves64 += (c + WAVE - 1) / WAVE;
@@ -933,16 +999,55 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (split)
       for (size_t c = 0; c < counts.size(); ++c)
         if (counts[c] < TINY_CLASS) solo[c] = 1;
+    // Of what stays, the wavefronts that end last are those of dense graphs (long ready lists, keys that go stale
+    // often).  The main kernel measures itself: per class, the time of its slowest wavefront on earlier launches and
+    // the heap pops per dispatch it needed (cls_pops16).  A wavefront of k_quad takes about 75 + nodes x (2.3 +
+    // 0.45 per pop) microseconds (fitted).  The classes are taken in the order of their measured time while one still
+    // ends later in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct` percent of
+    // the batch.  Nothing is known before the first launch of a class: it stays in the main kernel then.
+    if (split && e->quad_share_pct && waves64 <= (uint64_t)e->n_cu * 6) {
+      auto t_main = [&](uint32_t c) { return (double)(e->cls_pops16[cids[c]] >> 12); };
+      auto t_quad = [&](uint32_t c) {
+        const double nd = e->cls_nodes[cids[c]], p = (e->cls_pops16[cids[c]] & 0xFFFu) / 16.0;
+        return 75.0 + nd * (2.3 + 0.45 * p);
+      };
+      std::vector<uint32_t> cand;
+      for (uint32_t c = 0; c < counts.size(); ++c)
+        if (!solo[c] && e->cls_pops16[cids[c]]) cand.push_back(c);
+      std::sort(cand.begin(), cand.end(), [&](uint32_t x, uint32_t y) { return t_main(x) > t_main(y); });
+      double slowest_quad = 0.0;
+      uint64_t taken = 0;
+      for (uint32_t c : cand) {
+        const double tq = std::max(slowest_quad, t_quad(c));
+        if (t_main(c) <= tq) break;
+        if ((taken + counts[c]) * 100 > (uint64_t)n * e->quad_share_pct) break;
+        const uint32_t nodes = e->cls_nodes[cids[c]], slots = e->cls_slots[cids[c]];
+        if (kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, std::max(quad_nodes, nodes), std::max(quad_slots, slots), e->max_v, (uint32_t)KQ_PLANS) > 64 * 1024) continue;
+        quad[c] = 1;
+        taken += counts[c];
+        slowest_quad = tq;
+        quad_nodes = std::max(quad_nodes, nodes);
+        quad_slots = std::max(quad_slots, slots);
+      }
+    }
   }
-  uint32_t n_eval_waves = 0, n_solo = 0;
+  uint32_t n_eval_waves = 0, n_quad_waves = 0, n_solo = 0;
   for (size_t k = 0; k < order.size(); ++k) {
     const uint32_t c = order[k];
-    if (solo[c]) continue;
+    if (solo[c] || quad[c]) continue;
     first[c] = n_eval_waves;
     n_eval_waves += (counts[c] + clpw[c] - 1) / clpw[c];
   }
+  for (size_t k = 0; k < order.size(); ++k) {   // the tasks of k_quad follow those of the main kernel
+    const uint32_t c = order[k];
+    if (!quad[c]) continue;
+    clpw[c] = (uint32_t)(uint32_t)KQ_PLANS;
+    first[c] = n_eval_waves + n_quad_waves;
+    n_quad_waves += (counts[c] + clpw[c] - 1) / clpw[c];
+  }
+  const uint32_t n_lane_waves = n_eval_waves + n_quad_waves;
   const uint32_t pstride = one ? 1u : (uint32_t)WAVE;
-  const uint64_t n_sorted = (uint64_t)n_eval_waves * pstride;   // permutation entries of the main kernel
+  const uint64_t n_sorted = (uint64_t)n_lane_waves * pstride;   // permutation entries of the main kernel and k_quad
   for (size_t k = 0; k < order.size(); ++k) {
     const uint32_t c = order[k];
     if (!solo[c]) continue;
@@ -954,7 +1059,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   e->stats[1] = n_new;
   e->stats[6] = 0;
   if (n_sorted + n_solo == 0) return 0;
-  if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_eval_waves + n_solo)) return rc;
+  if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_lane_waves + n_solo)) return rc;
   uint32_t* const h_cfirst = e->h_ccount + (size_t)ncls * shards;   // behind the shard offsets
   uint32_t* const h_clpw = h_cfirst + ncls;
   uint32_t* const h_coff = h_clpw + ncls;
@@ -963,7 +1068,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   const uint32_t* const d_coff = d_clpw + ncls;
   // tasks of one plan get their class from the scatter kernel, not from the host: with one plan per wavefront
   // throughout that is every task of the launch, otherwise the tasks of the classes taken out of the main kernel
-  const uint32_t n_host_tasks = one ? 0u : n_eval_waves;
+  const uint32_t n_host_tasks = one ? 0u : n_lane_waves;
   // their class offsets ride behind the per-class tables when the block has room, else in a copy of their own
   const size_t block_words = (size_t)ncls * shards + 3 * (size_t)ncls;
   const bool tasks_in_block = block_words + n_host_tasks <= 4 * (size_t)e->ccap + COUNT_SLOTS;
@@ -987,7 +1092,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (solo[c] || one) {
       continue;
     } else {
-      const uint32_t flag = few_in_lds && clpw[c] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
+      // (never for a task of k_quad, whose eight plans of eight lanes each are not that layout)
+      const uint32_t flag = !quad[c] && few_in_lds && clpw[c] == (uint32_t)KE_FEW ? KE_CLS_LDS : 0u;
       const uint32_t nw = (counts[c] + clpw[c] - 1) / clpw[c];
       for (uint32_t t = 0; t < nw; ++t) h_tasks[first[c] + t] = offs[c] | flag;
     }
@@ -1004,7 +1110,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   const uint64_t n_waves = n_eval_waves;
   const unsigned grid = (unsigned)std::min<uint64_t>(std::max<uint64_t>(n_waves, 1), (uint64_t)e->n_cu * (one ? 32 : 16));
   const size_t wsb = ls || one ? 0 : ke_ws_bytes(e->max_nodes, e->max_slots);
-  if (!ls && !one)
+  if (!ls && !one && n_waves)
     if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
   EvalLaunch L;
   L.P = e->dP; L.vert = plans->vert; L.head = plans->head; L.stride = plans->stride;
@@ -1020,14 +1126,15 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // an overflow is final (RPEG_MASK_LIMIT), and a flag left standing would be redone by a later call's fix-up.
   L.ovf = short_list ? e->d_ovf : nullptr;
   L.need = !ls && !one ? e->d_need : nullptr;
+  L.cstat = !ls && !one && e->quad_share_pct ? e->d_cstat : nullptr;
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
   L.prof = nullptr;
   if (e->prof_on) {
     if (e->d_prof) hipFree(e->d_prof);
-    HIP_TRY(e, hipMalloc(&e->d_prof, (n_waves + n_solo) * 64));
-    HIP_TRY(e, hipMemsetAsync(e->d_prof, 0, (n_waves + n_solo) * 64, s));
-    e->prof_waves = n_waves + n_solo;
+    HIP_TRY(e, hipMalloc(&e->d_prof, (n_waves + n_quad_waves + n_solo) * 64));
+    HIP_TRY(e, hipMemsetAsync(e->d_prof, 0, (n_waves + n_quad_waves + n_solo) * 64, s));
+    e->prof_waves = n_waves + n_quad_waves + n_solo;
     L.prof = e->d_prof;
   }
   const size_t lds = one ? kp_lds_bytes(e->max_nodes, e->max_slots)
@@ -1040,7 +1147,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     HIP_TRY(e, hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     e->lds_attr_set[ki] = true;
   }
-  e->stats[2] = n_waves + n_solo;
+  e->stats[2] = n_waves + n_quad_waves + n_solo;
+  e->stats[7] = n_quad_waves;
   e->stats[3] = lds;
   e->stats[4] = wsb * grid;
   e->stats[5] = one ? 1u : (uint64_t)ls;
@@ -1048,13 +1156,35 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
   // The main kernel is submitted first: it needs 26 KB of LDS per wavefront, and once single-plan wavefronts
   // fill a compute unit its wavefronts only fit in as those retire.
-  if (n_solo) {
+  if (n_solo || n_quad_waves) {
     if (!e->s2) {
       HIP_TRY(e, hipStreamCreateWithFlags(&e->s2, hipStreamNonBlocking));
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_fork, hipEventDisableTiming));
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join, hipEventDisableTiming));
     }
+    if (n_quad_waves && !e->s3) {
+      HIP_TRY(e, hipStreamCreateWithFlags(&e->s3, hipStreamNonBlocking));
+      HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join3, hipEventDisableTiming));
+    }
     HIP_TRY(e, hipEventRecord(e->ev_fork, s));
+  }
+  if (n_quad_waves) {   // the four-lanes-per-plan wavefronts, beside the main kernel
+    EvalLaunch Q = L;
+    Q.perm = e->d_perm + (uint64_t)n_eval_waves * WAVE;
+    Q.wave_cls = L.wave_cls + n_eval_waves;
+    Q.n_waves = n_quad_waves;
+    Q.ws_nodes = quad_nodes; Q.ws_slots = quad_slots;
+    Q.ovf = nullptr; Q.need = nullptr; Q.cstat = nullptr;   // (32 entries are as many as the main kernel's full list holds: an overflow is final)
+    if (L.prof) Q.prof = L.prof + n_waves * 8;
+    const size_t qlds = kq_lds_bytes(L.cls_bytes, quad_nodes, quad_slots, e->max_v, (uint32_t)KQ_PLANS);
+    if (qlds > 64 * 1024 && !e->quad_attr_set) {
+      HIP_TRY(e, hipFuncSetAttribute((const void*)k_quad, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      e->quad_attr_set = true;
+    }
+    HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
+    hipLaunchKernelGGL(k_quad, dim3((unsigned)std::min<uint64_t>(n_quad_waves, (uint64_t)e->n_cu * 16)), dim3(WAVE), qlds, e->s3, Q);
+    HIP_TRY(e, hipGetLastError());
+    HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
   }
   if (n_waves == 0) {
   } else if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
@@ -1069,9 +1199,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (n_solo) {   // the single-plan wavefronts, beside the main kernel
     EvalLaunch S = L;
     S.perm = e->d_perm + n_sorted;
-    S.wave_cls = e->d_cls + n_eval_waves;
+    S.wave_cls = e->d_cls + n_host_tasks;
     S.n_waves = n_solo;
-    if (L.prof) S.prof = L.prof + n_waves * 8;
+    if (L.prof) S.prof = L.prof + (n_waves + n_quad_waves) * 8;
     HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
     hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n_solo, (uint64_t)e->n_cu * 32)), dim3(WAVE),
                        kp_lds_bytes(e->max_nodes, e->max_slots), e->s2, S);
@@ -1093,6 +1223,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     hipLaunchKernelGGL(k_eval<0>, dim3(std::min<unsigned>(grid, (unsigned)e->n_cu * 2u)), dim3(WAVE), lds_full, s, F);
     HIP_TRY(e, hipGetLastError());
   }
+  if (n_quad_waves) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join3, 0));
   if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
   if (e->timing) {
     HIP_TRY(e, hipEventRecord(e->ev1, s));
@@ -1460,7 +1591,7 @@ static int eval_host_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* p
   const int16_t* vert = plans->vert;
   const uint8_t* head = plans->head;
   const uint64_t stride = plans->stride;
-  if (e->state_lanes != 0 && e->state_lanes < 8 && n <= (uint64_t)e->host_small_max) {
+  if ((e->state_lanes == -1 || e->state_lanes == 1) && n <= (uint64_t)e->host_small_max) {
     auto get = [&](uint64_t i, PlanHead& h, VPlan (&a)[RPEG_MAX_V]) {
       h = load_head(head, stride, i);
       const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;

@@ -56,6 +56,8 @@ struct EvalLaunch {              // uniform launch parameters
                                  // consumed by the KE_FIXUP launch with the full one), or null
   uint32_t* need;                // KE_NEED_SHARDS running maxima of the ready-list length, then one word that
                                  // counts the plans flagged in `ovf` and not yet redone; or null
+  uint32_t* cstat = nullptr;     // per class (ClassHdr::id), of its slowest 64-plan wavefront so far: microseconds
+                                 // << 12 | heap pops per dispatch in sixteenths; or null
 };
 constexpr uint32_t KE_FIXUP = 0x80000000u;   // EvalLaunch::flags: only the plans flagged in `ovf` are evaluated
 constexpr int KE_NEED_SHARDS = 64;
@@ -177,6 +179,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   if (pi == KE_IDLE) return;
   first_lane = __builtin_ctzll(__ballot(1));
   KE_STAMP(0);
+  const unsigned long long t_begin = LS == 0 && L.cstat ? wall_clock64() : 0ull;   // (100 MHz)
 
   // ---- workspace rows of this lane
   double *g_time, *g_rank, *g_dur;
@@ -609,6 +612,21 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   }
   KE_STAMP(5);
   if (L.prof) atomicMax(&L.prof[w * 8 + 7], ((unsigned long long)n << 32) | (unsigned long long)guard_total);
+  if (LS == 0 && L.cstat && !(L.flags & KE_FIXUP) && n > 0) {
+    // what the wavefront paid per dispatch: the pops of its slowest plan.  The host reads it to decide which
+    // classes are worth four lanes per plan.
+    uint32_t g = (uint32_t)guard_total;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const uint32_t o = (uint32_t)__shfl_xor((int)g, off);
+      g = o > g ? o : g;
+    }
+    const uint32_t per16 = g * 16u / (uint32_t)n;
+    const unsigned long long us = (wall_clock64() - t_begin) / 100ull;
+    const uint32_t word = ((uint32_t)(us < 0xFFFFFull ? us : 0xFFFFFull) << 12) | (per16 < 0xFFFu ? per16 : 0xFFFu);
+    uint32_t* slot = L.cstat + cv.h->id;
+    if (lane == first_lane && word > *slot) atomicMax(slot, word);
+  }
 
   // ---- outputs
   uint8_t mask = RPEG_MASK_VALID;

@@ -4,7 +4,7 @@
 
 Runs the seeded candidate set of the configuration through rpeg_eval_batch with the per-wavefront stamps switched
 on (rpeg_engine_profile) and prints, for the main kernel (k_eval) and for the one-plan-per-wavefront kernel
-(k_plan) beside it: when their tasks start and end, how many run at a time, the longest tasks, and the durations
+(k_plan) and the four-lanes-per-plan kernel (k_quad) beside it: when their tasks start and end, how many run at a time, the longest tasks, and the durations
 by node count.  A kernel ends with its slowest wavefront, so the table of the longest tasks is the critical
 path of the step.
 
@@ -27,6 +27,7 @@ def main() -> None:
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--plans", type=int, default=0, help="plans of the seeded set (default: the configuration's own size)")
     ap.add_argument("--sections", action="store_true", help="section clocks of the scheduling loop (measurement build)")
+    ap.add_argument("--quad-share", type=int, default=-1, help="percent of the batch for the four-lanes-per-plan kernel (default: the engine's)")
     args = ap.parse_args()
     import torch
     from .. import build as B, configs
@@ -41,6 +42,8 @@ def main() -> None:
     n = args.plans or cfg.n_plans
     batch = candidates.generate(cfg.problem, n, cfg.tau_choices, seed=42, tag=args.config)
     eng = R.Engine(cfg.problem)
+    if args.quad_share >= 0:
+        eng.set_quad_share(args.quad_share)
     lib = eng.lib
     lib.rpeg_engine_profile.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_uint64]
     db = R.DeviceBatch(batch)
@@ -58,12 +61,13 @@ def main() -> None:
     buf = np.zeros((rows, 8), np.uint64)
     got = lib.rpeg_engine_profile(eng._h, 1, buf.ctypes.data, rows)
     buf = buf[:got]
-    n_eval = s["wave_tasks"] - s["single_plan_tasks"]
+    n_eval = s["wave_tasks"] - s["single_plan_tasks"] - s["quad_tasks"]
+    n_lane = n_eval + s["quad_tasks"]
     b = buf.astype(np.float64)
     nodes = (buf[:, 7] >> np.uint64(32)).astype(np.int64)
     t0 = b[:, 0][b[:, 0] > 0].min()
     start, end = (b[:, 0] - t0) / 100.0, (b[:, 6] - t0) / 100.0          # the stamps tick at 100 MHz: microseconds
-    for name, sl in (("k_eval", slice(0, n_eval)), ("k_plan", slice(n_eval, got))):
+    for name, sl in (("k_eval", slice(0, n_eval)), ("k_quad", slice(n_eval, n_lane)), ("k_plan", slice(n_lane, got))):
         S, E, N = start[sl], end[sl], nodes[sl]
         ok = E > 0
         S, E, N = S[ok], E[ok], N[ok]
@@ -78,9 +82,10 @@ def main() -> None:
         print("   longest tasks (nodes, start us, duration us):", [(int(N[k]), round(float(S[k]), 1), round(float(d[k]), 1)) for k in o])
         o = np.argsort(-E)[:6]
         print("   last to end   (nodes, start us, duration us):", [(int(N[k]), round(float(S[k]), 1), round(float(d[k]), 1)) for k in o])
-        if not args.sections:   # (the measurement build keeps the section clocks where the phase stamps are)
+        if not args.sections or name != "k_eval":   # (the measurement build keeps the section clocks where the phase stamps are)
             ph = np.diff(b[sl][ok][:, :7], axis=1) / 100.0
             names = ("plan fields", "durations", "memory model", "ranks", "scheduling", "outputs") if name == "k_eval" else \
+                    ("plan fields", "durations", "memory model", "ranks and positions", "scheduling", "outputs") if name == "k_quad" else \
                     ("plan fields", "durations", "memory model and ranks", "positions in the order", "scheduling", "outputs")
             print("   phases, mean us per task: " + ", ".join(f"{nm} {x:.1f}" for nm, x in zip(names, ph.mean(0))))
             slow = np.argsort(-d)[:40]

@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_quad_share", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
            "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static")
 
 
@@ -75,6 +75,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_last_kernel_ms.argtypes = [vp]
     lib.rpeg_engine_set_state_lanes.restype = C.c_int
     lib.rpeg_engine_set_state_lanes.argtypes = [vp, i32]
+    lib.rpeg_engine_set_quad_share.restype = C.c_int
+    lib.rpeg_engine_set_quad_share.argtypes = [vp, i32]
     lib.rpeg_engine_set_ready_cap.restype = C.c_int
     lib.rpeg_engine_set_ready_cap.argtypes = [vp, i32]
     lib.rpeg_engine_reset_classes.restype = C.c_int
@@ -194,8 +196,13 @@ class Engine:
         self.lib.rpeg_engine_set_timing(self._h, int(on))
 
     def set_state_lanes(self, lanes: int):
-        """-1 automatic; 0 scheduler state in HBM (64 plans per wavefront); 8/16/32/64 state in LDS."""
+        """-1 automatic; 0 scheduler state in HBM (64 plans per wavefront); 8/16/32/64 state in LDS; 1 a plan per
+        wavefront; 4 four lanes per plan."""
         self._check(self.lib.rpeg_engine_set_state_lanes(self._h, int(lanes)), "rpeg_engine_set_state_lanes")
+
+    def set_quad_share(self, percent: int):
+        """Percentage of a full batch that the four-lanes-per-plan kernel takes beside the main kernel (0: none)."""
+        self._check(self.lib.rpeg_engine_set_quad_share(self._h, int(percent)), "rpeg_engine_set_quad_share")
 
     def set_ready_cap(self, entries: int):
         """Ready-list entries per plan in the main kernel (8, 16, 24 or 32); plans that need more get MASK_LIMIT."""
@@ -208,10 +215,10 @@ class Engine:
         return float(self.lib.rpeg_engine_last_kernel_ms(self._h))
 
     def stats(self) -> Dict[str, int]:
-        buf = (C.c_uint64 * 7)()
-        self.lib.rpeg_engine_stats(self._h, buf, 7)
+        buf = (C.c_uint64 * 8)()
+        self.lib.rpeg_engine_stats(self._h, buf, 8)
         return dict(classes=buf[0], classes_lowered=buf[1], wave_tasks=buf[2], lds_bytes=buf[3], workspace_bytes=buf[4],
-                    state_lanes=buf[5], single_plan_tasks=buf[6])
+                    state_lanes=buf[5], single_plan_tasks=buf[6], quad_tasks=buf[7])
 
     def alloc_outputs(self, n: int):
         torch = _torch()

@@ -350,13 +350,13 @@ def test_drop_in_calls():
 @pytest.mark.parametrize("c,n", [(1, 2048), (2, 8192), (5, 1024)])
 def test_every_state_layout_gives_the_same_bits(c, n):
     """Scheduler state in the HBM workspace (64 plans per wavefront) or in LDS (8/16/32/64 plans per
-    wavefront), one plan per wavefront, and the per-batch automatic choice: identical outputs."""
+    wavefront), one plan per wavefront, four lanes per plan, and the per-batch automatic choice: identical outputs."""
     from rpeg_amd.engine.runtime import Engine, EngineError
     cfg, batch = seeded_batch(c, n)
     eng = Engine(cfg.problem)
     ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
     seen = set()
-    for lanes in (0, 1, 8, 16, 32, 64, -1):
+    for lanes in (0, 1, 4, 8, 16, 32, 64, -1):
         eng.set_state_lanes(lanes)
         try:
             out = eng.eval(batch, gate_stale=True)
@@ -364,6 +364,7 @@ def test_every_state_layout_gives_the_same_bits(c, n):
             assert lanes > 1 and "does not fit in LDS" in str(ex)   # the largest class is too big for that many plans
             continue
         seen.add(eng.stats()["state_lanes"])
+        assert (eng.stats()["quad_tasks"] > 0) == (lanes == 4)
         assert np.array_equal(out["mask"], ref["mask"]), lanes
         assert same_bits(out["makespan"], ref["makespan"]) and same_bits(out["score"], ref["score"]), lanes
         assert same_bits(out["peak"], ref["peak"]), lanes
@@ -387,6 +388,26 @@ def test_host_and_device_entry_points_agree(c, n):
             assert same_bits(out[k], ref[k]), k
         if "mass" in out:
             assert same_bits(out["mass"], ref["mass"])
+
+
+def test_dense_classes_move_to_four_lanes_per_plan_once_measured():
+    """A batch that fills the chip in one round: the first call runs every class in the main kernel, which records how
+    long the slowest wavefront of each class took; from the next call on the classes that end last there run four
+    lanes per plan beside it.  Outputs equal the host build's bit for bit in every call, also with the share at 0."""
+    from rpeg_amd.engine.runtime import Engine
+    cfg, batch = seeded_batch(2, 65536)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16, want_mass=True)
+    eng = Engine(cfg.problem)
+    quad = []
+    for call in range(4):
+        if call == 3:
+            eng.set_quad_share(0)
+        out = eng.eval(batch, gate_stale=True, mass=(call == 2))
+        quad.append(eng.stats()["quad_tasks"])
+        assert np.array_equal(out["mask"], ref["mask"]), call
+        for k in ("makespan", "peak", "score") + (("mass",) if call == 2 else ()):
+            assert same_bits(out[k], ref[k]), (call, k)
+    assert quad[0] == 0 and quad[1] > 0 and quad[2] > 0 and quad[3] == 0, quad
 
 
 def test_small_batches_pick_the_latency_layout():
@@ -564,21 +585,26 @@ def test_transfer_resource_policies_equal_reference(c):
 def test_a_horizon_beyond_the_ready_list_is_reported_as_a_limit():
     """DPO's unrolled steps are independent of each other, so every step's first node is ready at time zero: at a
     horizon of 128 steps the ready list would need 128 entries.  The engine says so (MASK_ERROR | MASK_LIMIT, NaN),
-    it does not return a number; the host build, whose list is unbounded in this range, evaluates the plans."""
+    it does not return a number; the host build, whose list is unbounded in this range, evaluates the plans.  The
+    same at 40 steps for the kernel that holds 32 entries in registers."""
     from dataclasses import replace
     from rpeg_amd.engine.runtime import Engine
     cfg, batch = seeded_batch(4, 2048)
-    for K, limited in ((24, False), (128, True)):
+    # (K, layout, limited): -1 is the automatic layout (one plan per wavefront, no bound, while a class has at most 384
+    # nodes; beyond that the plan-per-lane kernel with its 31 entries), 4 is four lanes per plan (32 entries in registers)
+    for K, lanes, limited in ((24, -1, False), (24, 4, False), (40, -1, False), (40, 4, True), (128, -1, True)):
         p = replace(cfg.problem, K_eval=K)
         eng = Engine(p)
+        eng.set_state_lanes(lanes)
         out = eng.eval(batch)
+        assert (eng.stats()["quad_tasks"] > 0) == (lanes == 4)
         valid = (out["mask"] & abi.MASK_VALID) != 0
         assert valid.sum() > 1000
-        assert np.all(((out["mask"][valid] & abi.MASK_LIMIT) != 0) == limited)
-        assert np.all(np.isnan(out["score"][valid]) == limited)
+        assert np.all(((out["mask"][valid] & abi.MASK_LIMIT) != 0) == limited), (K, lanes)
+        assert np.all(np.isnan(out["score"][valid]) == limited), (K, lanes)
         if not limited:
             ref = CpuPort(p).eval(batch, flags=abi.GATE_STALE, threads=16)
-            assert same_bits(out["score"], ref["score"]) and np.array_equal(out["mask"], ref["mask"])
+            assert same_bits(out["score"], ref["score"]) and np.array_equal(out["mask"], ref["mask"]), (K, lanes)
         eng.close()
     with pytest.raises(ValueError, match="K_eval"):
         Engine(replace(cfg.problem, K_eval=5000))
