@@ -592,12 +592,28 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
 template <class VM>
 RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
                                const PlanMasks& pm, const VM& vm) {
+  static_assert(RPEG_MAX_V <= 6, "a vertex set is packed into six bits below");
   const StructMasks sm = struct_masks(st, order);
   const unsigned full = (1u << st.n_vertex) - 1u;
   double best = -1.0;
+  // First the maximal cliques of this plan (a graph on six vertices has at most nine: six bits each in one word),
+  // then their peaks.  On the GPU the lanes of a wavefront carry different plans: testing a set is cheap, the peak
+  // of a set is not, and this way a wavefront computes as many peaks as its plan with the most cliques has, not
+  // one for every set that is a clique in some lane.
+  uint64_t list = 0;
+  int cnt = 0;
   for (unsigned M = 1; M <= full; ++M) {
     if (!maximal_clique(st.n_vertex, pm, M)) continue;
-    const double peak = device_class_peak(P, st, order, sm, pm, vm, M);
+    if (cnt < 10) {
+      list |= (uint64_t)M << (6 * cnt);
+      ++cnt;
+    } else {   // (not reached with six vertices)
+      const double peak = device_class_peak(P, st, order, sm, pm, vm, M);
+      if (peak > best) best = peak;
+    }
+  }
+  for (int k = 0; k < cnt; ++k) {
+    const double peak = device_class_peak(P, st, order, sm, pm, vm, (unsigned)(list >> (6 * k)) & 63u);
     if (peak > best) best = peak;
   }
   return best;

@@ -443,6 +443,7 @@ struct rpeg_engine_s {
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   hipStream_t s3 = nullptr;                     // third stream: the four-lanes-per-plan wavefronts (k_quad)
   hipEvent_t ev_join3 = nullptr;
+  uint32_t dbg_heavy_pct = 0;
   uint32_t quad_share_pct = 25;                 // share of a full batch that k_quad takes (rpeg_engine_set_quad_share)
   bool quad_attr_set = false;
   int split_heavy = 1;                          // 0: the classes with the largest graphs stay in the main kernel
@@ -769,6 +770,8 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
 
 int rpeg_engine_set_quad_share(rpeg_engine_t* e, int32_t percent) {
   if (!e) return -1;
+  e->dbg_heavy_pct = (percent >> 8) & 0xFF;   // EXPERIMENT
+  percent &= 0xFF;
   if (percent < 0 || percent > 100) { e->err = "the share is a percentage"; return -1; }
   e->quad_share_pct = (uint32_t)percent;
   return 0;
@@ -967,6 +970,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       uint64_t w64 = 0;
       for (uint32_t c : counts) w64 += (c + WAVE - 1) / WAVE;
       if (split && e->quad_share_pct && w64 <= (uint64_t)e->n_cu * 6) share_pct = 10;
+      if (e->dbg_heavy_pct) share_pct = e->dbg_heavy_pct - 1;   // EXPERIMENT
     }
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t waves64 = 0;
@@ -1003,8 +1007,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     // often).  The main kernel measures itself: per class, the time of its slowest wavefront on earlier launches and
     // the heap pops per dispatch it needed (cls_pops16).  A wavefront of k_quad takes about 75 + nodes x (2.3 +
     // 0.45 per pop) microseconds (fitted).  The classes are taken in the order of their measured time while one still
-    // ends later in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct` percent of
-    // the batch.  Nothing is known before the first launch of a class: it stays in the main kernel then.
+    // ends a fifth later in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct`
+    // percent of the batch.  Nothing is known before the first launch of a class: it stays in the main kernel then.
     if (split && e->quad_share_pct && waves64 <= (uint64_t)e->n_cu * 6) {
       auto t_main = [&](uint32_t c) { return (double)(e->cls_pops16[cids[c]] >> 12); };
       auto t_quad = [&](uint32_t c) {
@@ -1019,7 +1023,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       uint64_t taken = 0;
       for (uint32_t c : cand) {
         const double tq = std::max(slowest_quad, t_quad(c));
-        if (t_main(c) <= tq) break;
+        if (t_main(c) <= 1.2 * tq) break;   // (a margin: beyond the classes that clearly end later, more wavefronts of k_quad cost more than they save)
         if ((taken + counts[c]) * 100 > (uint64_t)n * e->quad_share_pct) break;
         const uint32_t nodes = e->cls_nodes[cids[c]], slots = e->cls_slots[cids[c]];
         if (kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, std::max(quad_nodes, nodes), std::max(quad_slots, slots), e->max_v, (uint32_t)KQ_PLANS) > 64 * 1024) continue;
