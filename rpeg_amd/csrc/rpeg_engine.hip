@@ -93,6 +93,7 @@ __global__ void k_fill_u32(uint32_t* p, uint64_t n, uint32_t v) {
 // Integer validity gate, class signature, class id (open-addressing table of the classes lowered so far)
 // and the per-class plan counts.  Blocks of SIG_BLOCK plans; shard = block mod shards.
 constexpr int SIG_BLOCK = 256, SIG_TABLE = 512;
+constexpr uint32_t N_QUEUES = 4;   // task counters of a call's evaluation launches (main kernel, k_quad, k_plan, spare)
 struct SigPlans {   // the plan fields of one thread's plan, a column of an LDS array [field][thread]
   const int16_t* col;
   __device__ VPlan operator[](int v) const { return ke_vplan<SIG_BLOCK>(col, v); }
@@ -247,8 +248,9 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
                           const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
                           const uint32_t* __restrict__ cbase, uint32_t shards, uint32_t* __restrict__ perm,
                           uint32_t pstride, const uint32_t* __restrict__ coff, uint32_t* __restrict__ task_cls,
-                          uint32_t first_entry) {
+                          uint32_t first_entry, uint32_t* __restrict__ queues) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < N_QUEUES) queues[i] = 0u;   // the task counters of the evaluation kernels that follow on this stream
   if (i >= n) return;
   const uint32_t c = cid[i];
   if (c >= CID_UNKNOWN) return;
@@ -259,11 +261,20 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
   } else perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
 }
 
+// The next wave task of a launch whose wavefronts take tasks as they become free (every wavefront ends when the
+// counter has passed the last task), or the next of this block's own.
+__device__ inline uint64_t next_task(const EvalLaunch& L, uint64_t w) {
+  if (!L.queue) return w + gridDim.x;
+  uint32_t t = 0;
+  if (threadIdx.x == 0) t = atomicAdd(L.queue, 1u);
+  return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+}
+
 template <int LS>
 __global__ __launch_bounds__(WAVE) void k_eval(const EvalLaunch L) {
   extern __shared__ uint8_t ke_lds[];
   if ((L.flags & KE_FIXUP) && L.need && L.need[KE_NEED_SHARDS] == 0u) return;   // no plan outgrew its list
-  for (uint64_t w = blockIdx.x; w < L.n_waves; w += gridDim.x) {
+  for (uint64_t w = L.queue ? next_task(L, 0) : blockIdx.x; w < L.n_waves; w = next_task(L, w)) {
     if (LS == 0 && (L.wave_cls[w] & KE_CLS_LDS)) ke_eval_wave<KE_FEW>(L, w, ke_lds);   // uniform branch
     else ke_eval_wave<LS>(L, w, ke_lds);
   }
@@ -451,6 +462,7 @@ struct rpeg_engine_s {
   uint64_t* h_sig = nullptr;
   uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_cls = nullptr;   // lane -> plan; wavefront -> class blob
   uint8_t* d_ws = nullptr;
+  uint32_t* d_queues = nullptr;                 // N_QUEUES task counters, cleared by k_scatter
   size_t ws_cap = 0;
   // timing / stats
   bool timing = false;
@@ -470,6 +482,10 @@ static int ensure_batch(rpeg_engine_t* e, size_t n) {
   e->cap_n = 0;
   HIP_TRY(e, hipMalloc(&e->d_ovf, cap));
   HIP_TRY(e, hipMemset(e->d_ovf, 0, cap));   // flags are cleared again by the launch that consumes them
+  if (!e->d_queues) {
+    HIP_TRY(e, hipMalloc(&e->d_queues, N_QUEUES * 4));
+    HIP_TRY(e, hipMemset(e->d_queues, 0, N_QUEUES * 4));
+  }
   if (!e->d_need) {
     HIP_TRY(e, hipMalloc(&e->d_need, (KE_NEED_SHARDS + 1) * 4));
     HIP_TRY(e, hipMemset(e->d_need, 0, (KE_NEED_SHARDS + 1) * 4));
@@ -714,6 +730,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_pool) hipFree(e->d_pool);
   if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
   if (e->d_need) hipFree(e->d_need);
+  if (e->d_queues) hipFree(e->d_queues);
   if (e->d_cstat) hipFree(e->d_cstat);
   if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); hipFree(e->d_hoff); }
   if (e->h_static) hipHostFree(e->h_static);
@@ -828,6 +845,38 @@ int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, u
 }  // extern "C"
 
 constexpr uint32_t TINY_CLASS = 16;   // classes of fewer plans go to the single-plan kernel
+
+// When a step ends, for a batch of more than one round of wavefronts (microseconds).  The main kernel keeps r
+// wavefronts on every compute unit and lasts max(its longest task, its work / (units x r)); k_plan runs beside it in
+// the LDS and registers left (16 - 2r wavefronts of 128 registers), and what it has not done by then it does with
+// the units to itself, sixteen wavefronts each.  A plan costs k_plan about 40 + 2.2 x nodes microseconds of a wavefront.
+struct DeepModel {
+  double n_cu, lds_main, lds_plan;
+  uint64_t r_max;
+  double plan_cost(uint32_t plans, uint32_t nodes) const { return (double)plans * (40.0 + 2.2 * (double)nodes); }
+  double total(double w_main, double w_plan, double max_t, uint64_t r) const {
+    const double t_main = std::max(max_t, w_main / (n_cu * (double)r));
+    const double room = std::max(0.0, std::min(16.0 - 2.0 * (double)r, std::floor((160.0 * 1024 - (double)r * lds_main) / lds_plan)));
+    const double left = std::max(0.0, w_plan - t_main * n_cu * room);
+    return t_main + left / (n_cu * 16.0);
+  }
+  double best(double w_main, double w_plan, double max_t, uint64_t* r_best) const {
+    double b = 0.0;
+    for (uint64_t r = r_max; r >= 1; --r) {
+      const double t = total(w_main, w_plan, max_t, r);
+      if (r == r_max || t < b) { b = t; if (r_best) *r_best = r; }
+    }
+    return b;
+  }
+};
+static DeepModel deep_model(const rpeg_engine_t* e, uint32_t rcap) {
+  DeepModel m;
+  m.n_cu = (double)e->n_cu;
+  m.lds_main = (double)ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, rcap, 0, e->max_nodes, e->max_slots, e->max_v);
+  m.lds_plan = (double)kp_lds_bytes(e->max_nodes, e->max_slots);
+  m.r_max = std::max<uint64_t>(1, std::min<uint64_t>(8, (uint64_t)(160.0 * 1024 / m.lds_main)));
+  return m;
+}
 
 static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                            double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
@@ -948,6 +997,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // first[c]: first wavefront of class c in launch order (first permutation entry for a class of
   // single-plan wavefronts, which follow the others in the permutation and in the task list)
   std::vector<uint32_t> first(counts.size(), 0), clpw(counts.size(), lpw);
+  // ready-list capacity of the main kernel: the full list until the longest list of earlier launches is known
+  const uint32_t rcap_main = e->need > 0 ? std::min(e->ready_cap, std::max(8u, (e->need + 2 + 7) & ~7u)) : e->ready_cap;
   std::vector<uint8_t> solo(counts.size(), 0), quad(counts.size(), quad_all ? 1 : 0);
   uint32_t quad_nodes = quad_all ? e->max_nodes : 0, quad_slots = quad_all ? e->max_slots : 0;
   if (!ls && !one && !quad_all && !order.empty()) {
@@ -1003,6 +1054,41 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (split)
       for (size_t c = 0; c < counts.size(); ++c)
         if (counts[c] < TINY_CLASS) solo[c] = 1;
+    // More than one round of wavefronts: the main kernel ends when its work is done, unless one wavefront alone runs
+    // longer than that.  With the measured time of every class (its slowest wavefront on earlier launches) the
+    // longest classes are taken out, as many of them as make the modelled end of the step (deep_model) earliest.
+    if (split && e->quad_share_pct) {
+      const DeepModel dm = deep_model(e, rcap_main);
+      uint64_t main_tasks = 0;
+      double w_main = 0.0, w_plan = 0.0;
+      bool known = true;
+      std::vector<uint32_t> cand;
+      for (uint32_t c = 0; c < counts.size(); ++c) {
+        if (solo[c]) { w_plan += dm.plan_cost(counts[c], e->cls_nodes[cids[c]]); continue; }
+        const double t = (double)(e->cls_pops16[cids[c]] >> 12);
+        if (t == 0.0) known = false;
+        main_tasks += (counts[c] + WAVE - 1) / WAVE;
+        w_main += (double)((counts[c] + WAVE - 1) / WAVE) * t;
+        cand.push_back(c);
+      }
+      if (known && main_tasks > (uint64_t)e->n_cu * dm.r_max) {
+        auto t_of = [&](uint32_t c) { return (double)(e->cls_pops16[cids[c]] >> 12); };
+        std::sort(cand.begin(), cand.end(), [&](uint32_t x, uint32_t y) { return t_of(x) > t_of(y); });
+        // the modelled end with the k longest classes taken out, for every k: the best k wins (classes of nearly
+        // equal time form plateaus, so one class at a time would stop at the first)
+        double best_t = dm.best(w_main, w_plan, cand.empty() ? 0.0 : t_of(cand[0]), nullptr);
+        size_t best_k = 0;
+        double wm = w_main, wp = w_plan;
+        for (size_t k = 0; k < cand.size(); ++k) {
+          const uint32_t c = cand[k];
+          wm -= (double)((counts[c] + WAVE - 1) / WAVE) * t_of(c);
+          wp += dm.plan_cost(counts[c], e->cls_nodes[cids[c]]);
+          const double t = dm.best(wm, wp, k + 1 < cand.size() ? t_of(cand[k + 1]) : 0.0, nullptr);
+          if (t < 0.98 * best_t) { best_t = t; best_k = k + 1; }
+        }
+        for (size_t k = 0; k < best_k; ++k) solo[cand[k]] = 1;
+      }
+    }
     // Of what stays, the wavefronts that end last are those of dense graphs (long ready lists, keys that go stale
     // often).  The main kernel measures itself: per class, the time of its slowest wavefront on earlier launches and
     // the heap pops per dispatch it needed (cls_pops16).  A wavefront of k_quad takes about 75 + nodes x (2.3 +
@@ -1087,8 +1173,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // Ready-list capacity: the full 32 entries until the longest list of earlier launches is known, then a
   // short list (less LDS, more wavefronts per compute unit); plans that outgrow it are redone below.
   const uint32_t rcap_full = e->ready_cap;
-  const bool short_list = !ls && !one && e->need > 0 && ((e->need + 2 + 7) & ~7u) < rcap_full;
-  const uint32_t rcap = short_list ? std::max(8u, (e->need + 2 + 7) & ~7u) : rcap_full;
+  const bool short_list = !ls && !one && rcap_main < rcap_full;
+  const uint32_t rcap = short_list ? rcap_main : rcap_full;
   const bool few_in_lds = !ls && !one &&
       ke_lds_bytes(0, rcap, KE_FEW, e->max_nodes, e->max_slots, e->max_v) <= ke_lds_bytes(0, rcap, 0, e->max_nodes, e->max_slots, e->max_v);
   for (size_t k = 0; k < order.size(); ++k) {
@@ -1108,11 +1194,37 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
   hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
-                     d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted);
+                     d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted, e->d_queues);
   HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_eval_waves;
-  const unsigned grid = (unsigned)std::min<uint64_t>(std::max<uint64_t>(n_waves, 1), (uint64_t)e->n_cu * (one ? 32 : 16));
+  // The main kernel with the state in the workspace is launched with as many wavefronts as can be resident (LDS, and
+  // two per SIMD by registers), which take the wave tasks from a counter as they become free: the tasks are in the
+  // order of their graphs' sizes, so the longest start first and the rest fills in behind them, and the wavefronts
+  // keep their place on the chip while k_plan's smaller ones run beside them.
+  const bool queued = !ls && !one;
+  uint64_t resident_per_cu = 0;
+  if (queued) {
+    const size_t lds_main = ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, rcap, 0, e->max_nodes, e->max_slots, e->max_v);
+    const uint64_t r_max = std::max<uint64_t>(1, std::min<uint64_t>(8, 160 * 1024 / lds_main));
+    resident_per_cu = r_max;
+    // More than one round of wavefronts with work for k_plan beside them: the main kernel leaves k_plan room
+    // (deep_model: the number of its wavefronts per compute unit for which both kernels are done soonest).
+    const DeepModel dm = deep_model(e, rcap);
+    double w_main = 0.0, w_plan = 0.0, max_t = 0.0;
+    bool known = true;
+    for (size_t c = 0; c < counts.size(); ++c) {
+      if (solo[c]) w_plan += dm.plan_cost(counts[c], e->cls_nodes[cids[c]]);
+      else if (!quad[c]) {
+        const double t = (double)(e->cls_pops16[cids[c]] >> 12);
+        if (t == 0.0) known = false;
+        w_main += (double)((counts[c] + clpw[c] - 1) / clpw[c]) * t;
+        max_t = std::max(max_t, t);
+      }
+    }
+    if (known && n_solo && n_waves > (uint64_t)e->n_cu * r_max) dm.best(w_main, w_plan, max_t, &resident_per_cu);
+  }
+  const unsigned grid = (unsigned)std::min<uint64_t>(std::max<uint64_t>(n_waves, 1), (uint64_t)e->n_cu * (one ? 32 : queued ? resident_per_cu : 16));
   const size_t wsb = ls || one ? 0 : ke_ws_bytes(e->max_nodes, e->max_slots);
   if (!ls && !one && n_waves)
     if (int rc = ensure_ws(e, wsb * grid, s)) return rc;
@@ -1131,6 +1243,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.ovf = short_list ? e->d_ovf : nullptr;
   L.need = !ls && !one ? e->d_need : nullptr;
   L.cstat = !ls && !one && e->quad_share_pct ? e->d_cstat : nullptr;
+  L.queue = queued ? e->d_queues : nullptr;
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
   L.prof = nullptr;
@@ -1178,7 +1291,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     Q.wave_cls = L.wave_cls + n_eval_waves;
     Q.n_waves = n_quad_waves;
     Q.ws_nodes = quad_nodes; Q.ws_slots = quad_slots;
-    Q.ovf = nullptr; Q.need = nullptr; Q.cstat = nullptr;   // (32 entries are as many as the main kernel's full list holds: an overflow is final)
+    Q.ovf = nullptr; Q.need = nullptr; Q.cstat = nullptr; Q.queue = nullptr;   // (32 entries are as many as the main kernel's full list holds: an overflow is final)
     if (L.prof) Q.prof = L.prof + n_waves * 8;
     const size_t qlds = kq_lds_bytes(L.cls_bytes, quad_nodes, quad_slots, e->max_v, (uint32_t)KQ_PLANS);
     if (qlds > 64 * 1024 && !e->quad_attr_set) {
@@ -1202,6 +1315,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   HIP_TRY(e, hipGetLastError());
   if (n_solo) {   // the single-plan wavefronts, beside the main kernel
     EvalLaunch S = L;
+    S.queue = nullptr;
     S.perm = e->d_perm + n_sorted;
     S.wave_cls = e->d_cls + n_host_tasks;
     S.n_waves = n_solo;
@@ -1215,6 +1329,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // (after the submission of k_plan, which is the longer of the two kernels and should not wait for this one)
   if (short_list && n_waves) {   // the plans whose ready list outgrew the short one, with the full one
     EvalLaunch F = L;
+    F.queue = nullptr;
     F.rcap = rcap_full;
     F.flags = flags | KE_FIXUP;
     const size_t lds_full = ke_lds_bytes(F.cls_bytes, F.rcap, 0, e->max_nodes, e->max_slots, e->max_v);

@@ -56,6 +56,8 @@ struct EvalLaunch {              // uniform launch parameters
                                  // consumed by the KE_FIXUP launch with the full one), or null
   uint32_t* need;                // KE_NEED_SHARDS running maxima of the ready-list length, then one word that
                                  // counts the plans flagged in `ovf` and not yet redone; or null
+  uint32_t* queue = nullptr;     // next wave task to take (zero at launch): the wavefronts of the grid take tasks as
+                                 // they become free; null: block b takes tasks b, b + grid, ...
   uint32_t* cstat = nullptr;     // per class (ClassHdr::id), of its slowest 64-plan wavefront so far: microseconds
                                  // << 12 | heap pops per dispatch in sixteenths; or null
 };
