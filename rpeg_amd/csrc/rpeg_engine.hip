@@ -454,7 +454,6 @@ struct rpeg_engine_s {
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   hipStream_t s3 = nullptr;                     // third stream: the four-lanes-per-plan wavefronts (k_quad)
   hipEvent_t ev_join3 = nullptr;
-  uint32_t dbg_heavy_pct = 0;
   uint32_t quad_share_pct = 25;                 // share of a full batch that k_quad takes (rpeg_engine_set_quad_share)
   bool quad_attr_set = false;
   int split_heavy = 1;                          // 0: the classes with the largest graphs stay in the main kernel
@@ -787,8 +786,6 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
 
 int rpeg_engine_set_quad_share(rpeg_engine_t* e, int32_t percent) {
   if (!e) return -1;
-  e->dbg_heavy_pct = (percent >> 8) & 0xFF;   // EXPERIMENT
-  percent &= 0xFF;
   if (percent < 0 || percent > 100) { e->err = "the share is a percentage"; return -1; }
   e->quad_share_pct = (uint32_t)percent;
   return 0;
@@ -947,7 +944,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   const bool quad_all = ls == 4;   // every class in the four-lanes-per-plan kernel (k_quad)
   if (quad_all) {
     ls = 0;
-    if (kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, e->max_nodes, e->max_slots, e->max_v, (uint32_t)KQ_PLANS) > 160 * 1024) {
+    if (kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, e->max_nodes, e->max_slots, e->max_v, (uint32_t)KQ_PLANS, mass != nullptr) > 160 * 1024) {
       e->err = "per-plan state of this problem does not fit in LDS with sixteen plans per wavefront";
       return -8;
     }
@@ -1014,14 +1011,13 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     const bool split = e->split_heavy && one_fits;
     // node count from which a class counts as large: the smallest one, not under `floor` percent of the
     // largest, such that the large classes hold at most `share` percent of the batch
-    // (ten percent when k_quad takes the dense classes: a plan costs k_plan four times the instructions)
+    // (eight percent when k_quad takes the dense classes: a plan costs k_plan four times the instructions)
     const uint64_t floor_pct = split ? 60ull : 70ull;
     uint64_t share_pct = split ? 15ull : 25ull;
     {
       uint64_t w64 = 0;
       for (uint32_t c : counts) w64 += (c + WAVE - 1) / WAVE;
-      if (split && e->quad_share_pct && w64 <= (uint64_t)e->n_cu * 6) share_pct = 10;
-      if (e->dbg_heavy_pct) share_pct = e->dbg_heavy_pct - 1;   // EXPERIMENT
+      if (split && e->quad_share_pct && w64 <= (uint64_t)e->n_cu * 12) share_pct = 8;
     }
     const uint32_t top = e->cls_nodes[cids[order[0]]];
     uint64_t waves64 = 0;
@@ -1093,9 +1089,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     // often).  The main kernel measures itself: per class, the time of its slowest wavefront on earlier launches and
     // the heap pops per dispatch it needed (cls_pops16).  A wavefront of k_quad takes about 75 + nodes x (2.3 +
     // 0.45 per pop) microseconds (fitted).  The classes are taken in the order of their measured time while one still
-    // ends a fifth later in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct`
+    // ends 15 % later in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct`
     // percent of the batch.  Nothing is known before the first launch of a class: it stays in the main kernel then.
-    if (split && e->quad_share_pct && waves64 <= (uint64_t)e->n_cu * 6) {
+    if (split && e->quad_share_pct && waves64 <= (uint64_t)e->n_cu * 12) {
       auto t_main = [&](uint32_t c) { return (double)(e->cls_pops16[cids[c]] >> 12); };
       auto t_quad = [&](uint32_t c) {
         const double nd = e->cls_nodes[cids[c]], p = (e->cls_pops16[cids[c]] & 0xFFFu) / 16.0;
@@ -1105,16 +1101,24 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       for (uint32_t c = 0; c < counts.size(); ++c)
         if (!solo[c] && e->cls_pops16[cids[c]]) cand.push_back(c);
       std::sort(cand.begin(), cand.end(), [&](uint32_t x, uint32_t y) { return t_main(x) > t_main(y); });
+      // (k_quad's wavefronts are taken to have half of a compute unit's LDS: beyond one round of them the time of a
+      // wavefront counts as many times as there are rounds)
       double slowest_quad = 0.0;
-      uint64_t taken = 0;
+      uint64_t taken = 0, tasks = 0;
       for (uint32_t c : cand) {
-        const double tq = std::max(slowest_quad, t_quad(c));
-        if (t_main(c) <= 1.2 * tq) break;   // (a margin: beyond the classes that clearly end later, more wavefronts of k_quad cost more than they save)
-        if ((taken + counts[c]) * 100 > (uint64_t)n * e->quad_share_pct) break;
         const uint32_t nodes = e->cls_nodes[cids[c]], slots = e->cls_slots[cids[c]];
-        if (kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, std::max(quad_nodes, nodes), std::max(quad_slots, slots), e->max_v, (uint32_t)KQ_PLANS) > 64 * 1024) continue;
+        const size_t qlds = kq_lds_bytes((e->max_cls_bytes + 15u) & ~15u, std::max(quad_nodes, nodes), std::max(quad_slots, slots), e->max_v,
+                                         (uint32_t)KQ_PLANS, mass != nullptr);
+        if (qlds > 64 * 1024) continue;
+        const uint64_t c_tasks = (counts[c] + KQ_PLANS - 1) / KQ_PLANS;
+        const double room = (double)e->n_cu * (double)std::max<uint64_t>(1, 80 * 1024 / qlds);
+        const double tq = std::max(slowest_quad, t_quad(c));
+        const double rounds = std::max(1.0, (double)(tasks + c_tasks) / room);
+        if (t_main(c) <= 1.15 * tq * rounds) break;   // (a margin: beyond the classes that clearly end later, more wavefronts of k_quad cost more than they save)
+        if ((taken + counts[c]) * 100 > (uint64_t)n * e->quad_share_pct) break;
         quad[c] = 1;
         taken += counts[c];
+        tasks += c_tasks;
         slowest_quad = tq;
         quad_nodes = std::max(quad_nodes, nodes);
         quad_slots = std::max(quad_slots, slots);
@@ -1293,7 +1297,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     Q.ws_nodes = quad_nodes; Q.ws_slots = quad_slots;
     Q.ovf = nullptr; Q.need = nullptr; Q.cstat = nullptr; Q.queue = nullptr;   // (32 entries are as many as the main kernel's full list holds: an overflow is final)
     if (L.prof) Q.prof = L.prof + n_waves * 8;
-    const size_t qlds = kq_lds_bytes(L.cls_bytes, quad_nodes, quad_slots, e->max_v, (uint32_t)KQ_PLANS);
+    const size_t qlds = kq_lds_bytes(L.cls_bytes, quad_nodes, quad_slots, e->max_v, (uint32_t)KQ_PLANS, mass != nullptr);
     if (qlds > 64 * 1024 && !e->quad_attr_set) {
       HIP_TRY(e, hipFuncSetAttribute((const void*)k_quad, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       e->quad_attr_set = true;

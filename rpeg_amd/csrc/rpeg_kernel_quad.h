@@ -33,14 +33,16 @@ constexpr uint32_t KQ_EMPTY = 0xFFFFFFFFu;
 
 // LDS of one wavefront of `np` plans: class tables (node records, successor lists), the class's reverse order and its
 // nodes grouped by tie-break class (uint16 each, first-node table of 17 words), plan fields, memory terms, then the
-// per-plan state [row][plan]: time, rank (doubles per node), duration (double per slot), position (uint16 per node),
-// in-degree (byte per node).
+// per-plan state [row][plan]: time and rank (a double per node each; ONE array for both unless the critical-chain
+// masses are asked for: a rank is not read again once the positions are known, a ready time not written before),
+// duration (double per slot), position (uint16 per node), in-degree (byte per node).
 __host__ __device__ inline size_t kq_tab_bytes(uint32_t nodes) { return ((size_t)nodes * 4 + 17 * 2 + 15) & ~size_t(15); }
 __host__ __device__ inline size_t kq_dyn_bytes(uint32_t nv, uint32_t np) {
   return (((size_t)nv * RPEG_FIELDS * np * 2 + 15) & ~size_t(15)) + (size_t)nv * 4 * np * 8;
 }
-__host__ __device__ inline size_t kq_lds_bytes(uint32_t cls_bytes, uint32_t nodes, uint32_t slots, uint32_t nv, uint32_t np) {
-  return cls_bytes + kq_tab_bytes(nodes) + kq_dyn_bytes(nv, np) + (size_t)np * ((16ull * nodes + 8ull * slots + 3ull * nodes + 15) & ~15ull);
+__host__ __device__ inline size_t kq_lds_bytes(uint32_t cls_bytes, uint32_t nodes, uint32_t slots, uint32_t nv, uint32_t np, bool mass) {
+  return cls_bytes + kq_tab_bytes(nodes) + kq_dyn_bytes(nv, np) +
+         (size_t)np * (((mass ? 16ull : 8ull) * nodes + 8ull * slots + 3ull * nodes + 15) & ~15ull);
 }
 
 #if defined(__HIPCC__)
@@ -94,11 +96,12 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   int16_t* l_plan = (int16_t*)dyn + p;                                // [fields][RW]
   double* l_vm = (double*)(dyn + (((size_t)L.max_v * RPEG_FIELDS * NP * 2 + 15) & ~size_t(15))) + p;   // [4 * vertices][RW]
   uint8_t* sbase = dyn + kq_dyn_bytes(L.max_v, NP);
+  const size_t tr_rows = (L.mass ? 2 : 1) * (size_t)L.ws_nodes;   // rows of the time and rank arrays together
   double* g_time = (double*)sbase + p;
-  double* g_rank = g_time + (size_t)L.ws_nodes * RW;
-  double* g_dur = g_rank + (size_t)L.ws_nodes * RW;
-  uint16_t* g_pos = (uint16_t*)((double*)sbase + (2 * (size_t)L.ws_nodes + L.ws_slots) * RW) + p;
-  uint8_t* g_deg = (uint8_t*)((uint16_t*)((double*)sbase + (2 * (size_t)L.ws_nodes + L.ws_slots) * RW) + (size_t)L.ws_nodes * RW) + p;
+  double* g_rank = L.mass ? g_time + (size_t)L.ws_nodes * RW : g_time;
+  double* g_dur = (double*)sbase + tr_rows * RW + p;
+  uint16_t* g_pos = (uint16_t*)((double*)sbase + (tr_rows + L.ws_slots) * RW) + p;
+  uint8_t* g_deg = (uint8_t*)((uint16_t*)((double*)sbase + (tr_rows + L.ws_slots) * RW) + (size_t)L.ws_nodes * RW) + p;
 
   const uint64_t pi = (uint64_t)L.perm[w * KE_WAVE + p];
   __syncthreads();  // the previous task of this wavefront is done with LDS
@@ -201,6 +204,7 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     for (int j = b0; j < b1; ++j) cnt += g_rank[(int)l_bykey[j] * RW] > rv ? 1 : 0;
     g_pos[v * RW] = (uint16_t)cnt;
   }
+  __syncthreads();   // (the ranks are dead from here on: their array becomes the ready times)
   for (int v = q; v < n; v += QL) {
     g_deg[v * RW] = node_at(v).indeg;
     g_time[v * RW] = 0.0;
