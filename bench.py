@@ -30,13 +30,13 @@ ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
 ALG_FLOPS = {1: 3697.0, 2: 2165.3, 3: 6502.9, 4: 1245.8, 5: 4155.6}
 # Counter figures of one step, taken from the rocprofv3 --pmc summaries under profiles/ and valid only for the
 # kernel layout they were measured on (`layout`: wave tasks, LDS bytes, plans per wavefront with LDS state,
-# single-plan tasks of rpeg_engine_stats): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
+# single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats; the task counts to 5 %): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
 # by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS + VMEM_RD + VMEM_WR of the
 # evaluation kernels / plans).  A run whose layout differs prints null instead of a stale number.
 MEASURED = {
-    2: dict(layout=(9950, 15392, 0, 8915), traffic=244.2e6, instructions_per_plan=4821.1),
-    3: dict(layout=(24495, 29984, 0, 20184), traffic=6218.5e6, instructions_per_plan=9968.7),
-    4: dict(layout=(16396, 14640, 0, 6), traffic=2105.7e6, instructions_per_plan=687.7),
+    2: dict(layout=(9950, 15392, 0, 8915, 0), traffic=244.2e6, instructions_per_plan=4821.1),
+    3: dict(layout=(24495, 29984, 0, 20184, 0), traffic=6218.5e6, instructions_per_plan=9968.7),
+    4: dict(layout=(16396, 14640, 0, 6, 0), traffic=2105.7e6, instructions_per_plan=687.7),
 }
 
 
@@ -277,6 +277,8 @@ def main():
 
     # duration of the evaluation launch (k_eval, k_plan, or both side by side from fork to join): HIP events on
     # the launch stream, recorded by the library
+    for _ in range(max(args.warmup, 3)):   # (the cold steps forgot what the engine had learned about its classes)
+        eng.eval_device(db, out)
     eng.set_timing(True)
     k_ms = []
     for _ in range(args.steps):
@@ -298,7 +300,8 @@ def main():
     out2 = eng2.alloc_outputs(n)
     s2 = torch.cuda.Stream()
     with torch.cuda.stream(s2):
-        eng2.eval_device(db, out2)
+        for _ in range(4):
+            eng2.eval_device(db, out2)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
@@ -329,6 +332,9 @@ def main():
     # otherwise; else the throughput kernel, for mid-size batches with the largest graphs on a second stream
     if stats["state_lanes"] == 1:
         kernel_name = "k_plan"
+    elif stats["single_plan_tasks"] and stats.get("quad_tasks"):
+        kernel_name = (f"k_eval<0> beside k_quad ({stats['quad_tasks']} wavefronts of 16 plans) and k_plan "
+                       f"({stats['single_plan_tasks']} plans), one launch each, timed from fork to join")
     elif stats["single_plan_tasks"]:
         kernel_name = f"k_eval<0> beside k_plan ({stats['single_plan_tasks']} plans), one launch each, timed from fork to join"
     else:
@@ -341,9 +347,12 @@ def main():
             "frac": achieved_tflops / FP64_PEAK_TFLOPS, "algorithmic_flops_per_plan": ALG_FLOPS[c]}
     # the roofline of the line is the one with the larger fraction: achieved = max(bytes fraction, flops fraction)
     roofline = dict(fp64 if fp64["frac"] >= hbm["frac"] else hbm)
-    layout = (stats["wave_tasks"], stats["lds_bytes"], stats["state_lanes"], stats["single_plan_tasks"])
+    layout = (stats["wave_tasks"], stats["lds_bytes"], stats["state_lanes"], stats["single_plan_tasks"], stats.get("quad_tasks", 0))
     measured = MEASURED.get(c)
-    same_layout = measured is not None and tuple(measured["layout"]) == layout
+    # (which classes run where is decided from times the kernels measure on themselves: the task counts of two runs
+    # differ by a few percent)
+    same_layout = measured is not None and tuple(measured["layout"][1:3]) == layout[1:3] and all(
+        abs(a - b) <= 0.05 * max(a, b) + 8 for a, b in zip((measured["layout"][0],) + tuple(measured["layout"][3:]), (layout[0],) + layout[3:]))
     roofline.update(traffic=measured["traffic"] if same_layout else None, kernel=kernel_name, kernel_ms=kernel_ms,
                     layout=list(layout))
     ipp = measured["instructions_per_plan"] if same_layout else None
