@@ -205,12 +205,14 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   const PlanHead h = load_head(L.head, L.stride, pi);
   const rpeg_struct_t& st = P.st[cv.h->structure];   // uniform (the class fixes the structure)
   const int nv = st.n_vertex;
-  for (int f0 = 0; f0 < nv * RPEG_FIELDS; f0 += RPEG_FIELDS) {   // a vertex at a time: ten loads in flight
-    int16_t x[RPEG_FIELDS];
+  {   // every load of the plan in flight at once
+    int16_t x[RPEG_MAX_V * RPEG_FIELDS];
 #pragma unroll
-    for (int f = 0; f < RPEG_FIELDS; ++f) x[f] = L.vert[(uint64_t)(f0 + f) * L.stride + pi];
+    for (int f = 0; f < RPEG_MAX_V * RPEG_FIELDS; ++f)
+      if (f < nv * RPEG_FIELDS) x[f] = L.vert[(uint64_t)f * L.stride + pi];
 #pragma unroll
-    for (int f = 0; f < RPEG_FIELDS; ++f) l_plan[(f0 + f) * RW] = x[f];
+    for (int f = 0; f < RPEG_MAX_V * RPEG_FIELDS; ++f)
+      if (f < nv * RPEG_FIELDS) l_plan[f * RW] = x[f];
   }
 
   VPlan a[RPEG_MAX_V];

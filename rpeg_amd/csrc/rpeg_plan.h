@@ -56,19 +56,24 @@ RPEG_HD bool stale_layout_ok(const rpeg_struct_t& st, const PlanHead& h, uint64_
 RPEG_HD PlanMasks plan_masks(const VPlan* a, int nv) {
   PlanMasks m;
   m.ovl = m.eq = m.dpne = 0;
+  // the three relations are symmetric: every pair is tested once and entered for both orders
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
 #endif
   for (int u = 0; u < RPEG_MAX_V; ++u) {
+    if (u >= nv) continue;
+    const uint64_t self = 1ull << (9 * u);
+    if (!alloc_disjoint(a[u], a[u])) m.ovl |= self;
+    m.eq |= self;
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
 #endif
-    for (int v = 0; v < RPEG_MAX_V; ++v) {
-      if (u >= nv || v >= nv) continue;
-      const uint64_t bit = 1ull << (8 * u + v);
-      if (!alloc_disjoint(a[u], a[v])) m.ovl |= bit;
-      if (alloc_equal(a[u], a[v])) m.eq |= bit;
-      if (a[u].dp != a[v].dp) m.dpne |= bit;
+    for (int v = u + 1; v < RPEG_MAX_V; ++v) {
+      if (v >= nv) continue;
+      const uint64_t bits = (1ull << (8 * u + v)) | (1ull << (8 * v + u));
+      if (!alloc_disjoint(a[u], a[v])) m.ovl |= bits;
+      if (alloc_equal(a[u], a[v])) m.eq |= bits;
+      if (a[u].dp != a[v].dp) m.dpne |= bits;
     }
   }
   return m;
