@@ -1101,8 +1101,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       for (uint32_t c = 0; c < counts.size(); ++c)
         if (!solo[c] && e->cls_pops16[cids[c]]) cand.push_back(c);
       std::sort(cand.begin(), cand.end(), [&](uint32_t x, uint32_t y) { return t_main(x) > t_main(y); });
-      // (k_quad's wavefronts are taken to have half of a compute unit's LDS: beyond one round of them the time of a
-      // wavefront counts as many times as there are rounds)
+      // (k_quad's wavefronts have the LDS that the main kernel's wavefronts and a few of k_plan's leave on a compute
+      // unit: beyond one round of them the time of a wavefront counts as many times as there are rounds)
+      const size_t lds_main = ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, rcap_main, 0, e->max_nodes, e->max_slots, e->max_v);
+      uint64_t main_tasks = 0;
+      for (uint32_t c = 0; c < counts.size(); ++c)
+        if (!solo[c]) main_tasks += (counts[c] + WAVE - 1) / WAVE;
       double slowest_quad = 0.0;
       uint64_t taken = 0, tasks = 0;
       for (uint32_t c : cand) {
@@ -1111,7 +1115,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
                                          (uint32_t)KQ_PLANS, mass != nullptr);
         if (qlds > 64 * 1024) continue;
         const uint64_t c_tasks = (counts[c] + KQ_PLANS - 1) / KQ_PLANS;
-        const double room = (double)e->n_cu * (double)std::max<uint64_t>(1, 80 * 1024 / qlds);
+        const uint64_t main_left = main_tasks - std::min<uint64_t>(main_tasks, (counts[c] + WAVE - 1) / WAVE);
+        const double lds_left = 144.0 * 1024 - (double)((main_left + e->n_cu - 1) / e->n_cu) * (double)lds_main;
+        const double room = (double)e->n_cu * std::max(1.0, std::floor(lds_left / (double)qlds));
         const double tq = std::max(slowest_quad, t_quad(c));
         const double rounds = std::max(1.0, (double)(tasks + c_tasks) / room);
         if (t_main(c) <= 1.15 * tq * rounds) break;   // (a margin: beyond the classes that clearly end later, more wavefronts of k_quad cost more than they save)
@@ -1119,6 +1125,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
         quad[c] = 1;
         taken += counts[c];
         tasks += c_tasks;
+        main_tasks = main_left;
         slowest_quad = tq;
         quad_nodes = std::max(quad_nodes, nodes);
         quad_slots = std::max(quad_slots, slots);
