@@ -1296,7 +1296,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     }
     HIP_TRY(e, hipEventRecord(e->ev_fork, s));
   }
-  if (n_quad_waves) {   // the four-lanes-per-plan wavefronts, beside the main kernel
+  auto launch_quad = [&]() -> int {   // the four-lanes-per-plan wavefronts, beside the main kernel
+    if (!n_quad_waves) return 0;
     EvalLaunch Q = L;
     Q.perm = e->d_perm + (uint64_t)n_eval_waves * WAVE;
     Q.wave_cls = L.wave_cls + n_eval_waves;
@@ -1313,7 +1314,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     hipLaunchKernelGGL(k_quad, dim3((unsigned)std::min<uint64_t>(n_quad_waves, (uint64_t)e->n_cu * 16)), dim3(WAVE), qlds, e->s3, Q);
     HIP_TRY(e, hipGetLastError());
     HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
-  }
+    return 0;
+  };
   auto launch_main = [&]() {
     if (n_waves == 0) {
     } else if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
@@ -1329,6 +1331,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // (The main kernel first also when k_plan has only a handful of tasks, which then wait until wavefronts of the main
   // kernel retire: with those few in front the step was 30 us longer on config 4.)
   HIP_TRY(e, launch_main());
+  // (k_quad second: measured against k_quad first, 0.50 against 0.52-0.53 ms on config 2, and against k_quad last,
+  // 0.59 ms; its wavefronts need the most LDS after the main kernel's)
+  if (int rc = launch_quad()) return rc;
   if (n_solo) {   // the single-plan wavefronts, beside the main kernel
     EvalLaunch S = L;
     S.queue = nullptr;
