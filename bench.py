@@ -30,7 +30,7 @@ ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
 ALG_FLOPS = {1: 3697.0, 2: 2165.3, 3: 6502.9, 4: 1245.8, 5: 4155.6}
 # Counter figures of one step, taken from the rocprofv3 --pmc summaries under profiles/ and valid only for the
 # kernel layout they were measured on (`layout`: wave tasks, LDS bytes, plans per wavefront with LDS state,
-# single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats; the task counts to 5 %): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
+# single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats; the task counts to 5 %, k_quad's to 25 %): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
 # by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS + VMEM_RD + VMEM_WR of the
 # evaluation kernels / plans).  A run whose layout differs prints null instead of a stale number.
 MEASURED = {
@@ -350,9 +350,10 @@ def main():
     layout = (stats["wave_tasks"], stats["lds_bytes"], stats["state_lanes"], stats["single_plan_tasks"], stats.get("quad_tasks", 0))
     measured = MEASURED.get(c)
     # (which classes run where is decided from times the kernels measure on themselves: the task counts of two runs
-    # differ by a few percent)
+    # differ by a few percent, the number of k_quad's tasks by up to a quarter)
     same_layout = measured is not None and tuple(measured["layout"][1:3]) == layout[1:3] and all(
-        abs(a - b) <= 0.05 * max(a, b) + 8 for a, b in zip((measured["layout"][0],) + tuple(measured["layout"][3:]), (layout[0],) + layout[3:]))
+        abs(a - b) <= tol * max(a, b) + 8 for a, b, tol in zip((measured["layout"][0],) + tuple(measured["layout"][3:]),
+                                                               (layout[0],) + layout[3:], (0.05, 0.05, 0.25)))
     roofline.update(traffic=measured["traffic"] if same_layout else None, kernel=kernel_name, kernel_ms=kernel_ms,
                     layout=list(layout))
     ipp = measured["instructions_per_plan"] if same_layout else None
