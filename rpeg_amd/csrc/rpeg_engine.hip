@@ -1294,7 +1294,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       HIP_TRY(e, hipStreamCreateWithFlags(&e->s3, hipStreamNonBlocking));
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join3, hipEventDisableTiming));
     }
+    // (the three launches back to back: every call between them delays the start of the later kernels)
     HIP_TRY(e, hipEventRecord(e->ev_fork, s));
+    if (n_quad_waves) HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
+    if (n_solo) HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
   }
   auto launch_quad = [&]() -> int {   // the four-lanes-per-plan wavefronts, beside the main kernel
     if (!n_quad_waves) return 0;
@@ -1310,10 +1313,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       HIP_TRY(e, hipFuncSetAttribute((const void*)k_quad, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       e->quad_attr_set = true;
     }
-    HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
     hipLaunchKernelGGL(k_quad, dim3((unsigned)std::min<uint64_t>(n_quad_waves, (uint64_t)e->n_cu * 16)), dim3(WAVE), qlds, e->s3, Q);
     HIP_TRY(e, hipGetLastError());
-    HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
     return 0;
   };
   auto launch_main = [&]() {
@@ -1341,12 +1342,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     S.wave_cls = e->d_cls + n_host_tasks;
     S.n_waves = n_solo;
     if (L.prof) S.prof = L.prof + (n_waves + n_quad_waves) * 8;
-    HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
     hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n_solo, (uint64_t)e->n_cu * 32)), dim3(WAVE),
                        kp_lds_bytes(e->max_nodes, e->max_slots), e->s2, S);
     HIP_TRY(e, hipGetLastError());
-    HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
   }
+  if (n_quad_waves) HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
+  if (n_solo) HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
   // (after the submission of k_plan, which is the longer of the two kernels and should not wait for this one)
   if (short_list && n_waves) {   // the plans whose ready list outgrew the short one, with the full one
     EvalLaunch F = L;
