@@ -407,6 +407,9 @@ struct rpeg_engine_s {
                                                      // microseconds << 12 | heap pops per dispatch in sixteenths
   uint32_t* d_cstat = nullptr;                       // the device's copy, written by the main kernel
   uint32_t cstat_cap = 0;
+  std::vector<uint8_t> cls_split;                    // where every class ran when that was last decided: 0 main kernel, 1 k_plan,
+  uint64_t split_for_n = 0, split_at = 0;            // 2 k_quad, 255 not in that batch; the batch size and the call of that decision
+  bool split_mass = false;
   uint32_t learn_calls = 0;                          // calls left after which the statistic is read back
   uint64_t batch_calls = 0;
   uint64_t* d_hkey = nullptr;                        // device table signature -> class id
@@ -781,6 +784,7 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
     return -1;
   }
   e->state_lanes = lanes;
+  e->split_for_n = 0;
   return 0;
 }
 
@@ -788,6 +792,7 @@ int rpeg_engine_set_quad_share(rpeg_engine_t* e, int32_t percent) {
   if (!e) return -1;
   if (percent < 0 || percent > 100) { e->err = "the share is a percentage"; return -1; }
   e->quad_share_pct = (uint32_t)percent;
+  e->split_for_n = 0;
   return 0;
 }
 
@@ -798,6 +803,7 @@ int rpeg_engine_set_ready_cap(rpeg_engine_t* e, int32_t entries) {
     return -1;
   }
   e->ready_cap = (uint32_t)entries;
+  e->split_for_n = 0;
   return 0;
 }
 
@@ -810,6 +816,8 @@ int rpeg_engine_reset_classes(rpeg_engine_t* e) {
   e->cls_nodes.clear();
   e->cls_slots.clear();
   e->cls_pops16.clear();
+  e->cls_split.clear();
+  e->split_for_n = 0;
   if (e->d_cstat) { hipFree(e->d_cstat); e->d_cstat = nullptr; e->cstat_cap = 0; }
   e->cls_sorted.clear();
   e->tables_for = 0xFFFFFFFFu;
@@ -998,7 +1006,25 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   const uint32_t rcap_main = e->need > 0 ? std::min(e->ready_cap, std::max(8u, (e->need + 2 + 7) & ~7u)) : e->ready_cap;
   std::vector<uint8_t> solo(counts.size(), 0), quad(counts.size(), quad_all ? 1 : 0);
   uint32_t quad_nodes = quad_all ? e->max_nodes : 0, quad_slots = quad_all ? e->max_slots : 0;
-  if (!ls && !one && !quad_all && !order.empty()) {
+  // Where every class runs is decided from the class counts and what has been measured (below): on a batch of
+  // thousands of classes that is 0.2 ms of host work.  The decision is kept per class for the next fifteen calls on
+  // batches of about the same size (a class not seen then goes by the plain size rule), unless new measurements
+  // are about to be read.
+  const bool keep_split = !ls && !one && !quad_all && e->quad_share_pct && e->split_for_n && e->learn_calls == 0 &&
+                          n * 4 >= e->split_for_n * 3 && n * 3 <= e->split_for_n * 4 && e->batch_calls - e->split_at < 16 &&
+                          e->split_mass == (mass != nullptr);
+  if (keep_split) {
+    for (size_t c = 0; c < counts.size(); ++c) {
+      const uint8_t a = cids[c] < e->cls_split.size() ? e->cls_split[cids[c]] : (uint8_t)255;
+      if (a == 255) solo[c] = counts[c] < TINY_CLASS ? 1 : 0;
+      else if (a == 1) solo[c] = 1;
+      else if (a == 2) {
+        quad[c] = 1;
+        quad_nodes = std::max(quad_nodes, e->cls_nodes[cids[c]]);
+        quad_slots = std::max(quad_slots, e->cls_slots[cids[c]]);
+      }
+    }
+  } else if (!ls && !one && !quad_all && !order.empty()) {
     // The kernel ends with its slowest wavefront, and a wavefront is as slow as its slowest plan.  The
     // classes with the largest graphs (up to 15 % of the batch: beyond that the single-plan kernel would be
     // the one that ends last) are taken out of it, unless the batch is
@@ -1050,6 +1076,57 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     if (split)
       for (size_t c = 0; c < counts.size(); ++c)
         if (counts[c] < TINY_CLASS) solo[c] = 1;
+    // Where the work decides (more wavefronts of either kernel than are resident at once) and the main kernel has
+    // measured its classes, the threshold is chosen for the batch: of 4, 8, 12, 16 and 24 plans the one for which the
+    // modelled end of the step (deep_model) is earliest.  A class not measured yet counts with the measured time per
+    // node of the batch's other classes.  (Config 1 with 65,536 plans: 21,500 plans in classes of fewer than 16, the
+    // main kernel half empty beside them; with 8 the kernels take 1.4 instead of 2.15 ms.  Config 3 keeps 16.)
+    // (One pass over the classes: sums by class size below 24 plans, then the five thresholds from them.)
+    if (split && e->quad_share_pct) {
+      uint32_t best_th = TINY_CLASS;
+      const DeepModel dm = deep_model(e, rcap_main);
+      constexpr uint32_t TOP = 24;
+      double t_sum = 0.0, nodes_sum = 0.0;
+      uint64_t main_tasks = 0, solo_plans = 0;
+      for (size_t c = 0; c < counts.size(); ++c) {
+        const double t = (double)(e->cls_pops16[cids[c]] >> 12);
+        if (t > 0.0) { t_sum += t; nodes_sum += (double)e->cls_nodes[cids[c]]; }
+        if (solo[c]) solo_plans += counts[c];
+        else main_tasks += (counts[c] + WAVE - 1) / WAVE;
+      }
+      if (t_sum > 0.0 && (main_tasks > (uint64_t)e->n_cu * dm.r_max || solo_plans > (uint64_t)e->n_cu * 32)) {
+        const double per_node = t_sum / nodes_sum;
+        double plan_by[TOP] = {}, main_by[TOP] = {}, max_by[TOP] = {};   // by class size: cost in k_plan, time in the main kernel
+        double w_plan0 = 0.0, w_main0 = 0.0, max0 = 0.0;                  // the classes no threshold moves
+        for (size_t c = 0; c < counts.size(); ++c) {
+          const uint32_t nodes = e->cls_nodes[cids[c]];
+          if (nodes >= cut) { w_plan0 += dm.plan_cost(counts[c], nodes); continue; }
+          const double t0 = (double)(e->cls_pops16[cids[c]] >> 12), t = t0 > 0.0 ? t0 : per_node * (double)nodes;
+          if (counts[c] >= TOP) {
+            w_main0 += (double)((counts[c] + WAVE - 1) / WAVE) * t;
+            max0 = std::max(max0, t);
+          } else {
+            plan_by[counts[c]] += dm.plan_cost(counts[c], nodes);
+            main_by[counts[c]] += t;
+            max_by[counts[c]] = std::max(max_by[counts[c]], t);
+          }
+        }
+        double best_t = 0.0;
+        for (uint32_t th : {TINY_CLASS, 4u, 8u, 12u, TOP}) {
+          double w_main = w_main0, w_plan = w_plan0, max_t = max0;
+          for (uint32_t k = 0; k < TOP; ++k) {
+            if (k < th) w_plan += plan_by[k];
+            else { w_main += main_by[k]; max_t = std::max(max_t, max_by[k]); }
+          }
+          const double t = dm.best(w_main, w_plan, max_t, nullptr);
+          if (th == TINY_CLASS) best_t = t;
+          else if (t < 0.97 * best_t) { best_t = t; best_th = th; }
+        }
+      }
+      if (best_th != TINY_CLASS)
+        for (size_t c = 0; c < counts.size(); ++c)
+          if (e->cls_nodes[cids[c]] < cut) solo[c] = counts[c] < best_th ? 1 : 0;
+    }
     // More than one round of wavefronts: the main kernel ends when its work is done, unless one wavefront alone runs
     // longer than that.  With the measured time of every class (its slowest wavefront on earlier launches) the
     // longest classes are taken out, as many of them as make the modelled end of the step (deep_model) earliest.
@@ -1130,6 +1207,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
         quad_nodes = std::max(quad_nodes, nodes);
         quad_slots = std::max(quad_slots, slots);
       }
+    }
+    if (split && e->quad_share_pct) {   // kept for the next calls
+      e->cls_split.assign(ncls, (uint8_t)255);
+      for (size_t c = 0; c < counts.size(); ++c) e->cls_split[cids[c]] = solo[c] ? 1 : quad[c] ? 2 : 0;
+      e->split_for_n = n; e->split_at = e->batch_calls; e->split_mass = mass != nullptr;
     }
   }
   uint32_t n_eval_waves = 0, n_quad_waves = 0, n_solo = 0;
