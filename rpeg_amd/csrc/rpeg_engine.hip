@@ -437,7 +437,8 @@ struct rpeg_engine_s {
   size_t d_trace_nodes = 0;
   size_t hs_cap = 0;
   std::vector<uint32_t> hs_idx;
-  uint32_t one_plan_waves_per_cu = 128;   // batches of at most this many plans per compute unit take one wavefront per plan
+  uint64_t relearn_at = 0;                // the call that last asked for the measurements again
+  uint32_t one_plan_waves_per_cu = 64;    // batches of at most this many plans per compute unit take one wavefront per plan
   uint32_t host_small_max = 1024;          // rpeg_eval_host: largest batch whose classes the host looks up itself
   int state_lanes = -1;   // -1: chosen per batch; 0: per-plan state in HBM; 8/16/32/64: in LDS, that many plans per wavefront; 1: one plan per wavefront (k_plan)
   bool prof_on = false;
@@ -857,11 +858,12 @@ constexpr uint32_t TINY_CLASS = 16;   // classes of fewer plans go to the single
 // the units to itself, sixteen wavefronts each.  A plan costs k_plan about 40 + 2.2 x nodes microseconds of a wavefront.
 struct DeepModel {
   double n_cu, lds_main, lds_plan;
+  double eff = 1.0;   // the part of the modelled room beside the main kernel that k_plan really gets
   uint64_t r_max;
   double plan_cost(uint32_t plans, uint32_t nodes) const { return (double)plans * (40.0 + 2.2 * (double)nodes); }
   double total(double w_main, double w_plan, double max_t, uint64_t r) const {
     const double t_main = std::max(max_t, w_main / (n_cu * (double)r));
-    const double room = std::max(0.0, std::min(16.0 - 2.0 * (double)r, std::floor((160.0 * 1024 - (double)r * lds_main) / lds_plan)));
+    const double room = eff * std::max(0.0, std::min(16.0 - 2.0 * (double)r, std::floor((160.0 * 1024 - (double)r * lds_main) / lds_plan)));
     const double left = std::max(0.0, w_plan - t_main * n_cu * room);
     return t_main + left / (n_cu * 16.0);
   }
@@ -1127,29 +1129,36 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
         for (size_t c = 0; c < counts.size(); ++c)
           if (e->cls_nodes[cids[c]] < cut) solo[c] = counts[c] < best_th ? 1 : 0;
     }
-    // More than one round of wavefronts: the main kernel ends when its work is done, unless one wavefront alone runs
-    // longer than that.  With the measured time of every class (its slowest wavefront on earlier launches) the
+    // The main kernel ends when its work is done, unless one wavefront alone runs longer than that (in a batch of a
+    // single round of wavefronts it always does).  With the measured time of every class (its slowest wavefront on
+    // earlier launches; a class not measured yet counts with the measured time per node of the others) the
     // longest classes are taken out, as many of them as make the modelled end of the step (deep_model) earliest.
     if (split && e->quad_share_pct) {
-      const DeepModel dm = deep_model(e, rcap_main);
-      uint64_t main_tasks = 0;
-      double w_main = 0.0, w_plan = 0.0;
-      bool known = true;
+      DeepModel dm = deep_model(e, rcap_main);
+      // (where k_quad is going to take its share of a compute unit's wavefront slots and LDS, k_plan gets through
+      // about two thirds of what the model gives it beside the main kernel: measured on configs 2 and 5)
+      if (waves64 <= (uint64_t)e->n_cu * 12) dm.eff = 0.65;
+      double w_main = 0.0, w_plan = 0.0, t_sum = 0.0, nodes_sum = 0.0;
       std::vector<uint32_t> cand;
       for (uint32_t c = 0; c < counts.size(); ++c) {
-        if (solo[c]) { w_plan += dm.plan_cost(counts[c], e->cls_nodes[cids[c]]); continue; }
         const double t = (double)(e->cls_pops16[cids[c]] >> 12);
-        if (t == 0.0) known = false;
-        main_tasks += (counts[c] + WAVE - 1) / WAVE;
-        w_main += (double)((counts[c] + WAVE - 1) / WAVE) * t;
+        if (t > 0.0) { t_sum += t; nodes_sum += (double)e->cls_nodes[cids[c]]; }
+      }
+      const double per_node = nodes_sum > 0.0 ? t_sum / nodes_sum : 0.0;
+      auto t_of = [&](uint32_t c) {
+        const double t = (double)(e->cls_pops16[cids[c]] >> 12);
+        return t > 0.0 ? t : per_node * (double)e->cls_nodes[cids[c]];
+      };
+      for (uint32_t c = 0; c < counts.size(); ++c) {
+        if (solo[c]) { w_plan += dm.plan_cost(counts[c], e->cls_nodes[cids[c]]); continue; }
+        w_main += (double)((counts[c] + WAVE - 1) / WAVE) * t_of(c);
         cand.push_back(c);
       }
-      if (known && main_tasks > (uint64_t)e->n_cu * dm.r_max) {
-        auto t_of = [&](uint32_t c) { return (double)(e->cls_pops16[cids[c]] >> 12); };
+      if (t_sum > 0.0 && !cand.empty()) {
         std::sort(cand.begin(), cand.end(), [&](uint32_t x, uint32_t y) { return t_of(x) > t_of(y); });
         // the modelled end with the k longest classes taken out, for every k: the best k wins (classes of nearly
         // equal time form plateaus, so one class at a time would stop at the first)
-        double best_t = dm.best(w_main, w_plan, cand.empty() ? 0.0 : t_of(cand[0]), nullptr);
+        double best_t = dm.best(w_main, w_plan, t_of(cand[0]), nullptr);
         size_t best_k = 0;
         double wm = w_main, wp = w_plan;
         for (size_t k = 0; k < cand.size(); ++k) {
@@ -1212,6 +1221,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       e->cls_split.assign(ncls, (uint8_t)255);
       for (size_t c = 0; c < counts.size(); ++c) e->cls_split[cids[c]] = solo[c] ? 1 : quad[c] ? 2 : 0;
       e->split_for_n = n; e->split_at = e->batch_calls; e->split_mass = mass != nullptr;
+      // a class that runs in the main kernel for the first time is measured by this launch: read it in the next call
+      // (at most once in eight calls, so that a class whose measurement never arrives cannot keep the read-back on)
+      bool unmeasured = false;
+      for (size_t c = 0; c < counts.size() && !unmeasured; ++c) unmeasured = !solo[c] && !quad[c] && (e->cls_pops16[cids[c]] >> 12) == 0;
+      if (unmeasured && e->learn_calls == 0 && e->batch_calls - e->relearn_at >= 8) { e->learn_calls = 1; e->relearn_at = e->batch_calls; }
     }
   }
   uint32_t n_eval_waves = 0, n_quad_waves = 0, n_solo = 0;

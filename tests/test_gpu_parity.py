@@ -410,11 +410,13 @@ def test_dense_classes_move_to_four_lanes_per_plan_once_measured():
     assert quad[0] == 0 and quad[1] > 0 and quad[2] > 0 and quad[3] == 0, quad
 
 
-@pytest.mark.parametrize("c,n,what", [(3, 65536, "single_plan_tasks"), (5, 40000, "quad_tasks"), (2, 131072, "quad_tasks")])
+@pytest.mark.parametrize("c,n,what", [(3, 65536, "single_plan_tasks"), (5, 40000, "quad_tasks"), (2, 131072, "quad_tasks"),
+                                      (1, 20000, "single_plan_tasks"), (3, 32768, "single_plan_tasks"), (2, 20000, "single_plan_tasks")])
 def test_the_measured_split_changes_where_classes_run_and_not_one_bit(c, n, what):
     """Other batches whose layout the engine changes once it has measured its classes -- more than one round of
     wavefronts (the longest classes leave the main kernel for one plan per wavefront, fewer main-kernel wavefronts per
-    compute unit), other graphs for four lanes per plan --: every call of a fresh engine equals the host build."""
+    compute unit), other graphs for four lanes per plan, a single round of wavefronts whose longest classes leave for
+    one plan per wavefront --: every call of a fresh engine equals the host build."""
     from rpeg_amd.engine.runtime import Engine
     cfg, batch = seeded_batch(c, n)
     ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
@@ -426,7 +428,7 @@ def test_the_measured_split_changes_where_classes_run_and_not_one_bit(c, n, what
         assert np.array_equal(out["mask"], ref["mask"]), call
         for k in ("makespan", "peak", "score"):
             assert same_bits(out[k], ref[k]), (call, k)
-    assert seen[-1] > seen[0], seen
+    assert seen[-1] != seen[0], seen
 
 
 def test_small_batches_pick_the_latency_layout():
