@@ -30,11 +30,11 @@ ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
 ALG_FLOPS = {1: 3697.0, 2: 2165.3, 3: 6502.9, 4: 1245.8, 5: 4155.6}
 # Counter figures of one step, taken from the rocprofv3 --pmc summaries under profiles/ and valid only for the
 # kernel layout they were measured on (`layout`: wave tasks, LDS bytes, plans per wavefront with LDS state,
-# single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats; the task counts to 5 %, k_quad's to 25 %): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
+# single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats; the task counts to 25 %, k_quad's to 35 %): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
 # by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS + VMEM_RD + VMEM_WR of the
 # evaluation kernels / plans).  A run whose layout differs prints null instead of a stale number.
 MEASURED = {
-    2: dict(layout=(6265, 15392, 0, 4815, 474), traffic=245.8e6, instructions_per_plan=3757.3),
+    2: dict(layout=(7407, 15392, 0, 6011, 428), traffic=251.9e6, instructions_per_plan=4128.7),
     3: dict(layout=(26026, 29984, 0, 21741, 0), traffic=5720.0e6, instructions_per_plan=10773.5),
     4: dict(layout=(16396, 14640, 0, 6, 0), traffic=2130.5e6, instructions_per_plan=681.5),
 }
@@ -350,10 +350,10 @@ def main():
     layout = (stats["wave_tasks"], stats["lds_bytes"], stats["state_lanes"], stats["single_plan_tasks"], stats.get("quad_tasks", 0))
     measured = MEASURED.get(c)
     # (which classes run where is decided from times the kernels measure on themselves: the task counts of two runs
-    # differ by a few percent, the number of k_quad's tasks by up to a quarter)
+    # differ by up to a fifth, the number of k_quad's tasks by up to a third)
     same_layout = measured is not None and tuple(measured["layout"][1:3]) == layout[1:3] and all(
         abs(a - b) <= tol * max(a, b) + 8 for a, b, tol in zip((measured["layout"][0],) + tuple(measured["layout"][3:]),
-                                                               (layout[0],) + layout[3:], (0.05, 0.05, 0.25)))
+                                                               (layout[0],) + layout[3:], (0.25, 0.25, 0.35)))
     roofline.update(traffic=measured["traffic"] if same_layout else None, kernel=kernel_name, kernel_ms=kernel_ms,
                     layout=list(layout))
     ipp = measured["instructions_per_plan"] if same_layout else None
