@@ -90,10 +90,10 @@ __device__ inline bool kp_is_inf(double v) {   // on the bits, so that a uniform
 // Ranks, tie-break classes and the list scheduler for a class of at most 64 * NS nodes.  l_rank holds the
 // ranks while they are computed and the finish times afterwards; nd is the index of the neutral element.
 // Returns 0, 1 on a broken class (cycle), 2 when the push counter outgrew its field (a limit of this kernel).
-template <int NS>
+template <int NS, bool keep_trace>
 __device__ inline int kp_schedule(const ClassView& cv, const int n, const int lane, const uint64_t ovl,
                                    const uint64_t dpne, const int nd, const double* l_dur, double* l_rank,
-                                   double* l_start, uint8_t* l_pt, const bool keep_trace, uint16_t* l_order,
+                                   double* l_start, uint8_t* l_pt, uint16_t* l_order,
                                    double* out_makespan, long* out_pops, unsigned long long* stamp) {
   const double inf = __builtin_inf();
   double key[NS], tm[NS], dvc[NS], dur[NS], rk[NS];
@@ -190,6 +190,13 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
     for (int s = 0; s < NS; ++s) {
       ord[s] <<= KP_TIE_BITS;
       shared[s] = eq[s] > 1u;
+      // pt[s] from here on: the vertices whose allocations overlap one this node reserves.  The overlap relation
+      // is symmetric, so a dispatched node D delays node s exactly when D's reserved set meets this mask.
+      uint32_t touch = 0u;
+#pragma unroll
+      for (int x = 0; x < RPEG_MAX_V; ++x)
+        if ((info[s] >> x) & 1u) touch |= mask_row(ovl, x);
+      pt[s] = touch;
     }
   }
   __syncthreads();   // l_rank is reused for the finish times from here on
@@ -210,9 +217,9 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
   double makespan = 0.0;
   int done = 0;
   bool ok = true;
-  long pops = 0, slow_decisions = 0;
-  const long guard_max = (long)n * n + 64;
-  long guard = 0;
+  uint32_t pops = 0, slow_decisions = 0;
+  const uint32_t guard_max = (uint32_t)n * (uint32_t)n + 64u;   // (at most 384 nodes)
+  uint32_t guard = 0;
   while (done < n && guard < guard_max) {
     ++guard;
     ++pops;
@@ -250,14 +257,15 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
         // Lanes that agree in the high word nearly always hold the same time exactly (nodes released by one
         // finish, or waiting for one device): then the low words need no reduction of their own.
         const uint32_t lo0 = (uint32_t)__builtin_amdgcn_readlane((int)elo, __builtin_ctzll(m));
-        if (__ballot(cand && elo != lo0) != 0ull) {
+        // (ballots of single comparisons, combined on the scalar unit: every lane is active here)
+        if ((m & __ballot(elo != lo0)) != 0ull) {
           const uint32_t glo = kp_wave_umin(cand ? elo : 0xFFFFFFFFu);
           cand = cand && elo == glo;
-          m = __ballot(cand);
+          m &= __ballot(elo == glo);
         }
         if (m & (m - 1ull)) {
           const uint32_t go_ = kp_wave_umin(cand ? bo : 0xFFFFFFFFu);
-          m = __ballot(cand && bo == go_);
+          m &= __ballot(bo == go_);
         }
       }
       wl = __builtin_ctzll(m);
@@ -374,13 +382,10 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
     const double fin = gk + d;
     makespan = fin > makespan ? fin : makespan;
     ++done;
-    unsigned touched = 0;
-#pragma unroll
-    for (int x = 0; x < RPEG_MAX_V; ++x)
-      if ((binfo >> x) & 1u) touched |= mask_row(ovl, x);
+    const uint32_t reserved = binfo & 0xFFu;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-      const bool hit = (info[s] & touched) != 0u;
+      const bool hit = (pt[s] & reserved) != 0u;
       dvc[s] = hit && fin > dvc[s] ? fin : dvc[s];
       if (mine && s == ws) key[s] = inf;
     }
@@ -411,7 +416,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
   }
   if (done != n) ok = false;
   *out_makespan = makespan;
-  *out_pops = (slow_decisions << 20) | pops;
+  *out_pops = ((long)slow_decisions << 20) | (long)pops;
   if (ctr > KP_TIE_MASK) return 2;   // the push counter outgrew its field of the packed order: a limit of this kernel
   return ok ? 0 : 1;
 }
@@ -731,12 +736,17 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   uint16_t* const l_order = L.util ? l_ord : nullptr;
   if (!err) {
     int ok;
-    if (n <= 64) ok = kp_schedule<1>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
-    else if (n <= 128) ok = kp_schedule<2>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
-    else if (n <= 192) ok = kp_schedule<3>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
-    else if (n <= 256) ok = kp_schedule<4>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
-    else if (n <= 320) ok = kp_schedule<5>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
-    else ok = kp_schedule<6>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, keep, l_order, &makespan, &pops, stamp);
+    // (the trace of start and finish times is compiled out where no output needs it: its flags and pointers would
+    // otherwise be carried through the scheduling loop)
+#define KP_SCHEDULE(NS) (keep ? kp_schedule<NS, true>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, l_order, &makespan, &pops, stamp) \
+                              : kp_schedule<NS, false>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, nullptr, &makespan, &pops, stamp))
+    if (n <= 64) ok = KP_SCHEDULE(1);
+    else if (n <= 128) ok = KP_SCHEDULE(2);
+    else if (n <= 192) ok = KP_SCHEDULE(3);
+    else if (n <= 256) ok = KP_SCHEDULE(4);
+    else if (n <= 320) ok = KP_SCHEDULE(5);
+    else ok = KP_SCHEDULE(6);
+#undef KP_SCHEDULE
     err = ok != 0;
     limit = ok == 2;
   }
