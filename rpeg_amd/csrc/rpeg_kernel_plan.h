@@ -220,7 +220,9 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
   uint32_t pops = 0, slow_decisions = 0;
   const uint32_t guard_max = (uint32_t)n * (uint32_t)n + 64u;   // (at most 384 nodes)
   uint32_t guard = 0;
-  while (done < n && guard < guard_max) {
+  for (;;) {
+    if (done >= n) break;
+    if (guard >= guard_max) break;
     ++guard;
     ++pops;
     // ---- One decision of the heap: the pops up to the next dispatch.  The heap pops stale entries (key below
@@ -253,7 +255,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
       if (ghi >= 0x7FF00000u) { ok = false; break; }   // nothing is ready: cycle (scheduler.py:548-550)
       bool cand = ehi == ghi;
       unsigned long long m = __ballot(cand);
-      if (m & (m - 1ull)) {
+      if (__builtin_popcountll(m) > 1) {
         // Lanes that agree in the high word nearly always hold the same time exactly (nodes released by one
         // finish, or waiting for one device): then the low words need no reduction of their own.
         const uint32_t lo0 = (uint32_t)__builtin_amdgcn_readlane((int)elo, __builtin_ctzll(m));
@@ -263,7 +265,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
           cand = cand && elo == glo;
           m &= __ballot(elo == glo);
         }
-        if (m & (m - 1ull)) {
+        if (__builtin_popcountll(m) > 1) {
           const uint32_t go_ = kp_wave_umin(cand ? bo : 0xFFFFFFFFu);
           m &= __ballot(bo == go_);
         }
@@ -282,7 +284,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
         in_r[s] = (dvc[s] > key[s]) & ((key[s] < gk) | ((key[s] == gk) & (o < go)));
         n_shared += (in_r[s] & shared[s]) ? 1u : 0u;
       }
-      slow = (m & (m - 1ull)) != 0ull || __ballot(other) != 0ull;
+      slow = __builtin_popcountll(m) > 1 || __ballot(other) != 0ull;
       if (!slow) {
         // Fresh ties of the entries pushed back: the heap hands them out in pop order, i.e. in the order of
         // the old keys.  Entries that share their position with no other node never compare ties and take
@@ -291,7 +293,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
 #pragma unroll
         for (int s = 0; s < NS; ++s) rank[s] = 0u;
         const unsigned long long ms = __ballot(n_shared > 0u);
-        if ((ms & (ms - 1ull)) != 0ull || __ballot(n_shared > 1u) != 0ull) {
+        if (__builtin_popcountll(ms) > 1 || __ballot(n_shared > 1u) != 0ull) {
           total = 0u;
 #pragma unroll
           for (int s = 0; s < NS; ++s) {
@@ -336,11 +338,11 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
         const uint32_t ghi = kp_wave_umin(khi);
         bool cand = khi == ghi;
         unsigned long long m = __ballot(cand);
-        if (m & (m - 1ull)) {
+        if (__builtin_popcountll(m) > 1) {
           const uint32_t glo = kp_wave_umin(cand ? klo : 0xFFFFFFFFu);
           cand = cand && klo == glo;
           m = __ballot(cand);
-          if (m & (m - 1ull)) {
+          if (__builtin_popcountll(m) > 1) {
             const uint32_t go_ = kp_wave_umin(cand ? bo : 0xFFFFFFFFu);
             m = __ballot(cand && bo == go_);
           }
@@ -403,7 +405,7 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
       const bool me = lane == (wn & 63);
 #pragma unroll
       for (int s = 0; s < NS; ++s)
-        if (me && s == (wn >> 6)) {
+        if (me && (NS == 1 || s == (wn >> 6))) {   // (a successor is a node of the class: below 64 when NS is 1)
           tm[s] = fin > tm[s] ? fin : tm[s];
           deg[s] -= 1u;
           if (deg[s] == 0u) {
