@@ -494,19 +494,6 @@ RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) 
 // pairwise-overlap graph.  `order` lists the vertices in order of first appearance among the
 // lowered operator nodes (it fixes the insertion order of the reference's dicts and hence the
 // order of its float sums).  VM provides w_shard(v) (as double), mem_w(v), opt(v), extra(v).
-// Whether some device is covered by exactly the vertex set M and no other set dominates it: M is a maximal
-// clique of the overlap graph.
-RPEG_HD bool maximal_clique(int nv, const PlanMasks& pm, unsigned M) {
-  bool clique = true, maximal = true;
-  for (int v = 0; v < nv; ++v) {
-    const bool in = (M >> v) & 1u;
-    const bool fits = (M & ~mask_row(pm.ovl, v)) == 0;   // every member of M intersects v
-    if (in && !fits) clique = false;
-    if (!in && fits) maximal = false;
-  }
-  return clique && maximal;
-}
-
 // Peak of the devices covered by exactly the vertex set M.
 template <class VM>
 RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
@@ -589,31 +576,40 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
   return peak;
 }
 
+// The maximal cliques of the overlap graph among the vertex sets that contain no vertex below V, given the
+// set M of the vertices below V already chosen and c, the vertices that intersect every one of those: bit M of
+// `found` is set for every maximal clique M.  The relation is symmetric, so a vertex outside M that intersects
+// every member of M is in c, and one inside M that misses a member is not: M is a maximal clique exactly when
+// c == M.  (All 63 sets in 63 ANDs and 63 comparisons; rows of vertices the structure does not have are zero.)
+template <int V, unsigned M>
+RPEG_HD void clique_sets(const unsigned (&row)[RPEG_MAX_V], unsigned c, uint64_t& found) {
+  if constexpr (V == RPEG_MAX_V) {
+    if (M != 0u && c == M) found |= 1ull << M;
+  } else {
+    clique_sets<V + 1, M>(row, c, found);
+    clique_sets<V + 1, M | (1u << V)>(row, c & row[V], found);
+  }
+}
+
 template <class VM>
 RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
                                const PlanMasks& pm, const VM& vm) {
-  static_assert(RPEG_MAX_V <= 6, "a vertex set is packed into six bits below");
+  static_assert(RPEG_MAX_V <= 6, "a vertex set is one bit of a 64-bit word below");
   const StructMasks sm = struct_masks(st, order);
   const unsigned full = (1u << st.n_vertex) - 1u;
   double best = -1.0;
-  // First the maximal cliques of this plan (a graph on six vertices has at most nine: six bits each in one word),
-  // then their peaks.  On the GPU the lanes of a wavefront carry different plans: testing a set is cheap, the peak
-  // of a set is not, and this way a wavefront computes as many peaks as its plan with the most cliques has, not
-  // one for every set that is a clique in some lane.
-  uint64_t list = 0;
-  int cnt = 0;
-  for (unsigned M = 1; M <= full; ++M) {
-    if (!maximal_clique(st.n_vertex, pm, M)) continue;
-    if (cnt < 10) {
-      list |= (uint64_t)M << (6 * cnt);
-      ++cnt;
-    } else {   // (not reached with six vertices)
-      const double peak = device_class_peak(P, st, order, sm, pm, vm, M);
-      if (peak > best) best = peak;
-    }
-  }
-  for (int k = 0; k < cnt; ++k) {
-    const double peak = device_class_peak(P, st, order, sm, pm, vm, (unsigned)(list >> (6 * k)) & 63u);
+  // First the maximal cliques of this plan, then their peaks in ascending order of the sets.  On the GPU the lanes
+  // of a wavefront carry different plans: finding the sets is cheap, the peak of a set is not, and this way a
+  // wavefront computes as many peaks as its plan with the most cliques has, not one for every set that is a clique
+  // in some lane.
+  unsigned row[RPEG_MAX_V];
+  for (int v = 0; v < RPEG_MAX_V; ++v) row[v] = v < st.n_vertex ? (mask_row(pm.ovl, v) & full) : 0u;
+  uint64_t found = 0;
+  clique_sets<0, 0u>(row, full, found);
+  while (found) {
+    const unsigned M = (unsigned)__builtin_ctzll(found);
+    found &= found - 1ull;
+    const double peak = device_class_peak(P, st, order, sm, pm, vm, M);
     if (peak > best) best = peak;
   }
   return best;
