@@ -388,7 +388,8 @@ int rpeg_sa_propose(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t what,
                     uint64_t stream_c, const int16_t* plan, const double* mass, double T, int32_t vertex, int32_t r_lo,
                     int32_t r_hi, int16_t* out, int64_t* draws, int32_t* fallback);
 
-/* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch, [1] classes lowered
+/* Counters of the last rpeg_eval_batch call: [0] lowering classes in the batch (the classes the engine knows
+   when a small batch needed no layout on the host and was not counted by class), [1] classes lowered
    by this call, [2] wave tasks, [3] dynamic LDS bytes of the evaluation kernel, [4] workspace bytes,
    [5] plans per wavefront with LDS-resident state (0: state in the HBM workspace; 1: one plan per
    wavefront), [6] plans of a large batch that ran one per wavefront beside the main kernel (included

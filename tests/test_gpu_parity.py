@@ -431,6 +431,30 @@ def test_the_measured_split_changes_where_classes_run_and_not_one_bit(c, n, what
     assert seen[-1] != seen[0], seen
 
 
+def test_small_device_batches_skip_the_layout_and_go_the_long_way_for_new_classes():
+    """A small batch of device tensors whose classes the engine knows is two launches and one wait (every plan finds
+    its class through the table on the device, no layout on the host); plans of classes not lowered yet send the call
+    the long way, which lowers them and evaluates the batch again.  With and without the critical-chain masses, every
+    call equals the host build."""
+    from rpeg_amd.engine.runtime import Engine
+    cfg, a = seeded_batch(2, 1500)
+    cfg, b = seeded_batch(2, 1500, start=40000)
+    port = CpuPort(cfg.problem)
+    eng = Engine(cfg.problem)
+    lowered = []
+    for call, batch in enumerate((a, a, b, b, a)):
+        ref = port.eval(batch, flags=abi.GATE_STALE, threads=16, want_mass=True)
+        out = eng.eval_mass_device(batch, gate_stale=True) if call % 2 else eng.eval_resident(batch, gate_stale=True)
+        st = eng.stats()
+        lowered.append(st["classes_lowered"])
+        assert st["state_lanes"] == 1 and st["wave_tasks"] <= batch.n
+        out = {k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in out.items()}
+        assert np.array_equal(out["mask"], ref["mask"]), call
+        for k in ("makespan", "peak", "score") + (("mass",) if "mass" in out else ()):
+            assert same_bits(out[k], ref[k]), (call, k)
+    assert lowered[0] > 0 and lowered[1] == 0 and lowered[2] > 0 and lowered[3] == 0 and lowered[4] == 0, lowered
+
+
 def test_small_batches_pick_the_latency_layout():
     cfg, batch = seeded_batch(2, 512)
     eng = engine(2)
