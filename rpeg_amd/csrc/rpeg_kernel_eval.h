@@ -279,9 +279,19 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
         d_next = g_dur[(node_at(v_next).slot) * SS];
       }
       double best = 0.0;
-      for (int j = 0; j < nr.n_succ; ++j) {
-        const int sx = l_succ[nr.succ_begin + j], px = l_pos[sx];
-        const double r = (win > 0 && px - i <= win) ? ring[(px & (win - 1)) * KE_WAVE] : g_rank[(sx) * SS];
+      auto rank_of = [&](int sx) {
+        const int px = l_pos[sx];
+        return (win > 0 && px - i <= win) ? ring[(px & (win - 1)) * KE_WAVE] : g_rank[(sx) * SS];
+      };
+      int j = 0;
+      for (; j + 2 <= nr.n_succ; j += 2) {   // two successors' reads in flight at once
+        const int s0 = l_succ[nr.succ_begin + j], s1 = l_succ[nr.succ_begin + j + 1];
+        const double r0 = rank_of(s0), r1 = rank_of(s1);
+        best = r0 > best ? r0 : best;
+        best = r1 > best ? r1 : best;
+      }
+      if (j < nr.n_succ) {
+        const double r = rank_of(l_succ[nr.succ_begin + j]);
         best = r > best ? r : best;
       }
       const double rk = d + best;

@@ -174,11 +174,19 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     const int v = l_topo[i];
     const NodeRec nr = node_at(v);
     double best = 0.0;
-    for (int j = 0; j < nr.n_succ; ++j) {
+    const double dv = g_dur[nr.slot * RW];
+    int j = 0;
+    for (; j + 2 <= nr.n_succ; j += 2) {   // two independent pairs of LDS reads in flight
+      const int u0 = l_succ[nr.succ_begin + j], u1 = l_succ[nr.succ_begin + j + 1];
+      const double r0 = g_rank[u0 * RW], r1 = g_rank[u1 * RW];
+      best = r0 > best ? r0 : best;
+      best = r1 > best ? r1 : best;
+    }
+    if (j < nr.n_succ) {
       const double r = g_rank[(int)l_succ[nr.succ_begin + j] * RW];
       best = r > best ? r : best;
     }
-    g_rank[v * RW] = g_dur[nr.slot * RW] + best;
+    g_rank[v * RW] = dv + best;
   }
   for (unsigned g = 0; g < cv.h->n_groups; ++g) {
     const GroupRec gr = cv.group[g];
@@ -201,7 +209,13 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     const int b0 = l_kbeg[k], b1 = l_kbeg[k + 1];
     const double rv = g_rank[v * RW];
     int cnt = b0;
-    for (int j = b0; j < b1; ++j) cnt += g_rank[(int)l_bykey[j] * RW] > rv ? 1 : 0;
+    int j = b0;
+    for (; j + 4 <= b1; j += 4) {   // four independent pairs of LDS reads in flight
+      const int u0 = l_bykey[j], u1 = l_bykey[j + 1], u2 = l_bykey[j + 2], u3 = l_bykey[j + 3];
+      const double r0 = g_rank[u0 * RW], r1 = g_rank[u1 * RW], r2 = g_rank[u2 * RW], r3 = g_rank[u3 * RW];
+      cnt += (r0 > rv ? 1 : 0) + (r1 > rv ? 1 : 0) + (r2 > rv ? 1 : 0) + (r3 > rv ? 1 : 0);
+    }
+    for (; j < b1; ++j) cnt += g_rank[(int)l_bykey[j] * RW] > rv ? 1 : 0;
     g_pos[v * RW] = (uint16_t)cnt;
   }
   __syncthreads();   // (the ranks are dead from here on: their array becomes the ready times)
