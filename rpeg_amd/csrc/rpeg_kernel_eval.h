@@ -73,7 +73,7 @@ __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
 // in-degree per node, duration per slot) lives in LDS too, interleaved by lane.  One area serves, one after
 // the other, the plan fields (read by the cost model), the per-vertex memory terms and the ready list; nv is
 // the largest vertex count of the problem's structures.
-__host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls, uint32_t nv) {
+__host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls, uint32_t nv, uint32_t nodes = 0) {
   const size_t rw = ls ? ls : KE_WAVE;
   const size_t ready = (size_t)rcap * rw * 12;                 // key (8 bytes) and meta (4 bytes) per entry
   const size_t plan = (size_t)nv * RPEG_FIELDS * rw * 2, vmem = (size_t)nv * 4 * rw * 8;
@@ -81,11 +81,17 @@ __host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls, uint3
   // (2 KB more for the full-width kernel: measured, not derived.  With 1-3 KB of slack behind the ready list the
   // steps of configs 2, 3 and 4 are 2-3 % shorter on the same machine; from 4 KB on config 3 loses a wavefront
   // per compute unit and from 6 KB on config 4 does.)
-  return ((top + 15) & ~size_t(15)) + (ls ? 0 : 2048);
+  const size_t bytes = ((top + 15) & ~size_t(15)) + (ls ? 0 : 2048);
+  // The rank pass of the full-width kernel keeps the ranks of the last nodes of the order in this area (a ring of a
+  // power of two of rows of 64 doubles, and two bytes per node behind it); a successor further back is read from the
+  // workspace, a round trip through the L2 right after the store.  With the unrolled steps of a graph of more than
+  // 32 nodes the successors in the next step are 10-20 places on: 32 rows hold them, 16 do not.
+  const size_t ring = !ls && nodes > 32 ? (size_t)32 * KE_WAVE * 8 + ((2 * (size_t)nodes + 15) & ~size_t(15)) : 0;
+  return bytes > ring ? bytes : ring;
 }
 __host__ __device__ inline size_t ke_lds_bytes(uint32_t cls_bytes, uint32_t rcap, uint32_t ls, uint32_t nodes,
                                                uint32_t slots, uint32_t nv) {
-  return cls_bytes + ke_dyn_bytes(rcap, ls, nv) + (size_t)ls * ((16ull * nodes + 8ull * slots + nodes + 15) & ~15ull);
+  return cls_bytes + ke_dyn_bytes(rcap, ls, nv, nodes) + (size_t)ls * ((16ull * nodes + 8ull * slots + nodes + 15) & ~15ull);
 }
 
 #if defined(__HIPCC__)
@@ -256,7 +262,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     // memory model and the ready list) holds the ranks of the last `win` nodes of the order, interleaved by
     // lane, and the place of every node in the order; a successor further back is read from the workspace.
     // All lanes carry plans of one class, so the control flow is uniform.
-    const int dyn_bytes = (int)ke_dyn_bytes(L.rcap, 0, L.max_v);
+    const int dyn_bytes = (int)ke_dyn_bytes(L.rcap, 0, L.max_v, L.ws_nodes);
     int win = (dyn_bytes - ((2 * n + 15) & ~15)) / (KE_WAVE * 8);
     while (win & (win - 1)) win &= win - 1;   // a power of two: the place in the ring is a mask away
     uint16_t* l_pos = (uint16_t*)(dyn + (size_t)win * KE_WAVE * 8);
@@ -320,8 +326,11 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     }
     for (int j = 0; j < gr.count; ++j) g_rank[(cv.gmember[gr.begin + j]) * SS] = top;
   }
-  for (int v = 0; v < n; ++v) {
-    g_deg[(v) * SS] = cv.node[v].indeg;
+  for (int v = 0; v < n; ++v) {   // (the node records from their LDS copies: a scalar load from the pool per node waited for each)
+    NodeRec nr;
+    const uint64_t bits = l_node[v];
+    __builtin_memcpy(&nr, &bits, 8);
+    g_deg[(v) * SS] = nr.indeg;
     g_time[(v) * SS] = 0.0;
   }
 

@@ -180,7 +180,9 @@ def test_plans_that_outgrow_the_learned_ready_list_are_redone():
         assert same_bits(out["makespan"], ref["makespan"]) and same_bits(out["score"], ref["score"])
         assert eng.stats()["state_lanes"] == 0
         lds.append(eng.stats()["lds_bytes"])
-    assert lds[1] < lds[0] and lds[1] < lds[3]      # the second call ran with the capacity learned from the chains
+    # the second call ran with the capacity learned from the chains (the area of the ready lists also holds the ring of
+    # the rank pass, which keeps it from shrinking below 32 rows: the two short capacities may need the same LDS)
+    assert lds[1] < lds[0] and lds[1] <= lds[3]
     assert (ref["mask"] & abi.MASK_VALID).sum() > n // 2
     eng.close()
 
