@@ -248,6 +248,37 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
 int rpeg_eval_trace_metrics(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4,
                             double* utilization, int32_t* n_active);
 
+/* lower() of ONE plan (RPEG/passes/unroll.py:85-152 and RPEG/passes/lower.py:330-851), on the host: the lowered
+   graph in the reference's node order (the insertion order of its `nodes` dict) and edge order (the append order
+   of its `edges` list), as rpeg_eval_trace returns it, without evaluating anything.  Integer work only: it needs
+   no engine and no GPU, and reads of `problem` only the structure tables, K_eval, the generation phases and the
+   model parameter counts -- not the hardware record, the device space or the memory policy, which lower() is not
+   given either (the plan is not checked against is_valid, as the reference's lower() does not check it).
+   node_payload / node_ref as for rpeg_plan_detail.  Any output may be NULL.  Returns the node count; -7 when
+   `cap` (nodes, and edges) is too small; -5 when the class cannot be lowered. */
+int rpeg_lower_plan(const rpeg_problem_t* problem, const int16_t* vert_fields, const uint8_t* head4, int32_t* node_kind,
+                    int32_t* node_vertex, int32_t* node_step, int32_t* node_sub, int32_t* node_src, int64_t* node_payload,
+                    int32_t* node_ref, int32_t* edges, int32_t* n_edges, int32_t cap);
+
+/* Per-node and per-device quantities of ONE plan, for the host objects behind the reference's own names
+   (NodeCostModel.time(node), RPEG/model/cost.py:66-88; _device_peaks / mem_worst_violation / mem_feasible,
+   RPEG/model/memory.py:608-887; ExecNode.payload_in_bytes and .label, RPEG/passes/lower.py:396-403, 523-567,
+   711-724).  The plan is given as for rpeg_eval_trace; nodes are in the reference's node order.
+     node_time[i]     NodeCostModel.time of node i (NaN where the reference would raise ZeroDivisionError)
+     node_payload[i]  payload_in_bytes of a COMM / RESHARD node, 0 for an operator node
+     node_ref[i]      what the node's label names: the index of the template's data edge (the container of that
+                      edge) for an activation transfer, 16 + model for a weight transfer or reshard ("W_<model>"),
+                      -1 for an operator node
+     set_peak[M]      64 doubles: for a non-empty set M of template vertices (bit v = vertex v) whose allocations
+                      all intersect, the peak in bytes of a device that lies in the allocations of exactly the
+                      vertices of M (every such device has the same peak: _device_peaks groups the operator nodes
+                      by device, memory.py:626-636); 0 for any other M.  Which devices exist, and in which order
+                      the reference's dictionary holds them, is integer geometry the caller does.
+   Any output may be NULL.  Returns the node count, or a negative status (-6: the plan breaks an integer rule of
+   is_valid; -7: cap too small). */
+int rpeg_plan_detail(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* node_time,
+                     int64_t* node_payload, int32_t* node_ref, int32_t cap, double* set_peak);
+
 /* Batched simulated annealing: n_chains independent Metropolis-Hastings chains of n_steps steps.  One
    step of a chain is one iteration of the inner loop of optimize() (RPEG/search/optimizer.py:702-930):
    with probability alpha_pair*min(1,T/T_init) a donor/receiver proposal (multi_move_pair,

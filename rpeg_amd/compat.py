@@ -9,11 +9,18 @@ pipeline.py:40-60).  `install()` makes those statements resolve to `rpeg_amd.*`:
     from search.optimizer import optimize, polish, OptimizerConfig     # the GPU engine behind the same names
 
 Registered: core.types; ir.plan, ir.rpeg, ir.ppo, ir.grpo, ir.dpo, ir.ac_share, ir.serialize; model.cost,
-model.hardware, model.memory, model.models, model.workload; search.cache, search.evaluate, search.inter_model,
-search.moves, search.optimizer.  (The search part of pipeline.py is rpeg_amd.search.pipeline.search_plan; it has
-no module of the reference's tree to stand for.)  Not registered, because their work happens inside the engine
-and no host object stands for it: passes.unroll, passes.lower, schedule.scheduler (evaluate() returns the lowered
-graph and the trace they would produce), and the reference's runtime, scripts and logging packages.
+model.hardware, model.memory, model.models, model.workload; passes.unroll, passes.lower; schedule.scheduler,
+schedule.trace; search.cache, search.evaluate, search.inter_model, search.moves, search.optimizer.  (The search
+part of pipeline.py is rpeg_amd.search.pipeline.search_plan; it has no module of the reference's tree to stand
+for.)  With them the call sequence of the reference's pipeline runs on the engine:
+
+    lowered = lower(rpeg, unroll(rpeg, K_eval), plan, suite, K_eval, workload=workload)
+    trace = schedule(executable=lowered, cost_model=NodeCostModel(hw, suite, workload), device_space=space)
+    violation = mem_worst_violation(lowered, NodeMemoryModel(hw, suite, workload, trainable=...))
+    t = cost_model.time(node)
+
+Not registered: passes.transfer_resources (the reservations are `Trace.reserved_allocations`) and the reference's
+runtime, scripts and logging packages.
 """
 
 from __future__ import annotations
@@ -22,10 +29,11 @@ import importlib
 import sys
 import types
 
-PACKAGES = ("core", "ir", "model", "search")
+PACKAGES = ("core", "ir", "model", "passes", "schedule", "search")
 MODULES = ("core.types",
            "ir.plan", "ir.rpeg", "ir.ppo", "ir.grpo", "ir.dpo", "ir.ac_share", "ir.serialize",
            "model.cost", "model.hardware", "model.memory", "model.models", "model.workload",
+           "passes.unroll", "passes.lower", "schedule.scheduler", "schedule.trace",
            "search.cache", "search.evaluate", "search.inter_model", "search.moves", "search.optimizer")
 _installed: dict = {}
 

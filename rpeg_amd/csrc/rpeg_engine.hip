@@ -36,8 +36,7 @@ using namespace rpeg;
 namespace {
 
 constexpr int WAVE = 64;
-constexpr int READY_CAP = 64;
-constexpr uint32_t IDLE_LANE = 0xFFFFFFFFu;  // padding lane of a partly filled wavefront  // ready-list entries per plan (LDS); overflow sets RPEG_MASK_ERROR
+constexpr uint32_t IDLE_LANE = 0xFFFFFFFFu;  // padding lane of a partly filled wavefront
 
 #define HIP_TRY(e, call)                                                                   \
   do {                                                                                     \
@@ -53,7 +52,7 @@ struct DevMem {
   double* r;       // rank rows
   double* d;       // duration rows
   uint8_t* deg;    // in-degree rows
-  uint16_t* ready; // LDS, pre-offset by lane
+  uint16_t* ready; // ready list, one entry per node (the heap of the reference has no capacity), pre-offset by lane
   double* tr_start;
   double* tr_finish;
   int32_t* tr_seq;   // dispatch index per node
@@ -69,8 +68,9 @@ struct DevMem {
   }
 };
 
+// workspace of one wavefront of the generic kernel: time and rank rows, duration rows, in-degree rows, ready list
 __host__ __device__ inline size_t wave_ws_bytes(uint32_t nodes, uint32_t slots) {
-  size_t b = (size_t)WAVE * (16ull * nodes + 8ull * slots + nodes);
+  size_t b = (size_t)WAVE * (16ull * nodes + 8ull * slots + 2ull * nodes + nodes);
   return (b + 255) & ~size_t(255);
 }
 
@@ -312,7 +312,6 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
                                                uint8_t* __restrict__ ws, uint32_t ws_nodes, uint32_t ws_slots,
                                                uint32_t flags, double* makespan, double* peak, double* score,
                                                uint8_t* mask, double* tr_start, double* tr_finish, int32_t* tr_seq) {
-  extern __shared__ uint16_t lds_ready[];
   const int lane = threadIdx.x;
   const uint64_t n_waves = (n_sorted + WAVE - 1) / WAVE;
   uint8_t* base = ws + (size_t)blockIdx.x * wave_ws_bytes(ws_nodes, ws_slots);
@@ -320,8 +319,8 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
   mem.t = (double*)base + lane;
   mem.r = (double*)base + (size_t)ws_nodes * WAVE + lane;
   mem.d = (double*)base + 2 * (size_t)ws_nodes * WAVE + lane;
-  mem.deg = base + 8 * (2 * (size_t)ws_nodes + ws_slots) * WAVE + lane;
-  mem.ready = lds_ready + lane;
+  mem.ready = (uint16_t*)(base + 8 * (2 * (size_t)ws_nodes + ws_slots) * WAVE) + lane;
+  mem.deg = base + (8 * (2 * (size_t)ws_nodes + ws_slots) + 2 * (size_t)ws_nodes) * WAVE + lane;
   mem.tr_start = tr_start;
   mem.tr_finish = tr_finish;
   mem.tr_seq = tr_seq;
@@ -336,12 +335,46 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
     const int nv = P->st[h.structure].n_vertex;
     for (int v = 0; v < RPEG_MAX_V; ++v)
       if (v < nv) load_vertex(vert, stride, i, v, &a[v]);
-    PlanOut o = eval_plan(*P, cv, h, a, mem, READY_CAP, flags);
+    PlanOut o = eval_plan(*P, cv, h, a, mem, (int)ws_nodes, flags);
     if (makespan) makespan[i] = o.makespan;
     if (peak) peak[i] = o.peak;
     if (score) score[i] = o.score;
     if (mask) mask[i] = o.mask;
   }
+}
+
+// Per-node quantities of ONE plan, for the host objects of the reference's API: lane s evaluates
+// NodeCostModel.time of the nodes that share duration slot s (cost.py:66-88), lane M (a bit set of template
+// vertices) the peak of a device that lies in exactly the allocations of M (memory.py:686-839; 0 for a set whose
+// allocations do not all intersect).  All 64 lanes work on the same plan.
+__global__ __launch_bounds__(WAVE) void k_plan_detail(const rpeg_problem_t* __restrict__ P, const int16_t* __restrict__ vert,
+                                                      const uint8_t* __restrict__ head, const uint8_t* __restrict__ blob,
+                                                      double* __restrict__ dur, double* __restrict__ set_peak) {
+  const int lane = threadIdx.x;
+  const ClassView cv = class_view(blob);
+  const PlanHead h = load_head(head, 1, 0);
+  const rpeg_struct_t& st = P->st[h.structure];
+  const int nv = st.n_vertex;
+  VPlan a[RPEG_MAX_V];
+  for (int v = 0; v < RPEG_MAX_V; ++v)
+    if (v < nv) load_vertex(vert, 1, 0, v, &a[v]);
+  for (unsigned s = lane; s < cv.h->n_slots; s += WAVE) {
+    bool zd = false;
+    const double t = slot_duration(*P, st, h.split, cv.slot[s], a, &zd);
+    dur[s] = zd ? __builtin_nan("") : t;
+  }
+  const PlanMasks pm = plan_masks(a, nv);
+  const bool coresident = struct_coresident(st);
+  VMem vm[RPEG_MAX_V];
+  for (int v = 0; v < RPEG_MAX_V; ++v)
+    if (v < nv) vm[v] = vertex_memory(*P, st.vertex[v], a[v], coresident);
+  const VMemArray vma{vm};
+  const StructMasks sm = struct_masks(st, cv.h->vorder);
+  const unsigned M = (unsigned)lane;
+  bool clique = M != 0u && M < (1u << nv);
+  for (int v = 0; v < nv; ++v)
+    if ((M >> v) & 1u) clique = clique && (mask_row(pm.ovl, v) & M) == M;
+  set_peak[lane] = clique ? device_class_peak(*P, st, cv.h->vorder, sm, pm, vma, M) : 0.0;
 }
 
 __global__ void k_op_time(const rpeg_problem_t* __restrict__ P, uint64_t n, int structure, int vertex,
@@ -438,6 +471,7 @@ struct rpeg_engine_s {
   uint8_t* h_stage = nullptr;   // pinned mirror of the result region of d_stage
   size_t h_stage_cap = 0;
   uint8_t* d_trace = nullptr;   // rpeg_eval_trace: one plan's fields and header, then start / finish / dispatch index
+  uint8_t* d_detail = nullptr;  // rpeg_plan_detail: one plan's fields and header, then slot durations and vertex-set peaks
   size_t d_trace_nodes = 0;
   size_t hs_cap = 0;
   std::vector<uint32_t> hs_idx;
@@ -753,6 +787,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_stage) hipFree(e->d_stage);
   if (e->h_stage) hipHostFree(e->h_stage);
   if (e->d_trace) hipFree(e->d_trace);
+  if (e->d_detail) hipFree(e->d_detail);
   if (e->d_ws) hipFree(e->d_ws);
   if (e->ev0) hipEventDestroy(e->ev0);
   if (e->ev1) hipEventDestroy(e->ev1);
@@ -1637,7 +1672,7 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   const uint32_t o32 = (uint32_t)off;
   HIP_TRY(e, hipMemcpy(e->d_perm, lanes, sizeof lanes, hipMemcpyHostToDevice));
   HIP_TRY(e, hipMemcpy(e->d_cls, &o32, 4, hipMemcpyHostToDevice));
-  hipLaunchKernelGGL(k_eval_generic, dim3(1), dim3(WAVE), (size_t)READY_CAP * WAVE * 2, s, e->dP, (uint64_t)WAVE, d_vert, d_head,
+  hipLaunchKernelGGL(k_eval_generic, dim3(1), dim3(WAVE), 0, s, e->dP, (uint64_t)WAVE, d_vert, d_head,
                      (uint64_t)1, e->d_perm, e->d_cls, e->d_pool, e->d_ws, e->max_nodes, e->max_slots, 0u,
                      (double*)nullptr, (double*)nullptr, (double*)nullptr, (uint8_t*)nullptr, d_tr, d_tr + n,
                      (int32_t*)(d_tr + 2 * (size_t)n));
@@ -1660,6 +1695,113 @@ int rpeg_eval_trace(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t*
   if (edges)
     for (size_t j = 0; j < lc.edges.size(); ++j) { edges[2 * j] = lc.edges[j].first; edges[2 * j + 1] = lc.edges[j].second; }
   if (n_edges) *n_edges = (int32_t)lc.edges.size();
+  return n;
+}
+
+// lower() of ONE plan on the host (integer work only, no engine and no GPU needed): the plan's class signature
+// and the class lowering the engine itself uses.
+int rpeg_lower_plan(const rpeg_problem_t* problem, const int16_t* vert_fields, const uint8_t* head4, int32_t* node_kind,
+                    int32_t* node_vertex, int32_t* node_step, int32_t* node_sub, int32_t* node_src, int64_t* node_payload,
+                    int32_t* node_ref, int32_t* edges, int32_t* n_edges, int32_t cap) {
+  if (!problem || !vert_fields || !head4) return -1;
+  if (problem->abi_version != RPEG_ABI_VERSION) return -3;
+  const PlanHead h = load_head(head4, 1, 0);
+  if (h.structure < 0 || h.structure >= problem->n_struct || h.split < 0 || h.split >= problem->n_split || h.tau0 > 3 || h.tau1 > 3)
+    return -1;
+  const rpeg_struct_t& st = problem->st[h.structure];
+  VPlan a[RPEG_MAX_V];
+  std::memset(a, 0, sizeof a);
+  for (int v = 0; v < st.n_vertex; ++v) load_vertex(vert_fields, 1, 0, v, &a[v]);
+  const uint64_t sg = plan_signature(*problem, h.structure, h.split, h.tau0, h.tau1, a);
+  LoweredClass lc;
+  try { lc = lower_class(*problem, sg); } catch (const std::exception&) { return -5; }
+  const int n = (int)lc.nodes.size();
+  if (n > cap || (edges && (int)lc.edges.size() > cap)) return -7;
+  const ClassView cv = class_view(lc.blob.data());
+  for (int i = 0; i < n; ++i) {
+    const LoweredNode& nd = lc.nodes[i];
+    const SlotDesc sd = cv.slot[nd.slot];
+    if (node_kind) node_kind[i] = nd.kind;
+    if (node_vertex) node_vertex[i] = nd.kind == 0 ? nd.vertex : nd.a1;
+    if (node_step) node_step[i] = nd.step;
+    if (node_sub) node_sub[i] = nd.sub;
+    if (node_src) node_src[i] = nd.kind == 0 ? nd.vertex : nd.a0;
+    int64_t payload = 0;
+    int32_t ref = -1;
+    if (sd.type == SLOT_COMM_DATA) {
+      payload = sd.q == 0xFF ? st.edge[sd.a].full_bytes : st.edge[sd.a].sub_bytes[h.split][sd.q];
+      ref = sd.a;
+    } else if (sd.type == SLOT_COMM_PUB) {
+      const rpeg_pub_t& pb = st.pub[sd.a];
+      payload = pub_payload(*problem, a[pb.src], a[pb.dst], pb.model);
+      ref = 16 + pb.model;
+    } else if (sd.type == SLOT_RESHARD) {
+      payload = problem->model[sd.b].n_params * problem->model[sd.b].sb;
+      ref = 16 + sd.b;
+    }
+    if (node_payload) node_payload[i] = payload;
+    if (node_ref) node_ref[i] = ref;
+  }
+  if (edges)
+    for (size_t j = 0; j < lc.edges.size(); ++j) { edges[2 * j] = lc.edges[j].first; edges[2 * j + 1] = lc.edges[j].second; }
+  if (n_edges) *n_edges = (int32_t)lc.edges.size();
+  return n;
+}
+
+int rpeg_plan_detail(rpeg_engine_t* e, const int16_t* vert_fields, const uint8_t* head4, double* node_time,
+                     int64_t* node_payload, int32_t* node_ref, int32_t cap, double* set_peak) {
+  if (!e || !vert_fields || !head4) return -1;
+  e->err.clear();
+  PlanHead h = load_head(head4, 1, 0);
+  VPlan a[RPEG_MAX_V];
+  std::memset(a, 0, sizeof a);
+  if (h.structure >= e->P.n_struct) { e->err = "bad structure"; return -1; }
+  const rpeg_struct_t& st = e->P.st[h.structure];
+  for (int v = 0; v < st.n_vertex; ++v) load_vertex(vert_fields, 1, 0, v, &a[v]);
+  if (!plan_valid(e->P, h, a)) { e->err = "plan violates the integer validity rules"; return -6; }
+  const uint64_t sg = plan_signature(e->P, h.structure, h.split, h.tau0, h.tau1, a);
+  LoweredClass lc;
+  try { lc = lower_class(e->P, sg); } catch (const std::exception& ex) { e->err = ex.what(); return -5; }
+  const int n = (int)lc.nodes.size();
+  if ((node_time || node_payload || node_ref) && n > cap) { e->err = "node arrays too small"; return -7; }
+  const int64_t off = class_offset(e, sg, nullptr);
+  if (off < 0) return -5;
+  hipStream_t s = nullptr;
+  HIP_TRY(e, hipDeviceSynchronize());   // (null stream, shared buffers: as rpeg_eval_trace)
+  if (int rc = ensure_pool(e, s)) return rc;
+  constexpr size_t IN_BYTES = 256, SLOTS = 256;
+  if (!e->d_detail) HIP_TRY(e, hipMalloc(&e->d_detail, IN_BYTES + (SLOTS + WAVE) * 8));
+  int16_t* d_vert = (int16_t*)e->d_detail;
+  uint8_t* d_head = e->d_detail + RPEG_MAX_V * RPEG_FIELDS * 2;
+  double* d_out = (double*)(e->d_detail + IN_BYTES);
+  HIP_TRY(e, hipMemcpy(d_vert, vert_fields, RPEG_MAX_V * RPEG_FIELDS * 2, hipMemcpyHostToDevice));
+  HIP_TRY(e, hipMemcpy(d_head, head4, 4, hipMemcpyHostToDevice));
+  hipLaunchKernelGGL(k_plan_detail, dim3(1), dim3(WAVE), 0, s, e->dP, d_vert, d_head, e->d_pool + off, d_out, d_out + SLOTS);
+  HIP_TRY(e, hipGetLastError());
+  double out[SLOTS + WAVE];
+  HIP_TRY(e, hipMemcpy(out, d_out, sizeof out, hipMemcpyDeviceToHost));
+  const ClassView cv = class_view(e->pool.data() + off);
+  for (int i = 0; i < n; ++i) {
+    const LoweredNode& nd = lc.nodes[i];
+    const SlotDesc sd = cv.slot[nd.slot];
+    if (node_time) node_time[i] = out[nd.slot];
+    int64_t payload = 0;
+    int32_t ref = -1;
+    if (sd.type == SLOT_COMM_DATA) {
+      payload = sd.q == 0xFF ? st.edge[sd.a].full_bytes : st.edge[sd.a].sub_bytes[h.split][sd.q];
+      ref = sd.a;
+    } else if (sd.type == SLOT_COMM_PUB) {
+      const rpeg_pub_t& pb = st.pub[sd.a];
+      payload = pub_payload(e->P, a[pb.src], a[pb.dst], pb.model);
+      ref = 16 + pb.model;
+    } else if (sd.type == SLOT_RESHARD) {
+      payload = e->P.model[sd.b].n_params * e->P.model[sd.b].sb;
+      ref = 16 + sd.b;
+    }
+    if (node_payload) node_payload[i] = payload;
+    if (node_ref) node_ref[i] = ref;
+  }
+  if (set_peak) std::memcpy(set_peak, out + SLOTS, WAVE * 8);
   return n;
 }
 

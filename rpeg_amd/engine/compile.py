@@ -127,7 +127,8 @@ def _reach(vertices, data_edges):
     return out
 
 
-def compile_problem(problem: EvalProblem) -> abi.ProblemT:
+def compile_problem(problem: EvalProblem, check_sizes: bool = True) -> abi.ProblemT:
+    """`check_sizes=False` for tables that only the host lowering reads: no horizon bound, no message-size bound."""
     wl, hw, sp, pol = problem.workload, problem.hw, problem.device_space, problem.memory_policy
     P = abi.ProblemT()
     P.abi_version = abi.ABI_VERSION
@@ -136,7 +137,7 @@ def compile_problem(problem: EvalProblem) -> abi.ProblemT:
     P.n_struct, P.n_split, P.K_eval = len(problem.structures), problem.n_splits(), problem.K_eval
     if P.n_split > abi.MAX_SPLIT:
         raise ValueError(f"at most {abi.MAX_PH} generation quantiles are supported")
-    if problem.K_eval < 1 or problem.K_eval > 4095:
+    if problem.K_eval < 1 or (check_sizes and problem.K_eval > 4095):
         # (what bounds the horizon is the size of a lowered graph: 4,095 nodes per class, reported by the engine
         # when a plan's class exceeds it -- a few hundred steps, depending on the template)
         raise ValueError("K_eval must be in 1..4095")
@@ -175,7 +176,7 @@ def compile_problem(problem: EvalProblem) -> abi.ProblemT:
         rec.params_formula = spec.L * rec.w_layer + spec.V * spec.d
         rec.n_params = transformer_parameter_count(spec, m)
         big = wl.B * wl.K * (wl.S + wl.T) * spec.d * spec.dtype_bytes
-        if max(big, 12 * rec.n_params * 4, rec.n_params * spec.dtype_bytes * sp.num_devices()) >= _LIMIT:
+        if check_sizes and max(big, 12 * rec.n_params * 4, rec.n_params * spec.dtype_bytes * sp.num_devices()) >= _LIMIT:
             raise ValueError("workload too large for exact float64 message sizes")
 
     total = wl.B * wl.K

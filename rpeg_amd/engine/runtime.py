@@ -24,7 +24,8 @@ EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
            "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_quad_share", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
-           "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static")
+           "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static", "rpeg_plan_detail",
+           "rpeg_lower_plan")
 
 
 class EngineError(RuntimeError):
@@ -39,6 +40,9 @@ def load_library(path: Optional[str] = None):
     p = path or _LIB_PATH
     if not os.path.exists(p):
         raise EngineError(f"{p} is missing: build it with `python -m rpeg_amd.build` (hipcc, gfx950)")
+    # torch first: it brings its own HIP runtime, and the library must bind to that copy -- loaded the other way
+    # round the process holds a runtime that sees no device (rpeg_engine_create then fails with status -4)
+    import torch  # noqa: F401
     lib = C.CDLL(p)
     vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int32
     lib.rpeg_engine_create.restype = C.c_int
@@ -67,6 +71,10 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_eval_trace.argtypes = [vp] * 13 + [i32, vp]
     lib.rpeg_eval_trace_metrics.restype = C.c_int
     lib.rpeg_eval_trace_metrics.argtypes = [vp] * 5
+    lib.rpeg_lower_plan.restype = C.c_int
+    lib.rpeg_lower_plan.argtypes = [vp] * 12 + [i32]
+    lib.rpeg_plan_detail.restype = C.c_int
+    lib.rpeg_plan_detail.argtypes = [vp, vp, vp, vp, vp, vp, i32, vp]
     lib.rpeg_engine_stats.restype = C.c_int
     lib.rpeg_engine_stats.argtypes = [vp, vp, i32]
     lib.rpeg_engine_set_timing.restype = C.c_int
@@ -442,6 +450,20 @@ class Engine:
         self._check(n, "rpeg_eval_trace")
         return dict(start=start[:n], finish=finish[:n], order=order[:n], kind=kind[:n], vertex=vertex[:n], step=step[:n],
                     sub=sub[:n], src=src[:n], edges=edges[:2 * ne.value].reshape(-1, 2), reserved=reserved[:n])
+
+    def plan_detail(self, batch: PlanBatch, i: int, cap: int = 4096):
+        """NodeCostModel.time, payload bytes and label reference of every lowered node of plan i (the reference's
+        node order), and the device peak of every set of template vertices whose allocations all intersect
+        (rpeg_plan_detail)."""
+        torch = _torch()
+        vert = np.ascontiguousarray(batch.vert[:, i], dtype=np.int16)
+        head = np.ascontiguousarray(batch.head[:, i], dtype=np.uint8)
+        time, payload, ref, peaks = np.zeros(cap), np.zeros(cap, np.int64), np.zeros(cap, np.int32), np.zeros(64)
+        with torch.cuda.device(self.device):
+            n = self.lib.rpeg_plan_detail(self._h, vert.ctypes.data, head.ctypes.data, time.ctypes.data,
+                                          payload.ctypes.data, ref.ctypes.data, cap, peaks.ctypes.data)
+        self._check(n, "rpeg_plan_detail")
+        return dict(time=time[:n], payload=payload[:n], ref=ref[:n], set_peak=peaks)
 
     def trace_metrics(self, batch: PlanBatch, i: int):
         """(Trace.utilization(), Trace.n_active()) of plan i, folded by the library (rpeg_eval_trace_metrics)."""

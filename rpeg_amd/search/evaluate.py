@@ -29,6 +29,8 @@ from ..model.hardware import Hardware
 from ..model.memory import MemoryPolicy, NodeMemoryModel
 from ..model.models import ModelSuite
 from ..model.workload import Workload
+from ..passes.lower import ExecEdge, ExecNode, ExecNodeType, ExecutableRPEG, lower   # noqa: F401  (re-exported)
+from ..schedule.trace import Trace   # noqa: F401  (re-exported: the reference's evaluate module names it)
 from .cache import EvalCache, config_hash
 
 _OOM_BETA = 40.0
@@ -128,17 +130,19 @@ def _engine_for(rpeg: RPEG, suite: ModelSuite, workload: Workload, hw: Hardware,
     return eng, st
 
 
-def _engine_like(rpeg, space: DeviceSpace, suite=None, workload=None, vertex=None):
+def _engine_like(rpeg, space: Optional[DeviceSpace], suite=None, workload=None, vertex=None, hw=None, policy=None):
     """The most recently used engine that holds the template of `rpeg` as a structure on device space `space`
-    (and, when given, for these models and this workload), with the index of that structure -- for calls of the
+    (any space when that is None; and, when given, for these models, this workload, this hardware record and this
+    (optimizer stage, activation checkpointing) pair), with the index of that structure -- for calls of the
     reference's API that name neither the hardware nor the horizon (the proposal functions of search.moves),
     whose results depend on neither.  With `vertex` in place of `rpeg`: an engine with a template that holds that
     vertex, the structure and the vertex's slot in it."""
     want = None if rpeg is None else _structure_of(rpeg).name
     for eng in reversed(list(_engines.values())):
         p = eng.problem
-        if p.device_space != space or (suite is not None and p.suite.specs != suite.specs) or \
-                (workload is not None and p.workload != workload):
+        if (space is not None and p.device_space != space) or (suite is not None and p.suite.specs != suite.specs) or \
+                (workload is not None and p.workload != workload) or (hw is not None and p.hw != hw) or \
+                (policy is not None and (p.memory_policy.optimizer_stage, p.memory_policy.activation_checkpointing) != tuple(policy)):
             continue
         for k, st in enumerate(p.structures):
             if vertex is not None:
@@ -149,6 +153,29 @@ def _engine_like(rpeg, space: DeviceSpace, suite=None, workload=None, vertex=Non
                 return eng, k
     raise LookupError("no evaluation engine for this template and device space yet: evaluate a configuration of it "
                       "(evaluate, evaluate_cached, evaluate_batch) before asking for proposals")
+
+
+def _engine_space_for(rpeg, plan, suite, workload, hw) -> DeviceSpace:
+    """A device space for calls of the reference's API that name none (NodeCostModel.time, mem_worst_violation):
+    node durations and device peaks do not depend on it, only the engine's validity gate does.  The space of the
+    most recently used engine for this template, these models, workload and hardware under which every vertex of
+    the plan is placed validly; else the smallest space that encloses the plan, with the devices per node for which
+    the plan's packing is valid."""
+    def fits(space):
+        return all(is_compatible(plan.sigma[v], plan.pi[v], space) for v in rpeg.vertices)
+    want = _structure_of(rpeg).name
+    for eng in reversed(list(_engines.values())):
+        p = eng.problem
+        if p.suite.specs == suite.specs and p.workload == workload and p.hw == hw and \
+                any(st.name == want for st in p.structures) and fits(p.device_space):
+            return p.device_space
+    R = max(plan.sigma[v].origin[0] + plan.sigma[v].extent[0] for v in rpeg.vertices)
+    N = max(plan.sigma[v].origin[1] + plan.sigma[v].extent[1] for v in rpeg.vertices)
+    g_lo = max(plan.sigma[v].origin[2] + plan.sigma[v].extent[2] for v in rpeg.vertices)
+    for G in range(g_lo, 8 * g_lo + 1):
+        if fits(DeviceSpace(R=R, N=N, G=G)):
+            return DeviceSpace(R=R, N=N, G=G)
+    raise ValueError("the plan's allocations are no valid packing on any device space")
 
 
 def _check_supported(config: Configuration):
@@ -218,137 +245,14 @@ def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload
 
 
 # ----------------------------------------------------------------------------- trace objects
-@dataclass(frozen=True, eq=False)
-class ExecNode:
-    """Lowered node as the reference exposes it to its callers (lower.py:30-81), rebuilt from the
-    engine's per-node arrays."""
-    id: str
-    kind: str                       # "op" | "comm" | "reshard"
-    allocs: Tuple[Allocation, ...]
-    template_vertex: object = None  # operator nodes
-    k: Optional[int] = None
-    model: object = None
-    pi: Optional[Tuple[int, int, int]] = None
-    mb: Optional[int] = None
-
-    def __hash__(self):
-        return hash(self.id)
-
-    def __eq__(self, other):
-        return isinstance(other, ExecNode) and self.id == other.id
-
-
-@dataclass(frozen=True)
-class ExecEdge:
-    src: ExecNode
-    dst: ExecNode
-
-
-@dataclass(frozen=True)
-class ExecutableRPEG:
-    nodes: Tuple[ExecNode, ...]
-    edges: Tuple[ExecEdge, ...]
-    composite_operators: tuple = ()
-
-
-def _devices(alloc: Allocation):
-    o, e = alloc.origin, alloc.extent
-    return [(r, n, g) for r in range(o[0], o[0] + e[0]) for n in range(o[1], o[1] + e[1])
-            for g in range(o[2], o[2] + e[2])]
-
-
-@dataclass(frozen=True)
-class Trace:
-    """Start/finish times per lowered node and the allocations reserved for each (mirror of
-    RPEG/schedule/trace.py:18-118).  The times and the reservations come from the engine; the two summary
-    metrics below fold them on the host exactly as the reference does, device by device in the insertion
-    order of its dictionaries, so they equal the reference's floats."""
-    start: Dict[ExecNode, float]
-    finish: Dict[ExecNode, float]
-    reserved_allocations: Optional[dict] = None
-
-    def makespan(self) -> float:
-        return max(self.finish.values())
-
-    def throughput(self, W_step: float, K: int) -> float:
-        return K * W_step / self.makespan()
-
-    def utilization(self) -> float:
-        """Mean over the devices any node reserves of merged busy time / makespan (trace.py:53-101)."""
-        ms = self.makespan()
-        if ms <= 0:
-            return 0.0
-        intervals: Dict[tuple, list] = {}
-        for node, s in self.start.items():
-            allocs = (self.reserved_allocations[node] if self.reserved_allocations is not None
-                      else node.allocs[-1:] if node.kind in ("comm", "reshard") else node.allocs)
-            for alloc in allocs:
-                for dv in _devices(alloc):
-                    intervals.setdefault(dv, []).append((s, self.finish[node]))
-        if not intervals:
-            return 0.0
-        total = 0.0
-        for spans in intervals.values():
-            merged = 0.0
-            cs = ce = None
-            for s, e in sorted(spans):
-                if ce is None or s > ce:
-                    if ce is not None:
-                        merged += ce - cs
-                    cs, ce = s, e
-                else:
-                    ce = max(ce, e)
-            if ce is not None:
-                merged += ce - cs
-            total += merged / ms
-        return total / len(intervals)
-
-    def n_active(self) -> int:
-        """Number of devices inside any allocation of any node (trace.py:103-118)."""
-        devices = set()
-        for node in self.start:
-            for alloc in node.allocs:
-                devices.update(_devices(alloc))
-        return len(devices)
-
-
-def _trace_of(eng, st, config: Configuration, batch: PlanBatch):
-    tr = eng.trace(batch, 0)
-    verts = config.rpeg.vertices
-    nodes: List[ExecNode] = []
-    n_comm = n_reshard = 0
-    for kind, vertex, step, sub, src in zip(tr["kind"], tr["vertex"], tr["step"], tr["sub"], tr["src"]):
-        v = verts[vertex]
-        if kind == 0:
-            tag = "" if sub < 0 else f":{'g' if v.kind.role.value == 'GEN' else 'i'}{sub}"
-            nodes.append(ExecNode(id=f"{v.id}@{step}{tag}", kind="op", allocs=(config.plan.sigma[v],),
-                                  template_vertex=v, k=int(step), model=v.kind.model, pi=config.plan.pi[v],
-                                  mb=config.plan.mb[v]))
-        else:
-            if kind == 1:
-                n_comm += 1
-                name = f"comm{n_comm}"
-            else:
-                n_reshard += 1
-                name = f"reshard{n_reshard}"
-            nodes.append(ExecNode(id=name, kind="comm" if kind == 1 else "reshard",
-                                  allocs=(config.plan.sigma[verts[src]], config.plan.sigma[v])))
-    # Trace.start / Trace.finish are filled in dispatch order (scheduler.py:517-518)
-    by_dispatch = sorted(range(len(nodes)), key=lambda i: int(tr["order"][i]))
-    start = {nodes[i]: float(tr["start"][i]) for i in by_dispatch}
-    finish = {nodes[i]: float(tr["finish"][i]) for i in by_dispatch}
-    edges = tuple(ExecEdge(nodes[a], nodes[b]) for a, b in tr["edges"])
-    # the allocations the scheduler reserved: of a node's allocations (source first) those whose vertex the
-    # engine reserved, identical allocations once (transfer_resources.py:138-148)
-    reserved = {}
-    for i, node in enumerate(nodes):
-        mask = int(tr["reserved"][i])
-        if tr["kind"][i] == 0:
-            owners = (int(tr["vertex"][i]),)
-        else:
-            owners = (int(tr["src"][i]), int(tr["vertex"][i]))
-        reserved[node] = tuple(dict.fromkeys(config.plan.sigma[verts[x]] for x in owners if (mask >> x) & 1))
-    return Trace(start=start, finish=finish, reserved_allocations=reserved), ExecutableRPEG(nodes=tuple(nodes), edges=edges)
+def _trace_of(eng, st, config: Configuration, batch: PlanBatch, workload=None, suite=None, lowered=None):
+    """(Trace, ExecutableRPEG) of the one plan of `batch`: the lowered graph (passes.lower.lower) and the engine's
+    start / finish time, dispatch position and reserved vertices of every node of it."""
+    from ..schedule.scheduler import trace_on
+    if lowered is None:
+        lowered = lower(config.rpeg, None, config.plan, suite if suite is not None else eng.problem.suite,
+                        eng.problem.K_eval, workload=workload if workload is not None else eng.problem.workload)
+    return trace_on(eng, lowered, batch), lowered
 
 
 # ----------------------------------------------------------------------------- reference API
@@ -360,7 +264,7 @@ def evaluate(config: Configuration, suite: ModelSuite, workload: Workload, hw: H
     eng, st = _engine_for(config.rpeg, suite, workload, hw, config.device_space, K_eval, memory_policy,
                           transfer_policy=config.transfer_resource_policy)
     batch = _pack([config], st, workload)
-    trace, lowered = _trace_of(eng, st, config, batch)
+    trace, lowered = _trace_of(eng, st, config, batch, workload, suite)
     score = trace.throughput(W_step=workload.B * workload.K * (workload.S + workload.T), K=K_eval)
     return score, trace, lowered
 
@@ -402,7 +306,7 @@ def _score_one(config, suite, workload, hw, K_eval, memory_policy, gate_stale):
                           transfer_policy=config.transfer_resource_policy)
     batch = _pack([config], st, workload)
     res = evaluate_batch([config], suite, workload, hw, K_eval, memory_policy, gate_stale=gate_stale)
-    trace, _ = _trace_of(eng, st, config, batch)
+    trace, _ = _trace_of(eng, st, config, batch, workload, suite)
     return float(res.score[0]), trace, res
 
 

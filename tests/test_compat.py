@@ -18,7 +18,11 @@ WANTED = {
     "ir.serialize": ["save_plan"],
     "model.cost": ["NodeCostModel"],
     "model.hardware": ["Hardware"],
-    "model.memory": ["MemoryPolicy", "NodeMemoryModel"],
+    "model.memory": ["MemoryPolicy", "NodeMemoryModel", "_device_peaks", "mem_worst_violation", "mem_feasible"],
+    "passes.unroll": ["unroll", "UnrolledNode"],
+    "passes.lower": ["lower", "ExecNodeType", "ExecNode", "ExecutableRPEG"],
+    "schedule.scheduler": ["schedule"],
+    "schedule.trace": ["Trace"],
     "model.models": ["ModelSuite", "ModelSpec", "Model"],
     "model.workload": ["Workload"],
     "search.cache": ["EvalCache"],
@@ -27,7 +31,7 @@ WANTED = {
     "search.moves": ["build_candidate_directory", "move_gen", "multi_move_pair", "sample_expl", "MoveStats"],
     "search.optimizer": ["optimize", "polish", "OptimizerConfig"],
 }
-INSIDE_THE_ENGINE = ["passes.unroll", "passes.lower", "schedule.scheduler"]
+NOT_MIRRORED = ["passes.transfer_resources", "runtime.job_plan"]
 
 
 @pytest.fixture
@@ -50,7 +54,7 @@ def test_reference_import_statements_resolve_to_this_package(names):
     assert search.optimizer is rpeg_amd.search.optimizer      # one module object: module switches are shared
     import search.moves
     assert search.moves.ABLATION_FIXED_MB is False
-    for module in INSIDE_THE_ENGINE:
+    for module in NOT_MIRRORED:
         with pytest.raises(ModuleNotFoundError):
             exec(f"import {module}", {})
 
@@ -82,8 +86,6 @@ def test_cost_model_record_validates_like_the_reference():
         NodeCostModel(p.hw, p.suite, p.workload, optimizer_stage=3)
     with pytest.raises(ValueError, match="reshard_scale"):
         NodeCostModel(dataclasses.replace(p.hw, reshard_scale=0.0), p.suite, p.workload)
-    with pytest.raises(NotImplementedError):
-        NodeCostModel(p.hw, p.suite, p.workload).time(None)
 
 
 @pytest.mark.gpu
