@@ -46,10 +46,14 @@ enum {
   RPEG_MASK_MEM_OK = 4,    /* no device peak above capacity (memory.py:864-887)               */
   RPEG_MASK_ERROR = 8,     /* the reference would raise (division by zero, cycle) or an engine
                               limit was hit; the numeric outputs of this plan are NaN           */
-  RPEG_MASK_LIMIT = 16     /* set with RPEG_MASK_ERROR when the cause is a limit of this engine
-                              (more than 31 ready nodes at once, a node that reserves more than
-                              two vertex allocations, more than 2^23 heap pushes): the reference
-                              would have evaluated the plan                                      */
+  RPEG_MASK_LIMIT = 16     /* set with RPEG_MASK_ERROR when the cause is a limit of this engine: the
+                              reference would have evaluated the plan.  No evaluation path sets it
+                              for a graph within the stated bounds (4,095 lowered nodes per plan):
+                              a plan whose ready set outgrows what a kernel holds -- 31 or 32 entries
+                              in the plan-per-lane and four-lanes-per-plan kernels -- is redone by
+                              the launch that ends the call with a ready list of one entry per
+                              node, as the reference's heap has no capacity
+                              (RPEG/schedule/scheduler.py:423-546)                                */
 };
 
 /* eval flags */
@@ -434,8 +438,8 @@ int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
    of the problem's largest class does not fit.  lanes = 1: one plan per wavefront, its nodes spread
    over the lanes (the layout of lowest latency, for batches of a few thousand plans at most; classes of
    up to 384 nodes).  lanes = 4: four lanes per plan, sixteen plans per wavefront, the ready entries (at most 32
-   at once) in the registers of the four lanes (the layout for dense graphs, whose plan-per-lane wavefronts end
-   last).
+   at once; a plan with more is redone by the launch that ends the call) in the registers of the four lanes (the
+   layout for dense graphs, whose plan-per-lane wavefronts end last).
    lanes = -1 (default): chosen per batch from its size.
    Results do not depend on the setting. */
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
@@ -448,10 +452,11 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
 int rpeg_engine_set_quad_share(rpeg_engine_t* e, int32_t percent);
 
 /* Ready-list entries per plan in the main kernel: 8, 16, 24 or 32 (default).  A plan with that many nodes
-   ready at once is not evaluated: NaN outputs, RPEG_MASK_ERROR | RPEG_MASK_LIMIT (the reference's heap has no
-   such bound; the longest list seen on the shipped problems is 24).  Fewer entries take less LDS per wavefront.
-   The kernel that runs one plan per wavefront (small batches) keeps its ready set in registers and has no
-   such bound.  No reference counterpart: tests use it to reach the limit. */
+   ready at once is redone, without a bound, by the launch that ends the call (one plan per lane, its state and
+   ready list in HBM: slow, and rare -- the longest list seen on the shipped problems is 24).  Fewer entries take
+   less LDS per wavefront.  The kernel that runs one plan per wavefront (small batches) keeps its ready set in
+   registers and has no such bound.  Results do not depend on the setting.  No reference counterpart: tests use
+   it to reach the redo path. */
 int rpeg_engine_set_ready_cap(rpeg_engine_t* e, int32_t entries);
 
 /* Forgets every lowered class, so that the next rpeg_eval_batch lowers all the classes of its batch

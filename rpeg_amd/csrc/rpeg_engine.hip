@@ -53,10 +53,11 @@ struct DevMem {
   double* d;       // duration rows
   uint8_t* deg;    // in-degree rows
   uint16_t* ready; // ready list, one entry per node (the heap of the reference has no capacity), pre-offset by lane
-  double* tr_start;
+  double* tr_start;   // optional start / finish time per node, elements `tr_stride` apart
   double* tr_finish;
-  int32_t* tr_seq;   // dispatch index per node
+  int32_t* tr_seq;    // optional dispatch index per node
   int32_t seq;
+  size_t tr_stride;
   __device__ double& time(int i) { return t[(size_t)i * WAVE]; }
   __device__ double& rank(int i) { return r[(size_t)i * WAVE]; }
   __device__ uint8_t& indeg(int i) { return deg[(size_t)i * WAVE]; }
@@ -64,7 +65,8 @@ struct DevMem {
   __device__ void set_dur(int s, double v) { d[(size_t)s * WAVE] = v; }
   __device__ uint16_t& rd_node(int j) { return ready[j * WAVE]; }
   __device__ void on_schedule(int v, double s, double f) {
-    if (tr_start) { tr_start[v] = s; tr_finish[v] = f; tr_seq[v] = seq++; }
+    if (tr_start) { tr_start[(size_t)v * tr_stride] = s; tr_finish[(size_t)v * tr_stride] = f; }
+    if (tr_seq) tr_seq[v] = seq++;
   }
 };
 
@@ -252,9 +254,10 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
                           const uint32_t* __restrict__ cfirst, const uint32_t* __restrict__ clpw,
                           const uint32_t* __restrict__ cbase, uint32_t shards, uint32_t* __restrict__ perm,
                           uint32_t pstride, const uint32_t* __restrict__ coff, uint32_t* __restrict__ task_cls,
-                          uint32_t first_entry, uint32_t* __restrict__ queues) {
+                          uint32_t first_entry, uint32_t* __restrict__ queues, uint32_t* __restrict__ limit) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < N_QUEUES) queues[i] = 0u;   // the task counters of the evaluation kernels that follow on this stream
+  if (i == 0) limit[0] = 0u;          // and the count of plans for the launch that ends the call
   if (i >= n) return;
   const uint32_t c = cid[i];
   if (c >= CID_UNKNOWN) return;
@@ -325,6 +328,7 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
   mem.tr_finish = tr_finish;
   mem.tr_seq = tr_seq;
   mem.seq = 0;
+  mem.tr_stride = 1;
   for (uint64_t w = blockIdx.x; w < n_waves; w += gridDim.x) {
     // every wavefront works on one class: the class tables are addressed uniformly (scalar loads)
     const ClassView cv = class_view(pool + wave_cls[w]);
@@ -340,6 +344,59 @@ __global__ __launch_bounds__(WAVE) void k_eval_generic(const rpeg_problem_t* __r
     if (peak) peak[i] = o.peak;
     if (score) score[i] = o.score;
     if (mask) mask[i] = o.mask;
+  }
+}
+
+// The launch that ends a batched call: the plans whose ready set outgrew what the evaluation kernels hold (flagged in
+// EvalLaunch::limit) once more, one plan per lane, through the scheduler template with a ready list of one entry per
+// node -- the reference's heap has no capacity (scheduler.py:423-546).  Lanes of a wavefront may work on different
+// classes.  Ends at once when nothing is flagged, which is the rule: 32 entries hold every plan of the shipped
+// configurations.  Per lane in `ws`: ready time, rank, start, finish per node, duration per slot, ready list,
+// in-degree, interleaved by lane.
+__host__ __device__ inline size_t limit_ws_bytes(uint32_t nodes, uint32_t slots) {
+  size_t b = (size_t)WAVE * (32ull * nodes + 8ull * slots + 2ull * nodes + nodes);
+  return (b + 255) & ~size_t(255);
+}
+__global__ __launch_bounds__(WAVE) void k_eval_limit(const EvalLaunch L, uint8_t* __restrict__ ws) {
+  const uint32_t n = L.limit[0];
+  if (n == 0) return;
+  const int lane = threadIdx.x;
+  const rpeg_problem_t& P = *L.P;
+  uint8_t* base = ws + (size_t)blockIdx.x * limit_ws_bytes(L.ws_nodes, L.ws_slots);
+  const size_t rows = (size_t)L.ws_nodes * WAVE;
+  DevMem mem;
+  mem.t = (double*)base + lane;
+  mem.r = mem.t + rows;
+  mem.tr_start = mem.r + rows;
+  mem.tr_finish = mem.tr_start + rows;
+  mem.d = mem.tr_finish + rows;
+  mem.ready = (uint16_t*)((double*)base + 4 * rows + (size_t)L.ws_slots * WAVE) + lane;
+  mem.deg = (uint8_t*)((uint16_t*)((double*)base + 4 * rows + (size_t)L.ws_slots * WAVE) + rows) + lane;
+  mem.tr_seq = nullptr;
+  mem.seq = 0;
+  mem.tr_stride = WAVE;
+  for (uint64_t k = (uint64_t)blockIdx.x * WAVE + lane; k < n; k += (uint64_t)gridDim.x * WAVE) {
+    const uint64_t i = L.limit[1 + 2 * k];
+    const ClassView cv = class_view(L.pool + L.limit[2 + 2 * k]);
+    const PlanHead h = load_head(L.head, L.stride, i);
+    VPlan a[RPEG_MAX_V];
+    const int nv = P.st[h.structure].n_vertex;
+    for (int v = 0; v < RPEG_MAX_V; ++v)
+      if (v < nv) load_vertex(L.vert, L.stride, i, v, &a[v]);
+    const PlanOut o = eval_plan(P, cv, h, a, mem, (int)cv.h->n_nodes, L.flags & RPEG_GATE_STALE);
+    if (L.makespan) L.makespan[i] = o.makespan;
+    if (L.peak) L.peak[i] = o.peak;
+    if (L.score) L.score[i] = o.score;
+    if (L.mask) L.mask[i] = o.mask;
+    if (L.mass) {
+      double m[RPEG_MAX_V];
+      if (o.mask & RPEG_MASK_ERROR) {
+        for (int x = 0; x < RPEG_MAX_V; ++x) m[x] = __builtin_nan("");
+      } else {
+        critical_mass(cv, [&](int v) { return mem.tr_finish[(size_t)v * WAVE]; }, [&](int v) { return mem.tr_start[(size_t)v * WAVE]; }, m);
+      }
+      for (int x = 0; x < RPEG_MAX_V; ++x) L.mass[i * RPEG_MAX_V + x] = m[x];
+    }
   }
 }
 
@@ -504,6 +561,10 @@ struct rpeg_engine_s {
   uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_cls = nullptr;   // lane -> plan; wavefront -> class blob
   uint8_t* d_ws = nullptr;
   uint32_t* d_queues = nullptr;                 // N_QUEUES task counters, cleared by k_scatter
+  uint32_t* d_limit = nullptr;                  // count, then (plan, class offset) pairs: plans to redo without a bound on the ready set
+  uint8_t* d_limit_ws = nullptr;                // state of the launch that redoes them
+  size_t limit_ws_cap = 0;
+  uint32_t limit_grid = 0;
   size_t ws_cap = 0;
   // timing / stats
   bool timing = false;
@@ -519,7 +580,7 @@ struct rpeg_engine_s {
 static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (n <= e->cap_n) return 0;
   size_t cap = std::max<size_t>(n, 4096);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); hipFree(e->d_limit); }
   e->cap_n = 0;
   HIP_TRY(e, hipMalloc(&e->d_ovf, cap));
   HIP_TRY(e, hipMemset(e->d_ovf, 0, cap));   // flags are cleared again by the launch that consumes them
@@ -537,6 +598,8 @@ static int ensure_batch(rpeg_engine_t* e, size_t n) {
   HIP_TRY(e, hipHostMalloc(&e->h_sig, cap * 8));
   HIP_TRY(e, hipMalloc(&e->d_cid, cap * 4));
   HIP_TRY(e, hipMalloc(&e->d_kidx, cap * 4));
+  HIP_TRY(e, hipMalloc(&e->d_limit, (1 + 2 * cap) * 4));
+  HIP_TRY(e, hipMemset(e->d_limit, 0, 4));
   e->cap_n = cap;
   return 0;
 }
@@ -715,6 +778,21 @@ static int ensure_ws(rpeg_engine_t* e, size_t bytes, hipStream_t s) {
   return 0;
 }
 
+// state of the launch that redoes flagged plans: as many wavefronts as 128 MiB hold, at most one per compute unit
+static int ensure_limit_ws(rpeg_engine_t* e, hipStream_t s) {
+  const size_t per_wave = limit_ws_bytes(e->max_nodes, e->max_slots);
+  const uint32_t grid = (uint32_t)std::max<size_t>(1, std::min<size_t>((size_t)e->n_cu, ((size_t)128 << 20) / per_wave));
+  if (per_wave * grid <= e->limit_ws_cap) { e->limit_grid = (uint32_t)std::min<size_t>(e->n_cu, e->limit_ws_cap / per_wave); return 0; }
+  HIP_TRY(e, hipStreamSynchronize(s));
+  if (e->d_limit_ws) hipFree(e->d_limit_ws);
+  e->d_limit_ws = nullptr;
+  e->limit_ws_cap = 0;
+  HIP_TRY(e, hipMalloc(&e->d_limit_ws, per_wave * grid));
+  e->limit_ws_cap = per_wave * grid;
+  e->limit_grid = grid;
+  return 0;
+}
+
 static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                            double* peak, double* score, uint8_t* mask, double* mass, void* stream);
 static int eval_host_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
@@ -769,7 +847,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   hipDeviceSynchronize();
   if (e->dP) hipFree(e->dP);
   if (e->d_pool) hipFree(e->d_pool);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); }
+  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); hipFree(e->d_limit); }
+  if (e->d_limit_ws) hipFree(e->d_limit_ws);
   if (e->d_need) hipFree(e->d_need);
   if (e->d_queues) hipFree(e->d_queues);
   if (e->d_cstat) hipFree(e->d_cstat);
@@ -1387,7 +1466,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
   hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
-                     d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted, e->d_queues);
+                     d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted, e->d_queues, e->d_limit);
   HIP_TRY(e, hipGetLastError());
 
   const uint64_t n_waves = n_eval_waves;
@@ -1440,6 +1519,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
   L.prof = nullptr;
+  const bool bounded = !one;   // some kernel of this call holds a bounded ready set
+  if (bounded) {
+    if (int rc = ensure_limit_ws(e, s)) return rc;
+    L.limit = e->d_limit;
+  }
   if (e->prof_on) {
     if (e->d_prof) hipFree(e->d_prof);
     HIP_TRY(e, hipMalloc(&e->d_prof, (n_waves + n_quad_waves + n_solo) * 64));
@@ -1488,7 +1572,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     Q.wave_cls = L.wave_cls + n_eval_waves;
     Q.n_waves = n_quad_waves;
     Q.ws_nodes = quad_nodes; Q.ws_slots = quad_slots;
-    Q.ovf = nullptr; Q.need = nullptr; Q.cstat = nullptr; Q.queue = nullptr;   // (32 entries are as many as the main kernel's full list holds: an overflow is final)
+    Q.ovf = nullptr; Q.need = nullptr; Q.cstat = nullptr; Q.queue = nullptr;   // (a plan that outgrows the 32 entries is flagged in Q.limit)
     if (L.prof) Q.prof = L.prof + n_waves * 8;
     const size_t qlds = kq_lds_bytes(L.cls_bytes, quad_nodes, quad_slots, e->max_v, (uint32_t)KQ_PLANS, mass != nullptr);
     if (qlds > 64 * 1024 && !e->quad_attr_set) {
@@ -1548,6 +1632,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   if (n_quad_waves) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join3, 0));
   if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
+  if (bounded) {   // the plans flagged by the kernels above, without a bound on the ready set (ends at once when there is none)
+    EvalLaunch U = L;
+    U.queue = nullptr;
+    hipLaunchKernelGGL(k_eval_limit, dim3(e->limit_grid), dim3(WAVE), 0, s, U, e->d_limit_ws);
+    HIP_TRY(e, hipGetLastError());
+  }
   if (e->timing) {
     HIP_TRY(e, hipEventRecord(e->ev1, s));
     HIP_TRY(e, hipEventSynchronize(e->ev1));

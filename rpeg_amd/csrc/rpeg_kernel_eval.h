@@ -60,7 +60,19 @@ struct EvalLaunch {              // uniform launch parameters
                                  // they become free; null: block b takes tasks b, b + grid, ...
   uint32_t* cstat = nullptr;     // per class (ClassHdr::id), of its slowest 64-plan wavefront so far: microseconds
                                  // << 12 | heap pops per dispatch in sixteenths; or null
+  uint32_t* limit = nullptr;     // plans whose ready set outgrew what this kernel holds for good (no launch with a
+                                 // longer list follows): limit[0] counts them, then (plan, class blob offset) pairs.
+                                 // The launch that ends the call redoes them with a ready list as long as the
+                                 // graph (the reference's heap has no capacity); or null
 };
+
+// Appends the plan of this lane to the list of plans to redo without a bound on the ready set.
+__device__ inline void ke_flag_limit(const EvalLaunch& L, uint64_t pi, uint32_t cls_off) {
+  if (!L.limit) return;
+  const uint32_t k = atomicAdd(L.limit, 1u);
+  L.limit[1 + 2 * (size_t)k] = (uint32_t)pi;
+  L.limit[2 + 2 * (size_t)k] = cls_off;
+}
 constexpr uint32_t KE_FIXUP = 0x80000000u;   // EvalLaunch::flags: only the plans flagged in `ovf` are evaluated
 constexpr int KE_NEED_SHARDS = 64;
 
@@ -618,6 +630,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   }
 #endif
   if (done != n) err = true;
+  if (limit || (ovf && (!L.ovf || (L.flags & KE_FIXUP)))) ke_flag_limit(L, pi, L.wave_cls[w] & ~KE_CLS_LDS);
   if (L.ovf) {
     const bool fix = (L.flags & KE_FIXUP) != 0;
     if (fix) L.ovf[pi] = 0;

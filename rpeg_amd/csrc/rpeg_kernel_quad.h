@@ -12,8 +12,9 @@
 // over the 32 entries (minima in each lane, two quad-permute steps across the lanes, no memory access), a stale
 // entry is re-keyed in place with a fresh tie (scheduler.py:437-443), a dispatched entry is cleared in place.  The
 // four lanes look at four successors at once; those that became ready are handed, in successor order, to the lanes
-// that have a free slot.  A plan with more than 32 entries ready at once, or more than 2^20 pushes, is not
-// evaluated (RPEG_MASK_LIMIT), as in the plan-per-lane kernel with its full list.
+// that have a free slot (one each per round, the rounds repeated until all are filed).  A plan with more than 32
+// entries ready at once, or more than 2^20 pushes, is not evaluated here: it is flagged (EvalLaunch::limit) and redone
+// by the launch that ends the call, whose ready list is as long as the graph.
 //
 // Per-plan state (ready time, rank, position, in-degree per node, duration per slot) is in LDS, interleaved by plan.
 // Before the scheduling loop the four lanes of a plan share the cost model (slots by lane), the per-vertex memory
@@ -356,26 +357,37 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
       const uint32_t rdy = (uint32_t)(__ballot(ready) >> group_shift) & ((1u << QL) - 1u);
       const int n_rdy = __builtin_popcount(rdy);
       if (n_rdy) {   // uniform within the plan
-        int u_free;
-        const int r = free_rank(u_free);
-        const uint32_t room = (uint32_t)(__ballot(r < QL) >> group_shift) & ((1u << QL) - 1u);
-        if (__builtin_popcount(room) < n_rdy) ovf = true;
-        // source lane of the r-th ready successor
-        uint32_t src_mask = rdy;
-        for (int k = 0; k < r && k < QL; ++k) src_mask &= src_mask - 1u;
-        const bool take = r < n_rdy;
-        const int src = (int)group_shift + (take ? __builtin_ctz(src_mask) : 0);
-        const double tk = __hiloint2double(__builtin_amdgcn_ds_bpermute(src << 2, __double2hiint(t)),
-                                           __builtin_amdgcn_ds_bpermute(src << 2, __double2loint(t)));
-        const uint32_t to = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)ord);
-        const uint32_t tm = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)node_blk);
-        file(take ? u_free : SL, tk, to | (tie + (uint32_t)r), tm);
+        // A round hands one entry to every lane that has room; the rounds repeat until every entry is filed, so that a
+        // plan overflows only when fewer free slots than entries are left in all four lanes together.
+        uint32_t rem = rdy;
+        int filed = 0;
+        while (rem) {
+          int u_free;
+          const int r = free_rank(u_free);
+          const uint32_t room = (uint32_t)(__ballot(r < QL) >> group_shift) & ((1u << QL) - 1u);
+          const int n_room = __builtin_popcount(room), n_rem = __builtin_popcount(rem);
+          if (n_room == 0) { ovf = true; break; }
+          // source lane of the r-th ready successor still to file
+          uint32_t src_mask = rem;
+          for (int k = 0; k < r && k < QL; ++k) src_mask &= src_mask - 1u;
+          const bool take = r < n_rem;
+          const int src = (int)group_shift + (take ? __builtin_ctz(src_mask) : 0);
+          const double tk = __hiloint2double(__builtin_amdgcn_ds_bpermute(src << 2, __double2hiint(t)),
+                                             __builtin_amdgcn_ds_bpermute(src << 2, __double2loint(t)));
+          const uint32_t to = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)ord);
+          const uint32_t tm = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)node_blk);
+          file(take ? u_free : SL, tk, to | (tie + (uint32_t)(filed + r)), tm);
+          const int k_done = n_room < n_rem ? n_room : n_rem;
+          for (int k = 0; k < k_done; ++k) rem &= rem - 1u;
+          filed += k_done;
+        }
         tie += (uint32_t)n_rdy;
       }
     }
     if (kq_or(ovf ? 1u : 0u) || tie >= KQ_TIE_MASK - 64u) { ovf = true; err = true; }
   }
   if (done != n) err = true;
+  if (ovf && q == 0) ke_flag_limit(L, pi, L.wave_cls[w] & ~KE_CLS_LDS);
   KE_STAMP(5);
   if (L.prof && q == 0) atomicMax(&L.prof[w * 8 + 7], ((unsigned long long)n << 32) | (unsigned long long)guard_total);
 

@@ -213,7 +213,8 @@ class Engine:
         self._check(self.lib.rpeg_engine_set_quad_share(self._h, int(percent)), "rpeg_engine_set_quad_share")
 
     def set_ready_cap(self, entries: int):
-        """Ready-list entries per plan in the main kernel (8, 16, 24 or 32); plans that need more get MASK_LIMIT."""
+        """Ready-list entries per plan in the main kernel (8, 16, 24 or 32); plans that need more are redone by the
+        launch that ends the call, without a bound."""
         self._check(self.lib.rpeg_engine_set_ready_cap(self._h, int(entries)), "rpeg_engine_set_ready_cap")
 
     def reset_classes(self):

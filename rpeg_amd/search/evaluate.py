@@ -232,9 +232,7 @@ def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload
     if np.any((mask & abi.MASK_VALID) == 0):
         raise ValueError("a configuration violates the integer validity rules of is_valid")
     if np.any(mask & abi.MASK_LIMIT):
-        raise EngineLimitError("a configuration exceeds a limit of the evaluation engine (more than 31 ready nodes at "
-                               "once, a node that reserves more than two vertex allocations, or more than 2^23 heap "
-                               "pushes): it was not evaluated")
+        raise EngineLimitError("a configuration exceeds a limit of the evaluation engine: it was not evaluated")
     if np.any(mask & abi.MASK_ERROR):
         raise ZeroDivisionError("a configuration has a degenerate node duration or makespan")
     feasible = ((mask & abi.MASK_MEM_OK) != 0) & ((mask & abi.MASK_STALE_OK) != 0)

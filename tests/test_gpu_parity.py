@@ -187,35 +187,37 @@ def test_plans_that_outgrow_the_learned_ready_list_are_redone():
     eng.close()
 
 
-def test_ready_list_limit_is_reported_and_leaves_nothing_behind():
-    """A plan that outgrows the FULL ready list is not evaluated: NaN outputs, MASK_ERROR | MASK_LIMIT, the other
-    plans of the batch unaffected.  The limit is 32 entries, above every list of the shipped problems, so the test
-    lowers it to 8.  Afterwards, with the limit back at 32, the same engine evaluates the set exactly again -- in
-    the launch that learns the short capacity and in the next one, whose fix-up launch must find no flag or count
-    left over from the overflowing call -- and the drop-in reports the condition under its own name."""
+def test_plans_beyond_a_short_ready_list_are_redone_and_nothing_is_left_behind():
+    """With the main kernel's ready list lowered to 8 entries thousands of plans of config 2 outgrow it.  They are
+    redone by the launch that ends the call and come back with the host build's bits; afterwards, with the list
+    back at 32 entries, the same engine evaluates the set exactly again -- in the launch that learns the short
+    capacity and in the next ones, whose fix-up launches must find no flag or count left over."""
     from rpeg_amd.engine.runtime import Engine
-    from rpeg_amd.search import evaluate as ev
     n = 40000
     cfg, batch = seeded_batch(2, n)
     ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    assert ref["max_ready"] > 8
     eng = Engine(cfg.problem)
-    eng.set_ready_cap(8)
-    out = eng.eval_resident(batch)
-    limit = (out["mask"] & abi.MASK_LIMIT) != 0
-    assert 0 < limit.sum() < (ref["mask"] & abi.MASK_VALID).sum()
-    assert np.all(out["mask"][limit] & abi.MASK_ERROR) and np.all(np.isnan(out["score"][limit]))
-    assert np.all(np.isnan(out["makespan"][limit]))
-    assert np.array_equal(out["mask"][~limit], ref["mask"][~limit])
-    assert same_bits(out["score"][~limit], ref["score"][~limit]) and same_bits(out["makespan"][~limit], ref["makespan"][~limit])
-    eng.set_ready_cap(32)
-    for _ in range(3):
-        out = eng.eval_resident(batch)
-        assert np.array_equal(out["mask"], ref["mask"]) and same_bits(out["score"], ref["score"])
+    eng.set_quad_share(0)      # (every class in the main kernel or, the largest graphs, one plan per wavefront)
+    for cap in (8, 32, 8, 16):
+        eng.set_ready_cap(cap)
+        for _ in range(2):
+            out = eng.eval_resident(batch)
+            assert not np.any(out["mask"] & abi.MASK_LIMIT)
+            assert np.array_equal(out["mask"], ref["mask"]), cap
+            assert same_bits(out["score"], ref["score"]) and same_bits(out["makespan"], ref["makespan"]), cap
     with pytest.raises(Exception, match="8, 16, 24 or 32"):
         eng.set_ready_cap(12)
     eng.close()
 
-    class Limited:                       # evaluate_batch names the condition instead of a division by zero
+
+def test_the_drop_in_names_an_engine_limit():
+    """evaluate_batch raises EngineLimitError for a mask with RPEG_MASK_LIMIT (no evaluation path sets it for a plan the
+    reference evaluates; the bit stays in the ABI for limits a later kernel may have) instead of a division by zero."""
+    from rpeg_amd.search import evaluate as ev
+    cfg, batch = seeded_batch(2, 4)
+
+    class Limited:
         def eval(self, b, gate_stale=True):
             m = np.full(b.n, abi.MASK_VALID | abi.MASK_ERROR | abi.MASK_LIMIT, np.uint8)
             nan = np.full(b.n, np.nan)
@@ -629,32 +631,56 @@ def test_transfer_resource_policies_equal_reference(c):
             assert float(trace.utilization()).hex() == want["utilization"], (i, pol)
 
 
-def test_a_horizon_beyond_the_ready_list_is_reported_as_a_limit():
+def test_a_horizon_beyond_the_ready_lists_is_evaluated_all_the_same():
     """DPO's unrolled steps are independent of each other, so every step's first node is ready at time zero: at a
-    horizon of 128 steps the ready list would need 128 entries.  The engine says so (MASK_ERROR | MASK_LIMIT, NaN),
-    it does not return a number; the host build, whose list is unbounded in this range, evaluates the plans.  The
-    same at 40 steps for the kernel that holds 32 entries in registers."""
+    horizon of 128 steps the ready set holds 128 entries, at 40 steps more than the 32 the four-lanes-per-plan kernel
+    keeps in registers.  The reference's heap has no capacity (scheduler.py:423-546), and neither has the call: plans
+    that outgrow a kernel's ready set are redone by the launch that ends the call, with a list as long as the graph.
+    Whatever the layout, every plan comes back with the host build's bits and no plan with RPEG_MASK_LIMIT."""
     from dataclasses import replace
     from rpeg_amd.engine.runtime import Engine
     cfg, batch = seeded_batch(4, 2048)
-    # (K, layout, limited): -1 is the automatic layout (one plan per wavefront, no bound, while a class has at most 384
-    # nodes; beyond that the plan-per-lane kernel with its 31 entries), 4 is four lanes per plan (32 entries in registers)
-    for K, lanes, limited in ((24, -1, False), (24, 4, False), (40, -1, False), (40, 4, True), (128, -1, True)):
+    for K, layouts in ((24, (-1, 4)), (33, (-1, 0, 1, 4)), (40, (-1, 0, 4)), (128, (-1, 0))):
         p = replace(cfg.problem, K_eval=K)
-        eng = Engine(p)
-        eng.set_state_lanes(lanes)
-        out = eng.eval(batch)
-        assert (eng.stats()["quad_tasks"] > 0) == (lanes == 4)
-        valid = (out["mask"] & abi.MASK_VALID) != 0
-        assert valid.sum() > 1000
-        assert np.all(((out["mask"][valid] & abi.MASK_LIMIT) != 0) == limited), (K, lanes)
-        assert np.all(np.isnan(out["score"][valid]) == limited), (K, lanes)
-        if not limited:
-            ref = CpuPort(p).eval(batch, flags=abi.GATE_STALE, threads=16)
-            assert same_bits(out["score"], ref["score"]) and np.array_equal(out["mask"], ref["mask"]), (K, lanes)
-        eng.close()
-    with pytest.raises(ValueError, match="K_eval"):
+        ref = CpuPort(p).eval(batch, flags=abi.GATE_STALE, threads=16)
+        assert ref["max_ready"] >= min(K, 33)
+        for lanes in layouts:
+            eng = Engine(p)
+            eng.set_state_lanes(lanes)
+            for _ in range(2):
+                out = eng.eval(batch)
+                assert (eng.stats()["quad_tasks"] > 0) == (lanes == 4)
+                assert not np.any(out["mask"] & abi.MASK_LIMIT), (K, lanes)
+                assert np.array_equal(out["mask"], ref["mask"]), (K, lanes)
+                assert same_bits(out["score"], ref["score"]) and same_bits(out["makespan"], ref["makespan"]), (K, lanes)
+            if K == 40:   # the critical-chain masses of redone plans come from the same launch
+                m = eng.eval_mass_device(batch)["mass"]
+                want = CpuPort(p).eval(batch, flags=0, threads=16, want_mass=True)["mass"]
+                assert same_bits(m, want), lanes
+            eng.close()
+    with pytest.raises(ValueError, match="K_eval"):     # a stated bound: graphs of at most 4,095 lowered nodes
         Engine(replace(cfg.problem, K_eval=5000))
+
+
+def test_short_ready_lists_and_dense_graphs_in_every_layout():
+    """Plans that outgrow a deliberately short ready list of the main kernel (8 entries), and a seeded subset of
+    config 3 (ready sets of up to 24 entries, fan-outs of four) in the four-lanes-per-plan kernel: the same bits as
+    the host build in every layout, and the same masks from every layout."""
+    from rpeg_amd.engine.runtime import Engine
+    cfg, batch = seeded_batch(3, 6000, start=40_000)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    assert ref["max_ready"] > 16
+    masks = []
+    for lanes, cap in ((0, 8), (0, 32), (4, 32), (1, 32), (-1, 16)):
+        eng = Engine(cfg.problem)
+        eng.set_state_lanes(lanes)
+        eng.set_ready_cap(cap)
+        for _ in range(2):
+            out = eng.eval(batch)
+            assert same_bits(out["score"], ref["score"]) and same_bits(out["peak"], ref["peak"]), (lanes, cap)
+            masks.append(out["mask"].copy())
+        eng.close()
+    assert all(np.array_equal(m, ref["mask"]) for m in masks)
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
