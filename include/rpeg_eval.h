@@ -58,8 +58,10 @@ enum {
 
 /* eval flags */
 enum {
-  RPEG_GATE_STALE = 1      /* score := 0 when the stale-layout rule fails (evaluate_cached, :372-374);
+  RPEG_GATE_STALE = 1,     /* score := 0 when the stale-layout rule fails (evaluate_cached, :372-374);
                               without it the score is what _eval_worker returns (:406-442)      */
+  RPEG_NO_WAIT = 2         /* rpeg_eval_batch_static only: enqueue the launches and return, without the
+                              copy and the wait that report plans of unknown classes            */
 };
 
 /* hardware parameter indices (RPEG/model/hardware.py:17-68, in field order) */
@@ -184,7 +186,12 @@ int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, 
        others their results).  Problems with a class above 384 nodes are rejected with status -8.
      - All engines on one GPU share that GPU's array and it keeps the last call's contents; the call resets
        what must start at zero.  Calls that overlap on one GPU (two host threads, two streams) race.
-   Returns after the results are in place (it waits for the stream to read back one counter). */
+   Without RPEG_NO_WAIT in `flags` the call returns after the results are in place: it copies one counter back and
+   waits for the stream, which is how it knows of status -11.  With RPEG_NO_WAIT it only enqueues its three kernel
+   launches on `stream` (a fill kernel, the class lookup, the evaluation) and returns 0: no copy, no wait and no
+   memset node, so that the call may stand inside a HIP stream capture and the captured graph be replayed on the
+   same buffers.  Plans of classes the engine has not met are then recognisable only by their outputs: NaN and
+   RPEG_MASK_VALID | RPEG_MASK_ERROR in the mask. */
 #define RPEG_STATIC_MAX_PLANS 32768
 int rpeg_eval_batch_static(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
                            double* makespan, double* peak, double* score, uint8_t* mask, void* stream);

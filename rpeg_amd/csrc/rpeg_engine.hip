@@ -1675,8 +1675,8 @@ int rpeg_eval_batch_static(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   hipStream_t s = (hipStream_t)stream;
   uint32_t* const d_cls = (uint32_t*)e->static_ptr;
   uint32_t* const d_counters = (uint32_t*)(e->static_ptr + STATIC_CLS_BYTES);
-  // the array keeps what the last call left: the counters start at zero (a fill kernel, so that a caller may
-  // capture the launches), the task list is rewritten for all n plans
+  // the array keeps what the last call left: the counters start at zero (a fill kernel, not a memset node: a caller
+  // may capture these launches into a HIP graph), the task list is rewritten for all n plans
   hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, s, d_counters, (uint64_t)(STATIC_COUNTER_BYTES / 4), 0u);
   hipLaunchKernelGGL(k_class_direct, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n,
                      plans->vert, plans->head, plans->stride, makespan, peak, score, mask, (double*)nullptr, e->d_hkey, e->d_hoff,
@@ -1687,14 +1687,18 @@ int rpeg_eval_batch_static(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.perm = nullptr; L.wave_cls = d_cls; L.pool = e->d_pool; L.ws = nullptr;
   L.n_waves = n; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
   L.cls_bytes = 0; L.rcap = 0; L.max_v = e->max_v; L.ovf = nullptr; L.need = nullptr;
-  L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
+  L.flags = flags & RPEG_GATE_STALE; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = nullptr; L.prof = nullptr;
   const size_t lds = kp_lds_bytes(e->max_nodes, e->max_slots);
   hipLaunchKernelGGL(k_plan, dim3((unsigned)std::min<uint64_t>(n, (uint64_t)e->n_cu * 32)), dim3(WAVE), lds, s, L);
   HIP_TRY(e, hipGetLastError());
+  e->stats[0] = 0; e->stats[1] = 0; e->stats[2] = n; e->stats[3] = lds; e->stats[4] = 0; e->stats[5] = 1; e->stats[6] = 0;
+  e->stats[7] = 0;
+  // With RPEG_NO_WAIT the call ends here: three launches on the caller's stream, no copy and no wait (what a
+  // capturing stream accepts).  Plans of classes the engine has not met are then told by their mask alone.
+  if (flags & RPEG_NO_WAIT) return 0;
   HIP_TRY(e, hipMemcpyAsync(e->h_static, d_counters, 4, hipMemcpyDeviceToHost, s));
   HIP_TRY(e, hipStreamSynchronize(s));
-  e->stats[0] = 0; e->stats[1] = 0; e->stats[2] = n; e->stats[3] = lds; e->stats[4] = 0; e->stats[5] = 1; e->stats[6] = 0;
   if (e->h_static[0] != 0u) {
     e->err = std::to_string(e->h_static[0]) + " plans belong to lowering classes the engine has not met: evaluate them through "
              "rpeg_eval_batch once (their outputs are NaN, their mask has RPEG_MASK_ERROR)";

@@ -10,6 +10,7 @@ MODEL = {"Pi": 0, "V": 1, "Ref": 2, "R": 3, "AC": 4}
 NEED_DISJ, NEED_PI = 1, 2
 MASK_VALID, MASK_STALE_OK, MASK_MEM_OK, MASK_ERROR, MASK_LIMIT = 1, 2, 4, 8, 16
 GATE_STALE = 1
+NO_WAIT = 2
 STATIC_MAX_PLANS = 32768
 HW_FIELDS = (
     "flops_per_gpu", "memory_per_gpu", "memory_bandwidth",

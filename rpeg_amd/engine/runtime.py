@@ -250,16 +250,19 @@ class Engine:
         self._check(rc, "rpeg_eval_batch")
         return out
 
-    def eval_device_static(self, dbatch: DeviceBatch, out=None, gate_stale: bool = True, n: Optional[int] = None):
+    def eval_device_static(self, dbatch: DeviceBatch, out=None, gate_stale: bool = True, n: Optional[int] = None,
+                           no_wait: bool = False):
         """eval_device through the entry point that allocates nothing (rpeg_eval_batch_static): at most
         abi.STATIC_MAX_PLANS plans whose lowering classes an earlier eval_device call has met.  `out` must be
-        given by a caller that may not allocate."""
+        given by a caller that may not allocate.  `no_wait`: only enqueue (RPEG_NO_WAIT), as a caller under HIP
+        stream capture needs it."""
         torch = _torch()
         n = dbatch.n if n is None else n
         out = out or self.alloc_outputs(n)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         with torch.cuda.device(self.device):
-            rc = self.lib.rpeg_eval_batch_static(self._h, n, C.addressof(dbatch.soa), abi.GATE_STALE if gate_stale else 0,
+            rc = self.lib.rpeg_eval_batch_static(self._h, n, C.addressof(dbatch.soa),
+                                                 (abi.GATE_STALE if gate_stale else 0) | (abi.NO_WAIT if no_wait else 0),
                                                  out["makespan"].data_ptr(), out["peak"].data_ptr(),
                                                  out["score"].data_ptr(), out["mask"].data_ptr(), stream)
         self._check(rc, "rpeg_eval_batch_static")
