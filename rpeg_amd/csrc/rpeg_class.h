@@ -79,6 +79,7 @@ struct ClassHdr {
   uint32_t n_nodes, n_slots, n_succ, n_init, n_groups, n_gmembers;
   uint32_t off_node, off_succ, off_init, off_topo, off_slot, off_group, off_gmember;  // byte offsets in the blob
   uint32_t off_pbeg, off_pred;       // predecessor lists in edge order: pred[pbeg[v] .. pbeg[v+1])
+  uint32_t off_umap;                 // per slot: its index in the structure's slot universe (slot_universe)
   uint32_t bytes;
   uint32_t structure, split, error;  // error != 0: the reference would raise for this class
   uint32_t id;                       // index of the class in the tables of the engine that holds it (0 elsewhere)
@@ -96,6 +97,7 @@ struct ClassView {
   const uint16_t* gmember;
   const uint16_t* pbeg;
   const uint16_t* pred;
+  const uint8_t* umap;
 };
 
 RPEG_HD ClassView class_view(const uint8_t* blob) {
@@ -110,6 +112,7 @@ RPEG_HD ClassView class_view(const uint8_t* blob) {
   v.gmember = (const uint16_t*)(blob + v.h->off_gmember);
   v.pbeg = (const uint16_t*)(blob + v.h->off_pbeg);
   v.pred = (const uint16_t*)(blob + v.h->off_pred);
+  v.umap = blob + v.h->off_umap;
   return v;
 }
 
@@ -133,6 +136,69 @@ RPEG_HD double slot_duration(const rpeg_problem_t& P, const rpeg_struct_t& st, i
     default:
       return reshard_time(P, a[sd.a], sd.b);
   }
+}
+
+// ------------------------------------------------------------------------------------- slot universe
+// Every duration slot a class of structure `st` can have, whatever the plan: the operator of every vertex unsplit and
+// by quantile phase, the transfer of every data edge whole and (generation -> inference edges) by phase, every
+// publication transfer, and the reshards lowering can place (between the vertices of a same-model pair, at the
+// source of a publication).  Durations depend on the plan only through the plan fields, so a launch of its own can
+// evaluate the whole universe for every plan before the classes of a batch are even known; a class's slot s is entry
+// ClassView::umap[s].  Entries by phase carry the phase in q: for a plan of split variant j only those with
+// q < P.n_phase[j] exist.  At most RPEG_MAX_UNIVERSE entries; returns their number.
+constexpr int RPEG_MAX_UNIVERSE = 96;
+RPEG_HD int slot_universe(const rpeg_problem_t& P, const rpeg_struct_t& st, SlotDesc* out) {
+  int n = 0, max_ph = 0;
+  for (int j = 1; j < P.n_split; ++j) max_ph = P.n_phase[j] > max_ph ? P.n_phase[j] : max_ph;
+  auto put = [&](uint8_t type, int a, int b, int q) {
+    for (int i = 0; i < n; ++i)
+      if (out[i].type == type && out[i].a == a && out[i].b == b && out[i].q == q) return;
+    if (n < RPEG_MAX_UNIVERSE) out[n] = SlotDesc{type, (uint8_t)a, (uint8_t)b, (uint8_t)q};
+    ++n;
+  };
+  for (int v = 0; v < st.n_vertex; ++v) put(SLOT_OP_UNSPLIT, v, 0, 0);
+  for (int v = 0; v < st.n_vertex; ++v)
+    if (st.vertex[v].role != RPEG_ROLE_TRAIN)
+      for (int q = 0; q < max_ph; ++q) put(SLOT_OP_SUB, v, 0, q);
+  for (int e = 0; e < st.n_edge; ++e) put(SLOT_COMM_DATA, e, 0, 0xFF);
+  for (int e = 0; e < st.n_edge; ++e)
+    if (st.edge[e].gen_inf)
+      for (int q = 0; q < max_ph; ++q) put(SLOT_COMM_DATA, e, 0, q);
+  for (int p = 0; p < st.n_pub; ++p) put(SLOT_COMM_PUB, p, 0, 0);
+  for (int p = 0; p < st.n_pair; ++p) put(SLOT_RESHARD, st.pair[p].u, st.pair[p].model, 0);
+  for (int p = 0; p < st.n_pub; ++p) put(SLOT_RESHARD, st.pub[p].src, st.pub[p].model, 0);
+  return n;
+}
+RPEG_HD bool slot_in_split(const rpeg_problem_t& P, int split, const SlotDesc& sd) {
+  const int nph = split > 0 ? P.n_phase[split] : 0;
+  if (sd.type == SLOT_OP_SUB) return sd.q < nph;
+  if (sd.type == SLOT_COMM_DATA && sd.q != 0xFF) return sd.q < nph;
+  return true;
+}
+
+// The order in which the template vertices first appear among a plan's lowered operator nodes (ClassHdr::vorder),
+// from the plan itself: template order, except that an inference vertex whose node is split into quantile phases
+// (its generation producer is split -- some inference consumer of it sits on disjoint devices -- and so is it:
+// lower.py:425-431, 528-558) is taken out and appended again, in the order of the data edges that split them.
+template <class PLANS>
+RPEG_HD void plan_vorder(const rpeg_problem_t& P, const rpeg_struct_t& st, int split, const PLANS& a, uint8_t* order) {
+  const int nv = st.n_vertex, nph = split > 0 ? P.n_phase[split] : 0;
+  unsigned gen_split = 0, moved = 0;
+  int n_tail = 0;
+  uint8_t tail[RPEG_MAX_V];
+  if (nph > 0) {
+    for (int e = 0; e < st.n_edge; ++e)
+      if (st.edge[e].gen_inf && alloc_disjoint(a[st.edge[e].src], a[st.edge[e].dst])) gen_split |= 1u << st.edge[e].src;
+    for (int e = 0; e < st.n_edge; ++e) {
+      const int u = st.edge[e].src, v = st.edge[e].dst;
+      if (!((gen_split >> u) & 1u) || st.vertex[v].role != RPEG_ROLE_INF || ((moved >> v) & 1u)) continue;
+      if (alloc_disjoint(a[u], a[v])) { moved |= 1u << v; tail[n_tail++] = (uint8_t)v; }
+    }
+  }
+  int c = 0;
+  for (int v = 0; v < nv; ++v)
+    if (!((moved >> v) & 1u)) order[c++] = (uint8_t)v;
+  for (int j = 0; j < n_tail; ++j) order[c++] = tail[j];
 }
 
 // ------------------------------------------------------------------------------------- scheduler

@@ -469,7 +469,8 @@ RPEG_HD bool struct_coresident(const rpeg_struct_t& st) {
   for (unsigned m = 0; m < sizeof(st.mem_trainable); ++m) any = any || st.mem_trainable[m] != 0;
   return !any;
 }
-RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) {
+template <class ORD>   // `order`: the vertices in order of first appearance, a byte array or anything indexable like one
+RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const ORD& order) {
   StructMasks m;
   m.train = m.trainable = 0;
   unsigned seen = 0;
@@ -495,8 +496,8 @@ RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const uint8_t* order) 
 // lowered operator nodes (it fixes the insertion order of the reference's dicts and hence the
 // order of its float sums).  VM provides w_shard(v) (as double), mem_w(v), opt(v), extra(v).
 // Peak of the devices covered by exactly the vertex set M.
-template <class VM>
-RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
+template <class VM, class ORD>
+RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& st, const ORD& order,
                                  const StructMasks& sm, const PlanMasks& pm, const VM& vm, unsigned M) {
   const int nv = st.n_vertex;
   double persistent = 0.0;
@@ -591,8 +592,8 @@ RPEG_HD void clique_sets(const unsigned (&row)[RPEG_MAX_V], unsigned c, uint64_t
   }
 }
 
-template <class VM>
-RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const uint8_t* order,
+template <class VM, class ORD>
+RPEG_HD double device_peak_max(const rpeg_problem_t& P, const rpeg_struct_t& st, const ORD& order,
                                const PlanMasks& pm, const VM& vm) {
   static_assert(RPEG_MAX_V <= 6, "a vertex set is one bit of a 64-bit word below");
   const StructMasks sm = struct_masks(st, order);

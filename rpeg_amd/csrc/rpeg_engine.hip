@@ -26,6 +26,7 @@
 
 #include "rpeg_kernel_eval.h"
 #include "rpeg_kernel_plan.h"
+#include "rpeg_kernel_prologue.h"
 #include "rpeg_kernel_quad.h"
 #include "rpeg_lower.h"
 #include "rpeg_plan.h"
@@ -266,6 +267,41 @@ __global__ void k_scatter(uint64_t n, const uint32_t* __restrict__ cid, const ui
     perm[(uint64_t)cfirst[c] + k] = (uint32_t)i;
     task_cls[cfirst[c] + k - first_entry] = coff[c];
   } else perm[(uint64_t)(cfirst[c] + k / l) * pstride + k % l] = (uint32_t)i;
+}
+
+// The prologue launches (rpeg_kernel_prologue.h), a thread per plan in the caller's order.  The structure decides
+// which tables a plan reads; it is made uniform (one pass per distinct structure among the plans of the wavefront) so
+// that those reads are scalar loads and the walk through the slot universe is one path.
+__global__ __launch_bounds__(WAVE) void k_prologue(const PrologueLaunch L) {
+  const uint64_t i = (uint64_t)blockIdx.x * WAVE + threadIdx.x;
+  const bool active = i < L.n && L.cid[i] != KPRO_INVALID;
+  int su = 0, split = 0;
+  if (active) { su = L.head[0 * L.stride + i]; split = L.head[1 * L.stride + i]; }
+  unsigned long long todo = __ballot(active);
+  while (todo) {
+    const int s0 = __builtin_amdgcn_readlane(su, __builtin_ctzll(todo));
+    const bool mine = active && su == s0;
+    todo &= ~__ballot(mine);
+    if (mine)
+      for (int row = (int)blockIdx.y; row < (int)(L.max_uni + 1 + RPEG_MAX_V); row += (int)gridDim.y) kpro_row(L, i, s0, split, row);
+  }
+}
+
+__global__ __launch_bounds__(WAVE) void k_peaks(const PrologueLaunch L) {
+  __shared__ double l_vm[RPEG_MAX_V * 4 * WAVE];
+  __shared__ uint8_t l_ord[8 * WAVE];
+  const uint64_t i = (uint64_t)blockIdx.x * WAVE + threadIdx.x;
+  const bool active = i < L.n && L.cid[i] != KPRO_INVALID;
+  PlanHead h;
+  h.structure = h.split = h.tau0 = h.tau1 = 0;
+  if (active) h = load_head(L.head, L.stride, i);
+  unsigned long long todo = __ballot(active);
+  while (todo) {
+    const int su = __builtin_amdgcn_readlane(h.structure, __builtin_ctzll(todo));
+    const bool mine = active && h.structure == su;
+    todo &= ~__ballot(mine);
+    if (mine) kpro_peaks(L, i, su, h, l_vm + threadIdx.x, l_ord + threadIdx.x);
+  }
 }
 
 // The next wave task of a launch whose wavefronts take tasks as they become free (every wavefront ends when the
@@ -551,6 +587,7 @@ struct rpeg_engine_s {
   uint32_t max_v = RPEG_MAX_V;   // largest vertex count of the problem's structures
   hipStream_t s2 = nullptr;                     // second stream: single-plan wavefronts of a large batch run beside the others
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  hipEvent_t ev_counts = nullptr;               // the class counts of a call have reached the host
   hipStream_t s3 = nullptr;                     // third stream: the four-lanes-per-plan wavefronts (k_quad)
   hipEvent_t ev_join3 = nullptr;
   uint32_t quad_share_pct = 25;                 // share of a full batch that k_quad takes (rpeg_engine_set_quad_share)
@@ -560,6 +597,16 @@ struct rpeg_engine_s {
   uint64_t* h_sig = nullptr;
   uint32_t *d_perm = nullptr, *d_cls = nullptr, *h_cls = nullptr;   // lane -> plan; wavefront -> class blob
   uint8_t* d_ws = nullptr;
+  // outputs of the prologue launches (rpeg_kernel_prologue.h), cap_n plans each: pair relations, penalty factor, gate
+  // bits; the durations of the slot universe ([slot][plan]); and the universe itself
+  uint64_t *d_aux_ovl = nullptr, *d_aux_dpne = nullptr, *d_aux_eq = nullptr;
+  double* d_vm = nullptr;
+  double* d_aux_pen = nullptr;
+  uint8_t* d_aux_mask = nullptr;
+  double* d_dur = nullptr;
+  size_t dur_cap = 0;
+  SlotDesc* d_uni = nullptr;
+  uint32_t n_uni[RPEG_MAX_STRUCT] = {0, 0, 0}, max_uni = 0;
   uint32_t* d_queues = nullptr;                 // N_QUEUES task counters, cleared by k_scatter
   uint32_t* d_limit = nullptr;                  // count, then (plan, class offset) pairs: plans to redo without a bound on the ready set
   uint8_t* d_limit_ws = nullptr;                // state of the launch that redoes them
@@ -580,7 +627,12 @@ struct rpeg_engine_s {
 static int ensure_batch(rpeg_engine_t* e, size_t n) {
   if (n <= e->cap_n) return 0;
   size_t cap = std::max<size_t>(n, 4096);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); hipFree(e->d_limit); }
+  if (e->d_sig) {
+    hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); hipFree(e->d_limit);
+    hipFree(e->d_aux_ovl); hipFree(e->d_aux_dpne); hipFree(e->d_aux_pen); hipFree(e->d_aux_mask); hipFree(e->d_dur);
+    hipFree(e->d_aux_eq); hipFree(e->d_vm);
+    e->d_dur = nullptr;
+  }
   e->cap_n = 0;
   HIP_TRY(e, hipMalloc(&e->d_ovf, cap));
   HIP_TRY(e, hipMemset(e->d_ovf, 0, cap));   // flags are cleared again by the launch that consumes them
@@ -600,6 +652,13 @@ static int ensure_batch(rpeg_engine_t* e, size_t n) {
   HIP_TRY(e, hipMalloc(&e->d_kidx, cap * 4));
   HIP_TRY(e, hipMalloc(&e->d_limit, (1 + 2 * cap) * 4));
   HIP_TRY(e, hipMemset(e->d_limit, 0, 4));
+  HIP_TRY(e, hipMalloc(&e->d_aux_ovl, cap * 8));
+  HIP_TRY(e, hipMalloc(&e->d_aux_dpne, cap * 8));
+  HIP_TRY(e, hipMalloc(&e->d_aux_pen, cap * 8));
+  HIP_TRY(e, hipMalloc(&e->d_aux_mask, cap));
+  HIP_TRY(e, hipMalloc(&e->d_aux_eq, cap * 8));
+  HIP_TRY(e, hipMalloc(&e->d_vm, cap * 8 * 4 * RPEG_MAX_V));
+  HIP_TRY(e, hipMalloc(&e->d_dur, cap * 8 * (size_t)std::max<uint32_t>(e->max_uni, 1)));
   e->cap_n = cap;
   return 0;
 }
@@ -832,6 +891,20 @@ int rpeg_engine_create(const rpeg_problem_t* problem, rpeg_engine_t** out) {
       return -2;
     }
   }
+  {   // the slot universe of every structure, for the duration launch
+    std::vector<SlotDesc> uni((size_t)RPEG_MAX_STRUCT * RPEG_MAX_UNIVERSE, SlotDesc{0, 0, 0, 0});
+    for (int q = 0; q < e->P.n_struct; ++q) {
+      const int nu = slot_universe(e->P, e->P.st[q], uni.data() + (size_t)q * RPEG_MAX_UNIVERSE);
+      if (nu > RPEG_MAX_UNIVERSE) { delete e; return -3; }
+      e->n_uni[q] = (uint32_t)nu;
+      e->max_uni = std::max(e->max_uni, (uint32_t)nu);
+    }
+    if (hipMalloc(&e->d_uni, uni.size() * sizeof(SlotDesc)) != hipSuccess ||
+        hipMemcpy(e->d_uni, uni.data(), uni.size() * sizeof(SlotDesc), hipMemcpyHostToDevice) != hipSuccess) {
+      delete e;
+      return -2;
+    }
+  }
   if (hipMalloc(&e->dP, sizeof(rpeg_problem_t)) != hipSuccess ||
       hipMemcpy(e->dP, problem, sizeof(rpeg_problem_t), hipMemcpyHostToDevice) != hipSuccess ||
       hipEventCreate(&e->ev0) != hipSuccess || hipEventCreate(&e->ev1) != hipSuccess) {
@@ -847,7 +920,11 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   hipDeviceSynchronize();
   if (e->dP) hipFree(e->dP);
   if (e->d_pool) hipFree(e->d_pool);
-  if (e->d_sig) { hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); hipFree(e->d_limit); }
+  if (e->d_sig) {
+    hipFree(e->d_sig); hipHostFree(e->h_sig); hipFree(e->d_cid); hipFree(e->d_kidx); hipFree(e->d_ovf); hipFree(e->d_limit);
+    hipFree(e->d_aux_ovl); hipFree(e->d_aux_dpne); hipFree(e->d_aux_pen); hipFree(e->d_aux_mask);
+    hipFree(e->d_aux_eq); hipFree(e->d_vm);
+  }
   if (e->d_limit_ws) hipFree(e->d_limit_ws);
   if (e->d_need) hipFree(e->d_need);
   if (e->d_queues) hipFree(e->d_queues);
@@ -859,9 +936,12 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
     hipHostFree(e->h_ccount);
   }
   if (e->d_perm) hipFree(e->d_perm);
+  if (e->d_dur) hipFree(e->d_dur);
+  if (e->d_uni) hipFree(e->d_uni);
   if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
   if (e->s2) { hipStreamDestroy(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
   if (e->s3) { hipStreamDestroy(e->s3); hipEventDestroy(e->ev_join3); }
+  if (e->ev_counts) hipEventDestroy(e->ev_counts);
   if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
   if (e->d_stage) hipFree(e->d_stage);
   if (e->h_stage) hipHostFree(e->h_stage);
@@ -1083,7 +1163,29 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     // that follow new classes, and now and then afterwards
     const bool read_stat = round == 0 && e->quad_share_pct && ncls && (e->learn_calls > 0 || (e->batch_calls & 63) == 0);
     if (read_stat) HIP_TRY(e, hipMemcpyAsync(e->cls_pops16.data(), e->d_cstat, (size_t)ncls * 4, hipMemcpyDeviceToHost, s));
-    HIP_TRY(e, hipStreamSynchronize(s));
+    if (round == 0) {
+      // Cost model, memory model and gates of every plan: they need the verdict of the gate (which plans to skip)
+      // and nothing of the classes, so they run behind the signature kernel while the host waits for the counts
+      // (the event, not the stream) and lays the batch out.
+      if (!e->ev_counts) HIP_TRY(e, hipEventCreateWithFlags(&e->ev_counts, hipEventDisableTiming));
+      HIP_TRY(e, hipEventRecord(e->ev_counts, s));
+      PrologueLaunch G;
+      G.P = e->dP; G.vert = plans->vert; G.head = plans->head; G.stride = plans->stride; G.n = n; G.cid = e->d_cid;
+      G.uni = e->d_uni;
+      for (int q = 0; q < RPEG_MAX_STRUCT; ++q) G.n_uni[q] = e->n_uni[q];
+      G.max_uni = e->max_uni;
+      G.dur = e->d_dur; G.dur_stride = e->cap_n;
+      G.aux_ovl = e->d_aux_ovl; G.aux_eq = e->d_aux_eq; G.aux_dpne = e->d_aux_dpne; G.vm = e->d_vm;
+      G.aux_pen = e->d_aux_pen; G.aux_mask = e->d_aux_mask;
+      G.peak = peak;
+      const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
+      hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, s, G);
+      hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
+      HIP_TRY(e, hipGetLastError());
+      HIP_TRY(e, hipEventSynchronize(e->ev_counts));
+    } else {
+      HIP_TRY(e, hipStreamSynchronize(s));
+    }
     if (read_stat && e->learn_calls > 0) --e->learn_calls;
     for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_ccount[n_count + q]);
     if (e->h_ccount[n_count - 1] == 0) break;
@@ -1519,6 +1621,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
   L.prof = nullptr;
+  L.dur = e->d_dur; L.aux_ovl = e->d_aux_ovl; L.aux_dpne = e->d_aux_dpne; L.aux_pen = e->d_aux_pen; L.aux_mask = e->d_aux_mask;
+  L.dur_stride = e->cap_n;
   const bool bounded = !one;   // some kernel of this call holds a bounded ready set
   if (bounded) {
     if (int rc = ensure_limit_ws(e, s)) return rc;

@@ -60,6 +60,14 @@ struct EvalLaunch {              // uniform launch parameters
                                  // they become free; null: block b takes tasks b, b + grid, ...
   uint32_t* cstat = nullptr;     // per class (ClassHdr::id), of its slowest 64-plan wavefront so far: microseconds
                                  // << 12 | heap pops per dispatch in sixteenths; or null
+  // What the prologue launches (rpeg_kernel_prologue.h) computed for every plan of the call, indexed by plan.  All null
+  // where a kernel computes these itself (the single-plan kernel without a layout).
+  const double* dur = nullptr;         // [universe slot][plan], rows dur_stride apart; NaN where the reference would raise
+  const uint64_t* aux_ovl = nullptr;   // PlanMasks::ovl
+  const uint64_t* aux_dpne = nullptr;  // PlanMasks::dpne
+  const double* aux_pen = nullptr;     // factor of the soft OOM penalty, 1.0 where the plan fits
+  const uint8_t* aux_mask = nullptr;   // RPEG_MASK_VALID | _STALE_OK | _MEM_OK
+  uint64_t dur_stride = 0;
   uint32_t* limit = nullptr;     // plans whose ready set outgrew what this kernel holds for good (no launch with a
                                  // longer list follows): limit[0] counts them, then (plan, class blob offset) pairs.
                                  // The launch that ends the call redoes them with a ready list as long as the
@@ -82,18 +90,16 @@ __host__ __device__ inline size_t ke_ws_bytes(uint32_t nodes, uint32_t slots) {
 }
 // Dynamic LDS of one wavefront.  ls = 0: the per-plan state lives in the HBM workspace and all 64 lanes
 // carry plans.  ls > 0: only the first `ls` lanes carry plans and their state (ready time, rank,
-// in-degree per node, duration per slot) lives in LDS too, interleaved by lane.  One area serves, one after
-// the other, the plan fields (read by the cost model), the per-vertex memory terms and the ready list; nv is
-// the largest vertex count of the problem's structures.
+// in-degree per node) lives in LDS too, interleaved by lane.  The area holds the ready list (and, during the
+// rank pass of the full-width kernel, a ring of ranks).
 __host__ __device__ inline size_t ke_dyn_bytes(uint32_t rcap, uint32_t ls, uint32_t nv, uint32_t nodes = 0) {
+  (void)nv;
   const size_t rw = ls ? ls : KE_WAVE;
   const size_t ready = (size_t)rcap * rw * 12;                 // key (8 bytes) and meta (4 bytes) per entry
-  const size_t plan = (size_t)nv * RPEG_FIELDS * rw * 2, vmem = (size_t)nv * 4 * rw * 8;
-  const size_t top = ready > plan ? (ready > vmem ? ready : vmem) : (plan > vmem ? plan : vmem);
   // (2 KB more for the full-width kernel: measured, not derived.  With 1-3 KB of slack behind the ready list the
   // steps of configs 2, 3 and 4 are 2-3 % shorter on the same machine; from 4 KB on config 3 loses a wavefront
   // per compute unit and from 6 KB on config 4 does.)
-  const size_t bytes = ((top + 15) & ~size_t(15)) + (ls ? 0 : 2048);
+  const size_t bytes = ((ready + 15) & ~size_t(15)) + (ls ? 0 : 2048);
   // The rank pass of the full-width kernel keeps the ranks of the last nodes of the order in this area (a ring of a
   // power of two of rows of 64 doubles, and two bytes per node behind it); a successor further back is read from the
   // workspace, a round trip through the L2 right after the store.  With the unrolled steps of a graph of more than
@@ -180,8 +186,6 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   uint64_t* l_node = (uint64_t*)lds;                                  // NodeRec[n]
   uint16_t* l_succ = (uint16_t*)(lds + (size_t)n * 8);                // uint16[n_succ]
   uint8_t* dyn = lds + L.cls_bytes;
-  int16_t* l_plan = (int16_t*)dyn + lane;                             // [60][64], aliased with the ready list
-  double* l_vm = (double*)dyn + lane;   // [4 * vertices][RW]: written once the cost model is done with the plan fields
   double* r_key = (double*)dyn + lane;                                       // [rcap][RW]
   uint32_t* r_nt = (uint32_t*)(dyn + (size_t)L.rcap * RW * 8) + lane;        // [rcap][RW] meta, see below
 
@@ -218,53 +222,29 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     g_dur = g_rank + (size_t)L.ws_nodes * KE_WAVE;
     g_deg = (uint8_t*)((double*)base + (2 * (size_t)L.ws_nodes + L.ws_slots) * KE_WAVE) + lane;
   }
-
-  // ---- plan fields -> LDS
-  const PlanHead h = load_head(L.head, L.stride, pi);
-  const rpeg_struct_t& st = P.st[cv.h->structure];   // uniform (the class fixes the structure)
-  const int nv = st.n_vertex;
-  {   // every load of the plan in flight at once
-    int16_t x[RPEG_MAX_V * RPEG_FIELDS];
-#pragma unroll
-    for (int f = 0; f < RPEG_MAX_V * RPEG_FIELDS; ++f)
-      if (f < nv * RPEG_FIELDS) x[f] = L.vert[(uint64_t)f * L.stride + pi];
-#pragma unroll
-    for (int f = 0; f < RPEG_MAX_V * RPEG_FIELDS; ++f)
-      if (f < nv * RPEG_FIELDS) l_plan[f * RW] = x[f];
-  }
-
-  VPlan a[RPEG_MAX_V];
-#pragma unroll
-  for (int v = 0; v < RPEG_MAX_V; ++v)
-    if (v < nv) a[v] = ke_vplan<RW>(l_plan, v);
-
-  // ---- per-plan relations
-  const PlanMasks pm = plan_masks(a, nv);
-  const uint64_t dpne = pm.dpne;
-
+  // Pair relations, penalty factor and gate bits of this lane's plan, and the durations of its class's slots out of
+  // the table of the slot universe: the prologue launches left them by plan index (one gather each, all in flight at
+  // once); the durations go into this lane's rows of the state, where the loops below read them coalesced.
+  const uint64_t ovl = L.aux_ovl[pi], dpne = L.aux_dpne[pi];
+  const double pen = L.aux_pen[pi];
+  const uint8_t gates = L.aux_mask[pi];
   KE_STAMP(1);
-  // ---- durations of the class's slots
-  bool err = cv.h->error != 0, zero_div = false;
-  const int split = (int)cv.h->split;
-  for (int s = 0; s < n_slots; ++s) g_dur[(s) * SS] = ke_slot_duration<RW>(P, st, split, cv.slot[s], l_plan, &zero_div);
-  err = err || zero_div;
-
-  KE_STAMP(2);
-  // ---- memory model and gates (plan fields in LDS are dead after this point)
-  const bool coresident = struct_coresident(st);
+  bool err = cv.h->error != 0;
+  {   // a slot whose duration the reference could not compute (division by zero) is NaN
+    bool bad = false;
+    const double* src = L.dur + pi;
+    for (int s0 = 0; s0 < n_slots; s0 += 8) {
+      double d[8];
 #pragma unroll
-  for (int v = 0; v < RPEG_MAX_V; ++v)
-    if (v < nv) {
-      const VMem m = vertex_memory(P, st.vertex[v], a[v], coresident);
-      l_vm[(v * 4 + 0) * RW] = (double)m.w_shard;
-      l_vm[(v * 4 + 1) * RW] = m.mem_w;
-      l_vm[(v * 4 + 2) * RW] = m.opt;
-      l_vm[(v * 4 + 3) * RW] = m.extra;
+      for (int u = 0; u < 8; ++u) d[u] = s0 + u < n_slots ? src[(size_t)cv.umap[s0 + u] * L.dur_stride] : 0.0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < n_slots) { g_dur[(s0 + u) * SS] = d[u]; bad = bad || d[u] != d[u]; }
     }
-  const KeVMem<RW> kvm{l_vm};
-  const double peak = device_peak_max(P, st, cv.h->vorder, pm, kvm);
-  const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
-  const bool mem_ok = !(peak > P.cap);
+    err = err || bad;
+  }
+  KE_STAMP(2);
+  const bool stale_ok = (gates & RPEG_MASK_STALE_OK) != 0, mem_ok = (gates & RPEG_MASK_MEM_OK) != 0;
 
   KE_STAMP(3);
   // ---- ranks: reverse topological pass, then chain inheritance (scheduler.py:71-100, 367-378)
@@ -569,7 +549,7 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     unsigned touched = 0;
 #pragma unroll
     for (int x = 0; x < RPEG_MAX_V; ++x)
-      if ((blocked >> x) & 1u) touched |= mask_row(pm.ovl, x);
+      if ((blocked >> x) & 1u) touched |= mask_row(ovl, x);
 #pragma unroll
     for (int x = 0; x < RPEG_MAX_V; ++x)
       if (((touched >> x) & 1u) && fin > lf[x]) lf[x] = fin;
@@ -681,13 +661,12 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     if (ovf || limit) mask |= RPEG_MASK_LIMIT;
   } else {
     double score = P.score_num / makespan;
-    if (!mem_ok) score = score * oom_penalty(peak, P.cap);
+    if (!mem_ok) score = score * pen;
     if ((L.flags & RPEG_GATE_STALE) && !stale_ok) score = 0.0;
     out_makespan = makespan;
     out_score = score;
   }
-  if (L.makespan) L.makespan[pi] = out_makespan;
-  if (L.peak) L.peak[pi] = peak;
+  if (L.makespan) L.makespan[pi] = out_makespan;   // (the peak is the prologue launch's output)
   if (L.score) L.score[pi] = out_score;
   if (L.mask) L.mask[pi] = mask;
   if (L.mass) {

@@ -654,80 +654,105 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
 
   __syncthreads();   // the previous plan of this wavefront is done with LDS
   KE_STAMP(0);
-  const PlanHead h = load_head(L.head, L.stride, pi);
   const rpeg_struct_t& st = P.st[cv.h->structure];
   const int nv = st.n_vertex;
-  if (lane < KP_PLAN_I16) l_plan[lane] = lane < nv * RPEG_FIELDS ? L.vert[(uint64_t)lane * L.stride + pi] : (int16_t)1;
-  __syncthreads();
-
-  // ---- pair relations: lane 8u+v tests vertices u and v, the ballots are the masks
   PlanMasks pm;
-  {
-    const int u = lane >> 3, v = lane & 7;
-    const bool valid = u < nv && v < nv;
-    const VPlan au = ke_vplan<1>(l_plan, valid ? u : 0), av = ke_vplan<1>(l_plan, valid ? v : 0);
-    pm.ovl = __ballot(valid && !alloc_disjoint(au, av));
-    pm.eq = 0;   // the memory model below works on position-indexed masks of its own
-    pm.dpne = __ballot(valid && au.dp != av.dp);
-  }
-  KE_STAMP(1);
+  pm.ovl = pm.eq = pm.dpne = 0;
+  bool err = cv.h->error != 0, limit = false, stale_ok = false, mem_ok = false;
+  double peak = -1.0, pen = 1.0;
+  if (L.dur) {
+    // a task of a laid-out batch: the prologue launches have left the durations of the slot universe, the pair
+    // relations, the penalty factor and the gate bits by plan index (and written the peak themselves)
+    const uint64_t sp = pi;
+    bool bad = false;
+    for (int s = lane; s < n_slots; s += KE_WAVE) {
+      const double d = L.dur[(size_t)cv.umap[s] * L.dur_stride + sp];
+      l_dur[s] = d;
+      bad = bad || d != d;
+    }
+    err = err || __ballot(bad) != 0ull;
+    pm.ovl = L.aux_ovl[sp];
+    pm.dpne = L.aux_dpne[sp];
+    pen = L.aux_pen[sp];
+    const uint8_t gates = L.aux_mask[sp];
+    stale_ok = (gates & RPEG_MASK_STALE_OK) != 0;
+    mem_ok = (gates & RPEG_MASK_MEM_OK) != 0;
+    __syncthreads();
+    KE_STAMP(1);
+    KE_STAMP(2);
+  } else {
+    const PlanHead h = load_head(L.head, L.stride, pi);
+    if (lane < KP_PLAN_I16) l_plan[lane] = lane < nv * RPEG_FIELDS ? L.vert[(uint64_t)lane * L.stride + pi] : (int16_t)1;
+    __syncthreads();
 
-  // ---- durations of the class's slots, one slot per lane
-  bool err = cv.h->error != 0, zero_div = false, limit = false;
-  const int split = (int)cv.h->split;
-  for (int s = lane; s < n_slots; s += KE_WAVE) l_dur[s] = ke_slot_duration<1>(P, st, split, cv.slot[s], l_plan, &zero_div);
-  err = err || __ballot(zero_div) != 0ull;
-  KE_STAMP(2);
+    // ---- pair relations: lane 8u+v tests vertices u and v, the ballots are the masks
+    {
+      const int u = lane >> 3, v = lane & 7;
+      const bool valid = u < nv && v < nv;
+      const VPlan au = ke_vplan<1>(l_plan, valid ? u : 0), av = ke_vplan<1>(l_plan, valid ? v : 0);
+      pm.ovl = __ballot(valid && !alloc_disjoint(au, av));
+      pm.eq = 0;   // the memory model below works on position-indexed masks of its own
+      pm.dpne = __ballot(valid && au.dp != av.dp);
+    }
+    KE_STAMP(1);
 
-  // ---- memory model (memory.py:608-841), in the order of first appearance of the vertices among the
-  // lowered operator nodes (position i = vertex vorder[i]): that order fixes the order of the float sums.
-  // One vertex per lane, then one vertex subset per lane tests whether it is a device class (a maximal clique
-  // of the overlap graph); the few that are get evaluated one after the other with uniform control flow.
-  const uint8_t* order = cv.h->vorder;
-  const bool coresident = struct_coresident(st);
-  if (lane < nv) {
-    const int v = order[lane];
-    const VMem m = vertex_memory(P, st.vertex[v], ke_vplan<1>(l_plan, v), coresident);
-    l_vm[lane * 4 + 0] = (double)m.w_shard;
-    l_vm[lane * 4 + 1] = m.mem_w;
-    l_vm[lane * 4 + 2] = m.opt;
-    l_vm[lane * 4 + 3] = m.extra;
-  }
-  KpOrdered om;
-  {
-    const int i = lane >> 3, j = lane & 7;
-    const bool valid = i < nv && j < nv;
-    const int vi = order[valid ? i : 0], vj = order[valid ? j : 0];
-    const VPlan ai = ke_vplan<1>(l_plan, vi), aj = ke_vplan<1>(l_plan, vj);
-    const rpeg_vertex_t &xi = st.vertex[vi], &xj = st.vertex[vj];
-    om.ovl = __ballot(valid && !alloc_disjoint(ai, aj));
-    om.eq = __ballot(valid && alloc_equal(ai, aj));
-    om.same_model = __ballot(valid && xi.model == xj.model);
-    om.train_same = __ballot(valid && xi.model == xj.model && xj.role == RPEG_ROLE_TRAIN);
-    const unsigned long long t = __ballot(valid && j == 0 && xi.role == RPEG_ROLE_TRAIN),
-                             tr = __ballot(valid && j == 0 && st.mem_trainable[xi.model] != 0);   // bit 8i: position i
-    om.train = om.trainable = 0u;
-    om.coresident = coresident;
+    // ---- durations of the class's slots, one slot per lane
+    bool zero_div = false;
+    const int split = (int)cv.h->split;
+    for (int s = lane; s < n_slots; s += KE_WAVE) l_dur[s] = ke_slot_duration<1>(P, st, split, cv.slot[s], l_plan, &zero_div);
+    err = err || __ballot(zero_div) != 0ull;
+    KE_STAMP(2);
+
+    // ---- memory model (memory.py:608-841), in the order of first appearance of the vertices among the
+    // lowered operator nodes (position i = vertex vorder[i]): that order fixes the order of the float sums.
+    // One vertex per lane, then one vertex subset per lane tests whether it is a device class (a maximal clique
+    // of the overlap graph); the few that are get evaluated one after the other with uniform control flow.
+    const uint8_t* order = cv.h->vorder;
+    const bool coresident = struct_coresident(st);
+    if (lane < nv) {
+      const int v = order[lane];
+      const VMem m = vertex_memory(P, st.vertex[v], ke_vplan<1>(l_plan, v), coresident);
+      l_vm[lane * 4 + 0] = (double)m.w_shard;
+      l_vm[lane * 4 + 1] = m.mem_w;
+      l_vm[lane * 4 + 2] = m.opt;
+      l_vm[lane * 4 + 3] = m.extra;
+    }
+    KpOrdered om;
+    {
+      const int i = lane >> 3, j = lane & 7;
+      const bool valid = i < nv && j < nv;
+      const int vi = order[valid ? i : 0], vj = order[valid ? j : 0];
+      const VPlan ai = ke_vplan<1>(l_plan, vi), aj = ke_vplan<1>(l_plan, vj);
+      const rpeg_vertex_t &xi = st.vertex[vi], &xj = st.vertex[vj];
+      om.ovl = __ballot(valid && !alloc_disjoint(ai, aj));
+      om.eq = __ballot(valid && alloc_equal(ai, aj));
+      om.same_model = __ballot(valid && xi.model == xj.model);
+      om.train_same = __ballot(valid && xi.model == xj.model && xj.role == RPEG_ROLE_TRAIN);
+      const unsigned long long t = __ballot(valid && j == 0 && xi.role == RPEG_ROLE_TRAIN),
+                               tr = __ballot(valid && j == 0 && st.mem_trainable[xi.model] != 0);   // bit 8i: position i
+      om.train = om.trainable = 0u;
+      om.coresident = coresident;
 #pragma unroll
-    for (int q = 0; q < RPEG_MAX_V; ++q) {
-      om.train |= (unsigned)((t >> (8 * q)) & 1ull) << q;
-      om.trainable |= (unsigned)((tr >> (8 * q)) & 1ull) << q;
+      for (int q = 0; q < RPEG_MAX_V; ++q) {
+        om.train |= (unsigned)((t >> (8 * q)) & 1ull) << q;
+        om.trainable |= (unsigned)((tr >> (8 * q)) & 1ull) << q;
+      }
     }
-  }
-  __syncthreads();
-  double peak = -1.0;
-  {
-    const unsigned M = (unsigned)lane + 1u;
-    unsigned long long classes = __ballot(M < (1u << nv) && kp_maximal_clique(nv, om.ovl, M));
-    while (classes) {
-      const unsigned Mu = (unsigned)__builtin_ctzll(classes) + 1u;
-      classes &= classes - 1ull;
-      const double p = kp_class_peak(P, st, order, nv, om, l_vm, Mu);
-      peak = p > peak ? p : peak;
+    __syncthreads();
+    {
+      const unsigned M = (unsigned)lane + 1u;
+      unsigned long long classes = __ballot(M < (1u << nv) && kp_maximal_clique(nv, om.ovl, M));
+      while (classes) {
+        const unsigned Mu = (unsigned)__builtin_ctzll(classes) + 1u;
+        classes &= classes - 1ull;
+        const double p = kp_class_peak(P, st, order, nv, om, l_vm, Mu);
+        peak = p > peak ? p : peak;
+      }
     }
+    stale_ok = stale_layout_ok(st, h, pm.ovl);
+    mem_ok = !(peak > P.cap);
+    if (!mem_ok) pen = oom_penalty(peak, P.cap);
   }
-  const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
-  const bool mem_ok = !(peak > P.cap);
   KE_STAMP(3);
   unsigned long long* stamp = L.prof && lane == 0 ? L.prof + w * 8 : nullptr;
 
@@ -766,7 +791,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     if (limit) mask |= RPEG_MASK_LIMIT;
   } else {
     double score = P.score_num / makespan;
-    if (!mem_ok) score = score * oom_penalty(peak, P.cap);
+    if (!mem_ok) score = score * pen;
     if ((L.flags & RPEG_GATE_STALE) && !stale_ok) score = 0.0;
     out_makespan = makespan;
     out_score = score;
@@ -789,7 +814,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   if (lane == 0) {
     if (L.util) L.util[pi] = util;
     if (L.makespan) L.makespan[pi] = out_makespan;
-    if (L.peak) L.peak[pi] = peak;
+    if (L.peak && !L.dur) L.peak[pi] = peak;   // (with a prologue launch the peak is that launch's output)
     if (L.score) L.score[pi] = out_score;
     if (L.mask) L.mask[pi] = mask;
     if (L.mass) {

@@ -39,7 +39,8 @@ constexpr uint32_t KQ_EMPTY = 0xFFFFFFFFu;
 // duration (double per slot), position (uint16 per node), in-degree (byte per node).
 __host__ __device__ inline size_t kq_tab_bytes(uint32_t nodes) { return ((size_t)nodes * 4 + 17 * 2 + 15) & ~size_t(15); }
 __host__ __device__ inline size_t kq_dyn_bytes(uint32_t nv, uint32_t np) {
-  return (((size_t)nv * RPEG_FIELDS * np * 2 + 15) & ~size_t(15)) + (size_t)nv * 4 * np * 8;
+  (void)nv; (void)np;   // (plan fields and memory terms used to sit here: the prologue launch computes from them now)
+  return 0;
 }
 __host__ __device__ inline size_t kq_lds_bytes(uint32_t cls_bytes, uint32_t nodes, uint32_t slots, uint32_t nv, uint32_t np, bool mass) {
   return cls_bytes + kq_tab_bytes(nodes) + kq_dyn_bytes(nv, np) +
@@ -94,8 +95,6 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   uint16_t* l_bykey = l_topo + L.ws_nodes;                            // uint16[n]: nodes grouped by tie-break class
   uint16_t* l_kbeg = l_bykey + L.ws_nodes;                            // uint16[17]: first place of every tie-break class
   uint8_t* dyn = lds + L.cls_bytes + kq_tab_bytes(L.ws_nodes);
-  int16_t* l_plan = (int16_t*)dyn + p;                                // [fields][RW]
-  double* l_vm = (double*)(dyn + (((size_t)L.max_v * RPEG_FIELDS * NP * 2 + 15) & ~size_t(15))) + p;   // [4 * vertices][RW]
   uint8_t* sbase = dyn + kq_dyn_bytes(L.max_v, NP);
   const size_t tr_rows = (L.mass ? 2 : 1) * (size_t)L.ws_nodes;   // rows of the time and rank arrays together
   double* g_time = (double*)sbase + p;
@@ -133,41 +132,27 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   first_lane = __builtin_ctzll(__ballot(1));
   KE_STAMP(0);
 
-  // ---- plan fields -> LDS, a share by each lane
-  const PlanHead h = load_head(L.head, L.stride, pi);
   const rpeg_struct_t& st = P.st[cv.h->structure];   // uniform (the class fixes the structure)
-  const int nv = st.n_vertex;
-  for (int f = q; f < nv * RPEG_FIELDS; f += QL) l_plan[f * RW] = L.vert[(uint64_t)f * L.stride + pi];
-  __syncthreads();
-  VPlan a[RPEG_MAX_V];
-#pragma unroll
-  for (int v = 0; v < RPEG_MAX_V; ++v)
-    if (v < nv) a[v] = ke_vplan<RW>(l_plan, v);
-  const PlanMasks pm = plan_masks(a, nv);
-  const uint64_t dpne = pm.dpne;
-
+  (void)st;
+  // pair relations, penalty factor and gate bits of this plan and the durations of its class's slots (out of the table
+  // of the slot universe) come from the prologue launches, by plan index
+  const uint64_t ovl = L.aux_ovl[pi], dpne = L.aux_dpne[pi];
+  const double pen = L.aux_pen[pi];
+  const uint8_t gates = L.aux_mask[pi];
   KE_STAMP(1);
-  // ---- durations of the class's slots, a share by each lane
-  bool err = cv.h->error != 0, zero_div = false;
-  const int split = (int)cv.h->split;
-  for (int s = q; s < n_slots; s += QL) g_dur[s * RW] = ke_slot_duration<RW>(P, st, split, cv.slot[s], l_plan, &zero_div);
-  err = err || kq_or(zero_div ? 1u : 0u) != 0u;
-
-  KE_STAMP(2);
-  // ---- memory model and gates: the per-vertex terms a vertex by each lane, the peak in all lanes alike
-  const bool coresident = struct_coresident(st);
-  for (int v = q; v < nv; v += QL) {
-    const VMem m = vertex_memory(P, st.vertex[v], ke_vplan<RW>(l_plan, v), coresident);
-    l_vm[(v * 4 + 0) * RW] = (double)m.w_shard;
-    l_vm[(v * 4 + 1) * RW] = m.mem_w;
-    l_vm[(v * 4 + 2) * RW] = m.opt;
-    l_vm[(v * 4 + 3) * RW] = m.extra;
+  bool err = cv.h->error != 0;
+  {   // a slot whose duration the reference could not compute (division by zero) is NaN; a share by each lane
+    bool bad = false;
+    for (int s = q; s < n_slots; s += QL) {
+      const double d = L.dur[(size_t)cv.umap[s] * L.dur_stride + pi];
+      g_dur[s * RW] = d;
+      bad = bad || d != d;
+    }
+    err = err || kq_or(bad ? 1u : 0u) != 0u;
   }
   __syncthreads();
-  const KeVMem<RW> kvm{l_vm};
-  const double peak = device_peak_max(P, st, cv.h->vorder, pm, kvm);
-  const bool stale_ok = stale_layout_ok(st, h, pm.ovl);
-  const bool mem_ok = !(peak > P.cap);
+  KE_STAMP(2);
+  const bool stale_ok = (gates & RPEG_MASK_STALE_OK) != 0, mem_ok = (gates & RPEG_MASK_MEM_OK) != 0;
 
   KE_STAMP(3);
   // ---- ranks: reverse topological pass, then chain inheritance (scheduler.py:71-100, 367-378); all lanes alike
@@ -323,7 +308,7 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     unsigned touched = 0;
 #pragma unroll
     for (int x = 0; x < RPEG_MAX_V; ++x)
-      if ((blocked >> x) & 1u) touched |= mask_row(pm.ovl, x);
+      if ((blocked >> x) & 1u) touched |= mask_row(ovl, x);
 #pragma unroll
     for (int x = 0; x < RPEG_MAX_V; ++x)
       if (((touched >> x) & 1u) && fin > lf[x]) lf[x] = fin;
@@ -402,14 +387,13 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
     if (ovf) mask |= RPEG_MASK_LIMIT;
   } else {
     double score = P.score_num / makespan;
-    if (!mem_ok) score = score * oom_penalty(peak, P.cap);
+    if (!mem_ok) score = score * pen;
     if ((L.flags & RPEG_GATE_STALE) && !stale_ok) score = 0.0;
     out_makespan = makespan;
     out_score = score;
   }
   if (q == 0) {
-    if (L.makespan) L.makespan[pi] = out_makespan;
-    if (L.peak) L.peak[pi] = peak;
+    if (L.makespan) L.makespan[pi] = out_makespan;   // (the peak is the prologue launch's output)
     if (L.score) L.score[pi] = out_score;
     if (L.mask) L.mask[pi] = mask;
     if (L.mass) {

@@ -277,6 +277,24 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
     for (int i = 0; i < n; ++i)
       if (out.nodes[i].kind == 0 && !seen_v[out.nodes[i].vertex]) { seen_v[out.nodes[i].vertex] = true; vorder[c++] = (uint8_t)out.nodes[i].vertex; }
     if (c != nv) throw std::runtime_error("a template vertex has no lowered operator node");
+    // The memory launch derives this order from the plan alone (plan_vorder): hold the two to each other here,
+    // from the signature's predicates, for every class that is ever lowered.
+    unsigned gs = 0, moved = 0;
+    std::vector<uint8_t> want, tail;
+    if (nph > 0) {
+      for (int e = 0; e < st.n_edge; ++e)
+        if (st.edge[e].gen_inf && sg.disjoint(st.edge[e].src, st.edge[e].dst)) gs |= 1u << st.edge[e].src;
+      for (int e = 0; e < st.n_edge; ++e) {
+        const int u = st.edge[e].src, v = st.edge[e].dst;
+        if (!((gs >> u) & 1u) || st.vertex[v].role != RPEG_ROLE_INF || ((moved >> v) & 1u)) continue;
+        if (sg.disjoint(u, v)) { moved |= 1u << v; tail.push_back((uint8_t)v); }
+      }
+    }
+    for (int v = 0; v < nv; ++v)
+      if (!((moved >> v) & 1u)) want.push_back((uint8_t)v);
+    want.insert(want.end(), tail.begin(), tail.end());
+    for (int v = 0; v < nv; ++v)
+      if (want[v] != vorder[v]) throw std::logic_error("vertex order of the lowered graph differs from the plan's own");
   }
 
   // blob
@@ -317,6 +335,20 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
     groups.push_back(GroupRec{(uint16_t)gmember.size(), (uint16_t)kv.second.size()});
     for (int i : kv.second) gmember.push_back((uint16_t)i);
   }
+  // every slot's place in the structure's slot universe
+  std::vector<uint8_t> umap(slots.size(), 0);
+  {
+    SlotDesc uni[RPEG_MAX_UNIVERSE];
+    const int nu = slot_universe(P, st, uni);
+    if (nu > RPEG_MAX_UNIVERSE) throw std::runtime_error("slot universe too large");
+    for (size_t k = 0; k < slots.size(); ++k) {
+      int hit = -1;
+      for (int u = 0; u < nu && hit < 0; ++u)
+        if (uni[u].type == slots[k].type && uni[u].a == slots[k].a && uni[u].b == slots[k].b && uni[u].q == slots[k].q) hit = u;
+      if (hit < 0) throw std::logic_error("a duration slot outside the slot universe");
+      umap[k] = (uint8_t)hit;
+    }
+  }
   std::vector<uint16_t> pbeg(n + 1, 0), pred(out.edges.size(), 0);
   {
     for (auto& ed : out.edges) ++pbeg[ed.second + 1];
@@ -340,6 +372,7 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   h.off_gmember = (uint32_t)off; off = align8(off + gmember.size() * 2);
   h.off_pbeg = (uint32_t)off; off = align8(off + pbeg.size() * 2);
   h.off_pred = (uint32_t)off; off = align8(off + pred.size() * 2);
+  h.off_umap = (uint32_t)off; off = align8(off + umap.size());
   h.bytes = (uint32_t)off;
   out.blob.assign(off, 0);
   std::memcpy(out.blob.data(), &h, sizeof h);
@@ -352,6 +385,7 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   if (!gmember.empty()) std::memcpy(out.blob.data() + h.off_gmember, gmember.data(), gmember.size() * 2);
   std::memcpy(out.blob.data() + h.off_pbeg, pbeg.data(), pbeg.size() * 2);
   if (!pred.empty()) std::memcpy(out.blob.data() + h.off_pred, pred.data(), pred.size() * 2);
+  if (!umap.empty()) std::memcpy(out.blob.data() + h.off_umap, umap.data(), umap.size());
   return out;
 }
 

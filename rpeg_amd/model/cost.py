@@ -51,7 +51,9 @@ class NodeCostModel:
         reference does (a degenerate phase), ValueError for a node the engine cannot place."""
         home = getattr(node, "_home", None)
         if home is not None:
-            graph, index = home
+            graph, index = home[0](), home[1]
+            if graph is None:
+                raise ValueError("the lowered graph this node belongs to no longer exists")
             t = float(_graph_detail(self, graph)["time"][index])
         else:
             t = self._mock_time(node)

@@ -10,6 +10,7 @@ It is integer work on the host and, like the reference's `lower()`, takes no har
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from dataclasses import dataclass, field
 from enum import Enum
 from typing import Dict, Optional, Tuple
@@ -48,7 +49,8 @@ class ExecNode:
     fusion_group: Optional[str] = None
     payload_in_bytes: int = 0
     label: Optional[str] = None
-    # where the node sits in the graph lower() built it for: (ExecutableRPEG, index); None for a node made by hand
+    # where the node sits in the graph lower() built it for: (weak reference to the ExecutableRPEG, index); None for a
+    # node made by hand
     _home: Optional[tuple] = field(default=None, repr=False, compare=False)
 
     def __hash__(self):
@@ -156,6 +158,7 @@ def lower(rpeg, unrolled: UnrolledRPEG, plan, suite, K_eval: int, workload: Opti
     verts = rpeg.vertices
     copies: Dict[tuple, UnrolledNode] = {} if unrolled is None else {(x.template_vertex, x.k): x for x in unrolled.nodes}
     graph = ExecutableRPEG.__new__(ExecutableRPEG)
+    home = weakref.ref(graph)      # (weak: a graph and its nodes must not keep each other alive in a cycle)
     nodes = []
     n_comm = n_reshard = 0
     for i in range(n):
@@ -173,19 +176,19 @@ def lower(rpeg, unrolled: UnrolledRPEG, plan, suite, K_eval: int, workload: Opti
                     tag = f":i{sub[i]}"
                     more = dict(n_seqs=n_seq)
             nodes.append(ExecNode(id=f"{v.id}@{step[i]}{tag}", kind=ExecNodeType.OP, allocs=(plan.sigma[v],), op=op,
-                                  model=v.kind.model, pi=plan.pi[v], mb=plan.mb.get(v, None), _home=(graph, i), **more))
+                                  model=v.kind.model, pi=plan.pi[v], mb=plan.mb.get(v, None), _home=(home, i), **more))
             continue
         allocs = (plan.sigma[verts[src[i]]], plan.sigma[v])
         label = rpeg.data_edges[ref[i]].container.name if ref[i] < 16 else f"W_{_MODEL_BY_CODE[ref[i] - 16].value}"
         if kind[i] == 1:
             n_comm += 1
             nodes.append(ExecNode(id=f"comm{n_comm}", kind=ExecNodeType.COMM, allocs=allocs,
-                                  payload_in_bytes=int(payload[i]), label=label, _home=(graph, i)))
+                                  payload_in_bytes=int(payload[i]), label=label, _home=(home, i)))
         else:
             n_reshard += 1
             nodes.append(ExecNode(id=f"reshard{n_reshard}", kind=ExecNodeType.RESHARD, allocs=allocs,
                                   model=_MODEL_BY_CODE[ref[i] - 16], payload_in_bytes=int(payload[i]), label=label,
-                                  _home=(graph, i)))
+                                  _home=(home, i)))
     pairs = edges[:2 * ne.value].reshape(-1, 2)
     object.__setattr__(graph, "nodes", tuple(nodes))
     object.__setattr__(graph, "edges", tuple(ExecEdge(nodes[a], nodes[b]) for a, b in pairs))

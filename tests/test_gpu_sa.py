@@ -553,7 +553,7 @@ def test_time_budget_ends_the_search_on_the_wall_clock():
                           T_cand={m: {0} for m in p.template(0, ()).tau})
     search_plan(p.suite, p.workload, p.hw, p.device_space, p.K_eval, opt, algorithm="ppo", no_polish=True)   # warm-up
     got = {}
-    for budget in (0.0, 0.05, 0.4):
+    for budget in (0.0, 0.1, 0.5):
         t0 = time.perf_counter()
         res = search_plan(p.suite, p.workload, p.hw, p.device_space, p.K_eval, opt, algorithm="ppo", no_polish=True,
                           time_budget=budget)
@@ -562,5 +562,6 @@ def test_time_budget_ends_the_search_on_the_wall_clock():
         assert budget <= res.seconds["optimize"] < budget + 0.1 + 2e-3 * res.cache.misses, (budget, res.seconds)
         assert time.perf_counter() - t0 < budget + 5.0
     assert got[0.0].scores["optimized"] == got[0.0].scores["start"]
-    assert got[0.0].scores["optimized"] <= got[0.05].scores["optimized"] <= got[0.4].scores["optimized"]
-    assert got[0.4].cache.misses > got[0.05].cache.misses > got[0.0].cache.misses
+    assert got[0.0].scores["optimized"] <= got[0.1].scores["optimized"] <= got[0.5].scores["optimized"]
+    counts = {b: (r.cache.misses, r.seconds) for b, r in got.items()}
+    assert got[0.5].cache.misses > got[0.1].cache.misses > got[0.0].cache.misses, counts
