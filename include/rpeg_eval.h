@@ -451,6 +451,14 @@ int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
    Results do not depend on the setting. */
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
 
+/* rpeg_sa_run deals its chains to `groups` groups (1..8, default 2; never fewer than 8 chains per group) that take
+   their steps in turn, each with a stream and staging buffers of its own: while the proposals of one group are being
+   evaluated, the host merges the results of another and draws its next proposals.  A chain's draws are keyed by
+   (seed, chain, step) and its decisions depend on its own evaluations only, so the result of a run does not depend
+   on the number of groups (the reference steps its chains one after the other, optimizer.py:683-786; it has no
+   counterpart of this setting). */
+int rpeg_engine_set_sa_groups(rpeg_engine_t* e, int32_t groups);
+
 /* With lanes = -1 and a batch that fills the chip in one round of wavefronts: the largest share of the batch's
    plans, in percent, that the four-lanes-per-plan kernel may take on a stream of its own (default 25; 0: none).
    Which classes it takes is learned: the main kernel records, per class, how long its slowest wavefront ran and how

@@ -200,6 +200,10 @@ void sa_context(Port* e, const rpeg_sa_params_t* prm, SaContext& cx) {
 }
 }  // namespace
 
+// groups of chains that SaRun steps in turn (1: all chains in one batch per step); the result must not depend on it
+static int g_sa_groups = 1;
+void port_set_sa_groups(int groups) { g_sa_groups = groups < 1 ? 1 : groups; }
+
 int port_sa_run(void* h, const rpeg_sa_params_t* prm, const int16_t* base_plan, rpeg_sa_result_t* res, int threads) {
   Port* e = (Port*)h;
   SaContext cx;
@@ -208,6 +212,7 @@ int port_sa_run(void* h, const rpeg_sa_params_t* prm, const int16_t* base_plan, 
   sa_settings_from(*prm, &st);
   CpuSaBackend be;
   be.e = e; be.threads = threads;
+  be.host_lanes = g_sa_groups;
   for (int k = 0; k < prm->n_variants; ++k) {
     be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;
     be.head_of[k][2] = prm->tau[k][0]; be.head_of[k][3] = prm->tau[k][1];

@@ -29,6 +29,8 @@ def lib():
         _lib.port_eval.restype = C.c_int
         _lib.port_eval.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint32] + \
             [C.c_void_p] * 6 + [C.c_int, C.c_void_p]
+        _lib.port_set_sa_groups.restype = None
+        _lib.port_set_sa_groups.argtypes = [C.c_int]
         _lib.port_sa_run.restype = C.c_int
         _lib.port_sa_run.argtypes = [C.c_void_p] * 4 + [C.c_int]
         _lib.port_sa_optimize.restype = C.c_int
@@ -111,8 +113,11 @@ class CpuPort:
                 params.dir[v] = None
         return keep
 
-    def sa_run(self, params, directory, base_plan=None, threads=1):
-        """The host annealing logic of rpeg_amd/csrc/rpeg_sa.h over this CPU evaluator."""
+    def sa_run(self, params, directory, base_plan=None, threads=1, groups=1):
+        """The host annealing logic of rpeg_amd/csrc/rpeg_sa.h over this CPU evaluator.  `groups`: the chains are
+        dealt to that many groups that take their steps in turn (what the GPU library does to overlap evaluation and
+        host work); the result does not depend on it."""
+        lib().port_set_sa_groups(int(groups))
         keep = self._set_directory(params, directory)
         nc, ns = params.n_chains, params.n_steps
         W = abi.MAX_V * abi.FIELDS

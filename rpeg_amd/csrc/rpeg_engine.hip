@@ -339,6 +339,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(4, 8))) vo
     const uint32_t off = L.wave_cls[w];
     if (off == KP_SKIP) continue;   // uniform: a task without a plan to evaluate
     kp_eval_plan(L, w, pi, class_view(L.pool + off), kp_lds);
+    // (lane 0 wrote the outputs of the task: its release store orders them before the flag)
+    if (L.done && threadIdx.x == 0) __hip_atomic_store(&L.done[w], L.done_tag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
@@ -524,6 +526,27 @@ static uint8_t* static_scratch_ptr(int dev, hipError_t* st) {
   return g_static_ptr[dev];
 }
 
+// Staging of one small host-pointer evaluation: plans and class offsets in (pinned, then device), results out (pinned,
+// written by the kernel itself), and which of the caller's plans went to the device.
+struct HostLane {
+  uint8_t *in = nullptr, *dev = nullptr, *out = nullptr;
+  // `direct`: the kernel reads the plans from the pinned block itself (no copy ahead of the launch) and flags every
+  // finished plan in the pinned result block, where the host polls for it instead of waiting for the launch to end:
+  // for the steps of an annealing run, whose latency is what counts
+  bool direct = false;
+  uint8_t *in_dev = nullptr, *out_dev = nullptr;   // the pinned blocks as the device addresses them
+  uint32_t tag = 0;
+  size_t cap = 0;
+  std::vector<uint32_t> idx;
+  size_t n = 0, stride = 0;
+  bool launched = false;
+  void release() {
+    if (in) { hipHostFree(in); hipFree(dev); hipHostFree(out); }
+    in = dev = out = in_dev = out_dev = nullptr;
+    cap = 0;
+  }
+};
+
 struct rpeg_engine_s {
   rpeg_problem_t P;
   rpeg_problem_t* dP = nullptr;
@@ -558,7 +581,7 @@ struct rpeg_engine_s {
   bool lds_attr_set[5] = {false, false, false, false, false};
   // staging of the host-pointer path: plans and class offsets in (pinned, then device), results out (pinned,
   // written by the kernel itself)
-  uint8_t *hs_in = nullptr, *ds_in = nullptr, *hs_out = nullptr;
+  HostLane lane0;
   uint8_t* d_stage = nullptr;   // device copy of host tensors and results for larger host-pointer batches
   size_t d_stage_cap = 0;
   uint8_t* h_stage = nullptr;   // pinned mirror of the result region of d_stage
@@ -566,8 +589,8 @@ struct rpeg_engine_s {
   uint8_t* d_trace = nullptr;   // rpeg_eval_trace: one plan's fields and header, then start / finish / dispatch index
   uint8_t* d_detail = nullptr;  // rpeg_plan_detail: one plan's fields and header, then slot durations and vertex-set peaks
   size_t d_trace_nodes = 0;
-  size_t hs_cap = 0;
-  std::vector<uint32_t> hs_idx;
+  int sa_lanes = 3;     // rpeg_sa_run: groups of chains whose evaluations overlap the host's work on the others
+  int lanes_busy = 0;   // evaluations submitted on lanes and not yet collected (their kernels read d_pool)
   uint64_t relearn_at = 0;                // the call that last asked for the measurements again
   uint32_t one_plan_waves_per_cu = 64;    // batches of at most this many plans per compute unit take one wavefront per plan
   uint32_t host_small_max = 1024;          // rpeg_eval_host: largest batch whose classes the host looks up itself
@@ -742,6 +765,7 @@ static int ensure_pool(rpeg_engine_t* e, hipStream_t s) {
     uint8_t* np = nullptr;
     HIP_TRY(e, hipMalloc(&np, cap));
     HIP_TRY(e, hipStreamSynchronize(s));
+    if (e->lanes_busy > 0) HIP_TRY(e, hipDeviceSynchronize());   // kernels of other lanes still read the old pool
     if (e->d_pool) hipFree(e->d_pool);
     e->d_pool = np;
     e->d_pool_cap = cap;
@@ -942,7 +966,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->s2) { hipStreamDestroy(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
   if (e->s3) { hipStreamDestroy(e->s3); hipEventDestroy(e->ev_join3); }
   if (e->ev_counts) hipEventDestroy(e->ev_counts);
-  if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
+  e->lane0.release();
   if (e->d_stage) hipFree(e->d_stage);
   if (e->h_stage) hipHostFree(e->h_stage);
   if (e->d_trace) hipFree(e->d_trace);
@@ -984,6 +1008,13 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
   }
   e->state_lanes = lanes;
   e->split_for_n = 0;
+  return 0;
+}
+
+int rpeg_engine_set_sa_groups(rpeg_engine_t* e, int32_t groups) {
+  if (!e) return -1;
+  if (groups < 1 || groups > 8) { e->err = "1 to 8 groups of chains"; return -1; }
+  e->sa_lanes = groups;
   return 0;
 }
 
@@ -2086,61 +2117,54 @@ int rpeg_eval_trace_metrics(rpeg_engine_t* e, const int16_t* vert_fields, const 
 namespace {
 
 constexpr size_t HS_IN_BYTES = (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 + 4 + 4;   // per plan: fields, header, class offset
-constexpr size_t HS_OUT_BYTES = 3 * 8 + (size_t)RPEG_MAX_V * 8 + 8 + 8;        // makespan, peak, score, mass, utilisation, mask (padded)
+constexpr size_t HS_OUT_BYTES = 3 * 8 + (size_t)RPEG_MAX_V * 8 + 8 + 8 + 8;    // makespan, peak, score, mass, utilisation, mask (padded), done flag (padded)
 
-int ensure_host_stage(rpeg_engine_t* e, size_t n, hipStream_t s) {
-  if (n <= e->hs_cap) return 0;
+int ensure_host_stage(rpeg_engine_t* e, HostLane& ln, size_t n, hipStream_t s) {
+  if (n <= ln.cap) return 0;
   HIP_TRY(e, hipStreamSynchronize(s));
-  if (e->hs_in) { hipHostFree(e->hs_in); hipFree(e->ds_in); hipHostFree(e->hs_out); }
-  e->hs_in = e->ds_in = e->hs_out = nullptr;
-  e->hs_cap = 0;
+  ln.release();
   const size_t cap = (std::max<size_t>(n + n / 2, 1024) + 63) & ~size_t(63);
-  HIP_TRY(e, hipHostMalloc(&e->hs_in, HS_IN_BYTES * cap));
-  HIP_TRY(e, hipMalloc(&e->ds_in, HS_IN_BYTES * cap));
-  HIP_TRY(e, hipHostMalloc(&e->hs_out, HS_OUT_BYTES * cap));
-  e->hs_cap = cap;
+  HIP_TRY(e, hipHostMalloc(&ln.in, HS_IN_BYTES * cap));
+  HIP_TRY(e, hipMalloc(&ln.dev, HS_IN_BYTES * cap));
+  HIP_TRY(e, hipHostMalloc(&ln.out, HS_OUT_BYTES * cap, hipHostMallocCoherent));   // (the host reads it while a launch runs)
+  std::memset(ln.out, 0, HS_OUT_BYTES * cap);
+  HIP_TRY(e, hipHostGetDevicePointer((void**)&ln.in_dev, ln.in, 0));
+  HIP_TRY(e, hipHostGetDevicePointer((void**)&ln.out_dev, ln.out, 0));
+  ln.cap = cap;
   return 0;
 }
 
 // Plans in host memory, results to host memory, for a batch small enough for one plan per wavefront: the
 // host computes the class of every plan itself (validity gate, signature, table lookup: ~100 ns per plan),
 // so the call is one copy to the device, one launch of k_plan, whose first lanes write the results straight
-// into pinned host memory, and one wait.  get(i, head, a) yields plan i.  Returns 1 when the batch is not
-// eligible (a class too large for k_plan); the caller then takes the device path.  Output arrays may be null.
+// into pinned host memory, and one wait.  get(i, head, a) yields plan i.  The work comes in two halves so that a
+// caller with several lanes (staging buffers and a stream each) can keep one evaluation running while it prepares
+// the next: host_small_submit stages and launches, host_small_collect waits and hands the results out.  Submit
+// returns 1 when the batch is not eligible (a class too large for k_plan); the caller then takes the device path.
 template <class GET>
-int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, double* makespan, double* peak, double* score,
-                    uint8_t* mask, double* mass, hipStream_t s, double* util = nullptr) {
-  e->last_ms = -1.0;
+int host_small_submit(rpeg_engine_t* e, HostLane& ln, uint64_t n, GET get, uint32_t flags, bool want_mass, bool want_util,
+                      hipStream_t s) {
+  ln.n = n; ln.launched = false; ln.idx.clear();
   if (n == 0) return 0;
   const size_t stride = ((size_t)n + 63) & ~size_t(63);
-  if (int rc = ensure_host_stage(e, stride, s)) return rc;
-  int16_t* in_vert = (int16_t*)e->hs_in;
-  uint8_t* in_head = e->hs_in + (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 * stride;
+  ln.stride = stride;
+  if (int rc = ensure_host_stage(e, ln, stride, s)) return rc;
+  int16_t* in_vert = (int16_t*)ln.in;
+  uint8_t* in_head = ln.in + (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 * stride;
   uint32_t* in_cls = (uint32_t*)(in_head + 4 * stride);
-  e->hs_idx.clear();
-  const double nan = __builtin_nan("");
   uint64_t n_new = 0;
   for (uint64_t i = 0; i < n; ++i) {
     PlanHead h;
     VPlan a[RPEG_MAX_V];
     get(i, h, a);
     const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;
-    if (nv == 0 || !plan_valid(e->P, h, a)) {
-      if (makespan) makespan[i] = nan;
-      if (peak) peak[i] = nan;
-      if (score) score[i] = nan;
-      if (mask) mask[i] = 0;
-      if (mass)
-        for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
-      if (util) util[i] = nan;
-      continue;
-    }
+    if (nv == 0 || !plan_valid(e->P, h, a)) continue;
     bool is_new = false;
     const int64_t off = class_offset(e, plan_signature(e->P, h.structure, h.split, h.tau0, h.tau1, a), &is_new);
     if (off < 0) return -5;
     n_new += is_new ? 1 : 0;
-    const size_t j = e->hs_idx.size();
-    e->hs_idx.push_back((uint32_t)i);
+    const size_t j = ln.idx.size();
+    ln.idx.push_back((uint32_t)i);
     for (int v = 0; v < nv; ++v) {
       int16_t* p = in_vert + (size_t)v * RPEG_FIELDS * stride + j;
       p[0 * stride] = (int16_t)a[v].dp; p[1 * stride] = (int16_t)a[v].pp; p[2 * stride] = (int16_t)a[v].tp; p[3 * stride] = (int16_t)a[v].mb;
@@ -2151,13 +2175,14 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
     in_head[2 * stride + j] = (uint8_t)h.tau0; in_head[3 * stride + j] = (uint8_t)h.tau1;
     in_cls[j] = (uint32_t)off;
   }
-  const size_t m = e->hs_idx.size();
+  const size_t m = ln.idx.size();
   e->stats[0] = 0; e->stats[1] = n_new; e->stats[2] = m; e->stats[3] = 0; e->stats[4] = 0; e->stats[5] = 1; e->stats[6] = 0;
   if (m == 0) return 0;
   if (e->max_nodes > (uint32_t)(WAVE * KP_MAX_NS) || kp_lds_bytes(e->max_nodes, e->max_slots) > 64 * 1024) return 1;
   if (int rc = ensure_pool(e, s)) return rc;
-  HIP_TRY(e, hipMemcpyAsync(e->ds_in, e->hs_in, HS_IN_BYTES * stride, hipMemcpyHostToDevice, s));
-  double* o_makespan = (double*)e->hs_out;
+  if (!ln.direct) HIP_TRY(e, hipMemcpyAsync(ln.dev, ln.in, HS_IN_BYTES * stride, hipMemcpyHostToDevice, s));
+  const uint8_t* d_in = ln.direct ? ln.in_dev : ln.dev;
+  double* o_makespan = (double*)ln.out_dev;
   double* o_peak = o_makespan + stride;
   double* o_score = o_peak + stride;
   double* o_mass = o_score + stride;
@@ -2165,8 +2190,8 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
   uint8_t* o_mask = (uint8_t*)(o_util + stride);
   EvalLaunch L;
   L.P = e->dP;
-  L.vert = (const int16_t*)e->ds_in;
-  L.head = e->ds_in + (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 * stride;
+  L.vert = (const int16_t*)d_in;
+  L.head = d_in + (size_t)RPEG_MAX_V * RPEG_FIELDS * 2 * stride;
   L.stride = stride;
   L.perm = nullptr;
   L.wave_cls = (const uint32_t*)(L.head + 4 * stride);
@@ -2174,9 +2199,25 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
   L.n_waves = m; L.ws_nodes = e->max_nodes; L.ws_slots = e->max_slots;
   L.cls_bytes = 0; L.rcap = 0; L.max_v = e->max_v; L.ovf = nullptr; L.need = nullptr;
   L.flags = flags; L.makespan = o_makespan; L.peak = o_peak; L.score = o_score; L.mask = o_mask;
-  L.mass = mass ? o_mass : nullptr;
-  L.util = util ? o_util : nullptr;
+  L.mass = want_mass ? o_mass : nullptr;
+  L.util = want_util ? o_util : nullptr;
   L.prof = nullptr;
+  if (e->prof_on) {   // phase clocks of this launch's wavefronts, read with rpeg_engine_profile
+    if (e->prof_waves < m) {
+      HIP_TRY(e, hipStreamSynchronize(s));
+      if (e->d_prof) hipFree(e->d_prof);
+      e->d_prof = nullptr;
+      HIP_TRY(e, hipMalloc(&e->d_prof, m * 64));
+    }
+    HIP_TRY(e, hipMemsetAsync(e->d_prof, 0, m * 64, s));
+    e->prof_waves = m;
+    L.prof = e->d_prof;
+  }
+  if (ln.direct) {
+    if (++ln.tag == 0) ++ln.tag;
+    L.done = (uint32_t*)(o_mask + stride);
+    L.done_tag = ln.tag;
+  }
   const size_t lds = kp_lds_bytes(e->max_nodes, e->max_slots);
   const unsigned grid = (unsigned)std::min<uint64_t>(m, (uint64_t)e->n_cu * 32);
   e->stats[3] = lds;
@@ -2184,14 +2225,60 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
   hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
   HIP_TRY(e, hipGetLastError());
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev1, s));
-  HIP_TRY(e, hipStreamSynchronize(s));
-  if (e->timing) {
-    float ms = 0.f;
-    HIP_TRY(e, hipEventElapsedTime(&ms, e->ev0, e->ev1));
-    e->last_ms = ms;
+  ln.launched = true;
+  ++e->lanes_busy;
+  return 0;
+}
+
+// Output arrays may be null; plans the validity gate refuses read NaN and a zero mask.
+int host_small_collect(rpeg_engine_t* e, HostLane& ln, double* makespan, double* peak, double* score, uint8_t* mask,
+                       double* mass, double* util, hipStream_t s) {
+  const size_t n = ln.n, m = ln.idx.size(), stride = ln.stride;
+  if (ln.launched) {
+    ln.launched = false;
+    --e->lanes_busy;
+    bool seen = false;
+    if (ln.direct) {
+      // the flags of all plans, in pinned memory: a plan's results are there once its flag is
+      const uint32_t* done = (const uint32_t*)(ln.out + (3 * 8 + (size_t)RPEG_MAX_V * 8 + 8) * stride + stride);
+      const auto t0 = std::chrono::steady_clock::now();
+      size_t j = 0;
+      for (uint64_t spins = 0;; ++spins) {
+        while (j < m && __atomic_load_n(&done[j], __ATOMIC_ACQUIRE) == ln.tag) ++j;
+        if (j == m) { seen = true; break; }
+        // a launch that does not come to an end is the stream's to report
+        if ((spins & 0xFFFFu) == 0xFFFFu && std::chrono::steady_clock::now() - t0 > std::chrono::seconds(2)) break;
+        __builtin_ia32_pause();
+      }
+    }
+    if (!seen) HIP_TRY(e, hipStreamSynchronize(s));
+    if (e->timing && !seen) {
+      float ms = 0.f;
+      HIP_TRY(e, hipEventElapsedTime(&ms, e->ev0, e->ev1));
+      e->last_ms = ms;
+    }
   }
+  if (m < n) {
+    const double nan = __builtin_nan("");
+    for (size_t i = 0; i < n; ++i) {
+      if (makespan) makespan[i] = nan;
+      if (peak) peak[i] = nan;
+      if (score) score[i] = nan;
+      if (mask) mask[i] = 0;
+      if (mass)
+        for (int x = 0; x < RPEG_MAX_V; ++x) mass[i * RPEG_MAX_V + x] = nan;
+      if (util) util[i] = nan;
+    }
+  }
+  if (m == 0) return 0;
+  const double* o_makespan = (const double*)ln.out;
+  const double* o_peak = o_makespan + stride;
+  const double* o_score = o_peak + stride;
+  const double* o_mass = o_score + stride;
+  const double* o_util = o_mass + (size_t)RPEG_MAX_V * stride;
+  const uint8_t* o_mask = (const uint8_t*)(o_util + stride);
   for (size_t j = 0; j < m; ++j) {
-    const uint32_t i = e->hs_idx[j];
+    const uint32_t i = ln.idx[j];
     if (makespan) makespan[i] = o_makespan[j];
     if (peak) peak[i] = o_peak[j];
     if (score) score[i] = o_score[j];
@@ -2201,6 +2288,15 @@ int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, doubl
     if (util) util[i] = o_util[j];
   }
   return 0;
+}
+
+template <class GET>
+int eval_host_small(rpeg_engine_t* e, uint64_t n, GET get, uint32_t flags, double* makespan, double* peak, double* score,
+                    uint8_t* mask, double* mass, hipStream_t s, double* util = nullptr) {
+  e->last_ms = -1.0;
+  const int rc = host_small_submit(e, e->lane0, n, get, flags, mass != nullptr, util != nullptr, s);
+  if (rc != 0) return rc;
+  return host_small_collect(e, e->lane0, makespan, peak, score, mask, mass, util, s);
 }
 
 }  // namespace
@@ -2295,8 +2391,24 @@ struct GpuSaBackend : SaBackend {
   double eval_s = 0.0;
   long n_launch = 0, n_plans = 0;
   int rc_alloc = 0;
+  // lanes of submit() / collect(): staging buffers and a stream each, so that the evaluation of one group of chains
+  // runs while the host merges and proposes for another
+  struct Lane {
+    HostLane st;
+    hipStream_t s = nullptr;
+    bool deferred = false;     // the batch is not one for k_plan: evaluated in collect()
+    int n = 0;
+    const SaPlan* plans = nullptr;
+    const uint8_t* variant = nullptr;
+  };
+  std::vector<Lane> lane;
 
-  GpuSaBackend(rpeg_engine_t* eng, hipStream_t st, int capacity) : e(eng), s(st), cap(capacity) {
+  GpuSaBackend(rpeg_engine_t* eng, hipStream_t st, int capacity, int n_lanes = 1) : e(eng), s(st), cap(capacity) {
+    lane.resize((size_t)std::max(1, n_lanes));
+    for (Lane& l : lane) {
+      l.st.direct = true;
+      if (hipStreamCreateWithFlags(&l.s, hipStreamNonBlocking) != hipSuccess) { rc_alloc = -2; e->err = "hipStreamCreate failed"; l.s = nullptr; }
+    }
     const size_t V = RPEG_MAX_V * RPEG_FIELDS;
     bool ok = hipHostMalloc(&h_vert, V * cap * 2) == hipSuccess && hipMalloc(&d_vert, V * cap * 2) == hipSuccess &&
               hipHostMalloc(&h_head, 4 * (size_t)cap) == hipSuccess && hipMalloc(&d_head, 4 * (size_t)cap) == hipSuccess &&
@@ -2310,6 +2422,11 @@ struct GpuSaBackend : SaBackend {
   }
   ~GpuSaBackend() override {
     hipStreamSynchronize(s);
+    for (Lane& l : lane) {
+      if (l.st.launched) { --e->lanes_busy; l.st.launched = false; }
+      if (l.s) { hipStreamSynchronize(l.s); hipStreamDestroy(l.s); }
+      l.st.release();
+    }
     if (h_vert) hipHostFree(h_vert);
     if (d_vert) hipFree(d_vert);
     if (h_head) hipHostFree(h_head);
@@ -2328,6 +2445,60 @@ struct GpuSaBackend : SaBackend {
   }
 
   int evaluate(int n, const SaPlan* plans, const uint8_t* variant, SaEval* out) override { return evaluate(n, plans, variant, out, false); }
+
+  int lanes() const override { return (int)lane.size(); }
+
+  int submit(int li, int n, const SaPlan* plans, const uint8_t* variant) override {
+    Lane& l = lane[(size_t)li];
+    l.n = n; l.plans = plans; l.variant = variant; l.deferred = false;
+    if (n > cap) { e->err = "annealing batch exceeds its buffers"; return -1; }
+    const auto t0 = std::chrono::steady_clock::now();
+    auto get = [&](uint64_t i, PlanHead& h, VPlan (&a)[RPEG_MAX_V]) {
+      const uint8_t* hd = head_of[variant[i]];
+      h.structure = hd[0]; h.split = hd[1]; h.tau0 = hd[2]; h.tau1 = hd[3];
+      const int nv = e->P.st[hd[0]].n_vertex;
+      for (int v = 0; v < nv; ++v) {
+        const int16_t* f = plans[i].f[v];
+        a[v].dp = f[0]; a[v].pp = f[1]; a[v].tp = f[2]; a[v].mb = f[3];
+        a[v].o[0] = f[4]; a[v].o[1] = f[5]; a[v].o[2] = f[6];
+        a[v].e[0] = f[7]; a[v].e[1] = f[8]; a[v].e[2] = f[9];
+      }
+    };
+    const int rc = host_small_submit(e, l.st, (uint64_t)n, get, 0u, true, false, l.s);
+    eval_s += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    if (rc == 1) { l.deferred = true; return 0; }
+    return rc;
+  }
+
+  int collect(int li, SaEval* out) override {
+    Lane& l = lane[(size_t)li];
+    if (l.deferred) { l.deferred = false; return evaluate(l.n, l.plans, l.variant, out, false); }
+    if (l.n == 0) return 0;
+    const auto t0 = std::chrono::steady_clock::now();
+    if (int rc = host_small_collect(e, l.st, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, l.s)) return rc;
+    const size_t n = l.st.n, m = l.st.idx.size(), stride = l.st.stride;
+    if (m < n) {
+      const double nan = __builtin_nan("");
+      for (size_t i = 0; i < n; ++i) {
+        out[i].score = nan;
+        out[i].mask = 0;
+        for (int x = 0; x < RPEG_MAX_V; ++x) out[i].mass[x] = nan;
+      }
+    }
+    const double* o_score = (const double*)l.st.out + 2 * stride;
+    const double* o_mass = o_score + stride;
+    const uint8_t* o_mask = (const uint8_t*)(o_mass + (size_t)RPEG_MAX_V * stride + stride);
+    for (size_t j = 0; j < m; ++j) {
+      SaEval& o = out[l.st.idx[j]];
+      o.score = o_score[j];
+      o.mask = o_mask[j];
+      for (int x = 0; x < RPEG_MAX_V; ++x) o.mass[x] = o_mass[j * RPEG_MAX_V + x];
+    }
+    eval_s += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    ++n_launch;
+    n_plans += l.n;
+    return 0;
+  }
 
   // with_util: Trace.utilization() of every plan from the same launch (out[i].util); 1 when this batch cannot
   // take that path (the caller then asks per plan)
@@ -2437,7 +2608,8 @@ int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* ba
   SaSettings st;
   sa_settings_from(*prm, &st);
   const int cap = prm->n_chains * std::max(prm->K_x, prm->restart_attempts);
-  GpuSaBackend be(e, (hipStream_t)stream, cap);
+  // chains in groups of at least 8, at most `sa_lanes` groups
+  GpuSaBackend be(e, (hipStream_t)stream, cap, std::max(1, std::min(e->sa_lanes, prm->n_chains / 8)));
   if (be.rc_alloc) return be.rc_alloc;
   for (int k = 0; k < prm->n_variants; ++k) {
     be.head_of[k][0] = (uint8_t)prm->structure; be.head_of[k][1] = (uint8_t)prm->split;

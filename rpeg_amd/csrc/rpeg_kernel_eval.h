@@ -68,6 +68,9 @@ struct EvalLaunch {              // uniform launch parameters
   const double* aux_pen = nullptr;     // factor of the soft OOM penalty, 1.0 where the plan fits
   const uint8_t* aux_mask = nullptr;   // RPEG_MASK_VALID | _STALE_OK | _MEM_OK
   uint64_t dur_stride = 0;
+  uint32_t* done = nullptr;      // k_plan only: done[w] = done_tag once the outputs of wave task w are written (a release
+  uint32_t done_tag = 0;         // store at system scope, for a host that polls pinned memory instead of waiting for the
+                                 // end of the launch); or null
   uint32_t* limit = nullptr;     // plans whose ready set outgrew what this kernel holds for good (no launch with a
                                  // longer list follows): limit[0] counts them, then (plan, class blob offset) pairs.
                                  // The launch that ends the call redoes them with a ready list as long as the

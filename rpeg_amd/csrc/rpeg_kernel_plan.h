@@ -36,8 +36,9 @@ constexpr int KP_PLAN_I16 = 80;                 // plan fields in LDS (60 used; 
 // per node (plus one neutral element each), tie-break class per node; busy-time table and dispatch order.
 __host__ __device__ inline size_t kp_lds_bytes(uint32_t nodes, uint32_t slots) {
   const size_t base = ((size_t)KP_PLAN_I16 * 2 + (size_t)RPEG_MAX_V * 4 * 8 + 8ull * slots + 16ull * (nodes + 1) + nodes + 7) & ~size_t(7);
-  // then, for the utilisation: busy time by allocation set (64 doubles) and the dispatch order (2 bytes per node)
-  return (base + 64 * 8 + 2ull * nodes + 15) & ~size_t(15);
+  // then, for the utilisation: busy time by allocation set (64 doubles) and the dispatch order (2 bytes per node);
+  // for the critical chain: the predecessor it follows at every node (2 bytes per node)
+  return (base + 64 * 8 + 2ull * nodes + 2ull * nodes + 15) & ~size_t(15);
 }
 
 #if defined(__HIPCC__)
@@ -217,6 +218,9 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
   double makespan = 0.0;
   int done = 0;
   bool ok = true;
+  // the trace (start and finish of every node) stays in registers while the loop runs where there is room for it
+  constexpr bool trace_regs = keep_trace && NS <= 4;
+  double t_fin[trace_regs ? NS : 1], t_start[trace_regs ? NS : 1];
   uint32_t pops = 0, slow_decisions = 0;
   const uint32_t guard_max = (uint32_t)n * (uint32_t)n + 64u;   // (at most 384 nodes)
   uint32_t guard = 0;
@@ -391,7 +395,15 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
       dvc[s] = hit && fin > dvc[s] ? fin : dvc[s];
       if (mine && s == ws) key[s] = inf;
     }
-    if (keep_trace && mine) {
+    if (trace_regs) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const bool here = mine && s == ws;
+        t_fin[trace_regs ? s : 0] = here ? fin : t_fin[trace_regs ? s : 0];
+        t_start[trace_regs ? s : 0] = here ? gk : t_start[trace_regs ? s : 0];
+      }
+      if (l_order && mine) l_order[done - 1] = (uint16_t)(ws * 64 + wl);
+    } else if (keep_trace && mine) {
       l_rank[ws * 64 + wl] = fin;
       l_start[ws * 64 + wl] = gk;
       if (l_order) l_order[done - 1] = (uint16_t)(ws * 64 + wl);
@@ -417,10 +429,60 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
     }
   }
   if (done != n) ok = false;
+  if (trace_regs && ok) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (s * 64 + lane < n) {
+        l_rank[s * 64 + lane] = t_fin[trace_regs ? s : 0];
+        l_start[s * 64 + lane] = t_start[trace_regs ? s : 0];
+      }
+  }
   *out_makespan = makespan;
   *out_pops = ((long)slow_decisions << 20) | (long)pops;
   if (ctr > KP_TIE_MASK) return 2;   // the push counter outgrew its field of the packed order: a limit of this kernel
   return ok ? 0 : 1;
+}
+
+// Critical-chain mass per template vertex (critical_mass of rpeg_class.h; moves.py:590-642) for one plan per
+// wavefront.  What the walk needs at a node -- the predecessor it goes on to (the first one, in edge order, of largest
+// finish time) and the vertex the node counts for -- is found for all nodes at once, a node per lane, and left in
+// LDS; the walk itself, one hop after the other from the first node of largest finish time, then reads LDS only.
+// Lane x < RPEG_MAX_V returns the mass of vertex x, summed in the order of the walk.
+__device__ inline double kp_critical_mass(const ClassView& cv, const int n, const int lane, const double* l_fin,
+                                          const double* l_start, uint16_t* l_next, uint8_t* l_vx) {
+  double bf = -1.0;
+  uint32_t bi = 0xFFFFFFFFu;
+  for (int v = lane; v < n; v += KE_WAVE) {
+    const double f = l_fin[v];
+    if (f > bf) { bf = f; bi = (uint32_t)v; }
+    const int pb = cv.pbeg[v], pe = cv.pbeg[v + 1];
+    uint32_t nx = 0xFFFFu;
+    if (pb != pe) {
+      nx = cv.pred[pb];
+      double b = l_fin[nx];
+      for (int j = pb + 1; j < pe; ++j) {
+        const uint32_t q = cv.pred[j];
+        const double fq = l_fin[q];
+        if (fq > b) { b = fq; nx = q; }
+      }
+    }
+    l_next[v] = (uint16_t)nx;
+    const SlotDesc sd = cv.slot[cv.node[v].slot];
+    l_vx[v] = sd.type <= SLOT_OP_SUB ? sd.a : (uint8_t)0xFF;
+  }
+  __syncthreads();
+  const double top = kp_wave_reduce(bf, KpMax());
+  int cur = (int)kp_wave_umin(bf == top ? bi : 0xFFFFFFFFu);
+  double m = 0.0;
+  for (int hops = 0; hops <= n; ++hops) {   // a chain visits a node at most once
+    const int vx = l_vx[cur];
+    const double d = l_fin[cur] - l_start[cur];
+    const int nx = __builtin_amdgcn_readfirstlane((int)l_next[cur]);
+    if (lane == vx) m += d;
+    if (nx == 0xFFFF) break;
+    cur = nx;
+  }
+  return m;
 }
 
 // Pair relations and vertex sets of one plan by POSITION in the order of first appearance (bit 8i+j of a
@@ -651,6 +713,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   uint8_t* l_pt = (uint8_t*)(l_start + (L.ws_nodes + 1));
   double* l_tab = (double*)(((uintptr_t)(l_pt + L.ws_nodes) + 7) & ~(uintptr_t)7);
   uint16_t* l_ord = (uint16_t*)(l_tab + 64);
+  uint16_t* l_next = l_ord + L.ws_nodes;
 
   __syncthreads();   // the previous plan of this wavefront is done with LDS
   KE_STAMP(0);
@@ -796,15 +859,10 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     out_makespan = makespan;
     out_score = score;
   }
-  double m[RPEG_MAX_V];
+  double m = __builtin_nan("");   // lane x < RPEG_MAX_V: mass of vertex x
   if (L.mass) {
     __syncthreads();
-    if (err) {
-#pragma unroll
-      for (int x = 0; x < RPEG_MAX_V; ++x) m[x] = __builtin_nan("");
-    } else {
-      critical_mass(cv, [&](int i) { return l_rank[i]; }, [&](int i) { return l_start[i]; }, m);
-    }
+    if (!err) m = kp_critical_mass(cv, n, lane, l_rank, l_start, l_next, l_pt);   // (the tie-break classes in l_pt are done with)
   }
   double util = 0.0;
   if (L.util) {
@@ -817,11 +875,8 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     if (L.peak && !L.dur) L.peak[pi] = peak;   // (with a prologue launch the peak is that launch's output)
     if (L.score) L.score[pi] = out_score;
     if (L.mask) L.mask[pi] = mask;
-    if (L.mass) {
-#pragma unroll
-      for (int x = 0; x < RPEG_MAX_V; ++x) L.mass[pi * RPEG_MAX_V + x] = m[x];
-    }
   }
+  if (L.mass && lane < RPEG_MAX_V) L.mass[pi * RPEG_MAX_V + lane] = m;
   KE_STAMP(6);
 }
 

@@ -87,6 +87,23 @@ struct SaBackend {
   }
   // Trace.utilization() of one plan (trace.py:53-101); backends without traces refuse
   virtual int utilization(const SaPlan& plan, uint8_t variant, double* out) { (void)plan; (void)variant; (void)out; return -1; }
+  // The same evaluation in two halves, for a caller that has other work while it runs: submit() starts the evaluation of
+  // `n` plans in lane `lane` (0 .. lanes() - 1; the arrays stay the caller's and must live until collect), collect()
+  // waits for it and fills `out`.  One evaluation per lane at a time; evaluate() may be called in between.  The default
+  // evaluates in collect().
+  virtual int lanes() const { return host_lanes; }
+  virtual int submit(int lane, int n, const SaPlan* plans, const uint8_t* variant) {
+    if ((int)pend.size() <= lane) pend.resize((size_t)lane + 1);
+    pend[(size_t)lane] = Pending{n, plans, variant};
+    return 0;
+  }
+  virtual int collect(int lane, SaEval* out) {
+    const Pending& q = pend[(size_t)lane];
+    return q.n > 0 ? evaluate(q.n, q.plans, q.variant, out) : 0;
+  }
+  int host_lanes = 1;
+  struct Pending { int n; const SaPlan* plans; const uint8_t* variant; };
+  std::vector<Pending> pend;
 };
 
 struct SaSettings {
@@ -484,70 +501,93 @@ struct SaRun {
       }
     }
 
-    std::vector<SaPlan> cand((size_t)p.n_chains * p.K_x);
-    std::vector<uint8_t> var((size_t)p.n_chains * p.K_x);
-    std::vector<SaEval> ev((size_t)p.n_chains * p.K_x);
-    std::vector<int> first(p.n_chains + 1), kind(p.n_chains);
-    std::vector<SaRng> rngs;
-    for (int step = 0; step < p.n_steps; ++step) {
-      // ---- proposals of every live chain
-      rngs.clear();
+    // The chains are independent of each other: they are dealt to `G` groups that take their steps in turn, so that
+    // the host proposes for one group and merges its results while the evaluations of the others run.  Every chain
+    // draws from its own stream keyed by (seed, chain, step), so its trajectory does not depend on the grouping.
+    const int G = std::max(1, std::min(be.lanes(), p.n_chains));
+    struct Group {
+      std::vector<int> who;              // chains of the group
+      std::vector<SaPlan> cand;
+      std::vector<uint8_t> var;
+      std::vector<SaEval> ev;
+      std::vector<int> first, kind;      // by position in `who`
+      std::vector<SaRng> rngs;
       int total = 0;
-      for (int c = 0; c < p.n_chains; ++c) {
+    };
+    std::vector<Group> groups(G);
+    for (int c = 0; c < p.n_chains; ++c) groups[c % G].who.push_back(c);
+    for (Group& g : groups) {
+      g.cand.resize(g.who.size() * (size_t)p.K_x);
+      g.var.resize(g.cand.size());
+      g.ev.resize(g.cand.size());
+      g.first.resize(g.who.size() + 1);
+      g.kind.resize(g.who.size());
+    }
+    // ---- proposals of every live chain of a group, and the start of their evaluation
+    auto propose = [&](int gi, int step) -> int {
+      Group& g = groups[gi];
+      g.rngs.clear();
+      int total = 0;
+      for (size_t k = 0; k < g.who.size(); ++k) {
+        const int c = g.who[k];
         SaChain& ch = chains[c];
-        rngs.emplace_back(p.seed, (uint64_t)c, (uint64_t)(step + 1), 0);
-        first[c] = total;
-        kind[c] = -1;
+        g.rngs.emplace_back(p.seed, (uint64_t)c, (uint64_t)(step + 1), 0);
+        g.first[k] = total;
+        g.kind[k] = -1;
         if (ch.dead) continue;
-        SaRng& rng = rngs.back();
+        SaRng& rng = g.rngs.back();
         const double frac = std::min(1.0, ch.T / p.T_init);
         if (rng.random() < p.alpha_pair * frac) {
-          kind[c] = 1;
-          if (sa_move_pair(rng, cx, ch.cur.plan, &cand[total])) total += 1;
-          else { ch.T = std::max(p.T_min, ch.T * p.T_cool); kind[c] = 2; }   // optimizer.py:737-740
+          g.kind[k] = 1;
+          if (sa_move_pair(rng, cx, ch.cur.plan, &g.cand[total])) total += 1;
+          else { ch.T = std::max(p.T_min, ch.T * p.T_cool); g.kind[k] = 2; }   // optimizer.py:737-740
         } else {
-          kind[c] = 0;
-          total += sa_move_gen(rng, cx, ch.cur.plan, ch.cur.ev.mass, p.K_x, p.T_max, ch.T, p.T_init, &cand[total]);
+          g.kind[k] = 0;
+          total += sa_move_gen(rng, cx, ch.cur.plan, ch.cur.ev.mass, p.K_x, p.T_max, ch.T, p.T_init, &g.cand[total]);
         }
-        for (int j = first[c]; j < total; ++j) var[j] = variant(c);
+        for (int j = g.first[k]; j < total; ++j) g.var[j] = variant(c);
       }
-      first[p.n_chains] = total;
-      if (total > 0)
-        if (int rc = be.evaluate(total, cand.data(), var.data(), ev.data())) return rc;
-      hard_oom(ev.data(), total);
-
-      // ---- best of K, one Metropolis-Hastings step, stagnation
+      g.first[g.who.size()] = total;
+      g.total = total;
+      return be.submit(gi, total, g.cand.data(), g.var.data());
+    };
+    // ---- best of K, one Metropolis-Hastings step, stagnation
+    auto merge = [&](int gi, int step) -> int {
+      Group& g = groups[gi];
+      if (int rc = be.collect(gi, g.ev.data())) return rc;
+      hard_oom(g.ev.data(), g.total);
       std::vector<int> random_who;
-      for (int c = 0; c < p.n_chains; ++c) {
+      for (size_t k = 0; k < g.who.size(); ++k) {
+        const int c = g.who[k];
         SaChain& ch = chains[c];
-        if (ch.dead || kind[c] < 0) continue;
+        if (ch.dead || g.kind[k] < 0) continue;
         uint8_t& lg = log[(size_t)c * p.n_steps + step];
-        if (kind[c] == 2) { lg = 1; continue; }
-        const int nc = first[c + 1] - first[c];
-        lg = (uint8_t)(kind[c] | nc << 1);
+        if (g.kind[k] == 2) { lg = 1; continue; }
+        const int nc = g.first[k + 1] - g.first[k];
+        lg = (uint8_t)(g.kind[k] | nc << 1);
         bool restart = false;
         if (nc == 0) {
           restart = true;   // "chain stuck" (optimizer.py:767-769)
         } else {
           int bi = -1;
           double bs = -INFINITY;
-          for (int j = first[c]; j < first[c + 1]; ++j) {
+          for (int j = g.first[k]; j < g.first[k + 1]; ++j) {
             ++ch.n_eval;
-            SaEntry e; e.plan = cand[j]; e.ev = ev[j];
-            const bool stale_ok = (ev[j].mask & RPEG_MASK_STALE_OK) != 0;
-            double s = p.gate_candidates ? gated(ev[j]) : ev[j].score;
-            if (ev[j].mask & RPEG_MASK_ERROR) s = -INFINITY;
-            const bool feas = (ev[j].mask & RPEG_MASK_MEM_OK) && !(ev[j].mask & RPEG_MASK_ERROR) &&
+            SaEntry e; e.plan = g.cand[j]; e.ev = g.ev[j];
+            const bool stale_ok = (g.ev[j].mask & RPEG_MASK_STALE_OK) != 0;
+            double sc = p.gate_candidates ? gated(g.ev[j]) : g.ev[j].score;
+            if (g.ev[j].mask & RPEG_MASK_ERROR) sc = -INFINITY;
+            const bool feas = (g.ev[j].mask & RPEG_MASK_MEM_OK) && !(g.ev[j].mask & RPEG_MASK_ERROR) &&
                               (stale_ok || !p.gate_candidates);
-            if (!(ev[j].mask & RPEG_MASK_ERROR)) note(ch, e, s, step, feas);
-            if (s > bs) { bs = s; bi = j; }
+            if (!(g.ev[j].mask & RPEG_MASK_ERROR)) note(ch, e, sc, step, feas);
+            if (sc > bs) { bs = sc; bi = j; }
           }
           if (bi >= 0) {
             const double delta = (bs - ch.score) / (std::fabs(ch.score) + 1e-12);
             if (std::fabs(delta) >= 1e-6) {
               const double prob = delta >= 0.0 ? 1.0 : exp_libm(delta / ch.T);
-              const bool acc = rngs[c].random() < prob;
-              if (acc) { ch.cur.plan = cand[bi]; ch.cur.ev = ev[bi]; ch.score = bs; ch.rej = 0; }
+              const bool acc = g.rngs[k].random() < prob;
+              if (acc) { ch.cur.plan = g.cand[bi]; ch.cur.ev = g.ev[bi]; ch.score = bs; ch.rej = 0; }
               else ++ch.rej;
               lg |= (uint8_t)((acc ? 2 : 1) << 4);
             }
@@ -572,7 +612,17 @@ struct SaRun {
           else { ch.T = p.T_warm; ch.rej = 0; }   // no valid restart: go on from the current plan
         }
       }
-    }
+      return 0;
+    };
+    if (p.n_steps > 0)
+      for (int gi = 0; gi < G; ++gi)
+        if (int rc = propose(gi, 0)) return rc;
+    for (int step = 0; step < p.n_steps; ++step)
+      for (int gi = 0; gi < G; ++gi) {
+        if (int rc = merge(gi, step)) return rc;
+        if (step + 1 < p.n_steps)
+          if (int rc = propose(gi, step + 1)) return rc;
+      }
     return 0;
   }
 };

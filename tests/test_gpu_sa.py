@@ -96,6 +96,34 @@ def test_chains_equal_host_replay(c, n_chains, n_steps, kw):
     assert got.n_launch >= n_steps
 
 
+def test_groups_of_chains_overlap_without_changing_the_run():
+    """rpeg_engine_set_sa_groups: 1, 2 and 3 groups (streams, staging buffers, polled completion flags of their own)
+    give the same decisions, plans and scores bit for bit, and as many launches as groups per step."""
+    p = configs.config(5).problem
+    eng = engine(5)
+    opt = OptimizerConfig(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)
+    rpeg0 = p.template(0, ())
+    table, _ = build_candidate_directory(rpeg0, p.suite, p.device_space, p.workload, eng)
+    arrays = directory_arrays(rpeg0, table)
+    runs = {}
+    try:
+        for groups in (1, 2, 3, 8):
+            eng.set_sa_groups(groups)
+            runs[groups] = optimize_chains(p, opt, 32, 150, _variants(p), seed=7, engine=eng, directory=arrays)
+    finally:
+        eng.set_sa_groups(3)
+    one = runs[1]
+    assert ((one.log >> 4) & 3 == 2).sum() > 0
+    for groups, got in runs.items():
+        assert np.array_equal(got.log, one.log), groups
+        assert np.array_equal(got.cur_plan, one.cur_plan) and same_bits(got.cur_score, one.cur_score), groups
+        assert np.array_equal(got.best_plan, one.best_plan) and same_bits(got.best_score, one.best_score), groups
+        assert np.array_equal(got.restarts, one.restarts) and np.array_equal(got.n_eval, one.n_eval), groups
+        assert got.n_launch >= min(groups, 4) * 150, groups     # (at least 8 chains to a group: 32 chains make 4)
+    with pytest.raises(Exception):
+        eng.set_sa_groups(0)
+
+
 def test_base_plan_start_and_gate():
     p = configs.config(1).problem
     eng = engine(1)

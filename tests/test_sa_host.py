@@ -102,6 +102,26 @@ def _log_byte(entry):
     return b
 
 
+def test_groups_of_chains_that_step_in_turn_change_nothing():
+    """SaRun deals the chains to groups whose steps interleave (so that a GPU evaluates one group while the host works
+    on another): every chain draws from its own (seed, chain, step) streams, so any grouping gives the same run."""
+    p = configs.config(1).problem
+    opt = OptimizerConfig(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=4)
+    rpeg0 = p.template(0, ())
+    _, _, arrays = _directory(p, rpeg0)
+    n_tau = len(p.structures[0].tau_models)
+    variants = [(0,) * n_tau, (1,) + (0,) * (n_tau - 1)]
+    params = sa_params(opt, 10, 60, variants, 0, 1 if p.workload.gen_quantiles else 0, 42)
+    one = CpuPort(p).sa_run(params, arrays, threads=4)
+    assert ((one["log"] >> 6) & 1).sum() > 0, "no restart in the run"
+    for groups in (2, 3, 7, 10, 16):
+        got = CpuPort(p).sa_run(params, arrays, threads=4, groups=groups)
+        for k in ("log", "cur_plan", "best_plan", "best_step", "best_feasible", "restarts", "n_eval", "dead"):
+            assert np.array_equal(got[k], one[k]), (groups, k)
+        for k in ("cur_score", "best_score"):
+            assert np.array_equal(got[k].view(np.uint64), one[k].view(np.uint64)), (groups, k)
+
+
 @pytest.mark.parametrize("c,n_chains,n_steps,kw", [
     (1, 6, 40, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=4)),
     (5, 4, 12, dict(T_init=0.05, T_min=0.05, T_warm=0.10, stag_window=10)),
