@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the batched plan evaluator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu] [--no-sa]
     python bench.py --config 5 [--chains 64] [--sa-steps 2000]      (batched simulated annealing)
 
 A step is one pass of the hot path (signature kernel, class grouping, evaluation kernel) over the
@@ -28,11 +28,12 @@ ALG_BYTES = {1: 149, 2: 109, 3: 149, 4: 89, 5: 149}
 # type) and averaged over the seeded set of the configuration (config 5: over 4,096 seeded plans);
 # tests/test_cpu_port.py holds these constants to a fresh count
 ALG_FLOPS = {1: 3697.0, 2: 2165.3, 3: 6502.9, 4: 1245.8, 5: 4155.6}
-# Counter figures of one step, taken from the rocprofv3 --pmc summaries under profiles/ and valid only for the
-# kernel layout they were measured on (`layout`: wave tasks, LDS bytes, plans per wavefront with LDS state,
-# single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats; the task counts to 25 %, k_quad's to 35 %): HBM bytes of the evaluation kernels (FETCH_SIZE / WRITE_SIZE scaled
-# by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS + VMEM_RD + VMEM_WR of the
-# evaluation kernels / plans).  A run whose layout differs prints null instead of a stale number.
+# Counter figures of one step.  A run cannot read hardware counters of itself: these come from the rocprofv3 --pmc
+# summaries under profiles/ and are printed only when the run's kernel layout (`layout`: wave tasks, LDS bytes, plans
+# per wavefront with LDS state, single-plan tasks, four-lanes-per-plan tasks of rpeg_engine_stats) is the profiled
+# one to within 5 % in every task count; any other run prints null.  HBM bytes of the evaluation kernels
+# (FETCH_SIZE / WRITE_SIZE scaled by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS +
+# VMEM_RD + VMEM_WR of the evaluation kernels / plans).
 MEASURED = {
     2: dict(layout=(6880, 17648, 0, 5497, 397), traffic=252.5e6, instructions_per_plan=3849.5),
     3: dict(layout=(26026, 29984, 0, 21741, 0), traffic=5775.0e6, instructions_per_plan=10402.0),
@@ -117,9 +118,10 @@ def parity_block(out, ref):
         max_rel_err=float(max(rel.max() if rel.size else 0.0, rel_m.max() if rel_m.size else 0.0)))
 
 
-def bench_sa(args):
-    """Config 5: 64 chains x 2000 steps of batched simulated annealing.  Prints one JSON line whose value
-    is the wall-clock of the whole run (directory build excluded and reported beside it)."""
+def sa_measure(args, deadlines=True):
+    """Config 5: `args.chains` chains x `args.sa_steps` steps of batched simulated annealing on the GPU evaluator, the
+    first steps of the same chains over the host build of the evaluator, and (deadlines=True) the serial optimize()
+    loop under wall-clock deadlines.  Returns the fields of the config-5 line."""
     import zlib
     import numpy as np
     import torch
@@ -140,7 +142,7 @@ def bench_sa(args):
     arrays = directory_arrays(rpeg0, table)
     dir_s = time.perf_counter() - t0
     runs = []
-    for rep in range(max(1, args.steps if args.steps < 20 else 2)):   # first run lowers every class it meets
+    for rep in range(3):   # the first run lowers every class it meets
         res = optimize_chains(p, opt, args.chains, args.sa_steps, variants, seed=42, engine=eng, directory=arrays)
         runs.append(res)
     cold, warm = runs[0], runs[-1]
@@ -158,42 +160,44 @@ def bench_sa(args):
         "best_plan_crc": zlib.crc32(cold.best_plan[c].tobytes()),
         "plans_evaluated": int(cold.n_plans), "launches": int(cold.n_launch),
         "evals_per_s": cold.n_plans / cold.wall_s, "eval_share_of_wall": cold.eval_s / cold.wall_s,
-        "warm_wall_s": warm.wall_s, "warm_time_to_best_s": float(warm.best_time[c]),
+        "wall_s_of_runs": [r.wall_s for r in runs], "warm_wall_s": warm.wall_s,
+        "warm_time_to_best_s": float(warm.best_time[c]),
         "directory_s": dir_s, "directory_sizes": [int(a.shape[0]) for a in arrays],
         "accept_rate": float((((cold.log >> 4) & 3) == 2).sum() / max(1, (((cold.log >> 4) & 3) != 0).sum())),
         "restarts": int(cold.restarts.sum()), "dead_chains": int(cold.dead.sum()),
         "feasible_chains": int(cold.best_feasible.sum()),
     }
-    # optimize() as the reference runs it (one chain at a time, cache, restarts), under a wall-clock deadline as
-    # `pipeline.py --time` sets it: the best score reached within t seconds, on the GPU evaluator and -- the same
-    # loop, the same generator -- on the host build of the evaluator
-    from rpeg_amd.engine import abi
-    from rpeg_amd.search import candidates
-    seeds = candidates.generate(p, 64, cfg.tau_choices, seed=42, tag=5)
-    verdict = eng.eval(seeds)["mask"]
-    start = next(i for i in range(seeds.n) if verdict[i] & abi.MASK_VALID and verdict[i] & abi.MASK_MEM_OK)
-    row = np.ascontiguousarray(seeds.vert[:, start])
     split = 1 if p.workload.gen_quantiles else 0
+    if deadlines:
+        # optimize() as the reference runs it (one chain at a time, cache, restarts), under a wall-clock deadline as
+        # `pipeline.py --time` sets it: the best score reached within t seconds, on the GPU evaluator and -- the same
+        # loop, the same generator -- on the host build of the evaluator
+        from rpeg_amd.engine import abi
+        from rpeg_amd.search import candidates
+        seeds = candidates.generate(p, 64, cfg.tau_choices, seed=42, tag=5)
+        verdict = eng.eval(seeds)["mask"]
+        start = next(i for i in range(seeds.n) if verdict[i] & abi.MASK_VALID and verdict[i] & abi.MASK_MEM_OK)
+        row = np.ascontiguousarray(seeds.vert[:, start])
 
-    def timed(seconds):
-        prm = sa_params(opt, 1, 1, [(0, 0)], 0, split, 42)
-        prm.timed, prm.deadline_s = 1, seconds
-        return prm
-    line["within_deadline"] = []
-    for seconds in (0.1, 0.3, 1.0):
-        r = eng.sa_optimize(timed(seconds), arrays, row, 10 ** 9, 10 ** 9, stream_key=(5, 0, 0))
-        line["within_deadline"].append(dict(seconds=seconds, best_score=r["best_score"], best_feasible=r["best_feasible"],
-                                            evaluations=r["E"], timed_out=r["timed_out"]))
+        def timed(seconds):
+            prm = sa_params(opt, 1, 1, [(0, 0)], 0, split, 42)
+            prm.timed, prm.deadline_s = 1, seconds
+            return prm
+        line["within_deadline"] = []
+        for seconds in (0.1, 0.3, 1.0):
+            r = eng.sa_optimize(timed(seconds), arrays, row, 10 ** 9, 10 ** 9, stream_key=(5, 0, 0))
+            line["within_deadline"].append(dict(seconds=seconds, best_score=r["best_score"], best_feasible=r["best_feasible"],
+                                                evaluations=r["E"], timed_out=r["timed_out"]))
     if not args.no_cpu:
         # the same host logic over the CPU build of the evaluator, all host cores, on a bounded number of steps
         from oracle.cpu_port import CpuPort
-        for rec in line["within_deadline"]:
-            r = CpuPort(p).sa_optimize(timed(rec["seconds"]), arrays, row, 10 ** 9, 10 ** 9, stream_key=(5, 0, 0),
-                                       threads=min(16, os.cpu_count() or 1))
-            rec.update(cpu_port_best_score=r["best_score"], cpu_port_evaluations=r["E"])
         threads = min(16, os.cpu_count() or 1)
+        if deadlines:
+            for rec in line["within_deadline"]:
+                r = CpuPort(p).sa_optimize(timed(rec["seconds"]), arrays, row, 10 ** 9, 10 ** 9, stream_key=(5, 0, 0),
+                                           threads=threads)
+                rec.update(cpu_port_best_score=r["best_score"], cpu_port_evaluations=r["E"])
         steps = max(1, min(args.sa_steps, 40))
-        split = 1 if p.workload.gen_quantiles else 0
         t0 = time.perf_counter()
         ref = CpuPort(p).sa_run(sa_params(opt, args.chains, steps, variants, 0, split, 42), arrays, threads=threads)
         dt = time.perf_counter() - t0
@@ -206,7 +210,13 @@ def bench_sa(args):
         line["host_cores"] = os.cpu_count()
     else:
         line["cpu_baseline"] = None
-    print(json.dumps(line))
+    eng.close()
+    return line
+
+
+def bench_sa(args):
+    """Prints the config-5 line: value = wall-clock of the whole run (directory build excluded, reported beside it)."""
+    print(json.dumps(sa_measure(args)))
 
 
 def main():
@@ -219,6 +229,7 @@ def main():
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="also run one device-to-device copy of this size (reference dispatch for scaling "
                          "FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--no-sa", action="store_true", help="leave the annealing run of config 5 out of the line")
     ap.add_argument("--chains", type=int, default=64)
     ap.add_argument("--sa-steps", type=int, default=2000)
     args = ap.parse_args()
@@ -258,12 +269,26 @@ def main():
         eng.eval_device(db, out)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    host_s = 0.0
     for _ in range(args.steps):
+        h0 = time.perf_counter()
         eng.eval_device(db, out)
+        host_s += time.perf_counter() - h0
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     value = n * args.steps / dt
+    # run-to-run spread: the same number of steps again, each one bracketed by a synchronisation of its own
+    each = []
+    for _ in range(args.steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.eval_device(db, out)
+        torch.cuda.synchronize()
+        each.append((time.perf_counter() - t0) * 1e3)
+    each.sort()
+    spread = {"min": each[0], "median": each[len(each) // 2], "max": each[-1],
+              "note": "ms per step over the same number of steps run again, each synchronised on its own"}
 
     # cold steps: every class of the batch is lowered again inside the step
     cold_steps = max(1, min(args.steps, 5))
@@ -352,8 +377,8 @@ def main():
     # (which classes run where is decided from times the kernels measure on themselves: the task counts of two runs
     # differ by up to a fifth, the number of k_quad's tasks by up to a third)
     same_layout = measured is not None and tuple(measured["layout"][1:3]) == layout[1:3] and all(
-        abs(a - b) <= tol * max(a, b) + 8 for a, b, tol in zip((measured["layout"][0],) + tuple(measured["layout"][3:]),
-                                                               (layout[0],) + layout[3:], (0.25, 0.25, 0.35)))
+        abs(a - b) <= 0.05 * max(a, b) + 8 for a, b in zip((measured["layout"][0],) + tuple(measured["layout"][3:]),
+                                                           (layout[0],) + layout[3:]))
     roofline.update(traffic=measured["traffic"] if same_layout else None, kernel=kernel_name, kernel_ms=kernel_ms,
                     layout=list(layout))
     ipp = measured["instructions_per_plan"] if same_layout else None
@@ -365,7 +390,8 @@ def main():
     line = {
         "metric": "cost-model plan evals/sec on 1 MI355X",
         "value": value, "unit": "plan evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms_per_step, "ms_per_step_spread": spread, "host_ms_in_calls_per_step": host_s / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64", "data": "synthetic",
         "config": {"workload": cfg.name, "n_plans": n, "seed": 42, "K_eval": cfg.problem.K_eval,
                    "device_mesh": [cfg.problem.device_space.R, cfg.problem.device_space.N, cfg.problem.device_space.G],
@@ -387,6 +413,13 @@ def main():
     else:
         line["cpu_baseline"] = None
         line["parity"] = None
+    if not args.no_sa:
+        # the second half of the metric: the annealing run of config 5, timed in the same process
+        eng.close()
+        sa = sa_measure(args, deadlines=False)
+        line["sa"] = {k: sa[k] for k in ("metric", "value", "unit", "config", "time_to_best_s", "best_step", "best_score",
+                                         "best_feasible", "best_plan_crc", "plans_evaluated", "launches", "evals_per_s",
+                                         "eval_share_of_wall", "wall_s_of_runs", "directory_s", "cpu_baseline")}
     print(json.dumps(line))
 
 
