@@ -222,9 +222,10 @@ int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, u
    node reserved of busy time / makespan, summed in the order in which the reference's trace first meets the
    devices, hence equal to the reference's number bit for bit (NaN for a plan with RPEG_MASK_ERROR or an
    invalid one).  This is the second factor of the utilisation objective of optimize() and polish()
-   (RPEG/search/optimizer.py:461-486, 1021-1044), which then costs no launch of its own.  At most 1,024 plans per
-   call, one plan per wavefront (status -8 beyond that, and for problems with a class above 384 nodes);
-   rpeg_eval_trace_metrics gives the same number for a single plan of any size. */
+   (RPEG/search/optimizer.py:461-486, 1021-1044), which then costs no launch of its own.  Any number of plans: one
+   launch of a plan per wavefront for every 1,024 of them.  A problem with a class above 384 nodes does not fit that
+   kernel: its batch takes the path of rpeg_eval_host and every plan is then traced on its own, as by
+   rpeg_eval_trace_metrics (the same numbers, one launch per plan). */
 int rpeg_eval_host_util(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                         double* peak, double* score, uint8_t* mask, double* utilization, void* stream);
 

@@ -2571,22 +2571,43 @@ int rpeg_eval_host_util(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* pla
   e->err.clear();
   e->last_ms = -1.0;
   if (n == 0) return 0;
+  if (n >= (1ull << 32)) { e->err = "at most 2^32-1 plans per call"; return -1; }
   if (!plans->vert || !plans->head || plans->stride < n) { e->err = "bad plan tensors"; return -1; }
-  if (n > (uint64_t)e->host_small_max) {
-    e->err = "rpeg_eval_host_util takes at most " + std::to_string(e->host_small_max) + " plans per call";
-    return -8;
-  }
   const int16_t* vert = plans->vert;
   const uint8_t* head = plans->head;
   const uint64_t stride = plans->stride;
-  auto get = [&](uint64_t i, PlanHead& h, VPlan (&a)[RPEG_MAX_V]) {
-    h = load_head(head, stride, i);
-    const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;
-    for (int v = 0; v < nv; ++v) load_vertex(vert, stride, i, v, &a[v]);
-  };
-  const int rc = eval_host_small(e, n, get, flags, makespan, peak, score, mask, nullptr, (hipStream_t)stream, utilization);
-  if (rc == 1) { e->err = "a class of this problem has too many nodes for one plan per wavefront"; return -8; }
-  return rc;
+  // one launch of a plan per wavefront for every `host_small_max` plans
+  const uint64_t piece = std::max<uint64_t>(1, e->host_small_max);
+  bool too_large = false;
+  for (uint64_t a = 0; a < n && !too_large; a += piece) {
+    const uint64_t m = std::min(piece, n - a);
+    auto get = [&](uint64_t i, PlanHead& h, VPlan (&pl)[RPEG_MAX_V]) {
+      h = load_head(head, stride, a + i);
+      const int nv = (h.structure >= 0 && h.structure < e->P.n_struct) ? e->P.st[h.structure].n_vertex : 0;
+      for (int v = 0; v < nv; ++v) load_vertex(vert, stride, a + i, v, &pl[v]);
+    };
+    const int rc = eval_host_small(e, m, get, flags, makespan ? makespan + a : nullptr, peak ? peak + a : nullptr,
+                                   score ? score + a : nullptr, mask ? mask + a : nullptr, nullptr, (hipStream_t)stream,
+                                   utilization + a);
+    if (rc == 1) too_large = true;
+    else if (rc) return rc;
+  }
+  if (!too_large) return 0;
+  // A class of this problem has more nodes than a wavefront holds: the batch takes the path of rpeg_eval_host and
+  // every plan is traced on its own for its utilisation (rpeg_eval_trace_metrics).
+  std::vector<uint8_t> own_mask;
+  if (!mask) { own_mask.resize(n); mask = own_mask.data(); }
+  if (int rc = eval_host_impl(e, n, plans, flags, makespan, peak, score, mask, nullptr, stream)) return rc;
+  for (uint64_t i = 0; i < n; ++i) {
+    utilization[i] = __builtin_nan("");
+    if (!(mask[i] & RPEG_MASK_VALID) || (mask[i] & RPEG_MASK_ERROR)) continue;
+    int16_t f[RPEG_MAX_V * RPEG_FIELDS] = {};
+    uint8_t h4[4];
+    for (int x = 0; x < RPEG_MAX_V * RPEG_FIELDS; ++x) f[x] = vert[(uint64_t)x * stride + i];
+    for (int x = 0; x < 4; ++x) h4[x] = head[(uint64_t)x * stride + i];
+    if (int rc = rpeg_eval_trace_metrics(e, f, h4, &utilization[i], nullptr)) return rc;
+  }
+  return 0;
 }
 
 int rpeg_sa_run(rpeg_engine_t* e, const rpeg_sa_params_t* prm, const int16_t* base_plan, rpeg_sa_result_t* res,

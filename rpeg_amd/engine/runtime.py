@@ -295,8 +295,8 @@ class Engine:
         return out
 
     def eval_util(self, batch: PlanBatch, gate_stale: bool = False) -> Dict[str, np.ndarray]:
-        """`eval` plus Trace.utilization() of every plan from the same launch (rpeg_eval_host_util; at most 1,024
-        plans): the dict of `eval` with "util", float64 [n]."""
+        """`eval` plus Trace.utilization() of every plan from the same launches (rpeg_eval_host_util): the dict of
+        `eval` with "util", float64 [n]."""
         torch = _torch()
         n = batch.n
         out = dict(makespan=np.empty(n), peak=np.empty(n), score=np.empty(n), mask=np.empty(n, np.uint8), util=np.empty(n))

@@ -224,8 +224,7 @@ def evaluate_batch(configs: Sequence[Configuration], suite: ModelSuite, workload
                           transfer_policy=pol)
     batch = _pack(configs, st, workload)
     if with_util:
-        parts = [eng.eval_util(batch.slice(a, min(a + 1024, batch.n)), gate_stale=gate_stale) for a in range(0, batch.n, 1024)]
-        out = {k: np.concatenate([q[k] for q in parts]) for k in parts[0]}
+        out = eng.eval_util(batch, gate_stale=gate_stale)
     else:
         out = eng.eval(batch, gate_stale=gate_stale)
     mask = out["mask"]

@@ -716,8 +716,33 @@ def test_utilization_from_the_batched_launch_equals_reference(c):
     more.vert[0, 3] = 3           # tp = 3 divides no G: not evaluated
     bad = eng.eval_util(more.slice(0, 8))
     assert bad["mask"][3] == 0 and np.isnan(bad["util"][3]) and not np.isnan(bad["util"][2])
-    with pytest.raises(EngineError, match="at most 1024"):
-        eng.eval_util(seeded_batch(c, 1025)[1])
+    # any number of plans: a launch for every 1,024 of them
+    _, many = seeded_batch(c, 2600, start=300_000)
+    whole = eng.eval_util(many)
+    plain = eng.eval(many, gate_stale=False)
+    assert same_bits(whole["score"], plain["score"]) and np.array_equal(whole["mask"], plain["mask"])
+    for a in (0, 1024, 2048):
+        part = eng.eval_util(many.slice(a, min(a + 1024, many.n)))
+        assert same_bits(whole["util"][a:a + 1024], part["util"]), a
+
+
+def test_utilization_of_classes_beyond_a_wavefront_is_traced_plan_by_plan():
+    """A problem whose graphs outgrow the plan-per-wavefront kernel (above 384 nodes): eval_util gives the numbers of
+    the single-plan trace and the other outputs of the plain call."""
+    from rpeg_amd.engine.runtime import Engine
+    import dataclasses
+    cfg, batch = seeded_batch(1, 24)
+    eng = Engine(dataclasses.replace(cfg.problem, K_eval=24))
+    out = eng.eval_util(batch, gate_stale=False)
+    plain = eng.eval(batch, gate_stale=False)
+    assert eng.stats()["classes"] > 0
+    assert same_bits(out["score"], plain["score"]) and np.array_equal(out["mask"], plain["mask"])
+    ok = np.flatnonzero(((out["mask"] & abi.MASK_VALID) != 0) & ((out["mask"] & abi.MASK_ERROR) == 0))
+    assert len(ok) > 8
+    for i in ok:
+        assert float(out["util"][i]).hex() == float(eng.trace_metrics(batch, int(i))[0]).hex(), i
+    assert np.all((out["util"][ok] > 0.0) & (out["util"][ok] <= 1.0))
+    eng.close()
 
 
 @pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
