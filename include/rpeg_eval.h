@@ -452,6 +452,15 @@ int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
    Results do not depend on the setting. */
 int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes);
 
+/* The nine fitted figures by which a full batch is split between the three scheduling kernels (microseconds of a
+   wavefront on an MI355X): cost of a plan in the one-plan-per-wavefront kernel a + b x nodes (40, 2.2); of a wavefront
+   of the four-lanes-per-plan kernel a + nodes x (b + c x heap pops per dispatch) (40, 1.6, 0.45); the share of the
+   modelled room that the former really gets beside the latter (0.65); how much later a class must end in the main
+   kernel to move to the four-lanes-per-plan kernel (1.15); the modelled gain that a split by class size (0.97) and by
+   measured time (0.98) must reach.  A measurement aid: the figures decide where a plan is evaluated, never what
+   the result is.  No counterpart in the reference. */
+int rpeg_engine_set_split_model(rpeg_engine_t* e, const double* values, int32_t n);
+
 /* rpeg_sa_run deals its chains to `groups` groups (1..8, default 2; never fewer than 8 chains per group) that take
    their steps in turn, each with a stream and staging buffers of its own: while the proposals of one group are being
    evaluated, the host merges the results of another and draws its next proposals.  A chain's draws are keyed by

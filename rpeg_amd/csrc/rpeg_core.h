@@ -456,10 +456,11 @@ struct PlanMasks {
 RPEG_HD unsigned mask_row(uint64_t m, int v) { return (unsigned)(m >> (8 * v)) & 0xFFu; }
 
 // Plan-independent vertex sets of one structure (bit v = vertex v).
-struct StructMasks {
-  uint8_t same_model[RPEG_MAX_V];   // vertices invoking the same model as v
-  uint8_t train_same[RPEG_MAX_V];   // TRAIN vertices of v's model
-  uint8_t before[RPEG_MAX_V];       // vertices that precede order[i] in first-appearance order
+struct StructMasks {                // (rows of 8 bits packed into words, read with mask_row: byte arrays indexed with
+                                    // run-time values would live in scratch memory on the GPU)
+  uint64_t same_model;              // row v: vertices invoking the same model as v
+  uint64_t train_same;              // row v: TRAIN vertices of v's model
+  uint64_t before;                  // row i: vertices that precede order[i] in first-appearance order
   uint8_t train, trainable;         // TRAIN vertices; vertices of trainable models
   bool coresident;                  // the memory model lists no trainable model at all: co-resident sum model
 };
@@ -474,17 +475,17 @@ RPEG_HD StructMasks struct_masks(const rpeg_struct_t& st, const ORD& order) {
   StructMasks m;
   m.train = m.trainable = 0;
   unsigned seen = 0;
-  for (int i = 0; i < RPEG_MAX_V; ++i) { m.same_model[i] = m.train_same[i] = m.before[i] = 0; }
+  m.same_model = m.train_same = m.before = 0;
   for (int v = 0; v < st.n_vertex; ++v) {
     if (st.vertex[v].role == RPEG_ROLE_TRAIN) m.train |= (uint8_t)(1u << v);
     if (st.mem_trainable[st.vertex[v].model]) m.trainable |= (uint8_t)(1u << v);
     for (int w = 0; w < st.n_vertex; ++w)
       if (st.vertex[w].model == st.vertex[v].model) {
-        m.same_model[v] |= (uint8_t)(1u << w);
-        if (st.vertex[w].role == RPEG_ROLE_TRAIN) m.train_same[v] |= (uint8_t)(1u << w);
+        m.same_model |= 1ull << (8 * v + w);
+        if (st.vertex[w].role == RPEG_ROLE_TRAIN) m.train_same |= 1ull << (8 * v + w);
       }
   }
-  for (int i = 0; i < st.n_vertex; ++i) { m.before[i] = (uint8_t)seen; seen |= 1u << order[i]; }
+  for (int i = 0; i < st.n_vertex; ++i) { m.before |= (uint64_t)seen << (8 * i); seen |= 1u << order[i]; }
   m.coresident = struct_coresident(st);
   return m;
 }
@@ -505,7 +506,7 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
   for (int i = 0; i < nv; ++i) {  // distinct (model, allocation) worker keys
     const int v = order[i];
     if (!((M >> v) & 1u)) continue;
-    if ((mask_row(pm.eq, v) & M & sm.same_model[v] & sm.before[i]) == 0) ++groups;
+    if ((mask_row(pm.eq, v) & M & mask_row(sm.same_model, v) & mask_row(sm.before, i)) == 0) ++groups;
   }
   if (sm.coresident) {
     // memory.py:706-742: every model present keeps its static footprint -- its largest shard among the vertices
@@ -517,8 +518,8 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
       const int v = order[i];
       if (!((M >> v) & 1u)) continue;
       transient = dmax(transient, vm.extra(v));
-      const unsigned same = M & sm.same_model[v];
-      if (same & sm.before[i]) continue;   // the model's entry exists
+      const unsigned same = M & mask_row(sm.same_model, v);
+      if (same & mask_row(sm.before, i)) continue;   // the model's entry exists
       double wmax = 0.0, dp = vm.opt(v);
       bool trained = false;
       for (int j = 0; j < nv; ++j) {
@@ -544,8 +545,8 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
   for (int i = 0; i < nv; ++i) {
     const int v = order[i];
     if (!(((M & sm.trainable & ~(unsigned)sm.train) >> v) & 1u)) continue;
-    const unsigned same_key = mask_row(pm.eq, v) & M & sm.same_model[v];
-    if (same_key & sm.train_same[v]) continue;
+    const unsigned same_key = mask_row(pm.eq, v) & M & mask_row(sm.same_model, v);
+    if (same_key & mask_row(sm.train_same, v)) continue;
     const bool first = (same_key & serving) == 0;
     serving |= 1u << v;
     if (!first) continue;
@@ -557,8 +558,8 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
   for (int i = 0; i < nv; ++i) {  // frozen weights: one entry per model, its largest shard
     const int v = order[i];
     if (!(((M & ~(unsigned)sm.trainable) >> v) & 1u)) continue;
-    const unsigned same = M & sm.same_model[v];
-    if (same & sm.before[i]) continue;
+    const unsigned same = M & mask_row(sm.same_model, v);
+    if (same & mask_row(sm.before, i)) continue;
     double wb = 0.0;
     for (int w = 0; w < nv; ++w)
       if ((same >> w) & 1u) wb = dmax(wb, vm.mem_w(w));
@@ -568,7 +569,7 @@ RPEG_HD double device_class_peak(const rpeg_problem_t& P, const rpeg_struct_t& s
   for (int i = 0; i < nv; ++i) {
     const int v = order[i];
     if (!((M >> v) & 1u)) continue;
-    const bool resident = !((sm.trainable >> v) & 1u) || (mask_row(pm.eq, v) & serving & sm.same_model[v]) != 0;
+    const bool resident = !((sm.trainable >> v) & 1u) || (mask_row(pm.eq, v) & serving & mask_row(sm.same_model, v)) != 0;
     const double c = resident ? vm.extra(v) : vm.mem_w(v) + vm.extra(v);
     top = dmax(top, c);
   }

@@ -526,6 +526,27 @@ static uint8_t* static_scratch_ptr(int dev, hipError_t* st) {
   return g_static_ptr[dev];
 }
 
+// The fitted figures behind the split of a full batch between the three scheduling kernels, in one place.  They are
+// microseconds of one wavefront on an MI355X, fitted to the per-wavefront clocks of configurations 2, 3 and 5
+// (python -m rpeg_amd.engine.profile) and then to the step time of configuration 2 over a sweep of each figure;
+// rpeg_engine_set_split_model replaces them (a measurement aid).  A wrong figure
+// costs time, never a result: every kernel computes the same bits.
+//   plan_a + plan_b x nodes                    what a plan costs k_plan (one plan per wavefront), beside the main kernel
+//   quad_a + nodes x (quad_b + quad_c x pops)  a wavefront of k_quad (sixteen plans); pops = heap pops per dispatch,
+//                                              as the main kernel measured them for the class
+//   eff_beside_quad                            the part of the modelled room beside the main kernel that k_plan really
+//                                              gets where k_quad takes its share of a compute unit too
+//   quad_margin                                a class moves to k_quad only if it ends this much later in the main kernel
+//   gain_threshold, gain_classes               a split by class size / by measured time must model this much earlier
+struct SplitModel {
+  double plan_a = 40.0, plan_b = 2.2;
+  double quad_a = 40.0, quad_b = 1.6, quad_c = 0.45;
+  double eff_beside_quad = 0.65;
+  double quad_margin = 1.15;
+  double gain_threshold = 0.97, gain_classes = 0.98;
+};
+constexpr int SPLIT_MODEL_FIELDS = 9;
+
 // Staging of one small host-pointer evaluation: plans and class offsets in (pinned, then device), results out (pinned,
 // written by the kernel itself), and which of the caller's plans went to the device.
 struct HostLane {
@@ -589,6 +610,7 @@ struct rpeg_engine_s {
   uint8_t* d_trace = nullptr;   // rpeg_eval_trace: one plan's fields and header, then start / finish / dispatch index
   uint8_t* d_detail = nullptr;  // rpeg_plan_detail: one plan's fields and header, then slot durations and vertex-set peaks
   size_t d_trace_nodes = 0;
+  SplitModel split_model;
   int sa_lanes = 3;     // rpeg_sa_run: groups of chains whose evaluations overlap the host's work on the others
   int lanes_busy = 0;   // evaluations submitted on lanes and not yet collected (their kernels read d_pool)
   uint64_t relearn_at = 0;                // the call that last asked for the measurements again
@@ -963,8 +985,9 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_dur) hipFree(e->d_dur);
   if (e->d_uni) hipFree(e->d_uni);
   if (e->d_cls) { hipFree(e->d_cls); hipHostFree(e->h_cls); }
-  if (e->s2) { hipStreamDestroy(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
-  if (e->s3) { hipStreamDestroy(e->s3); hipEventDestroy(e->ev_join3); }
+  // (the side streams belong to the device, not to the engine: side_streams)
+  if (e->s2) { hipStreamSynchronize(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
+  if (e->s3) { hipStreamSynchronize(e->s3); hipEventDestroy(e->ev_join3); }
   if (e->ev_counts) hipEventDestroy(e->ev_counts);
   e->lane0.release();
   if (e->d_stage) hipFree(e->d_stage);
@@ -1007,6 +1030,17 @@ int rpeg_engine_set_state_lanes(rpeg_engine_t* e, int32_t lanes) {
     return -1;
   }
   e->state_lanes = lanes;
+  e->split_for_n = 0;
+  return 0;
+}
+
+int rpeg_engine_set_split_model(rpeg_engine_t* e, const double* values, int32_t n) {
+  if (!e || !values || n != SPLIT_MODEL_FIELDS) { if (e) e->err = "nine figures"; return -1; }
+  for (int i = 0; i < n; ++i)
+    if (!(values[i] >= 0.0)) { e->err = "the figures are non-negative"; return -1; }
+  SplitModel& m = e->split_model;
+  m.plan_a = values[0]; m.plan_b = values[1]; m.quad_a = values[2]; m.quad_b = values[3]; m.quad_c = values[4];
+  m.eff_beside_quad = values[5]; m.quad_margin = values[6]; m.gain_threshold = values[7]; m.gain_classes = values[8];
   e->split_for_n = 0;
   return 0;
 }
@@ -1081,15 +1115,17 @@ int rpeg_eval_host(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, u
 
 constexpr uint32_t TINY_CLASS = 16;   // classes of fewer plans go to the single-plan kernel
 
+
 // When a step ends, for a batch of more than one round of wavefronts (microseconds).  The main kernel keeps r
 // wavefronts on every compute unit and lasts max(its longest task, its work / (units x r)); k_plan runs beside it in
 // the LDS and registers left (16 - 2r wavefronts of 128 registers), and what it has not done by then it does with
-// the units to itself, sixteen wavefronts each.  A plan costs k_plan about 40 + 2.2 x nodes microseconds of a wavefront.
+// the units to itself, sixteen wavefronts each.  What a plan costs k_plan: SplitModel.
 struct DeepModel {
   double n_cu, lds_main, lds_plan;
   double eff = 1.0;   // the part of the modelled room beside the main kernel that k_plan really gets
   uint64_t r_max;
-  double plan_cost(uint32_t plans, uint32_t nodes) const { return (double)plans * (40.0 + 2.2 * (double)nodes); }
+  SplitModel sm;
+  double plan_cost(uint32_t plans, uint32_t nodes) const { return (double)plans * (sm.plan_a + sm.plan_b * (double)nodes); }
   double total(double w_main, double w_plan, double max_t, uint64_t r) const {
     const double t_main = std::max(max_t, w_main / (n_cu * (double)r));
     const double room = eff * std::max(0.0, std::min(16.0 - 2.0 * (double)r, std::floor((160.0 * 1024 - (double)r * lds_main) / lds_plan)));
@@ -1107,11 +1143,30 @@ struct DeepModel {
 };
 static DeepModel deep_model(const rpeg_engine_t* e, uint32_t rcap) {
   DeepModel m;
+  m.sm = e->split_model;
   m.n_cu = (double)e->n_cu;
   m.lds_main = (double)ke_lds_bytes((e->max_cls_bytes + 15u) & ~15u, rcap, 0, e->max_nodes, e->max_slots, e->max_v);
   m.lds_plan = (double)kp_lds_bytes(e->max_nodes, e->max_slots);
   m.r_max = std::max<uint64_t>(1, std::min<uint64_t>(8, (uint64_t)(160.0 * 1024 / m.lds_main)));
   return m;
+}
+
+// The two streams on which k_plan and k_quad run beside the main kernel, one pair per device for all engines of the
+// process (never destroyed).  A process has few hardware queues (four by default): with a pair of side streams per
+// engine, two engines that evaluate at the same time on two caller streams are six streams, several of which share
+// a queue and then wait for each other's kernels; with one pair they are four.
+static int side_streams(rpeg_engine_t* e, hipStream_t* plan_stream, hipStream_t* quad_stream) {
+  static std::mutex mu;
+  static hipStream_t pair[64][2] = {};
+  int dev = 0;
+  HIP_TRY(e, hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) { e->err = "device index out of range"; return -2; }
+  std::lock_guard<std::mutex> lock(mu);
+  for (int k = 0; k < 2; ++k)
+    if (!pair[dev][k]) HIP_TRY(e, hipStreamCreateWithFlags(&pair[dev][k], hipStreamNonBlocking));
+  if (plan_stream) *plan_stream = pair[dev][0];
+  if (quad_stream) *quad_stream = pair[dev][1];
+  return 0;
 }
 
 static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
@@ -1420,7 +1475,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
           }
           const double t = dm.best(w_main, w_plan, max_t, nullptr);
           if (th == TINY_CLASS) best_t = t;
-          else if (t < 0.97 * best_t) { best_t = t; best_th = th; }
+          else if (t < dm.sm.gain_threshold * best_t) { best_t = t; best_th = th; }
         }
       }
       if (best_th != TINY_CLASS)
@@ -1435,7 +1490,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       DeepModel dm = deep_model(e, rcap_main);
       // (where k_quad is going to take its share of a compute unit's wavefront slots and LDS, k_plan gets through
       // about two thirds of what the model gives it beside the main kernel: measured on configs 2 and 5)
-      if (waves64 <= (uint64_t)e->n_cu * 12) dm.eff = 0.65;
+      if (waves64 <= (uint64_t)e->n_cu * 12) dm.eff = dm.sm.eff_beside_quad;
       double w_main = 0.0, w_plan = 0.0, t_sum = 0.0, nodes_sum = 0.0;
       std::vector<uint32_t> cand;
       for (uint32_t c = 0; c < counts.size(); ++c) {
@@ -1464,22 +1519,22 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
           wm -= (double)((counts[c] + WAVE - 1) / WAVE) * t_of(c);
           wp += dm.plan_cost(counts[c], e->cls_nodes[cids[c]]);
           const double t = dm.best(wm, wp, k + 1 < cand.size() ? t_of(cand[k + 1]) : 0.0, nullptr);
-          if (t < 0.98 * best_t) { best_t = t; best_k = k + 1; }
+          if (t < dm.sm.gain_classes * best_t) { best_t = t; best_k = k + 1; }
         }
         for (size_t k = 0; k < best_k; ++k) solo[cand[k]] = 1;
       }
     }
     // Of what stays, the wavefronts that end last are those of dense graphs (long ready lists, keys that go stale
     // often).  The main kernel measures itself: per class, the time of its slowest wavefront on earlier launches and
-    // the heap pops per dispatch it needed (cls_pops16).  A wavefront of k_quad takes about 75 + nodes x (2.3 +
-    // 0.45 per pop) microseconds (fitted).  The classes are taken in the order of their measured time while one still
-    // ends 15 % later in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct`
+    // the heap pops per dispatch it needed (cls_pops16).  What a wavefront of k_quad takes: SplitModel.  The classes
+    // are taken in the order of their measured time while one still ends later by SplitModel::quad_margin
+    // in the main kernel than the slowest chosen class ends in k_quad, up to `quad_share_pct`
     // percent of the batch.  Nothing is known before the first launch of a class: it stays in the main kernel then.
     if (split && e->quad_share_pct && waves64 <= (uint64_t)e->n_cu * 12) {
       auto t_main = [&](uint32_t c) { return (double)(e->cls_pops16[cids[c]] >> 12); };
       auto t_quad = [&](uint32_t c) {
         const double nd = e->cls_nodes[cids[c]], p = (e->cls_pops16[cids[c]] & 0xFFFu) / 16.0;
-        return 75.0 + nd * (2.3 + 0.45 * p);
+        return e->split_model.quad_a + nd * (e->split_model.quad_b + e->split_model.quad_c * p);
       };
       std::vector<uint32_t> cand;
       for (uint32_t c = 0; c < counts.size(); ++c)
@@ -1504,7 +1559,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
         const double room = (double)e->n_cu * std::max(1.0, std::floor(lds_left / (double)qlds));
         const double tq = std::max(slowest_quad, t_quad(c));
         const double rounds = std::max(1.0, (double)(tasks + c_tasks) / room);
-        if (t_main(c) <= 1.15 * tq * rounds) break;   // (a margin: beyond the classes that clearly end later, more wavefronts of k_quad cost more than they save)
+        if (t_main(c) <= e->split_model.quad_margin * tq * rounds) break;   // (a margin: beyond the classes that clearly end later, more wavefronts of k_quad cost more than they save)
         if ((taken + counts[c]) * 100 > (uint64_t)n * e->quad_share_pct) break;
         quad[c] = 1;
         taken += counts[c];
@@ -1687,12 +1742,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // fill a compute unit its wavefronts only fit in as those retire.
   if (n_solo || n_quad_waves) {
     if (!e->s2) {
-      HIP_TRY(e, hipStreamCreateWithFlags(&e->s2, hipStreamNonBlocking));
+      if (int rc = side_streams(e, &e->s2, nullptr)) return rc;
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_fork, hipEventDisableTiming));
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join, hipEventDisableTiming));
     }
     if (n_quad_waves && !e->s3) {
-      HIP_TRY(e, hipStreamCreateWithFlags(&e->s3, hipStreamNonBlocking));
+      if (int rc = side_streams(e, nullptr, &e->s3)) return rc;
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join3, hipEventDisableTiming));
     }
     // (the three launches back to back: every call between them delays the start of the later kernels)

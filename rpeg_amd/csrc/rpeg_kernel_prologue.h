@@ -67,18 +67,21 @@ __device__ inline VPlan kpro_vplan(const int16_t* p, uint64_t stride, int v) {
 
 // (the pieces are functions of their own, not inlined: each gets the registers it needs instead of the kernel holding
 // the union of all of them, which costs it its residency)
+// (NaN where the reference would raise ZeroDivisionError: a flag handed in by address would live in scratch memory)
 __device__ __attribute__((noinline)) double kpro_op_time(const rpeg_problem_t& P, const rpeg_vertex_t& vx, const rpeg_opconst_t& oc,
-                                                         const int16_t* pl, uint64_t stride, int v, bool* zero_div) {
-  return op_time(P, vx, oc, kpro_vplan(pl, stride, v), zero_div);
+                                                         const int16_t* pl, uint64_t stride, int v) {
+  bool zero_div = false;
+  const double t = op_time(P, vx, oc, kpro_vplan(pl, stride, v), &zero_div);
+  return zero_div ? __builtin_nan("") : t;
 }
 
 __device__ inline double kpro_slot_duration(const rpeg_problem_t& P, const rpeg_struct_t& st, int split, const SlotDesc sd,
-                                            const int16_t* pl, uint64_t stride, bool* zero_div) {
+                                            const int16_t* pl, uint64_t stride) {
   switch (sd.type) {
     case SLOT_OP_UNSPLIT:
-      return kpro_op_time(P, st.vertex[sd.a], st.vertex[sd.a].unsplit, pl, stride, sd.a, zero_div);
+      return kpro_op_time(P, st.vertex[sd.a], st.vertex[sd.a].unsplit, pl, stride, sd.a);
     case SLOT_OP_SUB:
-      return kpro_op_time(P, st.vertex[sd.a], st.vertex[sd.a].sub[split][sd.q], pl, stride, sd.a, zero_div);
+      return kpro_op_time(P, st.vertex[sd.a], st.vertex[sd.a].sub[split][sd.q], pl, stride, sd.a);
     case SLOT_COMM_DATA: {
       const rpeg_edge_t& e = st.edge[sd.a];
       const int64_t payload = sd.q == 0xFF ? e.full_bytes : e.sub_bytes[split][sd.q];
@@ -94,25 +97,27 @@ __device__ inline double kpro_slot_duration(const rpeg_problem_t& P, const rpeg_
   }
 }
 
-__device__ __attribute__((noinline)) void kpro_masks(const PrologueLaunch& L, const uint64_t i, const int nv) {
-  const int16_t* pl = L.vert + i;
+// (these take what they need by value: the address of the launch record would force a copy of it into scratch memory
+// in every wavefront)
+__device__ __attribute__((noinline)) void kpro_masks(const int16_t* pl, const uint64_t stride, const int nv, uint64_t* ovl,
+                                                     uint64_t* eq, uint64_t* dpne) {
   VPlan a[RPEG_MAX_V];
 #pragma unroll
   for (int v = 0; v < RPEG_MAX_V; ++v)
-    if (v < nv) a[v] = kpro_vplan(pl, L.stride, v);
+    if (v < nv) a[v] = kpro_vplan(pl, stride, v);
   const PlanMasks pm = plan_masks(a, nv);
-  L.aux_ovl[i] = pm.ovl;
-  L.aux_eq[i] = pm.eq;
-  L.aux_dpne[i] = pm.dpne;
+  *ovl = pm.ovl;
+  *eq = pm.eq;
+  *dpne = pm.dpne;
 }
 
-__device__ __attribute__((noinline)) void kpro_vmem(const PrologueLaunch& L, const uint64_t i, const rpeg_struct_t& st, const int v) {
-  const VMem m = vertex_memory(*L.P, st.vertex[v], kpro_vplan(L.vert + i, L.stride, v), struct_coresident(st));
-  double* out = L.vm + (uint64_t)(v * 4) * L.dur_stride + i;
-  out[0 * L.dur_stride] = (double)m.w_shard;
-  out[1 * L.dur_stride] = m.mem_w;
-  out[2 * L.dur_stride] = m.opt;
-  out[3 * L.dur_stride] = m.extra;
+__device__ __attribute__((noinline)) void kpro_vmem(const rpeg_problem_t& P, const int16_t* pl, const uint64_t stride,
+                                                    const rpeg_struct_t& st, const int v, double* out, const uint64_t out_stride) {
+  const VMem m = vertex_memory(P, st.vertex[v], kpro_vplan(pl, stride, v), struct_coresident(st));
+  out[0 * out_stride] = (double)m.w_shard;
+  out[1 * out_stride] = m.mem_w;
+  out[2 * out_stride] = m.opt;
+  out[3 * out_stride] = m.extra;
 }
 
 // Plan i of this lane, structure su (uniform), one row of the first launch's grid (uniform): the duration of one slot
@@ -125,14 +130,12 @@ __device__ inline void kpro_row(const PrologueLaunch& L, const uint64_t i, const
     if (row >= (int)L.n_uni[su]) return;
     const SlotDesc sd = L.uni[(size_t)su * RPEG_MAX_UNIVERSE + row];   // uniform
     if (!slot_in_split(P, split, sd)) return;                          // this lane's split variant has no such phase
-    bool zd = false;
-    const double t = kpro_slot_duration(P, st, split, sd, pl, L.stride, &zd);
-    L.dur[(uint64_t)row * L.dur_stride + i] = zd ? __builtin_nan("") : t;
+    L.dur[(uint64_t)row * L.dur_stride + i] = kpro_slot_duration(P, st, split, sd, pl, L.stride);
   } else if (row == (int)L.max_uni) {
-    kpro_masks(L, i, st.n_vertex);
+    kpro_masks(pl, L.stride, st.n_vertex, L.aux_ovl + i, L.aux_eq + i, L.aux_dpne + i);
   } else {
     const int v = row - (int)L.max_uni - 1;
-    if (v < st.n_vertex) kpro_vmem(L, i, st, v);
+    if (v < st.n_vertex) kpro_vmem(P, pl, L.stride, st, v, L.vm + (uint64_t)(v * 4) * L.dur_stride + i, L.dur_stride);
   }
 }
 
