@@ -1228,6 +1228,28 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       return 0;
     }
   }
+  // A batch small enough to get a wavefront per plan whatever its classes are (k_plan) leaves the cost model and the
+  // memory model to that kernel, which spreads them over the lanes of a plan's wavefront: the prologue launches work a
+  // plan per lane, and a few thousand plans are a few dozen wavefronts that take as long as a full grid would.
+  const bool own_prologue = e->state_lanes == 1 || (e->state_lanes == -1 && n <= (uint64_t)e->n_cu * e->one_plan_waves_per_cu);
+  bool prologue_done = false;
+  auto launch_prologue = [&]() -> int {
+    PrologueLaunch G;
+    G.P = e->dP; G.vert = plans->vert; G.head = plans->head; G.stride = plans->stride; G.n = n; G.cid = e->d_cid;
+    G.uni = e->d_uni;
+    for (int q = 0; q < RPEG_MAX_STRUCT; ++q) G.n_uni[q] = e->n_uni[q];
+    G.max_uni = e->max_uni;
+    G.dur = e->d_dur; G.dur_stride = e->cap_n;
+    G.aux_ovl = e->d_aux_ovl; G.aux_eq = e->d_aux_eq; G.aux_dpne = e->d_aux_dpne; G.vm = e->d_vm;
+    G.aux_pen = e->d_aux_pen; G.aux_mask = e->d_aux_mask;
+    G.peak = peak;
+    const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
+    hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, s, G);
+    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
+    HIP_TRY(e, hipGetLastError());
+    prologue_done = true;
+    return 0;
+  };
   // classes of the batch: every plan looks its class id up on the device and counts itself; only the
   // per-class counts come back.  Plans of classes not lowered yet make the call take the slow round:
   // their signatures are read back, the classes are lowered on the host, the tables are rebuilt.
@@ -1255,19 +1277,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       // (the event, not the stream) and lays the batch out.
       if (!e->ev_counts) HIP_TRY(e, hipEventCreateWithFlags(&e->ev_counts, hipEventDisableTiming));
       HIP_TRY(e, hipEventRecord(e->ev_counts, s));
-      PrologueLaunch G;
-      G.P = e->dP; G.vert = plans->vert; G.head = plans->head; G.stride = plans->stride; G.n = n; G.cid = e->d_cid;
-      G.uni = e->d_uni;
-      for (int q = 0; q < RPEG_MAX_STRUCT; ++q) G.n_uni[q] = e->n_uni[q];
-      G.max_uni = e->max_uni;
-      G.dur = e->d_dur; G.dur_stride = e->cap_n;
-      G.aux_ovl = e->d_aux_ovl; G.aux_eq = e->d_aux_eq; G.aux_dpne = e->d_aux_dpne; G.vm = e->d_vm;
-      G.aux_pen = e->d_aux_pen; G.aux_mask = e->d_aux_mask;
-      G.peak = peak;
-      const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
-      hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, s, G);
-      hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
-      HIP_TRY(e, hipGetLastError());
+      if (!own_prologue)
+        if (int rc = launch_prologue()) return rc;
       HIP_TRY(e, hipEventSynchronize(e->ev_counts));
     } else {
       HIP_TRY(e, hipStreamSynchronize(s));
@@ -1707,8 +1718,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.flags = flags; L.makespan = makespan; L.peak = peak; L.score = score; L.mask = mask;
   L.mass = mass;
   L.prof = nullptr;
-  L.dur = e->d_dur; L.aux_ovl = e->d_aux_ovl; L.aux_dpne = e->d_aux_dpne; L.aux_pen = e->d_aux_pen; L.aux_mask = e->d_aux_mask;
-  L.dur_stride = e->cap_n;
+  if (!prologue_done && !one)   // (the classes lowered in this call changed what was foreseen for the batch)
+    if (int rc = launch_prologue()) return rc;
+  if (prologue_done) {
+    L.dur = e->d_dur; L.aux_ovl = e->d_aux_ovl; L.aux_dpne = e->d_aux_dpne; L.aux_pen = e->d_aux_pen; L.aux_mask = e->d_aux_mask;
+    L.dur_stride = e->cap_n;
+  }
   const bool bounded = !one;   // some kernel of this call holds a bounded ready set
   if (bounded) {
     if (int rc = ensure_limit_ws(e, s)) return rc;
