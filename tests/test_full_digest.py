@@ -73,8 +73,8 @@ def test_full_sets_equal_reference_digest(c):
 @pytest.mark.gpu
 @pytest.mark.parametrize("c", [1, 2, 3, 4])
 def test_violating_devices_of_the_first_chunk_equal_reference(c):
-    """The device mem_worst_violation names for each of the first 1,024 plans (the reference's own CRC covers the
-    first 4,096: the recorded chunk digest is met by computing all of them)."""
+    """The device mem_worst_violation names for each plan of the first chunk (4,096 plans), through the drop-in
+    `lower` and `mem_worst_violation`: the CRC of all of them equals the one the reference's own run recorded."""
     import rpeg_amd.compat as compat
     gen, gold = _generator(), _gold(c)
     m = min(gold["n"], gold["chunk"])
