@@ -94,7 +94,7 @@ __device__ inline bool kp_is_inf(double v) {   // on the bits, so that a uniform
 template <int NS, bool keep_trace>
 __device__ inline int kp_schedule(const ClassView& cv, const int n, const int lane, const uint64_t ovl,
                                    const uint64_t dpne, const int nd, const double* l_dur, double* l_rank,
-                                   double* l_start, uint8_t* l_pt, uint16_t* l_order,
+                                   double* l_start, uint16_t* l_order, double* l_tab,
                                    double* out_makespan, long* out_pops, unsigned long long* stamp) {
   const double inf = __builtin_inf();
   double key[NS], tm[NS], dvc[NS], dur[NS], rk[NS];
@@ -119,41 +119,49 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
     key[s] = inf;
     tm[s] = 0.0;
     dvc[s] = 0.0;
-    if (ok) {
-      l_rank[v] = rk[s];
-      l_pt[v] = nr.ptkey;
-    }
+    if (ok) l_rank[v] = rk[s];
   }
-  if (lane == 0) l_rank[nd] = 0.0;
+  if (lane == 0) l_rank[nd] = l_start[nd] = 0.0;
   __syncthreads();
 
-  // ---- ranks (scheduler.py:71-100): rounds until no rank changes, at most one per node
-  for (int round = 0; round <= n; ++round) {
-    bool changed = false;
+  // ---- ranks (scheduler.py:71-100): rounds until no rank changes, at most one per node.  A round reads the ranks of
+  // the round before from one array and writes its own into the other (l_start is free until the trace is written),
+  // so that one barrier per round is enough.
+  {
+    double* cur = l_rank;
+    double* nxt = l_start;
+    for (int round = 0; round <= n; ++round) {
+      bool changed = false;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const double r0 = l_rank[sxl[s] & 0xFFFFu], r1 = l_rank[sxl[s] >> 16], r2 = l_rank[sxh[s] & 0xFFFFu],
-                   r3 = l_rank[sxh[s] >> 16];
-      double best = 0.0;
-      best = r0 > best ? r0 : best;
-      best = r1 > best ? r1 : best;
-      best = r2 > best ? r2 : best;
-      best = r3 > best ? r3 : best;
-      const int ns = (int)((info[s] >> 8) & 0xFFu), sb = (int)(info[s] >> 16);
-      for (int j = 4; j < ns; ++j) {
-        const double r = l_rank[cv.succ[sb + j]];
-        best = r > best ? r : best;
+      for (int s = 0; s < NS; ++s) {
+        const double r0 = cur[sxl[s] & 0xFFFFu], r1 = cur[sxl[s] >> 16], r2 = cur[sxh[s] & 0xFFFFu], r3 = cur[sxh[s] >> 16];
+        double best = 0.0;
+        best = r0 > best ? r0 : best;
+        best = r1 > best ? r1 : best;
+        best = r2 > best ? r2 : best;
+        best = r3 > best ? r3 : best;
+        const int ns = (int)((info[s] >> 8) & 0xFFu), sb = (int)(info[s] >> 16);
+        for (int j = 4; j < ns; ++j) {
+          const double r = cur[cv.succ[sb + j]];
+          best = r > best ? r : best;
+        }
+        const double nr_ = dur[s] + best;
+        changed = changed || nr_ != rk[s];
+        rk[s] = nr_;
       }
-      const double nr_ = dur[s] + best;
-      changed = changed || nr_ != rk[s];
-      rk[s] = nr_;
-    }
-    __syncthreads();
 #pragma unroll
-    for (int s = 0; s < NS; ++s)
-      if (s * 64 + lane < n) l_rank[s * 64 + lane] = rk[s];
-    __syncthreads();
-    if (!__ballot(changed)) break;
+      for (int s = 0; s < NS; ++s)
+        if (s * 64 + lane < n) nxt[s * 64 + lane] = rk[s];
+      __syncthreads();
+      double* const t = cur; cur = nxt; nxt = t;
+      if (!__ballot(changed)) break;
+    }
+    if (cur != l_rank) {   // the fixed point, in l_rank for what follows
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        if (s * 64 + lane < n) l_rank[s * 64 + lane] = rk[s];
+      __syncthreads();
+    }
   }
   // chain inheritance (scheduler.py:367-378): the sub-nodes of one split vertex share the chain's top rank
   for (unsigned g = lane; g < cv.h->n_groups; g += KE_WAVE) {
@@ -174,19 +182,55 @@ __device__ inline int kp_schedule(const ClassView& cv, const int n, const int la
   // marks the nodes whose position another node has too: only among those does a tie counter ever decide
   bool shared[NS];
   {
-    uint32_t eq[NS];
+    // Only nodes of one tie-break class (comm_prio * 8 + topo_idx, below 16) compare ranks: the ranks are laid out
+    // class by class (l_start is free until the trace is written), and every node counts within its class's stretch.
+    uint32_t* l_cnt = (uint32_t*)l_tab;   // [16] members of every class, then [17] first place of every class
+    uint32_t* l_beg = l_cnt + 16;
+    uint32_t place[NS], eq[NS];
+    if (lane < 16) l_cnt[lane] = 0u;
+    __syncthreads();
 #pragma unroll
-    for (int s = 0; s < NS; ++s) ord[s] = eq[s] = 0;
-#pragma unroll 4
-    for (int u = 0; u < n; ++u) {
-      const double ru = l_rank[u];
-      const uint32_t pu = l_pt[u];
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        ord[s] += ((pu < pt[s]) | ((pu == pt[s]) & (ru > rk[s]))) ? 1u : 0u;
-        eq[s] += ((pu == pt[s]) & (ru == rk[s])) ? 1u : 0u;
-      }
+    for (int s = 0; s < NS; ++s) {
+      place[s] = 0u;
+      if (s * 64 + lane < n) place[s] = atomicAdd(&l_cnt[pt[s] & 15u], 1u);
     }
+    __syncthreads();
+    if (lane < 16) {
+      const uint32_t cnt = l_cnt[lane];
+      uint32_t beg = cnt;   // inclusive prefix over the 16 classes, then exclusive
+      for (int d = 1; d < 16; d <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_up((int)beg, d, 16);
+        if (lane >= d) beg += o;
+      }
+      beg -= cnt;
+      l_beg[lane] = beg;
+      if (lane == 15) l_beg[16] = beg + cnt;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (s * 64 + lane < n) l_start[l_beg[pt[s] & 15u] + place[s]] = rk[s];
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const bool ok = s * 64 + lane < n;
+      const uint32_t b0 = ok ? l_beg[pt[s] & 15u] : 0u, b1 = ok ? l_beg[(pt[s] & 15u) + 1u] : 0u;
+      uint32_t before = 0u, same = 0u;
+      uint32_t j = b0;
+      for (; j + 4u <= b1; j += 4u) {   // four independent LDS reads in flight
+        const double r0 = l_start[j], r1 = l_start[j + 1], r2 = l_start[j + 2], r3 = l_start[j + 3];
+        before += (r0 > rk[s] ? 1u : 0u) + (r1 > rk[s] ? 1u : 0u) + (r2 > rk[s] ? 1u : 0u) + (r3 > rk[s] ? 1u : 0u);
+        same += (r0 == rk[s] ? 1u : 0u) + (r1 == rk[s] ? 1u : 0u) + (r2 == rk[s] ? 1u : 0u) + (r3 == rk[s] ? 1u : 0u);
+      }
+      for (; j < b1; ++j) {
+        const double ru = l_start[j];
+        before += ru > rk[s] ? 1u : 0u;
+        same += ru == rk[s] ? 1u : 0u;
+      }
+      ord[s] = b0 + before;
+      eq[s] = same;
+    }
+    __syncthreads();   // (l_start is the trace's from here on)
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       ord[s] <<= KP_TIE_BITS;
@@ -828,8 +872,8 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     int ok;
     // (the trace of start and finish times is compiled out where no output needs it: its flags and pointers would
     // otherwise be carried through the scheduling loop)
-#define KP_SCHEDULE(NS) (keep ? kp_schedule<NS, true>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, l_order, &makespan, &pops, stamp) \
-                              : kp_schedule<NS, false>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_pt, nullptr, &makespan, &pops, stamp))
+#define KP_SCHEDULE(NS) (keep ? kp_schedule<NS, true>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, l_order, l_tab, &makespan, &pops, stamp) \
+                              : kp_schedule<NS, false>(cv, n, lane, pm.ovl, pm.dpne, nd, l_dur, l_rank, l_start, nullptr, l_tab, &makespan, &pops, stamp))
     if (n <= 64) ok = KP_SCHEDULE(1);
     else if (n <= 128) ok = KP_SCHEDULE(2);
     else if (n <= 192) ok = KP_SCHEDULE(3);
@@ -862,7 +906,7 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
   double m = __builtin_nan("");   // lane x < RPEG_MAX_V: mass of vertex x
   if (L.mass) {
     __syncthreads();
-    if (!err) m = kp_critical_mass(cv, n, lane, l_rank, l_start, l_next, l_pt);   // (the tie-break classes in l_pt are done with)
+    if (!err) m = kp_critical_mass(cv, n, lane, l_rank, l_start, l_next, l_pt);
   }
   double util = 0.0;
   if (L.util) {
