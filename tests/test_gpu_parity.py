@@ -414,6 +414,39 @@ def test_dense_classes_move_to_four_lanes_per_plan_once_measured():
     assert quad[0] == 0 and quad[1] > 0 and quad[2] > 0 and quad[3] == 0, quad
 
 
+def test_the_fitted_figures_of_the_split_move_plans_between_kernels_and_no_bit():
+    """rpeg_engine_set_split_model: with the single-plan kernel made to look free, or the four-lanes-per-plan kernel,
+    or both dear, other classes change kernels (the task counts say so); every call equals the host build."""
+    from rpeg_amd.engine.runtime import Engine, EngineError
+    cfg, batch = seeded_batch(2, 65536)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+    layouts = []
+    for model in ([40.0, 2.2, 40.0, 1.6, 0.45, 0.65, 1.15, 0.97, 0.98],    # the defaults
+                  [1.0, 0.1, 40.0, 1.6, 0.45, 1.0, 1.15, 0.97, 0.98],      # a plan costs k_plan next to nothing
+                  [40.0, 2.2, 1.0, 0.1, 0.0, 0.65, 1.0, 0.97, 0.98],       # a wavefront of k_quad costs next to nothing
+                  [400.0, 20.0, 4000.0, 20.0, 5.0, 0.1, 2.0, 0.5, 0.5]):   # both dear
+        eng = Engine(cfg.problem)
+        eng.set_split_model(model)
+        try:
+            for call in range(3):
+                out = eng.eval(batch, gate_stale=True)
+                assert np.array_equal(out["mask"], ref["mask"]), (model, call)
+                for k in ("makespan", "peak", "score"):
+                    assert same_bits(out[k], ref[k]), (model, call, k)
+            st = eng.stats()
+            layouts.append((st["single_plan_tasks"], st["quad_tasks"]))
+        finally:
+            eng.close()
+    assert len(set(layouts)) >= 2, layouts
+    assert layouts[1][0] >= layouts[0][0] and layouts[2][1] >= layouts[0][1] and layouts[3][1] == 0, layouts
+    eng = Engine(cfg.problem)
+    with pytest.raises(EngineError):
+        eng.set_split_model([1.0] * 8)
+    with pytest.raises(EngineError):
+        eng.set_split_model([-1.0] + [1.0] * 8)
+    eng.close()
+
+
 @pytest.mark.parametrize("c,n,what", [(3, 65536, "single_plan_tasks"), (5, 40000, "quad_tasks"), (2, 131072, "quad_tasks"),
                                       (1, 20000, "single_plan_tasks"), (3, 32768, "single_plan_tasks"), (2, 20000, "single_plan_tasks")])
 def test_the_measured_split_changes_where_classes_run_and_not_one_bit(c, n, what):
