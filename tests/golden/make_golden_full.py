@@ -5,6 +5,8 @@ Run in the development container only (it needs the read-only reference tree; ho
 configurations 3 and 4):
 
     python tests/golden/make_golden_full.py [--ref /root/reference] [--configs 1,2,3,4] [--workers 6]
+    python tests/golden/make_golden_full.py --configs 5 --limit 16384      (ref_full_cfg5_first16384.json: the first
+                                                  16,384 seeded plans of the annealing configuration, which has no fixed set)
 
 Every plan of a set goes through the reference's own passes exactly as `make_golden.py` sends the first few
 hundred (`unroll`, `lower`, `NodeCostModel`, `schedule`, `Trace.throughput`, `mem_worst_violation`,

@@ -1,4 +1,5 @@
-"""The WHOLE seeded candidate sets of configurations 1-4 (4,096 / 65,536 / 262,144 / 1,048,576 plans) against digests
+"""The WHOLE seeded candidate sets of configurations 1-4 (4,096 / 65,536 / 262,144 / 1,048,576 plans), and the first
+16,384 seeded plans of configuration 5 (the annealing configuration, which has no fixed set), against digests
 the reference itself wrote (tests/golden/ref_full_cfg{c}.json, make_golden_full.py): per chunk of 4,096 plans the CRC
 of every makespan, peak, score (with and without the stale-layout gate) and feasibility flag, the best plan and the 32
 best plans in ranking order.  Bit-exact; a mismatch names its chunk."""
@@ -23,7 +24,7 @@ def _generator():
 
 
 def _gold(c):
-    path = os.path.join(GOLDEN, f"ref_full_cfg{c}.json")
+    path = os.path.join(GOLDEN, f"ref_full_cfg{c}.json" if c != 5 else "ref_full_cfg5_first16384.json")
     if not os.path.exists(path):
         pytest.skip(f"{os.path.basename(path)} has not been generated")
     with open(path) as f:
@@ -46,7 +47,7 @@ def check(gold, plain, gated):
     assert np.array_equal(gated["makespan"].view(np.uint64), plain["makespan"].view(np.uint64))
 
 
-@pytest.mark.parametrize("c", [1, 2, 3, 4])
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_host_build_equals_reference_digest(c):
     """The host build of the kernels' arithmetic headers (the checker of the full-size GPU tests) on the whole set."""
     from oracle.cpu_port import CpuPort
@@ -57,7 +58,7 @@ def test_host_build_equals_reference_digest(c):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("c", [1, 2, 3, 4])
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_full_sets_equal_reference_digest(c):
     from rpeg_amd.engine.runtime import Engine
     gold = _gold(c)
@@ -71,7 +72,7 @@ def test_full_sets_equal_reference_digest(c):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("c", [1, 2, 3, 4])
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
 def test_violating_devices_of_the_first_chunk_equal_reference(c):
     """The device mem_worst_violation names for each plan of the first chunk (4,096 plans), through the drop-in
     `lower` and `mem_worst_violation`: the CRC of all of them equals the one the reference's own run recorded."""
