@@ -304,6 +304,28 @@ __global__ __launch_bounds__(WAVE) void k_peaks(const PrologueLaunch L) {
   }
 }
 
+// The verdicts of the memory-model launch put into the outputs of the scheduling kernels, where that launch ran beside
+// them instead of ahead of them: the gate bits of the mask, the soft OOM penalty and the stale-layout gate of the
+// score (evaluate.py:372-374, 396-401), the same operations in the same order as the scheduling kernels apply them.
+__global__ void k_finish(uint64_t n, const uint32_t* __restrict__ cid, const double* __restrict__ pen,
+                         const uint8_t* __restrict__ gates, uint32_t flags, double* __restrict__ score, uint8_t* __restrict__ mask) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n || cid[i] == KPRO_INVALID) return;   // (a plan the gate rejected has its outputs from k_signature)
+  const uint8_t g = gates[i];
+  const bool stale_ok = (g & RPEG_MASK_STALE_OK) != 0, mem_ok = (g & RPEG_MASK_MEM_OK) != 0;
+  if (mask) {
+    const uint8_t m = mask[i];
+    mask[i] = (uint8_t)((m & ~(RPEG_MASK_STALE_OK | RPEG_MASK_MEM_OK)) | (g & (RPEG_MASK_STALE_OK | RPEG_MASK_MEM_OK)));
+  }
+  if (score) {
+    double sc = score[i];
+    if (sc != sc) return;   // RPEG_MASK_ERROR: the NaN stays
+    if (!mem_ok) sc = sc * pen[i];
+    if ((flags & RPEG_GATE_STALE) && !stale_ok) sc = 0.0;
+    score[i] = sc;
+  }
+}
+
 // The next wave task of a launch whose wavefronts take tasks as they become free (every wavefront ends when the
 // counter has passed the last task), or the next of this block's own.
 __device__ inline uint64_t next_task(const EvalLaunch& L, uint64_t w) {
@@ -1232,9 +1254,11 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // memory model to that kernel, which spreads them over the lanes of a plan's wavefront: the prologue launches work a
   // plan per lane, and a few thousand plans are a few dozen wavefronts that take as long as a full grid would.
   const bool own_prologue = e->state_lanes == 1 || (e->state_lanes == -1 && n <= (uint64_t)e->n_cu * e->one_plan_waves_per_cu);
-  bool prologue_done = false;
-  auto launch_prologue = [&]() -> int {
-    PrologueLaunch G;
+  bool prologue_done = false, peaks_deferred = false;
+  PrologueLaunch G;
+  // defer: only the cost-model launch now; the memory-model launch (k_peaks) goes out beside the scheduling kernels,
+  // which need nothing of it, and k_finish applies its verdicts when all of them are done
+  auto launch_prologue = [&](bool defer) -> int {
     G.P = e->dP; G.vert = plans->vert; G.head = plans->head; G.stride = plans->stride; G.n = n; G.cid = e->d_cid;
     G.uni = e->d_uni;
     for (int q = 0; q < RPEG_MAX_STRUCT; ++q) G.n_uni[q] = e->n_uni[q];
@@ -1245,9 +1269,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     G.peak = peak;
     const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
     hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, s, G);
-    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
+    if (!defer) hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
     HIP_TRY(e, hipGetLastError());
     prologue_done = true;
+    peaks_deferred = defer;
     return 0;
   };
   // classes of the batch: every plan looks its class id up on the device and counts itself; only the
@@ -1278,7 +1303,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       if (!e->ev_counts) HIP_TRY(e, hipEventCreateWithFlags(&e->ev_counts, hipEventDisableTiming));
       HIP_TRY(e, hipEventRecord(e->ev_counts, s));
       if (!own_prologue)
-        if (int rc = launch_prologue()) return rc;
+        if (int rc = launch_prologue(true)) return rc;
       HIP_TRY(e, hipEventSynchronize(e->ev_counts));
     } else {
       HIP_TRY(e, hipStreamSynchronize(s));
@@ -1719,9 +1744,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   L.mass = mass;
   L.prof = nullptr;
   if (!prologue_done && !one)   // (the classes lowered in this call changed what was foreseen for the batch)
-    if (int rc = launch_prologue()) return rc;
+    if (int rc = launch_prologue(false)) return rc;
   if (prologue_done) {
-    L.dur = e->d_dur; L.aux_ovl = e->d_aux_ovl; L.aux_dpne = e->d_aux_dpne; L.aux_pen = e->d_aux_pen; L.aux_mask = e->d_aux_mask;
+    L.dur = e->d_dur; L.aux_ovl = e->d_aux_ovl; L.aux_dpne = e->d_aux_dpne;
+    if (!peaks_deferred) { L.aux_pen = e->d_aux_pen; L.aux_mask = e->d_aux_mask; }
     L.dur_stride = e->cap_n;
   }
   const bool bounded = !one;   // some kernel of this call holds a bounded ready set
@@ -1755,19 +1781,23 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
   // The main kernel is submitted first: it needs 26 KB of LDS per wavefront, and once single-plan wavefronts
   // fill a compute unit its wavefronts only fit in as those retire.
-  if (n_solo || n_quad_waves) {
+  // The memory-model launch, where it was deferred: on k_quad's stream when that kernel has nothing to do in this call
+  // (the launch then runs beside all scheduling kernels), else behind the main kernel on the caller's stream, where
+  // it runs beside the tails of the two other kernels.
+  const bool peaks_aside = peaks_deferred && !n_quad_waves;
+  if (n_solo || n_quad_waves || peaks_aside) {
     if (!e->s2) {
       if (int rc = side_streams(e, &e->s2, nullptr)) return rc;
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_fork, hipEventDisableTiming));
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join, hipEventDisableTiming));
     }
-    if (n_quad_waves && !e->s3) {
+    if ((n_quad_waves || peaks_aside) && !e->s3) {
       if (int rc = side_streams(e, nullptr, &e->s3)) return rc;
       HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join3, hipEventDisableTiming));
     }
     // (the three launches back to back: every call between them delays the start of the later kernels)
     HIP_TRY(e, hipEventRecord(e->ev_fork, s));
-    if (n_quad_waves) HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
+    if (n_quad_waves || peaks_aside) HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
     if (n_solo) HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
   }
   auto launch_quad = [&]() -> int {   // the four-lanes-per-plan wavefronts, beside the main kernel
@@ -1817,7 +1847,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
                        kp_lds_bytes(e->max_nodes, e->max_slots), e->s2, S);
     HIP_TRY(e, hipGetLastError());
   }
-  if (n_quad_waves) HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
+  if (peaks_deferred) {
+    const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
+    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, peaks_aside ? e->s3 : s, G);
+    HIP_TRY(e, hipGetLastError());
+  }
+  if (n_quad_waves || peaks_aside) HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
   if (n_solo) HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
   // (after the submission of k_plan, which is the longer of the two kernels and should not wait for this one)
   if (short_list && n_waves) {   // the plans whose ready list outgrew the short one, with the full one
@@ -1835,8 +1870,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     hipLaunchKernelGGL(k_eval<0>, dim3(std::min<unsigned>(grid, (unsigned)e->n_cu * 2u)), dim3(WAVE), lds_full, s, F);
     HIP_TRY(e, hipGetLastError());
   }
-  if (n_quad_waves) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join3, 0));
+  if (n_quad_waves || peaks_aside) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join3, 0));
   if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
+  if (peaks_deferred) {   // (before k_eval_limit, whose plans get their final outputs from that kernel itself)
+    hipLaunchKernelGGL(k_finish, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_aux_pen, e->d_aux_mask, flags, score, mask);
+    HIP_TRY(e, hipGetLastError());
+  }
   if (bounded) {   // the plans flagged by the kernels above, without a bound on the ready set (ends at once when there is none)
     EvalLaunch U = L;
     U.queue = nullptr;

@@ -67,6 +67,8 @@ struct EvalLaunch {              // uniform launch parameters
   const uint64_t* aux_dpne = nullptr;  // PlanMasks::dpne
   const double* aux_pen = nullptr;     // factor of the soft OOM penalty, 1.0 where the plan fits
   const uint8_t* aux_mask = nullptr;   // RPEG_MASK_VALID | _STALE_OK | _MEM_OK
+                                       // (both null while `dur` is set: the kernel writes the score without penalty and
+                                       // gate and sets both gate bits; k_finish puts the verdicts in afterwards)
   uint64_t dur_stride = 0;
   uint32_t* done = nullptr;      // k_plan only: done[w] = done_tag once the outputs of wave task w are written (a release
   uint32_t done_tag = 0;         // store at system scope, for a host that polls pinned memory instead of waiting for the
@@ -229,8 +231,9 @@ __device__ inline void ke_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   // the table of the slot universe: the prologue launches left them by plan index (one gather each, all in flight at
   // once); the durations go into this lane's rows of the state, where the loops below read them coalesced.
   const uint64_t ovl = L.aux_ovl[pi], dpne = L.aux_dpne[pi];
-  const double pen = L.aux_pen[pi];
-  const uint8_t gates = L.aux_mask[pi];
+  // (null: the memory-model launch runs beside this kernel, and the launch that ends the call applies its verdicts)
+  const double pen = L.aux_pen ? L.aux_pen[pi] : 1.0;
+  const uint8_t gates = L.aux_mask ? L.aux_mask[pi] : (uint8_t)(RPEG_MASK_VALID | RPEG_MASK_STALE_OK | RPEG_MASK_MEM_OK);
   KE_STAMP(1);
   bool err = cv.h->error != 0;
   {   // a slot whose duration the reference could not compute (division by zero) is NaN

@@ -780,8 +780,8 @@ __device__ inline void kp_eval_plan(const EvalLaunch& L, const uint64_t w, const
     err = err || __ballot(bad) != 0ull;
     pm.ovl = L.aux_ovl[sp];
     pm.dpne = L.aux_dpne[sp];
-    pen = L.aux_pen[sp];
-    const uint8_t gates = L.aux_mask[sp];
+    pen = L.aux_pen ? L.aux_pen[sp] : 1.0;
+    const uint8_t gates = L.aux_mask ? L.aux_mask[sp] : (uint8_t)(RPEG_MASK_VALID | RPEG_MASK_STALE_OK | RPEG_MASK_MEM_OK);
     stale_ok = (gates & RPEG_MASK_STALE_OK) != 0;
     mem_ok = (gates & RPEG_MASK_MEM_OK) != 0;
     __syncthreads();

@@ -137,8 +137,8 @@ __device__ inline void kq_eval_wave(const EvalLaunch& L, uint64_t w, uint8_t* ld
   // pair relations, penalty factor and gate bits of this plan and the durations of its class's slots (out of the table
   // of the slot universe) come from the prologue launches, by plan index
   const uint64_t ovl = L.aux_ovl[pi], dpne = L.aux_dpne[pi];
-  const double pen = L.aux_pen[pi];
-  const uint8_t gates = L.aux_mask[pi];
+  const double pen = L.aux_pen ? L.aux_pen[pi] : 1.0;
+  const uint8_t gates = L.aux_mask ? L.aux_mask[pi] : (uint8_t)(RPEG_MASK_VALID | RPEG_MASK_STALE_OK | RPEG_MASK_MEM_OK);
   KE_STAMP(1);
   bool err = cv.h->error != 0;
   {   // a slot whose duration the reference could not compute (division by zero) is NaN; a share by each lane
