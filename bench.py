@@ -286,6 +286,7 @@ def main():
         eng.eval_device(db, out)
         torch.cuda.synchronize()
         each.append((time.perf_counter() - t0) * 1e3)
+    host_us = eng.host_us()   # of the last of those calls
     each.sort()
     spread = {"min": each[0], "median": each[len(each) // 2], "max": each[-1],
               "note": "ms per step over the same number of steps run again, each synchronised on its own"}
@@ -391,6 +392,7 @@ def main():
         "metric": "cost-model plan evals/sec on 1 MI355X",
         "value": value, "unit": "plan evals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "ms_per_step_spread": spread, "host_ms_in_calls_per_step": host_s / args.steps * 1e3,
+        "host_us_of_a_call": host_us,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64", "data": "synthetic",
         "config": {"workload": cfg.name, "n_plans": n, "seed": 42, "K_eval": cfg.problem.K_eval,

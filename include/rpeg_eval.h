@@ -439,6 +439,13 @@ int rpeg_sa_propose(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t what,
    in [2]), [7] wave tasks of the four-lanes-per-plan kernel (included in [2]). */
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
 
+/* Host time of the last rpeg_eval_batch call that laid its batch out, in microseconds of the steady clock: [0] from
+   the call to the end of the launches behind the gate (signature kernel, copies of the counts, cost-model launch),
+   [1] the wait for the class counts, [2] the layout of the batch, the split between the kernels and the copy of the
+   tables, [3] scatter, fork, the scheduling launches, join and the launches that end the call.  A measurement aid with
+   no counterpart in the reference. */
+int rpeg_engine_host_us(const rpeg_engine_t* e, double* out, int32_t n);
+
 /* Where the evaluation kernel keeps the scheduler state of a plan (ready time, rank and remaining
    in-degree per node, duration per slot).  lanes = 0: in an HBM workspace, 64 plans per wavefront (the
    throughput layout).  lanes = 8, 16, 32 or 64: in LDS, that many plans per wavefront (the latency

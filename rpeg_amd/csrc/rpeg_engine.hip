@@ -15,6 +15,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -685,6 +686,7 @@ struct rpeg_engine_s {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   double last_ms = -1.0;
   uint64_t stats[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  double host_us[4] = {0, 0, 0, 0};   // host time of the last laid-out rpeg_eval_batch call: rpeg_engine_host_us
   int n_cu = 256;
   uint8_t* static_ptr = nullptr;    // this device's copy of the file-scope scratch array (rpeg_eval_batch_static)
   uint32_t* h_static = nullptr;     // pinned: the counters of that array, read back after a call
@@ -1275,6 +1277,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     peaks_deferred = defer;
     return 0;
   };
+  const auto t_call = std::chrono::steady_clock::now();
+  auto t_counts = t_call, t_waited = t_call;
   // classes of the batch: every plan looks its class id up on the device and counts itself; only the
   // per-class counts come back.  Plans of classes not lowered yet make the call take the slow round:
   // their signatures are read back, the classes are lowered on the host, the tables are rebuilt.
@@ -1304,7 +1308,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       HIP_TRY(e, hipEventRecord(e->ev_counts, s));
       if (!own_prologue)
         if (int rc = launch_prologue(true)) return rc;
+      t_counts = std::chrono::steady_clock::now();
       HIP_TRY(e, hipEventSynchronize(e->ev_counts));
+      t_waited = std::chrono::steady_clock::now();
     } else {
       HIP_TRY(e, hipStreamSynchronize(s));
     }
@@ -1689,6 +1695,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   if (n_host_tasks && !tasks_in_block) HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, (size_t)n_host_tasks * 4, hipMemcpyHostToDevice, s));
   if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
+  const auto t_laid = std::chrono::steady_clock::now();
   hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
                      d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted, e->d_queues, e->d_limit);
   HIP_TRY(e, hipGetLastError());
@@ -1882,6 +1889,16 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     hipLaunchKernelGGL(k_eval_limit, dim3(e->limit_grid), dim3(WAVE), 0, s, U, e->d_limit_ws);
     HIP_TRY(e, hipGetLastError());
   }
+  {
+    const auto t_end = std::chrono::steady_clock::now();
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) {
+      return std::chrono::duration<double, std::micro>(b - a).count();
+    };
+    e->host_us[0] = us(t_call, t_counts);    // gate and signature launch, copies of the counts, prologue launch
+    e->host_us[1] = us(t_counts, t_waited);  // the wait for the counts
+    e->host_us[2] = us(t_waited, t_laid);    // layout of the batch and the split between the kernels, tables up
+    e->host_us[3] = us(t_laid, t_end);       // scatter, fork, the scheduling launches, join, the launches that end the call
+  }
   if (e->timing) {
     HIP_TRY(e, hipEventRecord(e->ev1, s));
     HIP_TRY(e, hipEventSynchronize(e->ev1));
@@ -1893,6 +1910,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
 }
 
 extern "C" {
+
+int rpeg_engine_host_us(const rpeg_engine_t* e, double* out, int32_t n) {
+  if (!e || !out) return -1;
+  for (int i = 0; i < n && i < 4; ++i) out[i] = e->host_us[i];
+  return 0;
+}
 
 // rpeg_eval_batch for callers that cannot allocate: every intermediate of the call lives in the file-scope
 // scratch array of this device, and the call makes no hipMalloc / hipFree.  One plan per wavefront (k_plan).

@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_sa_groups", "rpeg_engine_set_split_model", "rpeg_engine_set_quad_share", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_sa_groups", "rpeg_engine_host_us", "rpeg_engine_set_split_model", "rpeg_engine_set_quad_share", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
            "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static", "rpeg_plan_detail",
            "rpeg_lower_plan")
 
@@ -83,6 +83,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_last_kernel_ms.argtypes = [vp]
     lib.rpeg_engine_set_state_lanes.restype = C.c_int
     lib.rpeg_engine_set_state_lanes.argtypes = [vp, i32]
+    lib.rpeg_engine_host_us.restype = C.c_int
+    lib.rpeg_engine_host_us.argtypes = [vp, vp, i32]
     lib.rpeg_engine_set_split_model.restype = C.c_int
     lib.rpeg_engine_set_split_model.argtypes = [vp, vp, i32]
     lib.rpeg_engine_set_sa_groups.restype = C.c_int
@@ -211,6 +213,12 @@ class Engine:
         """-1 automatic; 0 scheduler state in HBM (64 plans per wavefront); 8/16/32/64 state in LDS; 1 a plan per
         wavefront; 4 four lanes per plan."""
         self._check(self.lib.rpeg_engine_set_state_lanes(self._h, int(lanes)), "rpeg_engine_set_state_lanes")
+
+    def host_us(self) -> Dict[str, float]:
+        """Host time of the last laid-out `eval_device` call, microseconds (rpeg_engine_host_us)."""
+        v = np.zeros(4)
+        self._check(self.lib.rpeg_engine_host_us(self._h, v.ctypes.data, 4), "rpeg_engine_host_us")
+        return dict(launch_gate=float(v[0]), wait_counts=float(v[1]), layout_and_split=float(v[2]), launch_schedulers=float(v[3]))
 
     def set_split_model(self, values):
         """The nine fitted figures of the split between the scheduling kernels (rpeg_engine_set_split_model)."""
