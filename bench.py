@@ -35,9 +35,9 @@ ALG_FLOPS = {1: 3697.0, 2: 2165.3, 3: 6502.9, 4: 1245.8, 5: 4155.6}
 # (FETCH_SIZE / WRITE_SIZE scaled by a 256 MiB copy) and instructions issued per plan (SQ_INSTS_VALU + SALU + LDS +
 # VMEM_RD + VMEM_WR of the evaluation kernels / plans).
 MEASURED = {
-    2: dict(layout=(6345, 17648, 0, 4815, 590), traffic=211.2e6, instructions_per_plan=3227.3),
-    3: dict(layout=(24495, 29984, 0, 20184, 0), traffic=4671.1e6, instructions_per_plan=None),
-    4: dict(layout=(16396, 14640, 0, 6, 0), traffic=1601.2e6, instructions_per_plan=None),
+    2: dict(layout=(6330, 17648, 0, 4815, 574), traffic=209.8e6, instructions_per_plan=3157.5),
+    3: dict(layout=(24672, 29984, 0, 20364, 0), traffic=4639.9e6, instructions_per_plan=None),
+    4: dict(layout=(16396, 14640, 0, 6, 0), traffic=1547.6e6, instructions_per_plan=None),
 }
 
 
