@@ -11,11 +11,8 @@
 #define RPEG_LOWER_H
 
 #include <cstring>
-#include <map>
-#include <set>
 #include <stdexcept>
 #include <string>
-#include <tuple>
 #include <utility>
 #include <vector>
 
@@ -73,27 +70,53 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   const int nv = st.n_vertex, K = P.K_eval, split = sg.split();
   const int nph = split > 0 ? P.n_phase[split] : 0;
 
+  // (A class is lowered on the critical path of the first call that meets it: flat arrays and one small open-addressing
+  // table instead of node-based containers; the orders -- of nodes, of edges, of slots -- are the reference's.)
   std::vector<LoweredNode> nodes;
   std::vector<std::pair<int, int>> edges;
-  std::set<std::pair<int, int>> seen;
+  nodes.reserve(512);
+  edges.reserve(1024);
+  std::vector<uint64_t> seen(2048, ~0ull);   // the edges met so far, keyed by (from << 32 | to)
+  size_t n_seen = 0;
+  auto seen_insert = [&](uint64_t key) {   // true when the key is new
+    if (2 * (n_seen + 1) > seen.size()) {
+      std::vector<uint64_t> old(seen.size() * 2, ~0ull);
+      old.swap(seen);
+      for (uint64_t k : old)
+        if (k != ~0ull) {
+          size_t h = (size_t)((k * 0x9E3779B97F4A7C15ull) >> 20) & (seen.size() - 1);
+          while (seen[h] != ~0ull) h = (h + 1) & (seen.size() - 1);
+          seen[h] = k;
+        }
+    }
+    size_t h = (size_t)((key * 0x9E3779B97F4A7C15ull) >> 20) & (seen.size() - 1);
+    while (seen[h] != ~0ull) {
+      if (seen[h] == key) return false;
+      h = (h + 1) & (seen.size() - 1);
+    }
+    seen[h] = key;
+    ++n_seen;
+    return true;
+  };
   std::vector<SlotDesc> slots;
-  std::map<std::tuple<int, int, int, int>, int> slot_of;
+  slots.reserve(64);
   auto slot = [&](SlotType t, int a, int b, int q) {
-    auto key = std::make_tuple((int)t, a, b, q);
-    auto it = slot_of.find(key);
-    if (it != slot_of.end()) return it->second;
+    const SlotDesc want{(uint8_t)t, (uint8_t)a, (uint8_t)b, (uint8_t)q};
+    for (size_t k = 0; k < slots.size(); ++k)
+      if (slots[k].type == want.type && slots[k].a == want.a && slots[k].b == want.b && slots[k].q == want.q) return (int)k;
     if (slots.size() >= 255) throw std::runtime_error("too many duration slots");
-    slots.push_back(SlotDesc{(uint8_t)t, (uint8_t)a, (uint8_t)b, (uint8_t)q});
-    return slot_of[key] = (int)slots.size() - 1;
+    slots.push_back(want);
+    return (int)slots.size() - 1;
   };
   auto add_edge = [&](int a, int b) {
-    if (seen.insert({a, b}).second) edges.push_back({a, b});
+    if (seen_insert((uint64_t)(uint32_t)a << 32 | (uint32_t)b)) edges.push_back({a, b});
   };
   auto add_node = [&](const LoweredNode& n) { nodes.push_back(n); return (int)nodes.size() - 1; };
 
-  // per (vertex, step): the unsplit node, generation sub-nodes, inference sub-nodes
-  std::vector<std::vector<int>> base(nv, std::vector<int>(K, -1));
-  std::vector<std::vector<std::vector<int>>> gsub(nv, std::vector<std::vector<int>>(K)), isub = gsub;
+  // per (vertex, step): the unsplit node; the first of the generation / inference sub-nodes (they are created one
+  // after the other, so sub-node q of a vertex and step is first + q; -1: none)
+  std::vector<int> base((size_t)nv * K, -1), gfirst((size_t)nv * K, -1), ifirst((size_t)nv * K, -1);
+  auto at = [&](int v, int k) { return (size_t)v * K + k; };
 
   // which generation vertices split: quantile phases exist and some inference consumer is disjoint
   std::vector<bool> gen_split(nv, false);
@@ -109,11 +132,13 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   for (int k = 0; k < K; ++k)
     for (int v = 0; v < nv; ++v) {
       if (nph > 0 && st.vertex[v].role == RPEG_ROLE_GEN && gen_split[v]) {
-        for (int q = 0; q < nph; ++q)
-          gsub[v][k].push_back(add_node({0, v, k, q, v, v, 0, st.vertex[v].model, slot(SLOT_OP_SUB, v, 0, q), true}));
-        for (int q = 1; q < nph; ++q) add_edge(gsub[v][k][q - 1], gsub[v][k][q]);
+        for (int q = 0; q < nph; ++q) {
+          const int id = add_node({0, v, k, q, v, v, 0, st.vertex[v].model, slot(SLOT_OP_SUB, v, 0, q), true});
+          if (q == 0) gfirst[at(v, k)] = id;
+        }
+        for (int q = 1; q < nph; ++q) add_edge(gfirst[at(v, k)] + q - 1, gfirst[at(v, k)] + q);
       } else {
-        base[v][k] = add_node({0, v, k, -1, v, v, 0, st.vertex[v].model, slot(SLOT_OP_UNSPLIT, v, 0, 0), true});
+        base[at(v, k)] = add_node({0, v, k, -1, v, v, 0, st.vertex[v].model, slot(SLOT_OP_UNSPLIT, v, 0, 0), true});
       }
     }
 
@@ -130,7 +155,7 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   for (int k = 0; k < K; ++k)
     for (int e = 0; e < st.n_edge; ++e) {
       const rpeg_edge_t& ed = st.edge[e];
-      if (!gsub[ed.src][k].empty() && st.vertex[ed.dst].role == RPEG_ROLE_INF) pass1.push_back({k, e});
+      if (gfirst[at(ed.src, k)] >= 0 && st.vertex[ed.dst].role == RPEG_ROLE_INF) pass1.push_back({k, e});
       else pass2.push_back({k, e});
     }
   pass1.insert(pass1.end(), pass2.begin(), pass2.end());
@@ -138,40 +163,43 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
     const int k = ke.first, e = ke.second;
     const rpeg_edge_t& ed = st.edge[e];
     const int u = ed.src, v = ed.dst;
-    const bool src_gen_split = !gsub[u][k].empty();
+    const int gu = gfirst[at(u, k)];
+    const bool src_gen_split = gu >= 0;
     if (src_gen_split && st.vertex[v].role == RPEG_ROLE_INF) {
       if (sg.disjoint(u, v)) {
-        if (isub[v][k].empty()) {
-          if (base[v][k] >= 0) { nodes[base[v][k]].alive = false; base[v][k] = -1; }
-          for (int q = 0; q < nph; ++q)
-            isub[v][k].push_back(add_node({0, v, k, q, v, v, 0, st.vertex[v].model, slot(SLOT_OP_SUB, v, 0, q), true}));
-          for (int q = 1; q < nph; ++q) add_edge(isub[v][k][q - 1], isub[v][k][q]);
+        if (ifirst[at(v, k)] < 0) {
+          if (base[at(v, k)] >= 0) { nodes[base[at(v, k)]].alive = false; base[at(v, k)] = -1; }
+          for (int q = 0; q < nph; ++q) {
+            const int id = add_node({0, v, k, q, v, v, 0, st.vertex[v].model, slot(SLOT_OP_SUB, v, 0, q), true});
+            if (q == 0) ifirst[at(v, k)] = id;
+          }
+          for (int q = 1; q < nph; ++q) add_edge(ifirst[at(v, k)] + q - 1, ifirst[at(v, k)] + q);
         }
-        for (int q = 0; q < nph; ++q) edge_or_comm(gsub[u][k][q], isub[v][k][q], e, q);
+        for (int q = 0; q < nph; ++q) edge_or_comm(gu + q, ifirst[at(v, k)] + q, e, q);
       } else {
-        edge_or_comm(gsub[u][k].back(), base[v][k], e, -1);
+        edge_or_comm(gu + nph - 1, base[at(v, k)], e, -1);
       }
     } else if (src_gen_split) {
-      edge_or_comm(gsub[u][k].back(), base[v][k], e, -1);
-    } else if (!isub[u][k].empty()) {
-      if (base[v][k] < 0) throw std::runtime_error("destination node of a split inference edge not found");
-      edge_or_comm(isub[u][k].back(), base[v][k], e, -1);
+      edge_or_comm(gu + nph - 1, base[at(v, k)], e, -1);
+    } else if (ifirst[at(u, k)] >= 0) {
+      if (base[at(v, k)] < 0) throw std::runtime_error("destination node of a split inference edge not found");
+      edge_or_comm(ifirst[at(u, k)] + nph - 1, base[at(v, k)], e, -1);
     } else {
-      if (base[u][k] < 0 || base[v][k] < 0) throw std::runtime_error("edge endpoint missing");
-      edge_or_comm(base[u][k], base[v][k], e, -1);
+      if (base[at(u, k)] < 0 || base[at(v, k)] < 0) throw std::runtime_error("edge endpoint missing");
+      edge_or_comm(base[at(u, k)], base[at(v, k)], e, -1);
     }
   }
 
   // 3) within-step weight reshards between consecutive vertices of one trainable model (lower.py:626-681)
   auto last_of = [&](int v, int k) {
-    if (!gsub[v][k].empty()) return gsub[v][k].back();
-    if (!isub[v][k].empty()) return isub[v][k].back();
-    return base[v][k];
+    if (gfirst[at(v, k)] >= 0) return gfirst[at(v, k)] + nph - 1;
+    if (ifirst[at(v, k)] >= 0) return ifirst[at(v, k)] + nph - 1;
+    return base[at(v, k)];
   };
   auto first_of = [&](int v, int k) {
-    if (!gsub[v][k].empty()) return gsub[v][k].front();
-    if (!isub[v][k].empty()) return isub[v][k].front();
-    return base[v][k];
+    if (gfirst[at(v, k)] >= 0) return gfirst[at(v, k)];
+    if (ifirst[at(v, k)] >= 0) return ifirst[at(v, k)];
+    return base[at(v, k)];
   };
   std::vector<bool> resharded(nv, false);
   auto make_reshard = [&](int a, int b, int model) {
@@ -201,7 +229,7 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
       const int t = sg.tau(pb.tau_slot);
       if (k <= t) continue;
       const int ks = k - (t + 1) > 0 ? k - (t + 1) : 0;
-      const int a = base[pb.src][ks];
+      const int a = base[at(pb.src, ks)];
       const int b = first_of(pb.dst, k);
       if (a < 0 || b < 0) throw std::runtime_error("publication endpoint missing");
       if (resharded[pb.dst]) continue;
@@ -216,16 +244,21 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
 
   // 4b) lifetime barriers between colocated trainable layouts (lower.py:730-793)
   {
-    std::vector<std::vector<int>> preds(nodes.size()), succs(nodes.size());
-    for (auto& ed : edges) { preds[ed.second].push_back(ed.first); succs[ed.first].push_back(ed.second); }
+    // operator predecessors / successors of the reshard nodes: how many, and one of them
+    std::vector<int> n_po(nodes.size(), 0), n_so(nodes.size(), 0), a_po(nodes.size(), -1), a_so(nodes.size(), -1);
+    bool any_reshard = false;
+    for (auto& nd : nodes) any_reshard = any_reshard || (nd.alive && nd.kind == 2);
+    if (any_reshard)
+      for (auto& ed : edges) {
+        if (nodes[ed.second].kind == 2 && nodes[ed.first].kind == 0) { ++n_po[ed.second]; a_po[ed.second] = ed.first; }
+        if (nodes[ed.first].kind == 2 && nodes[ed.second].kind == 0) { ++n_so[ed.first]; a_so[ed.first] = ed.second; }
+      }
     struct Tr { int node, pred, succ; };
     std::vector<Tr> to_train, to_serving;
-    for (int i = 0; i < (int)nodes.size(); ++i) {
+    for (int i = 0; any_reshard && i < (int)nodes.size(); ++i) {
       if (!nodes[i].alive || nodes[i].kind != 2) continue;
-      std::vector<int> po, so;
-      for (int x : preds[i]) if (nodes[x].kind == 0) po.push_back(x);
-      for (int x : succs[i]) if (nodes[x].kind == 0) so.push_back(x);
-      if (po.size() != 1 || so.size() != 1) continue;
+      if (n_po[i] != 1 || n_so[i] != 1) continue;
+      const int po[1] = {a_po[i]}, so[1] = {a_so[i]};
       const LoweredNode &pn = nodes[po[0]], &sn = nodes[so[0]];
       if (pn.model != sn.model || !st.trainable[pn.model]) continue;
       const int pr = st.vertex[pn.vertex].role, sr = st.vertex[sn.vertex].role;
@@ -245,6 +278,8 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   // compact to alive nodes, keep order
   std::vector<int> remap(nodes.size(), -1);
   LoweredClass out;
+  out.nodes.reserve(nodes.size());
+  out.edges.reserve(edges.size());
   for (int i = 0; i < (int)nodes.size(); ++i)
     if (nodes[i].alive) { remap[i] = (int)out.nodes.size(); out.nodes.push_back(nodes[i]); }
   for (auto& ed : edges) {
@@ -255,19 +290,33 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   if (n > 65535) throw std::runtime_error("too many lowered nodes");
 
   // adjacency in edge order, in-degrees, Kahn order (scheduler.py:28-67)
-  std::vector<std::vector<int>> adj(n);
+  std::vector<int> adj_beg(n + 1, 0), adj_to(out.edges.size(), 0);   // (successors of a node in the order of its edges)
   std::vector<int> indeg(n, 0);
-  for (auto& ed : out.edges) { adj[ed.first].push_back(ed.second); ++indeg[ed.second]; }
+  for (auto& ed : out.edges) { ++adj_beg[ed.first + 1]; ++indeg[ed.second]; }
+  for (int i = 0; i < n; ++i) adj_beg[i + 1] += adj_beg[i];
+  {
+    std::vector<int> cur(adj_beg.begin(), adj_beg.end() - 1);
+    for (auto& ed : out.edges) adj_to[cur[ed.first]++] = ed.second;
+  }
   std::vector<int> topo, deg = indeg;
+  topo.reserve(n);
   for (int i = 0; i < n; ++i) if (deg[i] == 0) topo.push_back(i);
   for (size_t h = 0; h < topo.size(); ++h)
-    for (int w : adj[topo[h]]) if (--deg[w] == 0) topo.push_back(w);
+    for (int j = adj_beg[topo[h]]; j < adj_beg[topo[h] + 1]; ++j) if (--deg[adj_to[j]] == 0) topo.push_back(adj_to[j]);
   const bool cycle = (int)topo.size() != n;
 
-  // chain groups: quantile sub-nodes of one (vertex, step) (scheduler.py:369-378)
-  std::map<std::pair<int, int>, std::vector<int>> chains;
+  // chain groups: quantile sub-nodes of one (vertex, step) (scheduler.py:369-378), the groups in the order of
+  // (vertex, step), the members of a group in node order
+  std::vector<int> chain_beg((size_t)nv * K + 1, 0), chain_of;
   for (int i = 0; i < n; ++i)
-    if (out.nodes[i].kind == 0 && out.nodes[i].sub >= 0) chains[{out.nodes[i].vertex, out.nodes[i].step}].push_back(i);
+    if (out.nodes[i].kind == 0 && out.nodes[i].sub >= 0) ++chain_beg[at(out.nodes[i].vertex, out.nodes[i].step) + 1];
+  for (size_t k = 0; k < (size_t)nv * K; ++k) chain_beg[k + 1] += chain_beg[k];
+  chain_of.assign(chain_beg.back(), 0);
+  {
+    std::vector<int> cur(chain_beg.begin(), chain_beg.end() - 1);
+    for (int i = 0; i < n; ++i)
+      if (out.nodes[i].kind == 0 && out.nodes[i].sub >= 0) chain_of[cur[at(out.nodes[i].vertex, out.nodes[i].step)]++] = i;
+  }
 
   // vertex order of first appearance among operator nodes (dict orders of memory.py:763-808)
   uint8_t vorder[8] = {0, 1, 2, 3, 4, 5, 6, 7};
@@ -301,14 +350,17 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   std::vector<NodeRec> recs(n);
   std::vector<uint16_t> succ, init, topo16, gmember;
   std::vector<GroupRec> groups;
+  succ.reserve(out.edges.size());
+  topo16.reserve(n);
   for (int i = 0; i < n; ++i) {
     const LoweredNode& nd = out.nodes[i];
     NodeRec r{};
     r.succ_begin = (uint16_t)succ.size();
-    if (adj[i].size() > 255 || indeg[i] > 255 || succ.size() + adj[i].size() > 65535)
+    const int n_adj = adj_beg[i + 1] - adj_beg[i];
+    if (n_adj > 255 || indeg[i] > 255 || succ.size() + (size_t)n_adj > 65535)
       throw std::runtime_error("node degree out of range");
-    r.n_succ = (uint8_t)adj[i].size();
-    for (int w : adj[i]) succ.push_back((uint16_t)w);
+    r.n_succ = (uint8_t)n_adj;
+    for (int j = adj_beg[i]; j < adj_beg[i + 1]; ++j) succ.push_back((uint16_t)adj_to[j]);
     r.slot = (uint8_t)nd.slot;
     r.indeg = (uint8_t)indeg[i];
     if (nd.kind == 0) {
@@ -331,9 +383,10 @@ inline LoweredClass lower_class(const rpeg_problem_t& P, uint64_t sig_bits) {
   }
   for (int v : topo) topo16.push_back((uint16_t)v);
   topo16.resize(n, 0);
-  for (auto& kv : chains) {
-    groups.push_back(GroupRec{(uint16_t)gmember.size(), (uint16_t)kv.second.size()});
-    for (int i : kv.second) gmember.push_back((uint16_t)i);
+  for (size_t k = 0; k < (size_t)nv * K; ++k) {
+    if (chain_beg[k + 1] == chain_beg[k]) continue;
+    groups.push_back(GroupRec{(uint16_t)gmember.size(), (uint16_t)(chain_beg[k + 1] - chain_beg[k])});
+    for (int j = chain_beg[k]; j < chain_beg[k + 1]; ++j) gmember.push_back((uint16_t)chain_of[j]);
   }
   // every slot's place in the structure's slot universe
   std::vector<uint8_t> umap(slots.size(), 0);
