@@ -2380,7 +2380,9 @@ int host_small_collect(rpeg_engine_t* e, HostLane& ln, double* makespan, double*
         if (j == m) { seen = true; break; }
         // a launch that does not come to an end is the stream's to report
         if ((spins & 0xFFFFu) == 0xFFFFu && std::chrono::steady_clock::now() - t0 > std::chrono::seconds(2)) break;
+#if defined(__x86_64__) || defined(__i386__)
         __builtin_ia32_pause();
+#endif
       }
     }
     if (!seen) HIP_TRY(e, hipStreamSynchronize(s));
