@@ -82,7 +82,7 @@ def main() -> None:
         print("   longest tasks (nodes, start us, duration us):", [(int(N[k]), round(float(S[k]), 1), round(float(d[k]), 1)) for k in o])
         o = np.argsort(-E)[:6]
         print("   last to end   (nodes, start us, duration us):", [(int(N[k]), round(float(S[k]), 1), round(float(d[k]), 1)) for k in o])
-        if not args.sections or name != "k_eval":   # (the measurement build keeps the section clocks where the phase stamps are)
+        if not args.sections:   # (the measurement build keeps the section clocks where the phase stamps are, in every kernel)
             ph = np.diff(b[sl][ok][:, :7], axis=1) / 100.0
             names = ("plan fields", "durations", "memory model", "ranks", "scheduling", "outputs") if name == "k_eval" else \
                     ("plan fields", "durations", "memory model", "ranks and positions", "scheduling", "outputs") if name == "k_quad" else \
