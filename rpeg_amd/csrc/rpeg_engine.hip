@@ -94,6 +94,45 @@ __global__ void k_fill_u32(uint32_t* p, uint64_t n, uint32_t v) {
   if (i < n) p[i] = v;
 }
 
+// The layout of a call from the pinned buffer the host wrote it to (read in place, sixteen bytes per thread: a copy
+// command ahead of the kernels costs a dozen microseconds before its first byte moves), and the idle marks of the
+// permutation, in one launch.  n_quads: sixteen-byte words of the layout.
+__global__ void k_upload_fill(const uint4* __restrict__ host_src, uint4* __restrict__ dst, uint64_t n_quads, uint32_t* __restrict__ p,
+                              uint64_t n, uint32_t v) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_quads) dst[i] = host_src[i];
+  if (i < n) p[i] = v;
+}
+
+// The counters of the signature kernel, summed over the shards of every class by a block of its own.  The shards'
+// counters become their offsets within the class, in place (k_scatter reads them there); the totals go to the host:
+// written into pinned host memory, then a flag the host polls -- there several microseconds before a copy command
+// behind the kernel would have moved its first byte.  host_count: n_classes totals, the count of the plans of classes
+// not lowered yet, then the KE_NEED_SHARDS running maxima of the ready-list length.
+constexpr int HAND_BLOCK = 1024;
+__global__ __launch_bounds__(HAND_BLOCK) void k_hand_counts(uint32_t* __restrict__ count, const uint32_t* __restrict__ need, uint32_t n_classes,
+                                                            uint32_t shards, uint32_t* __restrict__ host_count, uint32_t* __restrict__ host_flag,
+                                                            uint32_t tag) {
+  for (uint32_t c = threadIdx.x; c < n_classes; c += HAND_BLOCK) {
+    uint32_t* row = count + (size_t)c * shards;
+    uint32_t total = 0;
+    for (uint32_t s0 = 0; s0 < shards; s0 += 8) {   // eight loads in flight
+      uint32_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = s0 + u < shards ? row[s0 + u] : 0u;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < shards) { row[s0 + u] = total; total += v[u]; }
+    }
+    host_count[c] = total;
+  }
+  if (threadIdx.x == 0) host_count[n_classes] = count[(size_t)n_classes * shards];
+  if (threadIdx.x < KE_NEED_SHARDS) host_count[n_classes + 1 + threadIdx.x] = need[threadIdx.x];
+  __threadfence_system();
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(host_flag, tag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Integer validity gate, class signature, class id (open-addressing table of the classes lowered so far)
 // and the per-class plan counts.  Blocks of SIG_BLOCK plans; shard = block mod shards.
 constexpr int SIG_BLOCK = 256, SIG_TABLE = 512;
@@ -148,7 +187,7 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
     const uint8_t* __restrict__ head, uint64_t stride, uint64_t* __restrict__ sig, double* makespan, double* peak,
     double* score, uint8_t* mask, double* mass, const uint64_t* __restrict__ hkey, const uint32_t* __restrict__ hval,
     uint32_t hmask, uint32_t* __restrict__ cid, uint32_t* __restrict__ kidx, uint32_t* __restrict__ count,
-    uint32_t n_classes, uint32_t shards, const uint32_t* __restrict__ need) {
+    uint32_t n_classes, uint32_t shards) {
   // counters met in this block: key, plans of the block, and the block's first arrival index
   __shared__ uint32_t t_key[SIG_TABLE], t_cnt[SIG_TABLE], t_base[SIG_TABLE];
   // plan fields: the gate and the signature index the vertices with run-time values, which would put a
@@ -204,8 +243,6 @@ __global__ __launch_bounds__(SIG_BLOCK) void k_signature(
     if (t_cnt[j]) t_base[j] = atomicAdd(&count[t_key[j]], t_cnt[j]);
   __syncthreads();
   if (key != NONE) kidx[i] = t_base[slot] + local;
-  // the running maxima of the ready-list length ride behind the counters, so that one copy brings both to the host
-  if (blockIdx.x == 0 && threadIdx.x < KE_NEED_SHARDS) count[(size_t)n_classes * shards + 1 + threadIdx.x] = need[threadIdx.x];
 }
 
 // The plan -> class step of the entry point that allocates nothing: validity gate, signature and, through the
@@ -617,6 +654,10 @@ struct rpeg_engine_s {
   // per-class tables of a call, one block on each side: counters per (class, shard), which become the shards'
   // offsets, then first wavefront and plans per wavefront of every class
   uint32_t *d_ccount = nullptr, *h_ccount = nullptr;
+  uint32_t* h_ccount_dev = nullptr;             // the same pinned buffer as the device addresses it
+  uint32_t *h_tot = nullptr, *h_tot_dev = nullptr;   // pinned: per-class totals of a call, written by k_hand_counts
+  uint32_t *h_sigflag = nullptr, *h_sigflag_dev = nullptr;   // pinned word: the tag of the call whose counters are in h_ccount
+  uint32_t sig_tag = 0;
   uint32_t *d_cid = nullptr, *d_kidx = nullptr;   // per plan: class id, arrival index within the class
   std::vector<uint8_t> pool;
   uint8_t* d_pool = nullptr;
@@ -658,6 +699,9 @@ struct rpeg_engine_s {
   hipEvent_t ev_counts = nullptr;               // the class counts of a call have reached the host
   hipStream_t s3 = nullptr;                     // third stream: the four-lanes-per-plan wavefronts (k_quad)
   hipEvent_t ev_join3 = nullptr;
+  hipEvent_t ev_sig = nullptr;                  // the signature kernel of a call is done (its class ids are there)
+  bool layout_ahead = true;                     // prologue, layout and main kernel on k_quad's stream (see `ahead` in eval_batch_impl)
+  int side_dev = 0;                             // device of the side streams
   uint32_t quad_share_pct = 25;                 // share of a full batch that k_quad takes (rpeg_engine_set_quad_share)
   bool quad_attr_set = false;
   int split_heavy = 1;                          // 0: the classes with the largest graphs stay in the main kernel
@@ -767,7 +811,19 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
     }
     e->d_ccount = nullptr; e->ccap = 0;
     HIP_TRY(e, hipMalloc(&e->d_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4));
-    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4));
+    // (the signature kernel writes the counters here itself while the host polls: coherent, and mapped)
+    HIP_TRY(e, hipHostMalloc(&e->h_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4, hipHostMallocCoherent));
+    e->h_ccount_dev = nullptr;
+    HIP_TRY(e, hipHostGetDevicePointer((void**)&e->h_ccount_dev, e->h_ccount, 0));
+    if (e->h_tot) hipHostFree(e->h_tot);
+    e->h_tot = e->h_tot_dev = nullptr;
+    HIP_TRY(e, hipHostMalloc(&e->h_tot, ((size_t)cap + 1 + KE_NEED_SHARDS) * 4, hipHostMallocCoherent));
+    HIP_TRY(e, hipHostGetDevicePointer((void**)&e->h_tot_dev, e->h_tot, 0));
+    if (!e->h_sigflag) {
+      HIP_TRY(e, hipHostMalloc(&e->h_sigflag, 64, hipHostMallocCoherent));
+      std::memset(e->h_sigflag, 0, 64);
+      HIP_TRY(e, hipHostGetDevicePointer((void**)&e->h_sigflag_dev, e->h_sigflag, 0));
+    }
     e->ccap = cap;
   }
   if (ncls > e->cstat_cap) {   // the per-class statistic keeps what it has learned
@@ -1001,6 +1057,8 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   if (e->d_cstat) hipFree(e->d_cstat);
   if (e->d_hkey) { hipFree(e->d_hkey); hipFree(e->d_hval); hipFree(e->d_hoff); }
   if (e->h_static) hipHostFree(e->h_static);
+  if (e->h_sigflag) hipHostFree(e->h_sigflag);
+  if (e->h_tot) hipHostFree(e->h_tot);
   if (e->d_ccount) {
     hipFree(e->d_ccount);
     hipHostFree(e->h_ccount);
@@ -1012,6 +1070,7 @@ void rpeg_engine_destroy(rpeg_engine_t* e) {
   // (the side streams belong to the device, not to the engine: side_streams)
   if (e->s2) { hipStreamSynchronize(e->s2); hipEventDestroy(e->ev_fork); hipEventDestroy(e->ev_join); }
   if (e->s3) { hipStreamSynchronize(e->s3); hipEventDestroy(e->ev_join3); }
+  if (e->ev_sig) hipEventDestroy(e->ev_sig);
   if (e->ev_counts) hipEventDestroy(e->ev_counts);
   e->lane0.release();
   if (e->d_stage) hipFree(e->d_stage);
@@ -1193,6 +1252,35 @@ static int side_streams(rpeg_engine_t* e, hipStream_t* plan_stream, hipStream_t*
   return 0;
 }
 
+// The engine's handles on the two side streams and the events of its forks and joins.
+static int ensure_side(rpeg_engine_t* e) {
+  if (!e->s2) {
+    if (int rc = side_streams(e, &e->s2, nullptr)) return rc;
+    HIP_TRY(e, hipEventCreateWithFlags(&e->ev_fork, hipEventDisableTiming));
+    HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join, hipEventDisableTiming));
+  }
+  if (!e->s3) {
+    if (int rc = side_streams(e, nullptr, &e->s3)) return rc;
+    HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join3, hipEventDisableTiming));
+    HIP_TRY(e, hipEventCreateWithFlags(&e->ev_sig, hipEventDisableTiming));
+    HIP_TRY(e, hipGetDevice(&e->side_dev));
+  }
+  return 0;
+}
+
+// Whether the side streams of the device are this engine's to plan with: it was the last engine that used them (what
+// they still hold is then its own earlier call, which the caller's stream follows anyway), or they are idle.  When
+// another engine of the process is in the middle of a call on them, work put there would wait for that call's kernels.
+static bool side_claim(rpeg_engine_t* e) {
+  static std::mutex mu;
+  static const void* owner[64] = {};
+  std::lock_guard<std::mutex> lock(mu);
+  const void* last = owner[e->side_dev];
+  owner[e->side_dev] = e;
+  if (last == e || last == nullptr) return true;
+  return hipStreamQuery(e->s2) == hipSuccess && hipStreamQuery(e->s3) == hipSuccess;
+}
+
 static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags, double* makespan,
                            double* peak, double* score, uint8_t* mask, double* mass, void* stream) {
   if (!e || !plans) return -1;
@@ -1257,6 +1345,18 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   // plan per lane, and a few thousand plans are a few dozen wavefronts that take as long as a full grid would.
   const bool own_prologue = e->state_lanes == 1 || (e->state_lanes == -1 && n <= (uint64_t)e->n_cu * e->one_plan_waves_per_cu);
   bool prologue_done = false, peaks_deferred = false;
+  // ahead: k_quad's stream becomes the main line of the call -- the cost-model launch goes there as soon as the class
+  // ids are written (beside the hand-over of the counters to the host), the layout and the scatter follow it there
+  // as soon as the host has them, and the main kernel follows those in order; the caller's stream carries k_quad
+  // and joins at the end.  Only when no other engine of the process is using the side streams.
+  bool ahead = false;
+  // (whatever way the call ends, the caller's stream follows what went to k_quad's stream)
+  struct AheadJoin {
+    rpeg_engine_t* e; hipStream_t s; bool* ahead; bool joined = false;
+    ~AheadJoin() {
+      if (*ahead && !joined && e->s3 && e->ev_join3 && hipEventRecord(e->ev_join3, e->s3) == hipSuccess) hipStreamWaitEvent(s, e->ev_join3, 0);
+    }
+  } ahead_join{e, s, &ahead};
   PrologueLaunch G;
   // defer: only the cost-model launch now; the memory-model launch (k_peaks) goes out beside the scheduling kernels,
   // which need nothing of it, and k_finish applies its verdicts when all of them are done
@@ -1270,7 +1370,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     G.aux_pen = e->d_aux_pen; G.aux_mask = e->d_aux_mask;
     G.peak = peak;
     const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
-    hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, s, G);
+    hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, ahead ? e->s3 : s, G);
     if (!defer) hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
     HIP_TRY(e, hipGetLastError());
     prologue_done = true;
@@ -1287,36 +1387,63 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   for (int round = 0;; ++round) {
     if (int rc = ensure_class_tables(e, s)) return rc;
     ncls = (uint32_t)e->cls_sig.size();
+    // (a counter that every block adds to takes the blocks one after the other, ~0.1 us each: no more than about
+    // sixteen blocks per counter, and no more counters than that asks for -- all of them are cleared and summed)
     shards = MAX_SHARDS;
-    while (shards > 1 && (uint64_t)ncls * shards > COUNT_SLOTS) shards >>= 1;
+    while (shards > 1 && ((uint64_t)ncls * shards > COUNT_SLOTS || (uint64_t)shards * 8 * SIG_BLOCK >= n)) shards >>= 1;
     const uint64_t n_count = (uint64_t)ncls * shards + 1;
-    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_count + blk - 1) / blk)), dim3(blk), 0, s, e->d_ccount, n_count, 0u);
-    hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
-                       e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
-                       e->d_kidx, e->d_ccount, ncls, shards, e->d_need);
-    HIP_TRY(e, hipGetLastError());
-    HIP_TRY(e, hipMemcpyAsync(e->h_ccount, e->d_ccount, (n_count + KE_NEED_SHARDS) * 4, hipMemcpyDeviceToHost, s));
     // what earlier launches of the main kernel learned about the classes (pops per dispatch): read in the calls
     // that follow new classes, and now and then afterwards
     const bool read_stat = round == 0 && e->quad_share_pct && ncls && (e->learn_calls > 0 || (e->batch_calls & 63) == 0);
+    // The counters go to the host through k_hand_counts; in the first round the host polls its flag instead of waiting
+    // for the stream, unless a copy of the statistic has to be waited for anyway.
+    const bool handed = round == 0 && !read_stat;
+    const uint32_t tag = ++e->sig_tag ? e->sig_tag : ++e->sig_tag;
+    if (round == 0 && !own_prologue) {
+      if (int rc = ensure_side(e)) return rc;
+      ahead = !e->prof_on && e->layout_ahead && side_claim(e);
+    }
+    if (round > 0 && ahead) HIP_TRY(e, hipStreamSynchronize(e->s3));   // (the cost-model launch reads the class ids)
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_count + blk - 1) / blk)), dim3(blk), 0, s, e->d_ccount, n_count, 0u);
+    hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
+                       e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
+                       e->d_kidx, e->d_ccount, ncls, shards);
+    HIP_TRY(e, hipGetLastError());
+    if (round == 0 && ahead) {   // (before the hand-over: the cost-model launch does not wait for that)
+      HIP_TRY(e, hipEventRecord(e->ev_sig, s));
+      HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_sig, 0));
+    }
+    hipLaunchKernelGGL(k_hand_counts, dim3(1), dim3(HAND_BLOCK), 0, s, e->d_ccount, e->d_need, ncls, shards, e->h_tot_dev, e->h_sigflag_dev, tag);
+    HIP_TRY(e, hipGetLastError());
     if (read_stat) HIP_TRY(e, hipMemcpyAsync(e->cls_pops16.data(), e->d_cstat, (size_t)ncls * 4, hipMemcpyDeviceToHost, s));
     if (round == 0) {
       // Cost model, memory model and gates of every plan: they need the verdict of the gate (which plans to skip)
       // and nothing of the classes, so they run behind the signature kernel while the host waits for the counts
-      // (the event, not the stream) and lays the batch out.
+      // (the flag or the event, not the stream) and lays the batch out.
       if (!e->ev_counts) HIP_TRY(e, hipEventCreateWithFlags(&e->ev_counts, hipEventDisableTiming));
       HIP_TRY(e, hipEventRecord(e->ev_counts, s));
       if (!own_prologue)
         if (int rc = launch_prologue(true)) return rc;
       t_counts = std::chrono::steady_clock::now();
-      HIP_TRY(e, hipEventSynchronize(e->ev_counts));
+      bool seen = false;
+      if (handed) {
+        for (uint64_t spins = 0;; ++spins) {
+          if (__atomic_load_n(e->h_sigflag, __ATOMIC_ACQUIRE) == tag) { seen = true; break; }
+          // a launch that does not come to an end is the stream's to report
+          if ((spins & 0xFFFFu) == 0xFFFFu && std::chrono::steady_clock::now() - t_counts > std::chrono::seconds(2)) break;
+#if defined(__x86_64__) || defined(__i386__)
+          __builtin_ia32_pause();
+#endif
+        }
+      }
+      if (!seen) HIP_TRY(e, hipEventSynchronize(e->ev_counts));
       t_waited = std::chrono::steady_clock::now();
     } else {
       HIP_TRY(e, hipStreamSynchronize(s));
     }
     if (read_stat && e->learn_calls > 0) --e->learn_calls;
-    for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_ccount[n_count + q]);
-    if (e->h_ccount[n_count - 1] == 0) break;
+    for (int q = 0; q < KE_NEED_SHARDS; ++q) e->need = std::max(e->need, e->h_tot[ncls + 1 + q]);
+    if (e->h_tot[ncls] == 0) break;
     if (round >= 2) { e->err = "class table did not converge"; return -5; }
     HIP_TRY(e, hipMemcpyAsync(e->h_sig, e->d_sig, n * 8, hipMemcpyDeviceToHost, s));
     HIP_TRY(e, hipStreamSynchronize(s));
@@ -1332,13 +1459,8 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   ++e->batch_calls;
   std::vector<uint32_t> offs, counts, cids;   // the classes present in this batch
-  for (uint32_t c = 0; c < ncls; ++c) {   // per-shard counts become the shards' offsets within the class
-    uint32_t total = 0;
-    for (uint32_t sh = 0; sh < shards; ++sh) {
-      const uint32_t cnt = e->h_ccount[(size_t)c * shards + sh];
-      e->h_ccount[(size_t)c * shards + sh] = total;
-      total += cnt;
-    }
+  for (uint32_t c = 0; c < ncls; ++c) {
+    const uint32_t total = e->h_tot[c];
     if (total) { cids.push_back(c); offs.push_back(e->cls_off[c]); counts.push_back(total); }
   }
   // Plans per wavefront and where their scheduler state lives.  A full batch keeps 64 plans per wavefront
@@ -1652,17 +1774,20 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   e->stats[6] = 0;
   if (n_sorted + n_solo == 0) return 0;
   if (int rc = ensure_perm(e, n_sorted + n_solo, (size_t)n_lane_waves + n_solo)) return rc;
-  uint32_t* const h_cfirst = e->h_ccount + (size_t)ncls * shards;   // behind the shard offsets
+  // the per-class tables of the layout: on the device behind the shard offsets (which k_hand_counts left there), from
+  // a sixteen-byte boundary on
+  const size_t tab0 = ((size_t)ncls * shards + 1 + 3) & ~size_t(3);
+  uint32_t* const h_cfirst = e->h_ccount + tab0;
   uint32_t* const h_clpw = h_cfirst + ncls;
   uint32_t* const h_coff = h_clpw + ncls;
-  const uint32_t* const d_cfirst = e->d_ccount + (size_t)ncls * shards;
+  const uint32_t* const d_cfirst = e->d_ccount + tab0;
   const uint32_t* const d_clpw = d_cfirst + ncls;
   const uint32_t* const d_coff = d_clpw + ncls;
   // tasks of one plan get their class from the scatter kernel, not from the host: with one plan per wavefront
   // throughout that is every task of the launch, otherwise the tasks of the classes taken out of the main kernel
   const uint32_t n_host_tasks = one ? 0u : n_lane_waves;
   // their class offsets ride behind the per-class tables when the block has room, else in a copy of their own
-  const size_t block_words = (size_t)ncls * shards + 3 * (size_t)ncls;
+  const size_t block_words = tab0 + 3 * (size_t)ncls;
   const bool tasks_in_block = block_words + n_host_tasks <= 4 * (size_t)e->ccap + COUNT_SLOTS;
   uint32_t* const h_tasks = tasks_in_block ? e->h_ccount + block_words : e->h_cls;
   for (size_t c = 0; c < counts.size(); ++c) {
@@ -1691,12 +1816,28 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     }
   }
   if (int rc = ensure_pool(e, s)) return rc;
-  HIP_TRY(e, hipMemcpyAsync(e->d_ccount, e->h_ccount, (block_words + (tasks_in_block ? n_host_tasks : 0u)) * 4, hipMemcpyHostToDevice, s));
-  if (n_host_tasks && !tasks_in_block) HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, (size_t)n_host_tasks * 4, hipMemcpyHostToDevice, s));
-  if (!one && n_sorted)   // with one plan per wavefront every entry is written by the scatter
-    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_sorted + blk - 1) / blk)), dim3(blk), 0, s, e->d_perm, n_sorted, IDLE_LANE);
+  // (with `ahead`, the layout goes up and the plans are dealt to their tasks on k_quad's stream, right behind the
+  // cost-model launch; the host has seen the counts, so all that the upload and the scatter read or overwrite is at
+  // rest)
+  if (ahead && (one || !prologue_done || !peaks_deferred)) {   // (not the call that was foreseen: back to the caller's stream)
+    HIP_TRY(e, hipStreamSynchronize(e->s3));
+    ahead = false;
+  }
+  const hipStream_t sl = ahead ? e->s3 : s;
+  const uint64_t n_idle = !one ? n_sorted : 0;   // with one plan per wavefront every entry is written by the scatter
+  if (e->h_ccount_dev && (tasks_in_block || !n_host_tasks)) {
+    const uint64_t n_quads = (block_words - tab0 + (tasks_in_block ? n_host_tasks : 0u) + 3) / 4;
+    const uint64_t threads = std::max<uint64_t>(n_quads, n_idle);
+    hipLaunchKernelGGL(k_upload_fill, dim3((unsigned)((threads + blk - 1) / blk)), dim3(blk), 0, sl, (const uint4*)(e->h_ccount_dev + tab0),
+                       (uint4*)(e->d_ccount + tab0), n_quads, e->d_perm, n_idle, IDLE_LANE);
+  } else {
+    HIP_TRY(e, hipMemcpyAsync(e->d_ccount + tab0, e->h_ccount + tab0, (block_words - tab0 + (tasks_in_block ? n_host_tasks : 0u)) * 4, hipMemcpyHostToDevice, sl));
+    if (n_host_tasks && !tasks_in_block) HIP_TRY(e, hipMemcpyAsync(e->d_cls, e->h_cls, (size_t)n_host_tasks * 4, hipMemcpyHostToDevice, sl));
+    if (n_idle)
+      hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_idle + blk - 1) / blk)), dim3(blk), 0, sl, e->d_perm, n_idle, IDLE_LANE);
+  }
   const auto t_laid = std::chrono::steady_clock::now();
-  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
+  hipLaunchKernelGGL(k_scatter, dim3(nblk), dim3(blk), 0, sl, n, e->d_cid, e->d_kidx, d_cfirst, d_clpw, e->d_ccount, shards, e->d_perm, pstride,
                      d_coff, e->d_cls + n_host_tasks, one ? 0u : (uint32_t)n_sorted, e->d_queues, e->d_limit);
   HIP_TRY(e, hipGetLastError());
 
@@ -1785,27 +1926,26 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   e->stats[4] = wsb * grid;
   e->stats[5] = one ? 1u : (uint64_t)ls;
   e->stats[6] = n_solo;
-  if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
   // The main kernel is submitted first: it needs 26 KB of LDS per wavefront, and once single-plan wavefronts
   // fill a compute unit its wavefronts only fit in as those retire.
   // The memory-model launch, where it was deferred: on k_quad's stream when that kernel has nothing to do in this call
-  // (the launch then runs beside all scheduling kernels), else behind the main kernel on the caller's stream, where
-  // it runs beside the tails of the two other kernels.
+  // (the launch then runs beside all scheduling kernels), else behind the main kernel, where it runs beside the tails
+  // of the two other kernels.
+  // With the layout ahead on k_quad's stream, that stream and the caller's change places until the join: the main
+  // kernel follows the scatter in order (it starts first, as it must: the kernels of the two other streams see the
+  // fork event a few microseconds later), and k_quad follows the cost-model launch on the caller's stream.
   const bool peaks_aside = peaks_deferred && !n_quad_waves;
-  if (n_solo || n_quad_waves || peaks_aside) {
-    if (!e->s2) {
-      if (int rc = side_streams(e, &e->s2, nullptr)) return rc;
-      HIP_TRY(e, hipEventCreateWithFlags(&e->ev_fork, hipEventDisableTiming));
-      HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join, hipEventDisableTiming));
-    }
-    if ((n_quad_waves || peaks_aside) && !e->s3) {
-      if (int rc = side_streams(e, nullptr, &e->s3)) return rc;
-      HIP_TRY(e, hipEventCreateWithFlags(&e->ev_join3, hipEventDisableTiming));
-    }
-    // (the three launches back to back: every call between them delays the start of the later kernels)
+  const hipStream_t sm = ahead ? e->s3 : s;    // the main kernel and what follows it
+  hipStream_t sq = ahead ? s : e->s3;          // k_quad, or the memory-model launch in its place
+  if (ahead) {
+    HIP_TRY(e, hipEventRecord(e->ev_fork, e->s3));   // (cost-model launch, layout and scatter are done)
+  } else if (n_solo || n_quad_waves || peaks_aside) {
+    if (int rc = ensure_side(e)) return rc;
+    sq = e->s3;
     HIP_TRY(e, hipEventRecord(e->ev_fork, s));
-    if (n_quad_waves || peaks_aside) HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
-    if (n_solo) HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
+    if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
+  } else if (e->timing) {
+    HIP_TRY(e, hipEventRecord(e->ev0, s));
   }
   auto launch_quad = [&]() -> int {   // the four-lanes-per-plan wavefronts, beside the main kernel
     if (!n_quad_waves) return 0;
@@ -1821,29 +1961,38 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       HIP_TRY(e, hipFuncSetAttribute((const void*)k_quad, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       e->quad_attr_set = true;
     }
-    hipLaunchKernelGGL(k_quad, dim3((unsigned)std::min<uint64_t>(n_quad_waves, (uint64_t)e->n_cu * 16)), dim3(WAVE), qlds, e->s3, Q);
+    hipLaunchKernelGGL(k_quad, dim3((unsigned)std::min<uint64_t>(n_quad_waves, (uint64_t)e->n_cu * 16)), dim3(WAVE), qlds, sq, Q);
     HIP_TRY(e, hipGetLastError());
     return 0;
   };
   auto launch_main = [&]() {
     if (n_waves == 0) {
-    } else if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, s, L);
+    } else if (one) hipLaunchKernelGGL(k_plan, dim3(grid), dim3(WAVE), lds, sm, L);
     else switch (ls) {
-      case 0: hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds, s, L); break;
-      case 8: hipLaunchKernelGGL(k_eval<8>, dim3(grid), dim3(WAVE), lds, s, L); break;
-      case 16: hipLaunchKernelGGL(k_eval<16>, dim3(grid), dim3(WAVE), lds, s, L); break;
-      case 32: hipLaunchKernelGGL(k_eval<32>, dim3(grid), dim3(WAVE), lds, s, L); break;
-      default: hipLaunchKernelGGL(k_eval<64>, dim3(grid), dim3(WAVE), lds, s, L); break;
+      case 0: hipLaunchKernelGGL(k_eval<0>, dim3(grid), dim3(WAVE), lds, sm, L); break;
+      case 8: hipLaunchKernelGGL(k_eval<8>, dim3(grid), dim3(WAVE), lds, sm, L); break;
+      case 16: hipLaunchKernelGGL(k_eval<16>, dim3(grid), dim3(WAVE), lds, sm, L); break;
+      case 32: hipLaunchKernelGGL(k_eval<32>, dim3(grid), dim3(WAVE), lds, sm, L); break;
+      default: hipLaunchKernelGGL(k_eval<64>, dim3(grid), dim3(WAVE), lds, sm, L); break;
     }
     return hipGetLastError();
   };
   // (The main kernel first also when k_plan has only a handful of tasks, which then wait until wavefronts of the main
   // kernel retire: with those few in front the step was 30 us longer on config 4.)
   HIP_TRY(e, launch_main());
+  // (the three launches back to back: every call between them delays the start of the later kernels)
+  const bool side_q = n_quad_waves || peaks_aside;
+  if (ahead) {
+    HIP_TRY(e, hipStreamWaitEvent(s, e->ev_fork, 0));
+    if (e->timing) HIP_TRY(e, hipEventRecord(e->ev0, s));
+  } else if (side_q) {
+    HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_fork, 0));
+  }
   // (k_quad second: measured against k_quad first, 0.50 against 0.52-0.53 ms on config 2, and against k_quad last,
   // 0.59 ms; its wavefronts need the most LDS after the main kernel's)
   if (int rc = launch_quad()) return rc;
   if (n_solo) {   // the single-plan wavefronts, beside the main kernel
+    HIP_TRY(e, hipStreamWaitEvent(e->s2, e->ev_fork, 0));
     EvalLaunch S = L;
     S.queue = nullptr;
     S.perm = e->d_perm + n_sorted;
@@ -1856,10 +2005,9 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   if (peaks_deferred) {
     const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
-    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, peaks_aside ? e->s3 : s, G);
+    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, peaks_aside ? sq : sm, G);
     HIP_TRY(e, hipGetLastError());
   }
-  if (n_quad_waves || peaks_aside) HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
   if (n_solo) HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));
   // (after the submission of k_plan, which is the longer of the two kernels and should not wait for this one)
   if (short_list && n_waves) {   // the plans whose ready list outgrew the short one, with the full one
@@ -1874,10 +2022,14 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       e->lds_attr_set[0] = true;
     }
     // a small grid: the launch almost always finds the count of flagged plans at zero and ends at once
-    hipLaunchKernelGGL(k_eval<0>, dim3(std::min<unsigned>(grid, (unsigned)e->n_cu * 2u)), dim3(WAVE), lds_full, s, F);
+    hipLaunchKernelGGL(k_eval<0>, dim3(std::min<unsigned>(grid, (unsigned)e->n_cu * 2u)), dim3(WAVE), lds_full, sm, F);
     HIP_TRY(e, hipGetLastError());
   }
-  if (n_quad_waves || peaks_aside) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join3, 0));
+  if (ahead || side_q) {   // whatever ran on k_quad's stream
+    HIP_TRY(e, hipEventRecord(e->ev_join3, e->s3));
+    HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join3, 0));
+    ahead_join.joined = true;
+  }
   if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
   if (peaks_deferred) {   // (before k_eval_limit, whose plans get their final outputs from that kernel itself)
     hipLaunchKernelGGL(k_finish, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_aux_pen, e->d_aux_mask, flags, score, mask);
