@@ -476,6 +476,13 @@ int rpeg_engine_set_split_model(rpeg_engine_t* e, const double* values, int32_t 
    counterpart of this setting). */
 int rpeg_engine_set_sa_groups(rpeg_engine_t* e, int32_t groups);
 
+/* on = 1 (default): in a full batched call the cost-model launch, the layout of the batch and the main scheduling
+   kernel follow each other on the device's second side stream, from the moment the class ids are written, while the
+   caller's stream hands the class totals to the host -- unless another engine of the process is in the middle of a
+   call on the side streams.  on = 0: all of it on the caller's stream.  A measurement aid: results do not depend on
+   it.  No counterpart in the reference. */
+int rpeg_engine_set_side_layout(rpeg_engine_t* e, int32_t on);
+
 /* With lanes = -1 and a batch that fills the chip in one round of wavefronts: the largest share of the batch's
    plans, in percent, that the four-lanes-per-plan kernel may take on a stream of its own (default 25; 0: none).
    Which classes it takes is learned: the main kernel records, per class, how long its slowest wavefront ran and how

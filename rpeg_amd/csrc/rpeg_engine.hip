@@ -113,16 +113,16 @@ constexpr int HAND_BLOCK = 1024;
 __global__ __launch_bounds__(HAND_BLOCK) void k_hand_counts(uint32_t* __restrict__ count, const uint32_t* __restrict__ need, uint32_t n_classes,
                                                             uint32_t shards, uint32_t* __restrict__ host_count, uint32_t* __restrict__ host_flag,
                                                             uint32_t tag) {
+  // the totals first, and on their way to the host before anything else is written
   for (uint32_t c = threadIdx.x; c < n_classes; c += HAND_BLOCK) {
-    uint32_t* row = count + (size_t)c * shards;
+    const uint32_t* row = count + (size_t)c * shards;
     uint32_t total = 0;
-    for (uint32_t s0 = 0; s0 < shards; s0 += 8) {   // eight loads in flight
-      uint32_t v[8];
+    for (uint32_t s0 = 0; s0 < shards; s0 += 16) {   // sixteen loads in flight
+      uint32_t v[16];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = s0 + u < shards ? row[s0 + u] : 0u;
+      for (int u = 0; u < 16; ++u) v[u] = s0 + u < shards ? row[s0 + u] : 0u;
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (s0 + u < shards) { row[s0 + u] = total; total += v[u]; }
+      for (int u = 0; u < 16; ++u) total += v[u];
     }
     host_count[c] = total;
   }
@@ -131,6 +131,19 @@ __global__ __launch_bounds__(HAND_BLOCK) void k_hand_counts(uint32_t* __restrict
   __threadfence_system();
   __syncthreads();
   if (threadIdx.x == 0) __hip_atomic_store(host_flag, tag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  // then the shards' counters become their offsets within the class (for the kernels that follow on the device)
+  for (uint32_t c = threadIdx.x; c < n_classes; c += HAND_BLOCK) {
+    uint32_t* row = count + (size_t)c * shards;
+    uint32_t total = 0;
+    for (uint32_t s0 = 0; s0 < shards; s0 += 16) {
+      uint32_t v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = s0 + u < shards ? row[s0 + u] : 0u;
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (s0 + u < shards) { row[s0 + u] = total; total += v[u]; }
+    }
+  }
 }
 
 // Integer validity gate, class signature, class id (open-addressing table of the classes lowered so far)
@@ -1128,6 +1141,12 @@ int rpeg_engine_set_split_model(rpeg_engine_t* e, const double* values, int32_t 
   return 0;
 }
 
+int rpeg_engine_set_side_layout(rpeg_engine_t* e, int32_t on) {
+  if (!e) return -1;
+  e->layout_ahead = on != 0;
+  return 0;
+}
+
 int rpeg_engine_set_sa_groups(rpeg_engine_t* e, int32_t groups) {
   if (!e) return -1;
   if (groups < 1 || groups > 8) { e->err = "1 to 8 groups of chains"; return -1; }
@@ -1409,20 +1428,24 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
                        e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
                        e->d_kidx, e->d_ccount, ncls, shards);
     HIP_TRY(e, hipGetLastError());
-    if (round == 0 && ahead) {   // (before the hand-over: the cost-model launch does not wait for that)
+    // Cost model, memory model and gates of every plan: they need the verdict of the gate (which plans to skip) and
+    // nothing of the classes, so they run behind the signature kernel while the host waits for the counts (their
+    // flag, not the stream) and lays the batch out.  On k_quad's stream the launch goes out first: it does not wait for
+    // the hand-over of the counts, and the hand-over has a few microseconds to spare.
+    if (round == 0 && ahead) {
       HIP_TRY(e, hipEventRecord(e->ev_sig, s));
       HIP_TRY(e, hipStreamWaitEvent(e->s3, e->ev_sig, 0));
+      if (int rc = launch_prologue(true)) return rc;
     }
     hipLaunchKernelGGL(k_hand_counts, dim3(1), dim3(HAND_BLOCK), 0, s, e->d_ccount, e->d_need, ncls, shards, e->h_tot_dev, e->h_sigflag_dev, tag);
     HIP_TRY(e, hipGetLastError());
     if (read_stat) HIP_TRY(e, hipMemcpyAsync(e->cls_pops16.data(), e->d_cstat, (size_t)ncls * 4, hipMemcpyDeviceToHost, s));
     if (round == 0) {
-      // Cost model, memory model and gates of every plan: they need the verdict of the gate (which plans to skip)
-      // and nothing of the classes, so they run behind the signature kernel while the host waits for the counts
-      // (the flag or the event, not the stream) and lays the batch out.
-      if (!e->ev_counts) HIP_TRY(e, hipEventCreateWithFlags(&e->ev_counts, hipEventDisableTiming));
-      HIP_TRY(e, hipEventRecord(e->ev_counts, s));
-      if (!own_prologue)
+      if (!handed) {   // (the copy of the statistic has to be waited for: an event, so that the wait leaves the launch below alone)
+        if (!e->ev_counts) HIP_TRY(e, hipEventCreateWithFlags(&e->ev_counts, hipEventDisableTiming));
+        HIP_TRY(e, hipEventRecord(e->ev_counts, s));
+      }
+      if (!own_prologue && !ahead)
         if (int rc = launch_prologue(true)) return rc;
       t_counts = std::chrono::steady_clock::now();
       bool seen = false;
@@ -1436,7 +1459,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
 #endif
         }
       }
-      if (!seen) HIP_TRY(e, hipEventSynchronize(e->ev_counts));
+      if (!seen) {
+        if (handed) HIP_TRY(e, hipStreamSynchronize(s));
+        else HIP_TRY(e, hipEventSynchronize(e->ev_counts));
+      }
       t_waited = std::chrono::steady_clock::now();
     } else {
       HIP_TRY(e, hipStreamSynchronize(s));

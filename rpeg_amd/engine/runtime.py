@@ -23,7 +23,7 @@ _lib = None
 EXPORTS = ("rpeg_engine_create", "rpeg_engine_destroy", "rpeg_last_error", "rpeg_eval_batch",
            "rpeg_op_time_batch", "rpeg_eval_trace", "rpeg_engine_stats", "rpeg_engine_set_timing",
            "rpeg_engine_last_kernel_ms", "rpeg_device_exp", "rpeg_engine_reset_classes", "rpeg_eval_batch_mass",
-           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_sa_groups", "rpeg_engine_host_us", "rpeg_engine_set_split_model", "rpeg_engine_set_quad_share", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
+           "rpeg_sa_run", "rpeg_sa_propose", "rpeg_eval_host_util", "rpeg_engine_set_state_lanes", "rpeg_engine_set_sa_groups", "rpeg_engine_set_side_layout", "rpeg_engine_host_us", "rpeg_engine_set_split_model", "rpeg_engine_set_quad_share", "rpeg_engine_set_ready_cap", "rpeg_engine_profile", "rpeg_sa_optimize", "rpeg_eval_host",
            "rpeg_sa_optimize_families", "rpeg_eval_trace_metrics", "rpeg_eval_batch_static", "rpeg_plan_detail",
            "rpeg_lower_plan")
 
@@ -89,6 +89,8 @@ def load_library(path: Optional[str] = None):
     lib.rpeg_engine_set_split_model.argtypes = [vp, vp, i32]
     lib.rpeg_engine_set_sa_groups.restype = C.c_int
     lib.rpeg_engine_set_sa_groups.argtypes = [vp, i32]
+    lib.rpeg_engine_set_side_layout.restype = C.c_int
+    lib.rpeg_engine_set_side_layout.argtypes = [vp, i32]
     lib.rpeg_engine_set_quad_share.restype = C.c_int
     lib.rpeg_engine_set_quad_share.argtypes = [vp, i32]
     lib.rpeg_engine_set_ready_cap.restype = C.c_int
@@ -228,6 +230,10 @@ class Engine:
     def set_sa_groups(self, groups: int):
         """Groups of chains (1..8) whose evaluations overlap the host's work on the others in `sa_run`."""
         self._check(self.lib.rpeg_engine_set_sa_groups(self._h, int(groups)), "rpeg_engine_set_sa_groups")
+
+    def set_side_layout(self, on: bool):
+        """Cost-model launch, layout and main kernel of a full batch on a side stream (default) or on the caller's."""
+        self._check(self.lib.rpeg_engine_set_side_layout(self._h, 1 if on else 0), "rpeg_engine_set_side_layout")
 
     def set_quad_share(self, percent: int):
         """Percentage of a full batch that the four-lanes-per-plan kernel takes beside the main kernel (0: none)."""

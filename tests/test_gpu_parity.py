@@ -447,6 +447,57 @@ def test_the_fitted_figures_of_the_split_move_plans_between_kernels_and_no_bit()
     eng.close()
 
 
+@pytest.mark.parametrize("c,n", [(2, 65536), (4, 200000), (3, 50000)])
+def test_the_stream_that_carries_the_layout_changes_no_bit(c, n):
+    """rpeg_engine_set_side_layout: cost-model launch, layout and main kernel on the side stream (the default) or on
+    the caller's; cold calls (classes lowered, several rounds) and warm ones; two engines that step in turn on two
+    threads, of which the one that finds the side streams taken stays on its own; a batch that no plan of is valid.
+    Every call equals the host build."""
+    import threading
+    from rpeg_amd.engine.runtime import Engine
+    cfg, batch = seeded_batch(c, n)
+    ref = CpuPort(cfg.problem).eval(batch, flags=abi.GATE_STALE, threads=16)
+
+    def check(out, what):
+        assert np.array_equal(out["mask"], ref["mask"]), what
+        for k in ("makespan", "peak", "score"):
+            assert same_bits(out[k], ref[k]), (what, k)
+
+    for on in (True, False):
+        eng = Engine(cfg.problem)
+        eng.set_side_layout(on)
+        try:
+            for call in range(3):
+                check(eng.eval(batch, gate_stale=True), (on, call))
+            bad = batch.slice(0, 30000)
+            bad.vert[0, :] = 0   # dp = 0 in every plan: the gate rejects the whole batch
+            out = eng.eval(bad, gate_stale=True)
+            assert not out["mask"].any() and np.all(np.isnan(out["score"]))
+            check(eng.eval(batch, gate_stale=True), (on, "after a batch without a valid plan"))
+        finally:
+            eng.close()
+    engines = [Engine(cfg.problem) for _ in range(2)]
+    errors = []
+
+    def work(eng, who):
+        try:
+            for call in range(4):
+                check(eng.eval(batch, gate_stale=True), ("two engines", who, call))
+        except Exception as exc:   # noqa: BLE001 - handed to the main thread
+            errors.append(exc)
+
+    try:
+        threads = [threading.Thread(target=work, args=(e, k)) for k, e in enumerate(engines)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not errors, errors
+    finally:
+        for e in engines:
+            e.close()
+
+
 @pytest.mark.parametrize("c,n,what", [(3, 65536, "single_plan_tasks"), (5, 40000, "quad_tasks"), (2, 131072, "quad_tasks"),
                                       (1, 20000, "single_plan_tasks"), (3, 32768, "single_plan_tasks"), (2, 20000, "single_plan_tasks")])
 def test_the_measured_split_changes_where_classes_run_and_not_one_bit(c, n, what):
