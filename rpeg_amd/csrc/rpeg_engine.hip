@@ -358,9 +358,13 @@ __global__ __launch_bounds__(WAVE) void k_peaks(const PrologueLaunch L) {
 // The verdicts of the memory-model launch put into the outputs of the scheduling kernels, where that launch ran beside
 // them instead of ahead of them: the gate bits of the mask, the soft OOM penalty and the stale-layout gate of the
 // score (evaluate.py:372-374, 396-401), the same operations in the same order as the scheduling kernels apply them.
+// (It also clears the class counters for the signature kernel of the engine's next call, which then starts without a
+// launch of its own for that: zero_n words at zero_p.)
 __global__ void k_finish(uint64_t n, const uint32_t* __restrict__ cid, const double* __restrict__ pen,
-                         const uint8_t* __restrict__ gates, uint32_t flags, double* __restrict__ score, uint8_t* __restrict__ mask) {
+                         const uint8_t* __restrict__ gates, uint32_t flags, double* __restrict__ score, uint8_t* __restrict__ mask,
+                         uint32_t* __restrict__ zero_p, uint32_t zero_n) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (uint64_t j = i; j < zero_n; j += (uint64_t)gridDim.x * blockDim.x) zero_p[j] = 0u;
   if (i >= n || cid[i] == KPRO_INVALID) return;   // (a plan the gate rejected has its outputs from k_signature)
   const uint8_t g = gates[i];
   const bool stale_ok = (g & RPEG_MASK_STALE_OK) != 0, mem_ok = (g & RPEG_MASK_MEM_OK) != 0;
@@ -667,6 +671,8 @@ struct rpeg_engine_s {
   // per-class tables of a call, one block on each side: counters per (class, shard), which become the shards'
   // offsets, then first wavefront and plans per wavefront of every class
   uint32_t *d_ccount = nullptr, *h_ccount = nullptr;
+  uint64_t count_clean = 0;                     // leading words of d_ccount that the last call left at zero,
+  hipStream_t count_clean_on = nullptr;         // on this stream
   uint32_t* h_ccount_dev = nullptr;             // the same pinned buffer as the device addresses it
   uint32_t *h_tot = nullptr, *h_tot_dev = nullptr;   // pinned: per-class totals of a call, written by k_hand_counts
   uint32_t *h_sigflag = nullptr, *h_sigflag_dev = nullptr;   // pinned word: the tag of the call whose counters are in h_ccount
@@ -823,6 +829,7 @@ static int ensure_class_tables(rpeg_engine_t* e, hipStream_t s) {
       hipHostFree(e->h_ccount);
     }
     e->d_ccount = nullptr; e->ccap = 0;
+    e->count_clean = 0;
     HIP_TRY(e, hipMalloc(&e->d_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4));
     // (the signature kernel writes the counters here itself while the host polls: coherent, and mapped)
     HIP_TRY(e, hipHostMalloc(&e->h_ccount, (4 * (size_t)cap + COUNT_SLOTS + 64) * 4, hipHostMallocCoherent));
@@ -1423,7 +1430,10 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
       ahead = !e->prof_on && e->layout_ahead && side_claim(e);
     }
     if (round > 0 && ahead) HIP_TRY(e, hipStreamSynchronize(e->s3));   // (the cost-model launch reads the class ids)
-    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_count + blk - 1) / blk)), dim3(blk), 0, s, e->d_ccount, n_count, 0u);
+    // (clear already where the launch that ended the engine's last call did it)
+    if (e->count_clean < n_count || e->count_clean_on != s)
+      hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n_count + blk - 1) / blk)), dim3(blk), 0, s, e->d_ccount, n_count, 0u);
+    e->count_clean = 0;
     hipLaunchKernelGGL(k_signature, dim3((unsigned)((n + SIG_BLOCK - 1) / SIG_BLOCK)), dim3(SIG_BLOCK), 0, s, e->dP, n, plans->vert, plans->head, plans->stride,
                        e->d_sig, makespan, peak, score, mask, mass, e->d_hkey, e->d_hval, e->hcap - 1, e->d_cid,
                        e->d_kidx, e->d_ccount, ncls, shards);
@@ -2058,8 +2068,12 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   if (n_solo) HIP_TRY(e, hipStreamWaitEvent(s, e->ev_join, 0));
   if (peaks_deferred) {   // (before k_eval_limit, whose plans get their final outputs from that kernel itself)
-    hipLaunchKernelGGL(k_finish, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_aux_pen, e->d_aux_mask, flags, score, mask);
+    // (the layout tables in the counters' buffer have been read by now: the counters of the next call are cleared here)
+    const uint32_t zero_n = (uint32_t)std::min<size_t>(std::max<size_t>((size_t)COUNT_SLOTS, ncls) + 1, 4 * (size_t)e->ccap + COUNT_SLOTS);
+    hipLaunchKernelGGL(k_finish, dim3(nblk), dim3(blk), 0, s, n, e->d_cid, e->d_aux_pen, e->d_aux_mask, flags, score, mask, e->d_ccount, zero_n);
     HIP_TRY(e, hipGetLastError());
+    e->count_clean = zero_n;
+    e->count_clean_on = s;
   }
   if (bounded) {   // the plans flagged by the kernels above, without a bound on the ready set (ends at once when there is none)
     EvalLaunch U = L;
