@@ -167,8 +167,10 @@ const char* rpeg_last_error(const rpeg_engine_t* e);
    makespan: Trace.makespan() (trace.py:31-38); peak: largest per-device peak in bytes
    (memory.py:608-841); score: throughput times the soft OOM penalty (evaluate.py:288, 396-401);
    mask: RPEG_MASK_* bits.  All four are device arrays of n elements; any may be NULL.
-   `stream` is a hipStream_t (NULL = default stream).  The call is synchronous with respect to
-   the host only where it must read back the list of new lowering classes. */
+   `stream` is a hipStream_t (NULL = default stream).  The call waits for the host once, for the per-class totals
+   of the batch (a few microseconds behind the kernel that writes the class ids), and again only where it must read
+   back the list of new lowering classes; the evaluation kernels are left running on `stream`.  Successive calls on
+   one engine use one stream, or the caller orders them. */
 int rpeg_eval_batch(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* plans, uint32_t flags,
                     double* makespan, double* peak, double* score, uint8_t* mask, void* stream);
 
@@ -440,9 +442,9 @@ int rpeg_sa_propose(rpeg_engine_t* e, const rpeg_sa_params_t* prm, int32_t what,
 int rpeg_engine_stats(const rpeg_engine_t* e, uint64_t* out, int32_t n);
 
 /* Host time of the last rpeg_eval_batch call that laid its batch out, in microseconds of the steady clock: [0] from
-   the call to the end of the launches behind the gate (signature kernel, copies of the counts, cost-model launch),
-   [1] the wait for the class counts, [2] the layout of the batch, the split between the kernels and the copy of the
-   tables, [3] scatter, fork, the scheduling launches, join and the launches that end the call.  A measurement aid with
+   the call to the end of the launches up to the wait (signature kernel, cost-model launch, hand-over of the class
+   totals), [1] the wait for the class totals, [2] the layout of the batch and the split between the kernels,
+   [3] tables up, scatter, fork, the scheduling launches, join and the launches that end the call.  A measurement aid with
    no counterpart in the reference. */
 int rpeg_engine_host_us(const rpeg_engine_t* e, double* out, int32_t n);
 

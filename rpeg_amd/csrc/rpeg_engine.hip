@@ -715,7 +715,7 @@ struct rpeg_engine_s {
   uint32_t max_v = RPEG_MAX_V;   // largest vertex count of the problem's structures
   hipStream_t s2 = nullptr;                     // second stream: single-plan wavefronts of a large batch run beside the others
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
-  hipEvent_t ev_counts = nullptr;               // the class counts of a call have reached the host
+  hipEvent_t ev_counts = nullptr;               // the statistic of a call has reached the host (the calls that read it)
   hipStream_t s3 = nullptr;                     // third stream: the four-lanes-per-plan wavefronts (k_quad)
   hipEvent_t ev_join3 = nullptr;
   hipEvent_t ev_sig = nullptr;                  // the signature kernel of a call is done (its class ids are there)

@@ -11,8 +11,8 @@
 // it is -- so every slot a class of the plan's structure COULD have (slot_universe) is evaluated, and a class picks
 // its own through ClassView::umap --, and the vertex order that fixes the memory model's float sums follows from the
 // plan (plan_vorder).  Both launches therefore run on the plans in the caller's own order, straight from the
-// caller's tensors (coalesced), right behind the signature kernel: while the host reads the class counts back and
-// lays the batch out, i.e. off the critical path of the call.
+// caller's tensors (coalesced), right behind the signature kernel: while the class totals are on their way to the
+// host, which lays the batch out, i.e. off the critical path of the call.
 //
 //   k_prologue   one wavefront per (64 plans, row); a row is one slot of the universe, or the pair relations, or one
 //                vertex's memory terms -- a wavefront holds one short piece of arithmetic, so that many are resident
