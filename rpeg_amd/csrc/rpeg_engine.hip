@@ -338,9 +338,13 @@ __global__ __launch_bounds__(WAVE) void k_prologue(const PrologueLaunch L) {
   }
 }
 
+// (LDS by the problem's largest vertex count, kpeaks_lds_bytes: beside a resident main kernel the blocks of this launch
+// get what LDS that kernel leaves, and with the 12.8 KB of six vertices a DPO batch of three had half as many of them)
+static size_t kpeaks_lds_bytes(uint32_t max_v) { return (size_t)max_v * 4 * WAVE * 8 + 8 * WAVE; }
 __global__ __launch_bounds__(WAVE) void k_peaks(const PrologueLaunch L) {
-  __shared__ double l_vm[RPEG_MAX_V * 4 * WAVE];
-  __shared__ uint8_t l_ord[8 * WAVE];
+  extern __shared__ double kpk_lds[];
+  double* l_vm = kpk_lds;                                        // [vertex * 4 + field][lane]
+  uint8_t* l_ord = (uint8_t*)(kpk_lds + (size_t)L.max_v * 4 * WAVE);   // [position][lane]
   const uint64_t i = (uint64_t)blockIdx.x * WAVE + threadIdx.x;
   const bool active = i < L.n && L.cid[i] != KPRO_INVALID;
   PlanHead h;
@@ -1391,13 +1395,14 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
     G.uni = e->d_uni;
     for (int q = 0; q < RPEG_MAX_STRUCT; ++q) G.n_uni[q] = e->n_uni[q];
     G.max_uni = e->max_uni;
+    G.max_v = e->max_v;
     G.dur = e->d_dur; G.dur_stride = e->cap_n;
     G.aux_ovl = e->d_aux_ovl; G.aux_eq = e->d_aux_eq; G.aux_dpne = e->d_aux_dpne; G.vm = e->d_vm;
     G.aux_pen = e->d_aux_pen; G.aux_mask = e->d_aux_mask;
     G.peak = peak;
     const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
     hipLaunchKernelGGL(k_prologue, dim3(pblk, KPRO_PARTS), dim3(WAVE), 0, ahead ? e->s3 : s, G);
-    if (!defer) hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, s, G);
+    if (!defer) hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), kpeaks_lds_bytes(e->max_v), s, G);
     HIP_TRY(e, hipGetLastError());
     prologue_done = true;
     peaks_deferred = defer;
@@ -2041,7 +2046,7 @@ static int eval_batch_impl(rpeg_engine_t* e, uint64_t n, const rpeg_plan_soa_t* 
   }
   if (peaks_deferred) {
     const unsigned pblk = (unsigned)((n + WAVE - 1) / WAVE);
-    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), 0, peaks_aside ? sq : sm, G);
+    hipLaunchKernelGGL(k_peaks, dim3(pblk), dim3(WAVE), kpeaks_lds_bytes(e->max_v), peaks_aside ? sq : sm, G);
     HIP_TRY(e, hipGetLastError());
   }
   if (n_solo) HIP_TRY(e, hipEventRecord(e->ev_join, e->s2));

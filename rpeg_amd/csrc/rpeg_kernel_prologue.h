@@ -43,6 +43,7 @@ struct PrologueLaunch {
   const SlotDesc* uni;         // [structure][RPEG_MAX_UNIVERSE]
   uint32_t n_uni[RPEG_MAX_STRUCT];
   uint32_t max_uni;            // rows of the grid: max_uni durations, one row of pair relations, then one per vertex
+  uint32_t max_v;              // largest vertex count of the problem's structures (sizes the LDS of the second launch)
   double* dur;
   uint64_t dur_stride;         // plans per row of dur and vm
   uint64_t* aux_ovl;
